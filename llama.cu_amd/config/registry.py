@@ -1,0 +1,51 @@
+"""One registry from an architecture's name (config.json's ``architectures[0]``) to
+its configuration class and to the function that lays its model out of parts.
+
+The reference switches on the architecture name in code
+(llama.cu/src/model/mod.rs:62-67: ``"llama"``, ``"qwen2"``, else panic); here the
+switch is a table that anyone may add to.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Any, Callable, Dict, List
+
+from .base import ConfigError, read_config_json
+
+
+@dataclass(frozen=True)
+class Architecture:
+    name: str
+    config_from_dict: Callable[[Dict[str, Any]], Any]   # dict of config.json -> typed configuration
+    build_spec: Callable[[Any], Any]                    # typed configuration -> parts.ModelSpec
+
+
+_REGISTRY: Dict[str, Architecture] = {}
+
+
+def register_architecture(name: str, config_from_dict, build_spec, replace: bool = False) -> None:
+    if name in _REGISTRY and not replace:
+        raise ValueError(f"architecture {name!r} is already registered")
+    _REGISTRY[name] = Architecture(name, config_from_dict, build_spec)
+
+
+def registered_architectures() -> List[str]:
+    return sorted(_REGISTRY)
+
+
+def architecture_of(data: Dict[str, Any], where: str = "config.json") -> Architecture:
+    names = data.get("architectures")
+    if not isinstance(names, list) or not names or not isinstance(names[0], str):
+        raise ConfigError(f"{where}: required key 'architectures' is missing or holds no name")
+    arch = _REGISTRY.get(names[0])
+    if arch is None:
+        raise ConfigError(f"{where}: architecture {names[0]!r} is not registered; "
+                          f"registered: {registered_architectures()}")
+    return arch
+
+
+def load_config(folder: str):
+    """(architecture, typed configuration) of a model folder."""
+    data = read_config_json(folder)
+    arch = architecture_of(data, where=f"{folder}/config.json")
+    return arch, arch.config_from_dict(data)

@@ -1,0 +1,69 @@
+// Shared device helpers for the gfx950 kernels: element types, conversions,
+// wave and block reductions.  A wave has 64 lanes.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#define LCU_API extern "C" __attribute__((visibility("default")))
+
+// Error codes returned by every entry point (0 = launched).
+enum { LCU_OK = 0, LCU_BAD_ARGUMENT = -1, LCU_UNSUPPORTED = -2 };
+
+// Element type codes shared with the Python side.
+enum { LCU_F32 = 0, LCU_BF16 = 1 };
+
+struct bf16_t {
+    uint16_t bits;
+};
+
+__device__ __forceinline__ float to_f32(float x) { return x; }
+__device__ __forceinline__ float to_f32(bf16_t x) { return __uint_as_float(((uint32_t)x.bits) << 16); }
+
+template <class T> __device__ __forceinline__ T from_f32(float x);
+template <> __device__ __forceinline__ float from_f32<float>(float x) { return x; }
+// round to nearest, ties to even; NaN stays NaN
+template <> __device__ __forceinline__ bf16_t from_f32<bf16_t>(float x) {
+    uint32_t u = __float_as_uint(x);
+    bf16_t r;
+    if ((u & 0x7fffffffu) > 0x7f800000u) {
+        r.bits = (uint16_t)((u >> 16) | 0x0040u);
+    } else {
+        u += 0x7fffu + ((u >> 16) & 1u);
+        r.bits = (uint16_t)(u >> 16);
+    }
+    return r;
+}
+
+constexpr int WAVE = 64;
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, WAVE);
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, WAVE));
+    return v;
+}
+
+// Sum over a block of up to 1024 threads; `scratch` holds 16 floats of LDS.  Every
+// thread gets the result.  The order of the additions depends on the block's size
+// only.
+__device__ __forceinline__ float block_sum(float v, float *scratch) {
+    v = wave_sum(v);
+    const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
+    const int nwaves = (blockDim.x + WAVE - 1) / WAVE;
+    __syncthreads();
+    if (lane == 0) scratch[wave] = v;
+    __syncthreads();
+    float t = 0.f;
+    for (int i = 0; i < nwaves; ++i) t += scratch[i];
+    return t;
+}
+
+#define LCU_LAUNCH_CHECK()                                   \
+    do {                                                     \
+        hipError_t e_ = hipGetLastError();                   \
+        if (e_ != hipSuccess) return (int)e_;                \
+    } while (0)

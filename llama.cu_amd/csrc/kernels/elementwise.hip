@@ -1,0 +1,168 @@
+// Row-wise kernels: embedding gather, row gather, RMS norm fused with the residual
+// sum, SwiGLU, residual add.  Sums, the norm and the activation are computed in
+// 32-bit whatever the storage type.
+#include "common.h"
+
+// ---------------------------------------------------------------- embedding gather
+// out[i, :] = table[ids[i], :].  An id outside the table writes NaN into the row
+// (the host checks ids before; this keeps a bad id from reading out of bounds).
+template <class TT, class TO>
+__global__ void embedding_gather_kernel(TO *__restrict__ out, const TT *__restrict__ table,
+                                        const int *__restrict__ ids, int d, int vocab) {
+    const int row = blockIdx.x;
+    const int id = ids[row];
+    TO *o = out + (size_t)row * d;
+    if (id < 0 || id >= vocab) {
+        for (int c = threadIdx.x; c < d; c += blockDim.x) o[c] = from_f32<TO>(__uint_as_float(0x7fc00000u));
+        return;
+    }
+    const TT *t = table + (size_t)id * d;
+    for (int c = threadIdx.x; c < d; c += blockDim.x) o[c] = from_f32<TO>(to_f32(t[c]));
+}
+
+LCU_API int lcu_embedding_gather(void *out, int out_type, const void *table, int table_type,
+                                 const int *ids, int n, int d, int vocab, hipStream_t stream) {
+    if (n <= 0) return LCU_OK;
+    if (d <= 0 || vocab <= 0) return LCU_BAD_ARGUMENT;
+    dim3 grid(n), block(256);
+#define GO(TT, TO) embedding_gather_kernel<TT, TO><<<grid, block, 0, stream>>>((TO *)out, (const TT *)table, ids, d, vocab)
+    if (table_type == LCU_F32 && out_type == LCU_F32) GO(float, float);
+    else if (table_type == LCU_BF16 && out_type == LCU_F32) GO(bf16_t, float);
+    else if (table_type == LCU_BF16 && out_type == LCU_BF16) GO(bf16_t, bf16_t);
+    else if (table_type == LCU_F32 && out_type == LCU_BF16) GO(float, bf16_t);
+    else return LCU_BAD_ARGUMENT;
+#undef GO
+    LCU_LAUNCH_CHECK();
+    return LCU_OK;
+}
+
+// ---------------------------------------------------------------- row gather
+template <class T>
+__global__ void gather_rows_kernel(T *__restrict__ out, const T *__restrict__ x,
+                                   const int *__restrict__ rows, int d, int n_src) {
+    const int r = rows[blockIdx.x];
+    T *o = out + (size_t)blockIdx.x * d;
+    if (r < 0 || r >= n_src) {
+        for (int c = threadIdx.x; c < d; c += blockDim.x) o[c] = from_f32<T>(__uint_as_float(0x7fc00000u));
+        return;
+    }
+    const T *s = x + (size_t)r * d;
+    for (int c = threadIdx.x; c < d; c += blockDim.x) o[c] = s[c];
+}
+
+LCU_API int lcu_gather_rows(void *out, const void *x, int type, const int *rows, int n_out, int d,
+                            int n_src, hipStream_t stream) {
+    if (n_out <= 0) return LCU_OK;
+    if (d <= 0) return LCU_BAD_ARGUMENT;
+    dim3 grid(n_out), block(256);
+    if (type == LCU_F32) gather_rows_kernel<float><<<grid, block, 0, stream>>>((float *)out, (const float *)x, rows, d, n_src);
+    else if (type == LCU_BF16) gather_rows_kernel<bf16_t><<<grid, block, 0, stream>>>((bf16_t *)out, (const bf16_t *)x, rows, d, n_src);
+    else return LCU_BAD_ARGUMENT;
+    LCU_LAUNCH_CHECK();
+    return LCU_OK;
+}
+
+// ---------------------------------------------------------------- RMS norm (+ residual sum)
+// One block per row.  If `delta` is given: x += delta first (in 32-bit, written back
+// when x is 32-bit: x is then the residual stream).  Then
+//   y = x * rsqrt(sum(x^2)/d + eps) * w        (32-bit, one rounding at the store)
+// The order of the sum depends on d and the block size only, not on the batch.
+template <class TX, class TD, class TW, class TO>
+__global__ void rmsnorm_kernel(TX *__restrict__ x, const TD *__restrict__ delta, const TW *__restrict__ w,
+                               TO *__restrict__ out, int d, float eps, int write_back) {
+    __shared__ float scratch[16];
+    TX *xr = x + (size_t)blockIdx.x * d;
+    const TD *dr = delta ? delta + (size_t)blockIdx.x * d : nullptr;
+    float acc = 0.f;
+    for (int c = threadIdx.x; c < d; c += blockDim.x) {
+        float v = to_f32(xr[c]);
+        if (dr) {
+            v += to_f32(dr[c]);
+            if (write_back) xr[c] = from_f32<TX>(v);
+        }
+        acc += v * v;
+    }
+    const float total = block_sum(acc, scratch);
+    const float rms = rsqrtf(total / (float)d + eps);
+    TO *o = out + (size_t)blockIdx.x * d;
+    for (int c = threadIdx.x; c < d; c += blockDim.x) {
+        float v = to_f32(xr[c]);
+        if (dr && !write_back) v += to_f32(dr[c]);
+        o[c] = from_f32<TO>(rms * v * to_f32(w[c]));
+    }
+}
+
+template <class TX, class TD, class TO>
+static int rmsnorm_w(void *x, const void *delta, const void *w, int w_type, void *out, int n, int d, float eps,
+                     int write_back, hipStream_t stream) {
+    dim3 grid(n), block(d >= 2048 ? 512 : 256);
+    if (w_type == LCU_F32)
+        rmsnorm_kernel<TX, TD, float, TO><<<grid, block, 0, stream>>>((TX *)x, (const TD *)delta, (const float *)w, (TO *)out, d, eps, write_back);
+    else if (w_type == LCU_BF16)
+        rmsnorm_kernel<TX, TD, bf16_t, TO><<<grid, block, 0, stream>>>((TX *)x, (const TD *)delta, (const bf16_t *)w, (TO *)out, d, eps, write_back);
+    else
+        return LCU_BAD_ARGUMENT;
+    LCU_LAUNCH_CHECK();
+    return LCU_OK;
+}
+
+// x: [n, d] of x_type (read; written when write_back and delta are set), delta: [n, d] of
+// act_type or null, out: [n, d] of act_type.
+LCU_API int lcu_rmsnorm(void *x, int x_type, const void *delta, const void *w, int w_type, void *out,
+                        int act_type, int n, int d, float eps, int write_back, hipStream_t stream) {
+    if (n <= 0) return LCU_OK;
+    if (d <= 0) return LCU_BAD_ARGUMENT;
+    if (x_type == LCU_F32 && act_type == LCU_F32) return rmsnorm_w<float, float, float>(x, delta, w, w_type, out, n, d, eps, write_back, stream);
+    if (x_type == LCU_F32 && act_type == LCU_BF16) return rmsnorm_w<float, bf16_t, bf16_t>(x, delta, w, w_type, out, n, d, eps, write_back, stream);
+    if (x_type == LCU_BF16 && act_type == LCU_BF16) return rmsnorm_w<bf16_t, bf16_t, bf16_t>(x, delta, w, w_type, out, n, d, eps, write_back, stream);
+    return LCU_BAD_ARGUMENT;
+}
+
+// ---------------------------------------------------------------- residual add: x (f32) += delta
+template <class TD>
+__global__ void residual_add_kernel(float *__restrict__ x, const TD *__restrict__ delta, size_t total) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < total) x[i] += to_f32(delta[i]);
+}
+
+LCU_API int lcu_residual_add(float *x, const void *delta, int delta_type, long long total, hipStream_t stream) {
+    if (total <= 0) return LCU_OK;
+    dim3 block(256), grid((unsigned)((total + 255) / 256));
+    if (delta_type == LCU_F32) residual_add_kernel<float><<<grid, block, 0, stream>>>(x, (const float *)delta, (size_t)total);
+    else if (delta_type == LCU_BF16) residual_add_kernel<bf16_t><<<grid, block, 0, stream>>>(x, (const bf16_t *)delta, (size_t)total);
+    else return LCU_BAD_ARGUMENT;
+    LCU_LAUNCH_CHECK();
+    return LCU_OK;
+}
+
+// ---------------------------------------------------------------- SwiGLU
+// out[r, c] = gate * (1 / (1 + exp(-gate))) * up with gate = gu[r, c], up = gu[r, di + c].
+template <class T>
+__global__ void swiglu_kernel(T *__restrict__ out, const T *__restrict__ gu, int di) {
+    const int c = blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= di) return;
+    const size_t r = blockIdx.y;
+    const float gate = to_f32(gu[r * 2 * di + c]);
+    const float up = to_f32(gu[r * 2 * di + di + c]);
+    const float sig = 1.0f / (1.0f + expf(-gate));
+    out[r * di + c] = from_f32<T>(gate * sig * up);
+}
+
+LCU_API int lcu_swiglu(void *out, const void *gate_up, int type, int n, int di, hipStream_t stream) {
+    if (n <= 0) return LCU_OK;
+    if (di <= 0) return LCU_BAD_ARGUMENT;
+    dim3 block(256);
+    // grid.y is limited to 65535 rows: larger batches go in slices
+    for (int r0 = 0; r0 < n; r0 += 65535) {
+        const int rows = (n - r0) < 65535 ? (n - r0) : 65535;
+        dim3 grid((di + 255) / 256, rows);
+        if (type == LCU_F32)
+            swiglu_kernel<float><<<grid, block, 0, stream>>>((float *)out + (size_t)r0 * di, (const float *)gate_up + (size_t)r0 * 2 * di, di);
+        else if (type == LCU_BF16)
+            swiglu_kernel<bf16_t><<<grid, block, 0, stream>>>((bf16_t *)out + (size_t)r0 * di, (const bf16_t *)gate_up + (size_t)r0 * 2 * di, di);
+        else
+            return LCU_BAD_ARGUMENT;
+    }
+    LCU_LAUNCH_CHECK();
+    return LCU_OK;
+}

@@ -1,0 +1,93 @@
+// Rotary position encoding of the queries and keys of one step, fused with the write
+// of the step's keys and values into their pages.
+//
+// The rotation of one pair (a, b) by the angle of its token's position:
+//   (a, b) -> (a*cos - b*sin, a*sin + b*cos)
+// computed in 32-bit from 32-bit tables [max_pos, rot_dim/2], one rounding at the
+// store.  pairing 0: the pair is (x[i], x[i + rot_dim/2]); pairing 1: (x[2i], x[2i+1]).
+// Dims at and above rot_dim are not rotated.  A null table means no rotation at all.
+#include "common.h"
+#include "kv_layout.h"
+
+template <class T>
+__global__ void rope_kv_store_kernel(T *__restrict__ qkv, int row_stride, const int *__restrict__ positions,
+                                     const int *__restrict__ slots, const float *__restrict__ cos_t,
+                                     const float *__restrict__ sin_t, int max_pos, T *__restrict__ cache,
+                                     int nh, int nkvh, int dh, int rot_dim, int pairing, int page,
+                                     int store_kv) {
+    const int t = blockIdx.x;
+    T *row = qkv + (size_t)t * row_stride;
+    const int pos = positions[t];
+    const int half = rot_dim / 2;
+    const bool in_table = pos >= 0 && pos < max_pos;
+    const bool rotate = cos_t != nullptr && in_table;
+    // a position outside the table (the host checks before) gives NaN, not a wrong value
+    const bool poison = cos_t != nullptr && !in_table;
+    const int slot = store_kv ? slots[t] : -1;
+    T *pg = nullptr;
+    int tok = 0;
+    if (slot >= 0) {
+        pg = cache + (size_t)(slot / page) * kv_page_elems(nkvh, dh, page);
+        tok = slot % page;
+    }
+    const int rot_heads = store_kv ? nh + nkvh : nh;
+    const int pairs_per_head = dh / 2;
+    // queries and keys: one work item per pair of dims
+    for (int w = threadIdx.x; w < rot_heads * pairs_per_head; w += blockDim.x) {
+        const int head = w / pairs_per_head, i = w % pairs_per_head;
+        T *x = row + (size_t)head * dh;
+        int ia, ib;
+        const bool rot = rotate && i < half;
+        if (i < half) {                // a rotated pair
+            if (pairing == 0) { ia = i; ib = i + half; } else { ia = 2 * i; ib = 2 * i + 1; }
+        } else {                       // dims at and above rot_dim pass through, two at a time
+            ia = rot_dim + 2 * (i - half); ib = ia + 1;
+        }
+        float a = to_f32(x[ia]), b = to_f32(x[ib]);
+        if (rot) {
+            const float c = cos_t[(size_t)pos * half + i], s = sin_t[(size_t)pos * half + i];
+            const float ra = a * c - b * s, rb = a * s + b * c;
+            a = ra; b = rb;
+        }
+        if (poison && i < half) a = b = __uint_as_float(0x7fc00000u);
+        const T va = from_f32<T>(a), vb = from_f32<T>(b);
+        if (head < nh) {
+            if (rot || poison) { x[ia] = va; x[ib] = vb; }
+        } else if (pg) {
+            const int kvh = head - nh;
+            pg[kv_key_offset(kvh, tok, ia, dh, page)] = va;
+            pg[kv_key_offset(kvh, tok, ib, dh, page)] = vb;
+        }
+    }
+    // values: copied as they are
+    if (pg) {
+        const T *v = row + (size_t)(nh + nkvh) * dh;
+        for (int w = threadIdx.x; w < nkvh * dh; w += blockDim.x) {
+            const int kvh = w / dh, c = w % dh;
+            pg[kv_value_offset(nkvh, kvh, tok, c, dh, page)] = v[w];
+        }
+    }
+}
+
+// qkv: [n, row_stride] with a token's q heads, then k heads, then v heads (k and v only
+// when store_kv).  cache: this layer's pages.  slots[t] = page * page_size + place in
+// the page, or -1 to store nothing for token t.
+LCU_API int lcu_rope_kv_store(void *qkv, int type, int n, int row_stride, const int *positions, const int *slots,
+                              const float *cos_t, const float *sin_t, int max_pos, void *cache, int nh, int nkvh,
+                              int dh, int rot_dim, int pairing, int page, int store_kv, hipStream_t stream) {
+    if (n <= 0) return LCU_OK;
+    if (dh <= 0 || dh % 8 || rot_dim % 2 || rot_dim > dh || rot_dim < 0 || page <= 0 || page % 8 || nh <= 0 ||
+        nkvh < 0 || (pairing != 0 && pairing != 1))
+        return LCU_BAD_ARGUMENT;
+    if (store_kv && (!cache || !slots || nkvh <= 0)) return LCU_BAD_ARGUMENT;
+    if (row_stride < (store_kv ? (nh + 2 * nkvh) : nh) * dh) return LCU_BAD_ARGUMENT;
+    dim3 grid(n), block(256);
+    if (type == LCU_F32)
+        rope_kv_store_kernel<float><<<grid, block, 0, stream>>>((float *)qkv, row_stride, positions, slots, cos_t, sin_t, max_pos, (float *)cache, nh, nkvh, dh, rot_dim, pairing, page, store_kv);
+    else if (type == LCU_BF16)
+        rope_kv_store_kernel<bf16_t><<<grid, block, 0, stream>>>((bf16_t *)qkv, row_stride, positions, slots, cos_t, sin_t, max_pos, (bf16_t *)cache, nh, nkvh, dh, rot_dim, pairing, page, store_kv);
+    else
+        return LCU_BAD_ARGUMENT;
+    LCU_LAUNCH_CHECK();
+    return LCU_OK;
+}

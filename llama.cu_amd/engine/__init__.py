@@ -1,0 +1,5 @@
+"""The step function, the scheduler above it, and the engine that ties them to sampling."""
+from .batch import BatchBuilder, StepContext
+from .runner import LayerCache, ModelRunner
+
+__all__ = ["BatchBuilder", "StepContext", "LayerCache", "ModelRunner"]

@@ -1,0 +1,145 @@
+"""The batch of one step, as the model's parts see it, and the builder that lays it
+out in pinned host memory and brings it to the device in one copy.
+
+The reference builds the same facts per round: the tokens, their positions
+(``pos()``), the rows whose output is wanted (``out_idx()``) and one ``Req{cache, pos,
+seq}`` per request (llama.cu/src/exec/engine.rs:352-371, llama.cu/src/exec/group.rs:19-24),
+staged through pinned buffers (llama.cu/src/exec/engine.rs:373-429).  Here a request's
+tokens may be any portion of its prompt or one decoded token, and the requests' pages
+come as block tables.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import List, Optional, Sequence
+
+import torch
+
+from ..cache import CacheManager
+
+
+@dataclass
+class StepContext:
+    """Everything about one step that kernels need.  All tensors are int32 on the device.
+
+    ``tokens, positions, req_of_token``: per token.  ``q_start``: [requests + 1] offsets
+    of each request's tokens; ``ctx_len``: tokens each request holds after this step;
+    ``state_slot``: each request's slot for per-request state; ``logit_rows``: the tokens
+    whose logits are wanted.  A request's tokens stand at positions
+    ``ctx_len - q_len .. ctx_len - 1``.  The lists hold the same facts on the host, for
+    the choice of kernels."""
+    n: int
+    n_req: int
+    tokens: torch.Tensor
+    positions: torch.Tensor
+    req_of_token: torch.Tensor
+    q_start: torch.Tensor
+    ctx_len: torch.Tensor
+    state_slot: torch.Tensor
+    logit_rows: torch.Tensor
+    n_logits: int
+    block_tables: List[torch.Tensor]
+    slot_maps: List[torch.Tensor]
+    q_lens: List[int] = field(default_factory=list)
+    ctx_lens: List[int] = field(default_factory=list)
+    req_ids: List[int] = field(default_factory=list)
+
+    def block_table(self, group: int) -> torch.Tensor:
+        return self.block_tables[group]
+
+    def slots(self, group: int) -> torch.Tensor:
+        return self.slot_maps[group]
+
+    @property
+    def max_q_len(self) -> int:
+        return max(self.q_lens) if self.q_lens else 0
+
+    @property
+    def max_ctx_len(self) -> int:
+        return max(self.ctx_lens) if self.ctx_lens else 0
+
+    @property
+    def decode_only(self) -> bool:
+        return self.max_q_len == 1
+
+
+class BatchBuilder:
+    """Lays the arrays of a step out in one pinned host buffer and one device buffer of
+    fixed capacity, so a step costs one host-to-device copy and the device addresses
+    never change (a captured graph can read them)."""
+
+    def __init__(self, cache: CacheManager, max_tokens: int, max_reqs: int, max_pages: Sequence[int],
+                 device: torch.device):
+        self.cache = cache
+        self.max_tokens, self.max_reqs = int(max_tokens), int(max_reqs)
+        self.max_pages = [int(m) for m in max_pages]
+        self.device = device
+        n, r = self.max_tokens, self.max_reqs
+        sizes = [("tokens", n), ("positions", n), ("req_of_token", n), ("logit_rows", n),
+                 ("q_start", r + 1), ("ctx_len", r), ("state_slot", r)]
+        for g, mp in enumerate(self.max_pages):
+            sizes += [(f"slots{g}", n), (f"block_table{g}", r * mp)]
+        self.offsets = {}
+        total = 0
+        for name, size in sizes:
+            self.offsets[name] = (total, size)
+            total += (size + 3) // 4 * 4
+        pin = device.type == "cuda"
+        self.host = torch.zeros(total, dtype=torch.int32, pin_memory=pin)
+        self.dev = torch.zeros(total, dtype=torch.int32, device=device)
+        self._copied: Optional[torch.cuda.Event] = None
+
+    def _h(self, name: str) -> torch.Tensor:
+        o, s = self.offsets[name]
+        return self.host[o:o + s]
+
+    def _d(self, name: str, count: int) -> torch.Tensor:
+        o, s = self.offsets[name]
+        return self.dev[o:o + count]
+
+    def build(self, req_ids: Sequence[int], tokens: Sequence[Sequence[int]], want: Sequence[Sequence[int]],
+              vocab_size: int) -> StepContext:
+        """The batch in which request ``req_ids[i]`` feeds ``tokens[i]`` and wants the logits
+        at the places ``want[i]`` among them.  The requests' pages must be reserved."""
+        n_req = len(req_ids)
+        n_new = [len(t) for t in tokens]
+        n = sum(n_new)
+        if n_req == 0 or n == 0:
+            raise ValueError("a step needs at least one request with at least one token")
+        if n > self.max_tokens or n_req > self.max_reqs:
+            raise ValueError(f"step of {n} tokens / {n_req} requests exceeds the builder's capacity "
+                             f"({self.max_tokens} / {self.max_reqs})")
+        if self._copied is not None:
+            self._copied.synchronize()          # the last copy out of the host buffer has ended
+        flat = [t for ts in tokens for t in ts]
+        lo, hi = min(flat), max(flat)
+        if lo < 0 or hi >= vocab_size:
+            raise ValueError(f"token id {lo if lo < 0 else hi} is outside the vocabulary of {vocab_size}")
+        self._h("tokens")[:n] = torch.tensor(flat, dtype=torch.int32)
+        rows = []
+        start = 0
+        for i, w in enumerate(want):
+            for k in w:
+                if not 0 <= k < n_new[i]:
+                    raise ValueError(f"request {req_ids[i]}: wanted place {k} is outside its {n_new[i]} tokens")
+                rows.append(start + k)
+            start += n_new[i]
+        if rows:
+            self._h("logit_rows")[:len(rows)] = torch.tensor(rows, dtype=torch.int32)
+        ptr = lambda name: self._h(name).data_ptr()
+        self.cache.fill_batch(req_ids, n_new, ptr("positions"), ptr("req_of_token"), ptr("q_start"), ptr("ctx_len"),
+                              ptr("state_slot"), [ptr(f"block_table{g}") for g in range(len(self.max_pages))],
+                              self.max_pages, [ptr(f"slots{g}") for g in range(len(self.max_pages))])
+        self.dev.copy_(self.host, non_blocking=True)
+        if self.device.type == "cuda":
+            self._copied = torch.cuda.Event()
+            self._copied.record()
+        ctx_lens = self._h("ctx_len")[:n_req].tolist()
+        return StepContext(
+            n=n, n_req=n_req, tokens=self._d("tokens", n), positions=self._d("positions", n),
+            req_of_token=self._d("req_of_token", n), q_start=self._d("q_start", n_req + 1),
+            ctx_len=self._d("ctx_len", n_req), state_slot=self._d("state_slot", n_req),
+            logit_rows=self._d("logit_rows", len(rows)), n_logits=len(rows),
+            block_tables=[self._d(f"block_table{g}", n_req * mp).view(n_req, mp) for g, mp in enumerate(self.max_pages)],
+            slot_maps=[self._d(f"slots{g}", n) for g in range(len(self.max_pages))],
+            q_lens=n_new, ctx_lens=ctx_lens, req_ids=list(req_ids))

@@ -1,0 +1,166 @@
+"""The model runner: the model on the device, its caches, and the one step function.
+
+``step`` is everything between a batch of (request, its next tokens) and the logits at
+the wanted places.  It runs only the tokens it is given, as one batch, from the cache
+that earlier steps left, whatever the mix: portions of prompts beside single decoded
+tokens, cut anywhere.  (The reference's counterpart is ``ModelGroup::load_inputs`` +
+``launch`` + ``OutputHead::launch``, llama.cu/src/exec/group.rs:89-157 and
+llama.cu/src/exec/output_head.rs:55-116, which feeds whole prompts only and returns
+sampled ids instead of logits.)
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Any, Dict, List, Optional, Sequence
+
+import torch
+
+from ..cache import CacheGroup, CacheManager, OutOfPages
+from ..config import load_config
+from ..parts import BuildContext, DecoderModel, ModelSpec, PagedKV, SlotState
+from ..weights import load_weights, open_safetensors, random_tensors
+from .batch import BatchBuilder, StepContext
+
+DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "f32": torch.float32,
+          "fp32": torch.float32, torch.bfloat16: torch.bfloat16, torch.float32: torch.float32}
+
+
+@dataclass
+class LayerCache:
+    """What one entry of the run order gets: the pages of its layer (``pages``,
+    ``[num_pages, 2, kv_heads * head_dim * page_size]``) with the group whose block tables
+    index them, whether the entry writes them, and/or its per-request state
+    (``state``, ``[slots, *shape]``)."""
+    group: int = -1
+    pages: Optional[torch.Tensor] = None
+    writes: bool = True
+    state: Optional[torch.Tensor] = None
+
+
+def require_gpu(device) -> torch.device:
+    device = torch.device(device)
+    if device.type != "cuda" or not torch.cuda.is_available():
+        raise RuntimeError("llama.cu_amd runs on a GPU only (gfx950); no GPU is visible to torch "
+                           "and there is no CPU fallback")
+    return device
+
+
+class ModelRunner:
+    def __init__(self, spec: ModelSpec, tensors: Dict[str, torch.Tensor], dtype, device="cuda:0",
+                 page_size: int = 16, max_tokens: Optional[int] = None, num_pages: Optional[int] = None,
+                 max_seqs: int = 8, max_batch_tokens: int = 2048, max_model_len: Optional[int] = None):
+        self.device = require_gpu(device)
+        self.dtype = DTYPES[dtype]
+        self.spec = spec
+        self.page_size = int(page_size)
+        if self.page_size % 8:
+            raise ValueError(f"page_size {page_size} must be a multiple of 8")
+        self.max_model_len = min(int(max_model_len or spec.max_positions), spec.max_positions)
+        self.max_seqs, self.max_batch_tokens = int(max_seqs), int(max_batch_tokens)
+        torch.cuda.set_device(self.device)
+        self.model = DecoderModel(spec)
+        build = BuildContext(self.dtype, self.device, spec.max_positions, self.page_size)
+        self.model.load(tensors, build)
+
+        # cache groups: one per distinct window among the layers that page keys and values
+        needs = self.model.cache_needs()
+        windows = sorted({n.window for n in needs if isinstance(n, PagedKV)})
+        if num_pages is None:
+            if max_tokens is None:
+                raise ValueError("give max_tokens or num_pages for the cache pool")
+            num_pages = (int(max_tokens) + self.page_size - 1) // self.page_size
+        self.num_pages = int(num_pages)
+        self.groups = [CacheGroup(self.num_pages, self.page_size, w) for w in windows]
+        self.cache = CacheManager(self.groups, self.max_seqs)
+        self.caches: List[LayerCache] = []
+        for i, (entry, need) in enumerate(zip(spec.run_order, needs)):
+            if entry.cache_of is not None:
+                src = self.caches[entry.cache_of]
+                self.caches.append(LayerCache(group=src.group, pages=src.pages, writes=False, state=src.state))
+            elif isinstance(need, PagedKV):
+                pages = torch.zeros((self.num_pages, 2, need.kv_heads * need.head_dim * self.page_size),
+                                    dtype=self.dtype, device=self.device)
+                self.caches.append(LayerCache(group=windows.index(need.window), pages=pages))
+            elif isinstance(need, SlotState):
+                state = torch.zeros((self.max_seqs,) + tuple(need.shape), dtype=need.dtype, device=self.device)
+                self.caches.append(LayerCache(state=state))
+            elif need is None:
+                self.caches.append(LayerCache())
+            else:
+                raise ValueError(f"run order entry {i}: unknown cache need {need!r}")
+        max_pages = [(self.max_model_len + self.page_size - 1) // self.page_size for _ in self.groups]
+        self.builder = BatchBuilder(self.cache, self.max_batch_tokens, self.max_seqs, max_pages, self.device)
+
+    # ------------------------------------------------------------ construction helpers
+    @classmethod
+    def from_folder(cls, folder: str, dtype="bfloat16", device="cuda:0", **kw) -> "ModelRunner":
+        """The model of a folder (config.json picks the architecture; model.safetensors)."""
+        from .. import models  # noqa: F401  (registers the architectures)
+        device = require_gpu(device)
+        arch, cfg = load_config(folder)
+        spec = arch.build_spec(cfg)
+        files = open_safetensors(folder)
+        tensors = load_weights(files, DecoderModel(spec).tensors(), DTYPES[dtype], device)
+        runner = cls(spec, tensors, dtype, device, **kw)
+        runner.config = cfg
+        return runner
+
+    @classmethod
+    def from_config(cls, cfg, seed: int, dtype="bfloat16", device="cuda:0", std: float = 0.02, **kw) -> "ModelRunner":
+        """Random weights made on the device (nothing is written or read)."""
+        from .. import models  # noqa: F401
+        from ..config import architecture_of
+        device = require_gpu(device)
+        spec = architecture_of(cfg.to_dict()).build_spec(cfg)
+        tensors = random_tensors(DecoderModel(spec).tensors(), seed, dtype=DTYPES[dtype], std=std, device=device)
+        runner = cls(spec, tensors, dtype, device, **kw)
+        runner.config = cfg
+        return runner
+
+    # ------------------------------------------------------------ the step function
+    def prepare(self, req_ids: Sequence[int], tokens: Sequence[Sequence[int]], want: Sequence[Sequence[int]]) -> StepContext:
+        """Give the requests their pages (new requests get a slot) and build the batch."""
+        added = []
+        reserved = []
+        try:
+            for rid, toks in zip(req_ids, tokens):
+                if not self.cache.has(rid):
+                    self.cache.add(rid)
+                    added.append(rid)
+                new_len = self.cache.length(rid) + len(toks)
+                if new_len > self.max_model_len:
+                    raise ValueError(f"request {rid}: {new_len} tokens exceed the context limit {self.max_model_len}")
+                if not self.cache.reserve(rid, new_len):
+                    raise OutOfPages(f"request {rid}: no free pages for {len(toks)} more tokens "
+                                     f"({self.cache.free_pages(0)} pages free)")
+                reserved.append(rid)
+        except Exception:
+            for rid in reserved:                       # give back what this call took
+                if rid not in added:
+                    self.cache.truncate(rid, self.cache.length(rid))
+            for rid in added:
+                self.cache.release(rid)
+            raise
+        return self.builder.build(req_ids, tokens, want, self.spec.vocab_size)
+
+    def run(self, step: StepContext) -> torch.Tensor:
+        return self.model.forward(step, self.caches)
+
+    def step(self, req_ids: Sequence[int], tokens: Sequence[Sequence[int]],
+             want: Optional[Sequence[Sequence[int]]] = None) -> torch.Tensor:
+        """Run one batch: request ``req_ids[i]`` feeds ``tokens[i]`` (its next tokens, after
+        what earlier steps fed).  Returns float32 logits ``[wanted, vocab]`` on the device, in
+        the order of the requests and of ``want[i]`` (places among ``tokens[i]``; default: the
+        last token of each request)."""
+        if want is None:
+            want = [[len(t) - 1] for t in tokens]
+        ctx = self.prepare(req_ids, tokens, want)
+        logits = self.run(ctx)
+        for rid in req_ids:
+            self.cache.commit(rid)
+        return logits
+
+    def end(self, req_id: int) -> None:
+        """The request is finished: its pages and slot are given back."""
+        if self.cache.has(req_id):
+            self.cache.release(req_id)

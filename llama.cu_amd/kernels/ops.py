@@ -1,0 +1,286 @@
+"""The hand-written gfx950 kernels as Python functions on torch tensors.
+
+Every function checks on the host that the operands' shapes, types, layout and
+device are what its kernel and its grid assume, and raises before anything is
+launched if they are not; then it launches on torch's current stream.  There is no
+CPU path: a tensor that is not on the GPU is an error.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Optional
+
+import torch
+
+from . import build
+
+F32, BF16 = 0, 1
+_TYPE = {torch.float32: F32, torch.bfloat16: BF16}
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+def _type(t: torch.Tensor, what: str) -> int:
+    code = _TYPE.get(t.dtype)
+    if code is None:
+        raise KernelError(f"{what}: type {t.dtype} is not supported (float32 or bfloat16)")
+    return code
+
+
+def _gpu(*tensors: Optional[torch.Tensor]) -> None:
+    dev = None
+    for t in tensors:
+        if t is None:
+            continue
+        if not t.is_cuda:
+            raise KernelError("kernel operands must be on the GPU (there is no CPU path)")
+        if dev is None:
+            dev = t.device
+        elif t.device != dev:
+            raise KernelError("kernel operands are on different devices")
+
+
+def _rows(t: torch.Tensor, what: str) -> None:
+    if t.dim() != 2 or t.stride(1) != 1:
+        raise KernelError(f"{what}: need a 2-d tensor with contiguous rows, got shape {tuple(t.shape)} "
+                          f"strides {tuple(t.stride())}")
+
+
+def _contig(t: torch.Tensor, what: str) -> None:
+    if not t.is_contiguous():
+        raise KernelError(f"{what}: must be contiguous")
+
+
+def _i32(t: torch.Tensor, what: str, n: Optional[int] = None) -> None:
+    if t.dtype != torch.int32 or not t.is_contiguous():
+        raise KernelError(f"{what}: must be a contiguous int32 tensor")
+    if n is not None and t.numel() != n:
+        raise KernelError(f"{what}: expected {n} entries, got {t.numel()}")
+
+
+def _stream() -> ctypes.c_void_p:
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _ptr(t: Optional[torch.Tensor]) -> ctypes.c_void_p:
+    return ctypes.c_void_p(0 if t is None else t.data_ptr())
+
+
+def _check(rc: int, name: str) -> None:
+    if rc == 0:
+        return
+    if rc == -1:
+        raise KernelError(f"{name}: the kernel refused its arguments (unsupported size or shape)")
+    if rc == -2:
+        raise KernelError(f"{name}: unsupported configuration")
+    raise KernelError(f"{name}: launch failed with HIP error {rc}")
+
+
+# ------------------------------------------------------------------ elementwise
+
+
+def embedding_gather(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """``out[i, :] = table[ids[i], :]`` (converted to ``out``'s type)."""
+    _gpu(table, ids, out)
+    _rows(table, "embedding table"); _contig(table, "embedding table"); _contig(out, "embedding out")
+    n = ids.numel()
+    _i32(ids, "token ids")
+    if out.shape != (n, table.shape[1]):
+        raise KernelError(f"embedding out: shape {tuple(out.shape)}, expected {(n, table.shape[1])}")
+    lib = build.load("elementwise")
+    _check(lib.lcu_embedding_gather(_ptr(out), _type(out, "embedding out"), _ptr(table), _type(table, "embedding table"),
+                                    _ptr(ids), n, table.shape[1], table.shape[0], _stream()), "embedding_gather")
+    return out
+
+
+def gather_rows(x: torch.Tensor, rows: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``out[i, :] = x[rows[i], :]``."""
+    _gpu(x, rows, out)
+    _rows(x, "gather source"); _contig(x, "gather source")
+    _i32(rows, "row indices")
+    n = rows.numel()
+    if out is None:
+        out = torch.empty((n, x.shape[1]), dtype=x.dtype, device=x.device)
+    if out.shape != (n, x.shape[1]) or out.dtype != x.dtype or not out.is_contiguous():
+        raise KernelError("gather out: wrong shape, type or layout")
+    lib = build.load("elementwise")
+    _check(lib.lcu_gather_rows(_ptr(out), _ptr(x), _type(x, "gather source"), _ptr(rows), n, x.shape[1], x.shape[0],
+                               _stream()), "gather_rows")
+    return out
+
+
+def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor,
+            delta: Optional[torch.Tensor] = None, write_back: bool = True) -> torch.Tensor:
+    """``y = x' * rsqrt(mean(x'^2) + eps) * weight`` with ``x' = x + delta`` (``x`` if there is
+    no ``delta``), all in 32-bit.  With ``write_back`` the sum ``x'`` replaces ``x`` (the
+    residual stream takes in the branch's output)."""
+    _gpu(x, weight, out, delta)
+    _rows(x, "norm input"); _contig(x, "norm input"); _contig(out, "norm out"); _contig(weight, "norm weight")
+    n, d = x.shape
+    if out.shape != (n, d):
+        raise KernelError(f"norm out: shape {tuple(out.shape)}, expected {(n, d)}")
+    if weight.shape != (d,):
+        raise KernelError(f"norm weight: shape {tuple(weight.shape)}, expected {(d,)}")
+    if delta is not None:
+        _contig(delta, "norm delta")
+        if delta.shape != (n, d) or delta.dtype != out.dtype:
+            raise KernelError("norm delta: must have the output's shape and type")
+    xt, at = _type(x, "norm input"), _type(out, "norm out")
+    if (xt, at) not in ((F32, F32), (F32, BF16), (BF16, BF16)):
+        raise KernelError(f"norm: input {x.dtype} with output {out.dtype} is not supported")
+    lib = build.load("elementwise")
+    _check(lib.lcu_rmsnorm(_ptr(x), xt, _ptr(delta), _ptr(weight), _type(weight, "norm weight"), _ptr(out), at,
+                           n, d, ctypes.c_float(eps), int(bool(write_back)), _stream()), "rmsnorm")
+    return out
+
+
+def residual_add(x: torch.Tensor, delta: torch.Tensor) -> torch.Tensor:
+    """``x += delta`` in 32-bit (``x`` is float32)."""
+    _gpu(x, delta)
+    _contig(x, "residual"); _contig(delta, "delta")
+    if x.dtype != torch.float32 or x.shape != delta.shape:
+        raise KernelError("residual_add: x must be float32 and delta of the same shape")
+    lib = build.load("elementwise")
+    _check(lib.lcu_residual_add(_ptr(x), _ptr(delta), _type(delta, "delta"), ctypes.c_longlong(x.numel()), _stream()),
+           "residual_add")
+    return x
+
+
+def swiglu(gate_up: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``out = gate * sigmoid(gate) * up`` for ``gate_up = [gate | up]`` of shape ``[n, 2*di]``."""
+    _gpu(gate_up, out)
+    _rows(gate_up, "gate_up"); _contig(gate_up, "gate_up")
+    n, two_di = gate_up.shape
+    if two_di % 2:
+        raise KernelError("swiglu: the input's width must be even (gate and up side by side)")
+    di = two_di // 2
+    if out is None:
+        out = torch.empty((n, di), dtype=gate_up.dtype, device=gate_up.device)
+    if out.shape != (n, di) or out.dtype != gate_up.dtype or not out.is_contiguous():
+        raise KernelError("swiglu out: wrong shape, type or layout")
+    lib = build.load("elementwise")
+    _check(lib.lcu_swiglu(_ptr(out), _ptr(gate_up), _type(gate_up, "gate_up"), n, di, _stream()), "swiglu")
+    return out
+
+
+# ------------------------------------------------------------------ rotation and cache write
+
+
+def rope_kv_store(qkv: torch.Tensor, positions: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: int,
+                  cos: Optional[torch.Tensor], sin: Optional[torch.Tensor], rot_dim: int, pairing: int,
+                  cache: Optional[torch.Tensor], slots: Optional[torch.Tensor], page_size: int) -> None:
+    """Rotate the queries (in place) and the keys of ``qkv [n, (heads + 2 kv_heads) * head_dim]``
+    and write keys and values into ``cache`` at ``slots``.  With ``cache=None`` the row holds
+    queries only and nothing is stored."""
+    _gpu(qkv, positions, cos, sin, cache, slots)
+    _rows(qkv, "qkv")
+    n = qkv.shape[0]
+    store = cache is not None
+    need = (n_heads + (2 * n_kv_heads if store else 0)) * head_dim
+    if qkv.shape[1] != need:
+        raise KernelError(f"qkv: width {qkv.shape[1]}, expected {need}")
+    _i32(positions, "positions", n)
+    if head_dim % 8:
+        raise KernelError(f"head_dim {head_dim} must be a multiple of 8")
+    max_pos = 0
+    if cos is not None:
+        if sin is None or cos.shape != sin.shape or cos.dtype != torch.float32 or sin.dtype != torch.float32 \
+                or cos.dim() != 2 or cos.shape[1] * 2 != rot_dim or not cos.is_contiguous() or not sin.is_contiguous():
+            raise KernelError("rotation tables must be two contiguous float32 tensors [max_pos, rot_dim/2]")
+        max_pos = cos.shape[0]
+    if store:
+        _i32(slots, "cache slots", n)
+        _contig(cache, "cache")
+        if cache.dtype != qkv.dtype:
+            raise KernelError("cache and qkv must have one type")
+        if cache.dim() != 3 or cache.shape[1] != 2 or cache.shape[2] != n_kv_heads * head_dim * page_size:
+            raise KernelError(f"cache: shape {tuple(cache.shape)}, expected [pages, 2, {n_kv_heads * head_dim * page_size}]")
+    lib = build.load("rope_kv")
+    _check(lib.lcu_rope_kv_store(_ptr(qkv), _type(qkv, "qkv"), n, qkv.stride(0), _ptr(positions), _ptr(slots),
+                                 _ptr(cos), _ptr(sin), max_pos, _ptr(cache), n_heads, n_kv_heads, head_dim, rot_dim,
+                                 pairing, page_size, int(store), _stream()), "rope_kv_store")
+
+
+# ------------------------------------------------------------------ attention
+
+
+def _attention_args(q, out, cache, block_table, q_start, ctx_len, req_of_token, n_heads, n_kv_heads, head_dim,
+                    page_size):
+    _gpu(q, out, cache, block_table, q_start, ctx_len, req_of_token)
+    _rows(q, "attention q"); _rows(out, "attention out")
+    n = q.shape[0]
+    if q.shape[1] < n_heads * head_dim or out.shape != (n, n_heads * head_dim) or out.dtype != q.dtype:
+        raise KernelError("attention: q or out has a wrong shape or type")
+    if cache.dtype != q.dtype or not cache.is_contiguous() or cache.dim() != 3 or cache.shape[1] != 2 \
+            or cache.shape[2] != n_kv_heads * head_dim * page_size:
+        raise KernelError("attention: cache has a wrong shape, type or layout")
+    if block_table.dim() != 2 or block_table.dtype != torch.int32 or not block_table.is_contiguous():
+        raise KernelError("attention: block_table must be a contiguous int32 [requests, pages]")
+    n_req = block_table.shape[0]
+    _i32(q_start, "q_start", n_req + 1); _i32(ctx_len, "ctx_len", n_req); _i32(req_of_token, "req_of_token", n)
+    if n_heads % n_kv_heads:
+        raise KernelError("attention: heads must be a multiple of kv heads")
+    return n
+
+
+def paged_attention_generic(q: torch.Tensor, out: torch.Tensor, cache: torch.Tensor, block_table: torch.Tensor,
+                            q_start: torch.Tensor, ctx_len: torch.Tensor, req_of_token: torch.Tensor,
+                            n_heads: int, n_kv_heads: int, head_dim: int, page_size: int, scale: float,
+                            window: int = 0) -> torch.Tensor:
+    """Causal attention of the step's queries over the paged cache (every shape)."""
+    n = _attention_args(q, out, cache, block_table, q_start, ctx_len, req_of_token, n_heads, n_kv_heads, head_dim,
+                        page_size)
+    if head_dim % 8 or head_dim > 256:
+        raise KernelError(f"attention: head_dim {head_dim} must be a multiple of 8, at most 256")
+    lib = build.load("attention_generic")
+    _check(lib.lcu_paged_attention_generic(_ptr(q), q.stride(0), _ptr(out), out.stride(0), _type(q, "q"), _ptr(cache),
+                                           _ptr(block_table), block_table.shape[1], _ptr(q_start), _ptr(ctx_len),
+                                           _ptr(req_of_token), n, n_heads, n_kv_heads, head_dim, page_size,
+                                           ctypes.c_float(scale), int(window), _stream()), "paged_attention_generic")
+    return out
+
+
+# ------------------------------------------------------------------ matrix products
+
+
+def gemm_nt(a: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = None,
+            out_dtype: Optional[torch.dtype] = None, accumulate: bool = False) -> torch.Tensor:
+    """``out (+)= a @ w.T`` with ``w [N, K]``, 32-bit accumulation, any mix of float32 and
+    bfloat16 operands.  With float32 operands this is a true 32-bit product."""
+    _gpu(a, w, out)
+    _rows(a, "gemm a"); _rows(w, "gemm w")
+    m, k = a.shape
+    nn, k2 = w.shape
+    if k != k2:
+        raise KernelError(f"gemm: a is [{m}, {k}] but w is [{nn}, {k2}]")
+    if out is None:
+        if accumulate:
+            raise KernelError("gemm: accumulate needs an output to add to")
+        out = torch.empty((m, nn), dtype=out_dtype or a.dtype, device=a.device)
+    _rows(out, "gemm out")
+    if out.shape != (m, nn):
+        raise KernelError(f"gemm out: shape {tuple(out.shape)}, expected {(m, nn)}")
+    lib = build.load("gemm_generic")
+    _check(lib.lcu_gemm_nt(_ptr(a), _type(a, "gemm a"), a.stride(0), _ptr(w), _type(w, "gemm w"), w.stride(0),
+                           _ptr(out), _type(out, "gemm out"), out.stride(0), m, nn, k, int(bool(accumulate)),
+                           _stream()), "gemm_nt")
+    return out
+
+
+def paged_attention(q: torch.Tensor, out: torch.Tensor, cache: torch.Tensor, step, group: int, n_heads: int,
+                    n_kv_heads: int, head_dim: int, page_size: int, scale: float, window: int = 0) -> torch.Tensor:
+    """Attention for the batch ``step`` (an engine.batch.StepContext) over cache group
+    ``group``: picks the kernel for the batch's shape."""
+    return paged_attention_generic(q, out, cache, step.block_table(group), step.q_start, step.ctx_len,
+                                   step.req_of_token, n_heads, n_kv_heads, head_dim, page_size, scale, window)
+
+
+def skinny_supported(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype) -> bool:
+    """Whether the weight-streaming kernel for few rows takes this product."""
+    return False
+
+
+def gemm_skinny(x, w, out=None, out_dtype=None, accumulate=False):
+    raise KernelError("gemm_skinny: not available")

@@ -1,0 +1,80 @@
+"""The attention mixer: grouped-query causal attention over the paged cache.
+
+q, k, v projections as one matrix product (rows q, then k, then v, the layout of the
+reference's fused tensor, llama.cu/src/model/mod.rs:114-119), position encoding of q
+and k and the write of k and v into the request's pages in one kernel, attention of
+the step's queries over the cache, output projection (llama.cu/src/model/mod.rs:125-130).
+The call contract of the attention itself is llama.cu/src/exec/step.rs:162-178: causal,
+offset by the request's position.  Scores, softmax and the output sum are 32-bit.
+"""
+from __future__ import annotations
+
+from typing import Dict, Optional
+
+import torch
+
+from ..kernels import ops
+from .base import BuildContext, PagedKV, Part, PartSpec, TensorSpec, make_part, register_part
+from .linear import linear
+
+
+class Attention(Part):
+    def __init__(self, hidden_size: int, heads: int, kv_heads: int, head_dim: int, scale: Optional[float] = None,
+                 window: int = 0, position: Optional[PartSpec] = None, shares_kv: bool = False):
+        if heads % kv_heads:
+            raise ValueError(f"attention: {heads} heads are no multiple of {kv_heads} key/value heads")
+        if head_dim % 16 or head_dim > 256:
+            raise ValueError(f"attention: head_dim {head_dim} is not supported by the kernels "
+                             f"(multiples of 16 up to 256)")
+        self.hidden_size, self.heads, self.kv_heads, self.head_dim = int(hidden_size), int(heads), int(kv_heads), int(head_dim)
+        self.scale = float(scale) if scale is not None else float(head_dim) ** -0.5
+        self.window = int(window or 0)
+        self.shares_kv = bool(shares_kv)          # reads another layer's keys and values: has q and o only
+        self.position = make_part("position", position or PartSpec("none"))
+        self.w_qkv = self.w_o = None
+        self.page_size = 0
+
+    def tensors(self) -> Dict[str, TensorSpec]:
+        d, nh, nkv, dh = self.hidden_size, self.heads, self.kv_heads, self.head_dim
+        t = {"q_proj.weight": TensorSpec((nh * dh, d)), "o_proj.weight": TensorSpec((d, nh * dh))}
+        if not self.shares_kv:
+            t["k_proj.weight"] = TensorSpec((nkv * dh, d))
+            t["v_proj.weight"] = TensorSpec((nkv * dh, d))
+        return t
+
+    def cache_need(self):
+        return PagedKV(self.kv_heads, self.head_dim, self.window)
+
+    def load(self, tensors, build: BuildContext) -> None:
+        if self.shares_kv:
+            self.w_qkv = tensors["q_proj.weight"].contiguous()
+        else:
+            parts = [tensors["q_proj.weight"], tensors["k_proj.weight"], tensors["v_proj.weight"]]
+            if len({p.dtype for p in parts}) != 1:
+                parts = [p.float() for p in parts]
+            self.w_qkv = torch.cat(parts, dim=0).contiguous()
+        self.w_o = tensors["o_proj.weight"].contiguous()
+        self.position.load({}, build)
+        self.page_size = build.page_size
+        self.dtype = build.dtype
+
+    def forward(self, h: torch.Tensor, step, cache) -> torch.Tensor:
+        nh, nkv, dh = self.heads, self.kv_heads, self.head_dim
+        qkv = linear(h, self.w_qkv, out_dtype=self.dtype)
+        self.position.apply(qkv, step.positions, nh, 0 if self.shares_kv else nkv, dh)
+        rot = self.position.rotary_tables()
+        cos, sin, rot_dim, pairing = rot if rot is not None else (None, None, 0, 0)
+        store = cache.writes and not self.shares_kv
+        if self.shares_kv == cache.writes:
+            raise ops.KernelError("attention: a layer that shares another's keys and values must be given that "
+                                  "layer's cache in the run order (and only such a layer)")
+        ops.rope_kv_store(qkv, step.positions, nh, nkv, dh, cos, sin, rot_dim, pairing,
+                          cache.pages if store else None, step.slots(cache.group) if store else None,
+                          self.page_size)
+        out = torch.empty((h.shape[0], nh * dh), dtype=self.dtype, device=h.device)
+        ops.paged_attention(qkv, out, cache.pages, step, cache.group, nh, nkv, dh, self.page_size, self.scale,
+                            self.window)
+        return linear(out, self.w_o, out_dtype=self.dtype)
+
+
+register_part("mixer", "attention", Attention)

@@ -1,0 +1,136 @@
+"""What a model is made of: specifications (data), parts (objects that hold weights
+and run kernels) and the registries that turn the first into the second.
+
+A *specification* is plain data: a kind, parameters, and the name under which the
+part's tensors lie in the weight file.  A *part* is built from a specification by
+the registry of its category:
+
+  ``norm``      ``forward(x, delta) -> y``             x: float32 [n, d] residual stream, updated in
+                                                    place by ``x += delta`` (``delta`` may be None);
+                                                    y: [n, d] in the compute type
+  ``mixer``     ``forward(h, step, cache) -> delta``   h, delta: [n, d] compute type; ``step`` is the
+                ``cache_need() -> need or None``       batch (engine.batch.StepContext); ``cache`` is
+                                                    what the engine made for ``cache_need()``
+  ``ffn``       ``forward(h) -> delta``
+  ``position``  ``tables(...)``/``apply(...)``         see parts.position
+  ``block``     ``forward(x, pending, step, cache) -> pending``   the arrangement of the four above
+
+Every part also has ``tensors() -> {relative name: TensorSpec}`` and
+``load(tensors, build)``.  No part knows which model it is in: sizes and constants
+arrive as parameters.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Any, Callable, Dict, List, Optional, Tuple
+
+import torch
+
+
+@dataclass(frozen=True)
+class TensorSpec:
+    """One tensor a part binds: its shape, and how a random model fills it
+    (``normal``: N(0, std); ``one_plus_normal``: 1 + N(0, std), for norm weights).
+    ``integer`` tensors are kept as int32, all others follow the weight policy."""
+    shape: Tuple[int, ...]
+    init: str = "normal"
+    integer: bool = False
+    optional: bool = False
+
+
+@dataclass
+class PartSpec:
+    kind: str
+    params: Dict[str, Any] = field(default_factory=dict)
+    name: str = ""           # the part's component in tensor names ("self_attn", "mlp", ...)
+
+
+@dataclass(frozen=True)
+class RunEntry:
+    """One step of the run order: which layer runs, and whose cache it uses.  ``cache_of``
+    None: a cache of its own.  ``cache_of = j``: it reads the cache that entry ``j`` of the
+    run order wrote (and writes none)."""
+    layer: int
+    cache_of: Optional[int] = None
+
+
+@dataclass
+class ModelSpec:
+    """A whole decoder as data."""
+    hidden_size: int
+    vocab_size: int
+    max_positions: int
+    embedding: PartSpec
+    layers: List[PartSpec]              # block specifications, each with its tensor-name prefix
+    run_order: List[RunEntry]
+    final_norm: PartSpec
+    head: PartSpec
+    eos_token_ids: Tuple[int, ...] = ()
+
+
+# ------------------------------------------------------------------ cache needs
+
+
+@dataclass(frozen=True)
+class PagedKV:
+    """Keys and values of every token (or of the last ``window`` tokens), in pages."""
+    kv_heads: int
+    head_dim: int
+    window: int = 0          # 0: all tokens
+
+
+@dataclass(frozen=True)
+class SlotState:
+    """A state of fixed size per request (``shape`` without the slot axis)."""
+    shape: Tuple[int, ...]
+    dtype: torch.dtype = torch.float32
+
+
+# ------------------------------------------------------------------ building
+
+
+@dataclass
+class BuildContext:
+    """What a part may need to know about the engine while it binds its weights."""
+    dtype: torch.dtype               # the compute type: torch.bfloat16 or torch.float32
+    device: torch.device
+    max_positions: int
+    page_size: int
+
+
+class Part:
+    def tensors(self) -> Dict[str, TensorSpec]:
+        return {}
+
+    def load(self, tensors: Dict[str, torch.Tensor], build: BuildContext) -> None:
+        pass
+
+
+_REGISTRIES: Dict[str, Dict[str, Callable[..., Part]]] = {
+    "norm": {}, "mixer": {}, "ffn": {}, "position": {}, "block": {}, "embedding": {}, "head": {}}
+
+
+def register_part(category: str, kind: str, factory: Callable[..., Part], replace: bool = False) -> None:
+    """Make ``kind`` known in ``category``; ``factory(**params)`` builds the part."""
+    reg = _REGISTRIES.get(category)
+    if reg is None:
+        raise ValueError(f"no part category {category!r}; categories: {sorted(_REGISTRIES)}")
+    if kind in reg and not replace:
+        raise ValueError(f"{category} part {kind!r} is already registered")
+    reg[kind] = factory
+
+
+def make_part(category: str, spec: PartSpec) -> Part:
+    reg = _REGISTRIES[category]
+    factory = reg.get(spec.kind)
+    if factory is None:
+        raise ValueError(f"no {category} part of kind {spec.kind!r}; registered: {sorted(reg)}")
+    return factory(**spec.params)
+
+
+def registered_parts(category: str) -> List[str]:
+    return sorted(_REGISTRIES[category])
+
+
+def prefixed(prefix: str, name: str) -> str:
+    return f"{prefix}.{name}" if prefix else name

@@ -1,0 +1,52 @@
+"""The arrangement of norm, mixer, norm and feed-forward in one layer.
+
+``prenorm``: ``x += mixer(norm1(x)); x += ffn(norm2(x))``
+(llama.cu/src/model/mod.rs:100-157, ``TransformerBlk::new(norm, attention, norm, mlp)``;
+the residual is added where the output and down projections end,
+llama.cu/src/op/linear.rs:35-62).  Here the residual stream ``x`` is float32 and each
+sum is made in 32-bit inside the norm kernel that follows it: a block returns its last
+branch's output as ``pending``, and whoever norms next adds it.
+"""
+from __future__ import annotations
+
+from typing import Dict, Optional
+
+import torch
+
+from .base import BuildContext, Part, PartSpec, TensorSpec, make_part, prefixed, register_part
+
+
+class PreNormBlock(Part):
+    def __init__(self, norm1: PartSpec, mixer: PartSpec, norm2: PartSpec, ffn: PartSpec):
+        self.specs = {"norm1": norm1, "mixer": mixer, "norm2": norm2, "ffn": ffn}
+        self.norm1 = make_part("norm", norm1)
+        self.mixer = make_part("mixer", mixer)
+        self.norm2 = make_part("norm", norm2)
+        self.ffn = make_part("ffn", ffn)
+
+    def _children(self):
+        return [(self.specs[k].name, getattr(self, k)) for k in ("norm1", "mixer", "norm2", "ffn")]
+
+    def tensors(self) -> Dict[str, TensorSpec]:
+        out = {}
+        for name, part in self._children():
+            for k, v in part.tensors().items():
+                out[prefixed(name, k)] = v
+        return out
+
+    def load(self, tensors, build: BuildContext) -> None:
+        for name, part in self._children():
+            pre = name + "." if name else ""
+            part.load({k[len(pre):]: v for k, v in tensors.items() if k.startswith(pre)}, build)
+
+    def cache_need(self):
+        return self.mixer.cache_need()
+
+    def forward(self, x: torch.Tensor, pending: Optional[torch.Tensor], step, cache) -> torch.Tensor:
+        h = self.norm1.forward(x, pending)
+        a = self.mixer.forward(h, step, cache)
+        h2 = self.norm2.forward(x, a)
+        return self.ffn.forward(h2)
+
+
+register_part("block", "prenorm", PreNormBlock)

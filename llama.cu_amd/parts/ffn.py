@@ -1,0 +1,43 @@
+"""The dense feed-forward: ``down(gate * sigmoid(gate) * up)``.
+
+gate and up projections as one matrix product (gate rows first, the layout of the
+reference's fused tensor, llama.cu/src/model/mod.rs:140-147), the activation of
+llama.cu/src/op/swiglu.cuh:1-20 in 32-bit, then the down projection
+(llama.cu/src/model/mod.rs:148-153).
+"""
+from __future__ import annotations
+
+from typing import Dict
+
+import torch
+
+from ..kernels import ops
+from .base import BuildContext, Part, TensorSpec, register_part
+from .linear import linear
+
+
+class SwiGLU(Part):
+    def __init__(self, hidden_size: int, intermediate_size: int):
+        self.hidden_size, self.intermediate_size = int(hidden_size), int(intermediate_size)
+        self.w_gate_up = self.w_down = None
+
+    def tensors(self) -> Dict[str, TensorSpec]:
+        d, di = self.hidden_size, self.intermediate_size
+        return {"gate_proj.weight": TensorSpec((di, d)), "up_proj.weight": TensorSpec((di, d)),
+                "down_proj.weight": TensorSpec((d, di))}
+
+    def load(self, tensors, build: BuildContext) -> None:
+        g, u = tensors["gate_proj.weight"], tensors["up_proj.weight"]
+        if g.dtype != u.dtype:
+            g, u = g.float(), u.float()
+        self.w_gate_up = torch.cat([g, u], dim=0).contiguous()
+        self.w_down = tensors["down_proj.weight"].contiguous()
+        self.dtype = build.dtype
+
+    def forward(self, h: torch.Tensor) -> torch.Tensor:
+        gu = linear(h, self.w_gate_up, out_dtype=self.dtype)
+        act = ops.swiglu(gu)
+        return linear(act, self.w_down, out_dtype=self.dtype)
+
+
+register_part("ffn", "swiglu", SwiGLU)

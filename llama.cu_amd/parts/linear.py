@@ -1,0 +1,35 @@
+"""``y = x @ W.T`` for a weight stored ``[out, in]`` (llama.cu/src/op/linear.rs:85-89).
+
+Which routine multiplies is decided here and nowhere else:
+
+* bfloat16 activations and weights, bfloat16 out: few rows (decoding) go to the
+  hand-written weight-streaming kernel, many rows to the library's matrix product
+  (hipBLASLt through torch), as the reference's engine calls its vendor library
+  (llama.cu/src/op/linear.rs:91-118);
+* everything else (float32 anywhere: the true 32-bit path, a weight that its file
+  stores in 32-bit, float32 logits): the hand-written kernel with 32-bit
+  multiply-adds.
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from ..kernels import ops
+
+
+def linear(x: torch.Tensor, weight: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
+           out: Optional[torch.Tensor] = None, accumulate: bool = False) -> torch.Tensor:
+    """``out (+)= x @ weight.T``.  ``accumulate`` adds into a float32 ``out`` in 32-bit."""
+    if not x.is_cuda:
+        raise ops.KernelError("linear: operands must be on the GPU (there is no CPU path)")
+    out_dtype = out.dtype if out is not None else (out_dtype or x.dtype)
+    all_bf16 = x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
+    if all_bf16 and ops.skinny_supported(x, weight, out_dtype):
+        return ops.gemm_skinny(x, weight, out=out, out_dtype=out_dtype, accumulate=accumulate)
+    if all_bf16 and out_dtype == torch.bfloat16 and not accumulate:
+        if out is None:
+            return torch.matmul(x, weight.t())
+        return torch.matmul(x, weight.t(), out=out)
+    return ops.gemm_nt(x, weight, out=out, out_dtype=out_dtype, accumulate=accumulate)

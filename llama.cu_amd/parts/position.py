@@ -1,0 +1,75 @@
+"""Position encodings of the attention mixer.
+
+A position encoding tells the attention mixer how queries and keys depend on a
+token's place.  The interface:
+
+  ``load(build)``                       make tables on the device
+  ``rotary_tables() -> (cos, sin, rot_dim, pairing) or None``
+        if not None, the mixer applies the rotation in the same kernel that writes
+        keys and values to the cache;
+  ``apply(qkv, positions, heads, kv_heads, head_dim)``
+        any other change of queries and keys, in place, before the cache write
+        (the default does nothing).
+"""
+from __future__ import annotations
+
+import numpy as np
+import torch
+
+from .base import BuildContext, Part, register_part
+
+
+class NoPosition(Part):
+    """Queries and keys are used as they are."""
+
+    def load(self, tensors, build: BuildContext) -> None:
+        pass
+
+    def rotary_tables(self):
+        return None
+
+    def apply(self, qkv, positions, heads, kv_heads, head_dim) -> None:
+        pass
+
+
+class Rotary(NoPosition):
+    """Rotation of pairs of dims by ``pos * theta^(-2i/rot_dim)``.
+
+    The tables follow llama.cu/src/model/mod.rs:200-209: the frequency
+    ``theta^(-2i/dh)`` and the angle ``pos * freq`` are 32-bit values; the table holds
+    the sine and cosine of that 32-bit angle (taken in 64-bit, rounded once).  The
+    pairing is a parameter: ``interleaved`` pairs neighbours ``(2i, 2i+1)`` as
+    llama.cu/src/op/rope.cuh:21-34 does; otherwise ``(i, i + rot_dim/2)``, the order in
+    which files with config.json's tensor names hold the rows of q and k.
+    """
+
+    def __init__(self, head_dim: int, theta: float, max_positions: int, interleaved: bool = False,
+                 rot_dim: int = 0):
+        self.head_dim = int(head_dim)
+        self.rot_dim = int(rot_dim) if rot_dim else int(head_dim)
+        if self.rot_dim % 2 or self.rot_dim > self.head_dim:
+            raise ValueError(f"rotary: rot_dim {self.rot_dim} must be even and at most head_dim {self.head_dim}")
+        self.theta = float(theta)
+        self.max_positions = int(max_positions)
+        self.interleaved = bool(interleaved)
+        self.cos = self.sin = None
+
+    def host_tables(self):
+        half = self.rot_dim // 2
+        i = np.arange(half, dtype=np.float64)
+        freq = np.power(np.float64(self.theta), -(2.0 * i) / self.rot_dim).astype(np.float32)
+        pos = np.arange(self.max_positions, dtype=np.float32)
+        ang = (pos[:, None] * freq[None, :]).astype(np.float32).astype(np.float64)   # the 32-bit product
+        return np.cos(ang).astype(np.float32), np.sin(ang).astype(np.float32)
+
+    def load(self, tensors, build: BuildContext) -> None:
+        cos, sin = self.host_tables()
+        self.cos = torch.from_numpy(cos).to(build.device).contiguous()
+        self.sin = torch.from_numpy(sin).to(build.device).contiguous()
+
+    def rotary_tables(self):
+        return self.cos, self.sin, self.rot_dim, 1 if self.interleaved else 0
+
+
+register_part("position", "none", NoPosition)
+register_part("position", "rotary", Rotary)

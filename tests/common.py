@@ -1,0 +1,208 @@
+"""Shared by the tests: the tiny configurations, model folders in temporary places,
+builders of traces, and the comparison with the plain implementation."""
+from __future__ import annotations
+
+import json
+import os
+import random
+import subprocess
+import sys
+import tempfile
+from typing import Dict, List, Optional, Sequence, Tuple
+
+import numpy as np
+import torch
+
+import plain
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+# Tiny configurations of the architecture that differ in every size and option.
+TINY_A = dict(architectures=["LlamaForCausalLM"], num_hidden_layers=2, hidden_size=64, num_attention_heads=4,
+              num_key_value_heads=4, head_dim=16, intermediate_size=172, vocab_size=256,
+              max_position_embeddings=128, rope_theta=10000.0, rms_norm_eps=1e-5, tie_word_embeddings=False)
+TINY_B = dict(architectures=["LlamaForCausalLM"], num_hidden_layers=3, hidden_size=128, num_attention_heads=4,
+              num_key_value_heads=1, head_dim=32, intermediate_size=352, vocab_size=384,
+              max_position_embeddings=256, rope_theta=500000.0, rms_norm_eps=1e-6, tie_word_embeddings=True)
+# no size a power of two, head_dim * heads != hidden_size, groups of 3, neighbour pairing, a large epsilon
+TINY_C = dict(architectures=["LlamaForCausalLM"], num_hidden_layers=1, hidden_size=80, num_attention_heads=6,
+              num_key_value_heads=2, head_dim=48, intermediate_size=100, vocab_size=301,
+              max_position_embeddings=200, rope_theta=777.0, rms_norm_eps=1e-3, tie_word_embeddings=False,
+              rope_interleaved=True)
+TINY = {"A": TINY_A, "B": TINY_B, "C": TINY_C}
+
+
+def make_folder(cfg_dict: dict, seed: int, dtype: torch.dtype, std: float = 0.15, folder: Optional[str] = None) -> str:
+    """A model folder with random weights, written by the test's own generator (so the
+    engine's writer is not what the comparison rests on)."""
+    folder = folder or tempfile.mkdtemp(prefix="lcu_model_")
+    pcfg = plain.PlainConfig.from_dict(cfg_dict)
+    w = plain.random_weights(pcfg, seed, std=std)
+    w = {k: v.to(dtype) for k, v in w.items()}
+    sys.path.insert(0, ROOT)
+    from llama_cu_amd.weights import write_safetensors
+    with open(os.path.join(folder, "config.json"), "w") as f:
+        json.dump(cfg_dict, f)
+    write_safetensors(os.path.join(folder, "model.safetensors"), w)
+    return folder
+
+
+def random_requests(vocab: int, lengths: Sequence[int], seed: int) -> Dict[str, List[int]]:
+    rng = random.Random(seed)
+    return {f"r{i}": [rng.randrange(vocab) for _ in range(n)] for i, n in enumerate(lengths)}
+
+
+def plain_logits(folder: str, reqs: Dict[str, List[int]]) -> Dict[str, torch.Tensor]:
+    cfg, w = plain.load_folder(folder)
+    return {name: plain.forward(cfg, w, toks) for name, toks in reqs.items()}
+
+
+# ----------------------------------------------------------------------------- traces
+def ceil64(n: int) -> int:
+    return (n + 63) // 64 * 64
+
+
+def trace_whole(reqs):
+    """Each request alone and whole: one step with all its tokens, all logits wanted."""
+    steps = []
+    for name, toks in reqs.items():
+        steps.append({"step": len(steps), "entries": [{"id": name, "tokens": toks, "want": list(range(len(toks)))}],
+                      "end": [name]})
+    return steps, max(ceil64(len(t)) for t in reqs.values())
+
+
+def trace_tail_decode(reqs, tail=32):
+    """Most of a request in one step, its last ``tail`` tokens one by one."""
+    steps = []
+    for name, toks in reqs.items():
+        head = max(len(toks) - tail, 0)
+        if head:
+            steps.append({"step": len(steps), "entries": [{"id": name, "tokens": toks[:head], "want": list(range(head))}], "end": []})
+        for i in range(head, len(toks)):
+            steps.append({"step": len(steps), "entries": [{"id": name, "tokens": [toks[i]], "want": [0]}],
+                          "end": [name] if i == len(toks) - 1 else []})
+    return steps, max(ceil64(len(t)) for t in reqs.values())
+
+
+def trace_portions(reqs, sizes=(7, 2, 16, 3, 48, 2, 1, 33, 5, 2)):
+    """Portions of changing size, down to two tokens (and one), across page edges."""
+    steps = []
+    k = 0
+    for name, toks in reqs.items():
+        fed = 0
+        while fed < len(toks):
+            n = min(sizes[k % len(sizes)], len(toks) - fed)
+            k += 1
+            steps.append({"step": len(steps), "entries": [{"id": name, "tokens": toks[fed:fed + n], "want": list(range(n))}],
+                          "end": [name] if fed + n == len(toks) else []})
+            fed += n
+    return steps, max(ceil64(len(t)) for t in reqs.values())
+
+
+def trace_mixed(reqs, seed=0, max_live=4, tail=12):
+    """Up to ``max_live`` requests at a time: portions of some beside single tokens of
+    others; requests sit steps out; finished requests' pages go to the next ones.  Returns
+    the steps and the smallest ``--max-tokens`` that holds them."""
+    rng = random.Random(seed)
+    pending = list(reqs.items())
+    live: Dict[str, int] = {}
+    steps = []
+    need = 0
+    while pending or live:
+        while pending and len(live) < max_live and (not live or rng.random() < 0.6):
+            name, _ = pending.pop(0)
+            live[name] = 0
+        entries, end = [], []
+        names = list(live)
+        for name in names:
+            toks, fed = reqs[name], live[name]
+            remaining = len(toks) - fed
+            if len(names) > 1 and rng.random() < 0.25:
+                continue                                   # sits this step out
+            if remaining <= tail:
+                n = 1
+            else:
+                n = min(remaining - tail, rng.choice([2, 2, 3, 5, 7, 16, 17, 31, 48]))
+            entries.append({"id": name, "tokens": toks[fed:fed + n], "want": list(range(n))})
+            live[name] = fed + n
+        if not entries:
+            name = names[0]
+            toks, fed = reqs[name], live[name]
+            entries.append({"id": name, "tokens": toks[fed:fed + 1], "want": [0]})
+            live[name] = fed + 1
+        need = max(need, sum(ceil64(v) for v in live.values()))
+        for name in list(live):
+            if live[name] == len(reqs[name]):
+                end.append(name)
+                del live[name]
+        steps.append({"step": len(steps), "entries": entries, "end": end})
+    return steps, need
+
+
+def collect(steps, outputs: Dict[int, np.ndarray], vocab: int) -> Dict[str, Dict[int, np.ndarray]]:
+    """Logits by request and position from the per-step outputs of a replay."""
+    fed: Dict[str, int] = {}
+    got: Dict[str, Dict[int, np.ndarray]] = {}
+    for st in steps:
+        out = outputs.get(st["step"])
+        row = 0
+        for e in st["entries"]:
+            base = fed.get(e["id"], 0)
+            for k in e.get("want", []):
+                got.setdefault(e["id"], {})[base + k] = out[row]
+                row += 1
+            fed[e["id"]] = base + len(e["tokens"])
+        if out is not None:
+            assert out.shape == (row, vocab), (out.shape, row, vocab)
+    return got
+
+
+def run_trace_inprocess(folder: str, dtype: str, steps, max_tokens: int) -> Dict[int, np.ndarray]:
+    sys.path.insert(0, ROOT)
+    import llama_cu_amd  # noqa: F401
+    from llama_cu_amd.engine.trace import TraceReplayer
+    rep = TraceReplayer(folder, dtype, max_tokens)
+    outputs = {}
+    for st in steps:
+        out = rep.step(st)
+        if out is not None:
+            outputs[st["step"]] = out
+    rep.runner.cache.check()
+    assert rep.runner.cache.live_requests() == 0
+    assert rep.runner.cache.free_pages(0) == rep.runner.num_pages
+    return outputs
+
+
+def run_trace_program(folder: str, dtype: str, steps, max_tokens: int, vocab: int) -> Dict[int, np.ndarray]:
+    """Through ``bin/trace_run`` as a user runs it."""
+    out_dir = tempfile.mkdtemp(prefix="lcu_trace_")
+    text = "".join(json.dumps(s) + "\n" for s in steps)
+    proc = subprocess.run([os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", dtype, "--out", out_dir,
+                           "--max-tokens", str(max_tokens)], input=text, capture_output=True, text=True, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    done = [l for l in proc.stdout.splitlines() if l.startswith("done ")]
+    assert done == [f"done {s['step']}" for s in steps]
+    outputs = {}
+    for s in steps:
+        p = os.path.join(out_dir, f"{s['step']}.f32")
+        if os.path.exists(p):
+            outputs[s["step"]] = np.fromfile(p, dtype="<f4").reshape(-1, vocab)
+    return outputs
+
+
+# tolerances, as a fraction of the largest logit of the sequence (set from the formats'
+# precision, not from what passes): float32 rounds at 6e-8 and sums a few hundred terms;
+# bfloat16 activations round at 4e-3 about ten times per layer.
+REL_TOL = {"float32": 1e-4, "bfloat16": 5e-2}
+
+
+def assert_matches_plain(got: Dict[str, Dict[int, np.ndarray]], want: Dict[str, torch.Tensor], dtype: str, what: str):
+    rel = REL_TOL[dtype]
+    for name, logits in want.items():
+        ref = logits.numpy()
+        scale = float(np.abs(ref).max())
+        assert set(got.get(name, {})) == set(range(ref.shape[0])), f"{what}: request {name}: positions missing"
+        for pos in range(ref.shape[0]):
+            err = float(np.abs(got[name][pos].astype(np.float64) - ref[pos]).max())
+            assert np.isfinite(err) and err <= rel * scale, \
+                f"{what}: request {name}, first wrong position {pos} of {ref.shape[0]}: error {err:.3e} > {rel * scale:.3e}"
