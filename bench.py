@@ -1,0 +1,172 @@
+#!/usr/bin/python3
+"""Measurement: decoded tokens a second of the Llama-3-8B shape on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A step is one decode step of the whole batch through the engine (scheduler, step
+function, sampling): W untimed steps, then exactly K timed ones between two
+synchronisations.  The default run has the layer sizes of the Llama-3-8B shape with random
+weights, a batch of 8 requests with prompts of 2,048 uniform random tokens and a context
+limit of 8,192.  One JSON line comes out: decoded tokens a second (``value``), the time of
+a 2,048-token prefill with its fraction of the bf16 matrix peak, the decode step's bytes
+against the HBM peak, and decoding at batch 1 and 64 (``points``).
+
+Peaks are MI355X's published ones: HBM 8 TB/s; dense matrix bf16 2.5 PFLOP/s, fp32
+157.3 TFLOP/s.  The reference publishes no numbers, so ``vs_baseline`` is null.
+"""
+import argparse
+import json
+import os
+import random
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK = 8.0e12
+MATRIX_PEAK = {"bf16": 2.5e15, "f32": 157.3e12}
+
+# BASELINE.json configs[2]: the Llama-3-8B shape
+SHAPE = dict(architectures=["LlamaForCausalLM"], num_hidden_layers=32, hidden_size=4096, num_attention_heads=32,
+             num_key_value_heads=8, head_dim=128, intermediate_size=14336, vocab_size=128256,
+             max_position_embeddings=8192, rope_theta=500000.0, rms_norm_eps=1e-5, tie_word_embeddings=False)
+PROMPT_LEN = 2048
+PREFILL_TOKENS = 2048
+
+
+def weight_bytes(c, elem):
+    """Bytes of the weights a decode step reads once: every matrix and norm weight (of the
+    embedding table only the batch's rows, which is negligible and left out)."""
+    d, dh, nh, nkv, di = c.hidden_size, c.head_dim, c.num_attention_heads, c.num_key_value_heads, c.intermediate_size
+    per_layer = (nh + 2 * nkv) * dh * d + d * nh * dh + 2 * di * d + d * di + 2 * d
+    return (c.num_hidden_layers * per_layer + d + c.vocab_size * d) * elem
+
+
+def kv_bytes_per_token(c, elem):
+    return c.num_hidden_layers * 2 * c.num_key_value_heads * c.head_dim * elem
+
+
+def prefill_flops(c, t):
+    d, dh, nh, nkv, di = c.hidden_size, c.head_dim, c.num_attention_heads, c.num_key_value_heads, c.intermediate_size
+    per_token = 2 * ((nh + 2 * nkv) * dh * d + d * nh * dh + 2 * di * d + d * di)
+    matmul = c.num_hidden_layers * per_token * t + 2 * c.vocab_size * d      # the output matrix for the last row only
+    attention = c.num_hidden_layers * 2 * 2 * nh * dh * t * (t + 1) / 2      # causal: QK^T and PV over t(t+1)/2 pairs
+    return matmul + attention
+
+
+def run_decode(engine, cfg, batch, steps, warmup, rng, sync):
+    """Prefill ``batch`` prompts, then time ``steps`` decode steps.  Returns (seconds,
+    tokens decoded in them, mean context length during the timed steps)."""
+    from llama_cu_amd.sampling import GREEDY
+    ids = [engine.add_request([rng.randrange(cfg.vocab_size) for _ in range(PROMPT_LEN)], GREEDY,
+                              max_steps=steps + warmup + 2 * batch + 8, ignore_eos=True) for _ in range(batch)]
+    # prefill rounds: until every request has produced its first token
+    while any(engine.sched.info(i).generated == 0 for i in ids):
+        engine.step()
+    for _ in range(warmup):
+        engine.step()
+    ctx0 = engine.sched.info(ids[0]).n_tokens
+    sync()
+    t0 = time.perf_counter()
+    produced = 0
+    for _ in range(steps):
+        produced += sum(1 for o in engine.step() if o.token is not None)
+    sync()
+    dt = time.perf_counter() - t0
+    ctx1 = engine.sched.info(ids[0]).n_tokens
+    for i in ids:
+        engine.abort(i)
+        engine.drop(i)
+    assert produced == batch * steps, (produced, batch, steps)
+    return dt, produced, (ctx0 + ctx1) / 2.0
+
+
+def run_prefill(engine, cfg, rng, sync, repeats=3):
+    """Best time of one step that feeds a whole prompt of PREFILL_TOKENS tokens."""
+    best = None
+    for k in range(repeats + 1):
+        toks = [rng.randrange(cfg.vocab_size) for _ in range(PREFILL_TOKENS)]
+        rid = 10_000 + k
+        sync()
+        t0 = time.perf_counter()
+        engine.runner.step([rid], [toks])
+        sync()
+        dt = time.perf_counter() - t0
+        engine.runner.end(rid)
+        if k > 0:                                   # the first run warms up
+            best = dt if best is None else min(best, dt)
+    return best
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=128)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--layers", type=int, default=None, help="fewer layers than the shape has (named in config)")
+    ap.add_argument("--dtype", choices=["bfloat16", "float32"], default="bfloat16")
+    ap.add_argument("--no-points", action="store_true", help="skip decoding at batch 1 and 64 and the prefill")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported (no multi-GPU path)")
+        return 2
+
+    import torch
+    import llama_cu_amd  # noqa: F401
+    from llama_cu_amd.config import LlamaConfig
+    from llama_cu_amd.engine.engine import Engine
+
+    shape = dict(SHAPE)
+    full_layers = shape["num_hidden_layers"]
+    if args.layers:
+        shape["num_hidden_layers"] = args.layers
+    cfg = LlamaConfig.from_dict(shape)
+    dt_name = "bf16" if args.dtype == "bfloat16" else "f32"
+    elem = 2 if args.dtype == "bfloat16" else 4
+    rng = random.Random(0)
+    sync = torch.cuda.synchronize
+    page = 16
+    biggest = max(args.batch, 1 if args.no_points else 64)
+    # a request decodes while later ones still prefill: room for that too
+    per_req = PROMPT_LEN + args.steps + args.warmup + 2 * biggest + 64
+    engine = Engine.from_config(cfg, seed=0, dtype=args.dtype, page_size=page,
+                                max_tokens=biggest * ((per_req + page - 1) // page * page) + PREFILL_TOKENS + page,
+                                max_seqs=biggest + 2, max_batch_tokens=max(PREFILL_TOKENS, biggest), prefill_chunk=PREFILL_TOKENS)
+
+    seconds, produced, mean_ctx = run_decode(engine, cfg, args.batch, args.steps, args.warmup, rng, sync)
+    ms_per_step = seconds / args.steps * 1e3
+    value = produced / seconds
+    step_bytes = weight_bytes(cfg, elem) + args.batch * mean_ctx * kv_bytes_per_token(cfg, elem)
+    achieved = step_bytes / (seconds / args.steps)
+    line = {
+        "metric": "decode tok/s (Llama-3-8B shape, prompts of 2048 tokens)", "value": round(value, 2), "unit": "tok/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": dt_name, "data": "synthetic",
+        "config": {"model": "Llama-3-8B shape, random weights", "global_batch": args.batch, "seq_len": PROMPT_LEN,
+                   "parallelism": "none (1 GPU)", "context": cfg.max_position_embeddings,
+                   "layers": cfg.num_hidden_layers, "layers_of_shape": full_layers, "hidden_size": cfg.hidden_size,
+                   "heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads, "head_dim": cfg.head_dim,
+                   "intermediate_size": cfg.intermediate_size, "vocab_size": cfg.vocab_size,
+                   "rope_theta": cfg.rope_theta, "rms_norm_eps": cfg.rms_norm_eps, "page_size": page,
+                   "sampling": "greedy"},
+        "roofline": {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK, 4)},
+    }
+    if not args.no_points:
+        pt = run_prefill(engine, cfg, rng, sync)
+        flops = prefill_flops(cfg, PREFILL_TOKENS)
+        line["prefill"] = {"value": round(PREFILL_TOKENS / pt, 1), "tokens": PREFILL_TOKENS, "ms": round(pt * 1e3, 3),
+                           "frac": round(flops / pt / MATRIX_PEAK[dt_name], 4)}
+        points = {}
+        for b in (1, 64):
+            s, p, _ = run_decode(engine, cfg, b, max(16, args.steps // 4), 4, rng, sync)
+            points[f"decode_b{b}"] = round(p / s, 2)
+        line["points"] = points
+    print(json.dumps(line), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

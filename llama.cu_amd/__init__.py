@@ -8,4 +8,28 @@ from . import config, parts, models, weights  # noqa: F401
 from .config import LlamaConfig, register_architecture
 from .parts import register_part
 
-__all__ = ["config", "parts", "models", "weights", "LlamaConfig", "register_architecture", "register_part"]
+from .sampling import SamplingParams
+
+
+def Engine(model: str, dtype: str = "bfloat16", device: str = "cuda:0", **kw):
+    """The engine for the model folder ``model`` (see engine.engine.Engine)."""
+    from .engine.engine import Engine as _Engine
+    return _Engine.from_folder(model, dtype=dtype, device=device, **kw)
+
+
+def generate(model: str, prompts, sampling: SamplingParams = SamplingParams(), max_steps: int = 1000,
+             dtype: str = "bfloat16", device: str = "cuda:0", **kw):
+    """Generate for ``prompts`` (lists of token ids, or strings that the folder's tokenizer
+    encodes) with the model of the folder ``model``; returns token ids, or strings for
+    string prompts."""
+    from . import text
+    engine = Engine(model, dtype=dtype, device=device, **kw)
+    as_text = len(prompts) > 0 and isinstance(prompts[0], str)
+    tok = text.load_tokenizer(model, engine.runner.spec.vocab_size) if as_text else None
+    ids = [tok.encode(p) for p in prompts] if as_text else [list(p) for p in prompts]
+    out = engine.generate(ids, sampling, max_steps)
+    return [tok.decode(o) for o in out] if as_text else out
+
+
+__all__ = ["config", "parts", "models", "weights", "LlamaConfig", "register_architecture", "register_part",
+           "SamplingParams", "Engine", "generate"]

@@ -1,0 +1,132 @@
+"""The command line, in the manner of the reference's ``xtask``
+(llama.cu/xtask/src/main.rs:25-73): ``generate MODEL [--max-steps N] [-p PROMPT] [-t]`` and
+``chat MODEL [--max-steps N]``.  ``--gpus``, ``--no-cuda-graph``, ``--tui`` and the
+``service`` and ``bench`` subcommands are not here: one GPU, no server.  Added: the
+compute type and the sampling options.
+"""
+from __future__ import annotations
+
+import argparse
+import sys
+import time
+from typing import List, Optional
+
+
+def _base(p: argparse.ArgumentParser) -> None:
+    p.add_argument("model", metavar="MODEL", help="model folder (config.json, model.safetensors[, tokenizer.json])")
+    p.add_argument("--max-steps", type=int, default=1000, help="most tokens to generate (default 1000)")
+    p.add_argument("--dtype", choices=["bfloat16", "float32"], default="bfloat16")
+    p.add_argument("--temperature", type=float, default=0.0)
+    p.add_argument("--top-p", type=float, default=1.0)
+    p.add_argument("--top-k", type=int, default=None)
+    p.add_argument("--seed", type=int, default=0)
+    p.add_argument("--max-tokens", type=int, default=None, help="size of the cache pool in tokens (default: from free memory)")
+
+
+def _engine(args):
+    from . import text
+    from .engine.engine import Engine
+    from .sampling import SamplingParams, TOP_K_ALL
+    kw = {}
+    if args.max_tokens:
+        kw["max_tokens"] = args.max_tokens
+    t0 = time.time()
+    engine = Engine.from_folder(args.model, dtype=args.dtype, max_seqs=4, **kw)
+    print(f"[info] model ready in {time.time() - t0:.2f} s", file=sys.stderr)
+    params = SamplingParams(args.temperature, args.top_p, args.top_k or TOP_K_ALL, args.seed)
+    tok = text.load_tokenizer(args.model, engine.runner.spec.vocab_size)
+    return engine, params, tok
+
+
+def _stream(engine, rid: int, decoder, out=sys.stdout):
+    """Run rounds until request ``rid`` ends; print its text as it comes.  Returns (time of
+    the first round, time of the later rounds, tokens)."""
+    prefill = decode = 0.0
+    ntoks = 0
+    first = True
+    while True:
+        t = time.time()
+        results = engine.step()
+        dt = time.time() - t
+        if first:
+            prefill, first = dt, False
+        else:
+            decode += dt
+        done = False
+        for o in results:
+            if o.req != rid:
+                continue
+            if o.token is not None:
+                ntoks += 1
+                out.write(decoder.push(o.token))
+                out.flush()
+            done = done or o.finished is not None
+        if done or engine.idle:
+            return prefill, decode, ntoks
+
+
+def generate(args) -> int:
+    """llama.cu/xtask/src/generate.rs:16-69: echo the prompt, stream the continuation, then
+    report prefill time, decode time, tokens, time per token and tokens per second."""
+    from . import text
+    engine, params, tok = _engine(args)
+    prompt = args.prompt if args.prompt is not None else "Once upon a time,"
+    sys.stdout.write(prompt)
+    sys.stdout.flush()
+    if args.use_template:
+        prompt = text.load_chat_template(args.model).render([text.user(prompt)])
+    rid = engine.add_request(tok.encode(prompt), params, args.max_steps)
+    prefill, decode, ntoks = _stream(engine, rid, text.StreamDecoder(tok))
+    print()
+    print(f"[info] prefill = {prefill * 1e3:.2f} ms, decode = {decode * 1e3:.2f} ms", file=sys.stderr)
+    if ntoks > 1 and decode > 0:
+        per = decode / (ntoks - 1)
+        print(f"[info] n toks = {ntoks}, perf: {per * 1e3:.3f} ms/tok, {1 / per:.1f} tok/s", file=sys.stderr)
+    return 0
+
+
+def chat(args) -> int:
+    """llama.cu/xtask/src/chat/mod.rs:38-77: one session whose cache lives across turns."""
+    from . import text
+    engine, params, tok = _engine(args)
+    template = text.load_chat_template(args.model)
+    rid: Optional[int] = None
+    while True:
+        line = ""
+        while not line:
+            sys.stdout.write("user> ")
+            sys.stdout.flush()
+            raw = sys.stdin.readline()
+            if not raw:
+                print()
+                return 0
+            line = raw.rstrip("\n")
+        tokens = tok.encode(template.render([text.user(line)]))
+        if rid is None:
+            rid = engine.add_request(tokens, params, args.max_steps, keep=True)
+        else:
+            engine.continue_request(rid, tokens, args.max_steps)
+        sys.stdout.write("assistant> ")
+        sys.stdout.flush()
+        _stream(engine, rid, text.StreamDecoder(tok))
+        print()
+        print("=== over ===")
+        if engine.sched.info(rid).reason == "length":
+            print("[info] the context is full; starting a new session", file=sys.stderr)
+            engine.drop(rid)
+            rid = None
+
+
+def main(argv: Optional[List[str]] = None) -> int:
+    ap = argparse.ArgumentParser(prog="llama.cu_amd")
+    sub = ap.add_subparsers(dest="command", required=True)
+    g = sub.add_parser("generate", help="text generation")
+    _base(g)
+    g.add_argument("-p", "--prompt", default=None)
+    g.add_argument("-t", "--use-template", action="store_true")
+    g.set_defaults(func=generate)
+    c = sub.add_parser("chat", help="chat in console")
+    _base(c)
+    c.set_defaults(func=chat)
+    args = ap.parse_args(argv)
+    return args.func(args)

@@ -60,6 +60,7 @@ int Scheduler::drop(int64_t id) {
     if (it->second.reason == NOT_FINISHED) return CACHE_BAD_ARGUMENT;
     if (cache_->has(id)) cache_->release(id);
     reqs_.erase(it);
+    finished_.erase(std::remove(finished_.begin(), finished_.end(), id), finished_.end());
     return CACHE_OK;
 }
 

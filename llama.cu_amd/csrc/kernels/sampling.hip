@@ -7,13 +7,14 @@
 // 186-207, with library sort, scan and reduce).  The same token comes out here without
 // sorting: the entry with c[i] >= p is found by a radix select over the bit patterns of
 // the logits, most significant byte first, on histograms of counts and of weights.
-// Weights are summed as 64-bit fixed-point integers (w * 2^40), so the sums do not
+// Weights are summed as 64-bit fixed-point integers (w * 2^45), so the sums do not
 // depend on the order of the additions and a draw is reproducible bit for bit.  Equal
 // logits are ordered by index, as a stable sort orders them.
 #include "common.h"
 
 constexpr int SAMPLE_THREADS = 1024;
-constexpr double FIXED_ONE = 1099511627776.0;   // 2^40
+constexpr double FIXED_ONE = 35184372088832.0;   // 2^45: the sum of 2^19 weights of 1 still fits 64 bits
+constexpr int MAX_VOCAB = 1 << 19;
 
 __device__ __forceinline__ uint32_t order_key(float x) {
     // ascending float order -> ascending unsigned order
@@ -210,7 +211,7 @@ sample_kernel(const float *__restrict__ logits, int ld, int vocab, const float *
 LCU_API int lcu_sample(const float *logits, int ld, int rows, int vocab, const float *temperature, const float *top_p,
                        const int *top_k, const float *uniform, int *out, hipStream_t stream) {
     if (rows <= 0) return LCU_OK;
-    if (vocab <= 0 || ld < vocab) return LCU_BAD_ARGUMENT;
+    if (vocab <= 0 || vocab > MAX_VOCAB || ld < vocab) return LCU_BAD_ARGUMENT;
     sample_kernel<<<dim3(rows), dim3(SAMPLE_THREADS), 0, stream>>>(logits, ld, vocab, temperature, top_p, top_k, uniform, out);
     LCU_LAUNCH_CHECK();
     return LCU_OK;

@@ -48,7 +48,8 @@ def require_gpu(device) -> torch.device:
 class ModelRunner:
     def __init__(self, spec: ModelSpec, tensors: Dict[str, torch.Tensor], dtype, device="cuda:0",
                  page_size: int = 16, max_tokens: Optional[int] = None, num_pages: Optional[int] = None,
-                 max_seqs: int = 8, max_batch_tokens: int = 2048, max_model_len: Optional[int] = None):
+                 max_seqs: int = 8, max_batch_tokens: int = 2048, max_model_len: Optional[int] = None,
+                 kv_fraction: float = 0.85):
         self.device = require_gpu(device)
         self.dtype = DTYPES[dtype]
         self.spec = spec
@@ -65,10 +66,16 @@ class ModelRunner:
         # cache groups: one per distinct window among the layers that page keys and values
         needs = self.model.cache_needs()
         windows = sorted({n.window for n in needs if isinstance(n, PagedKV)})
-        if num_pages is None:
-            if max_tokens is None:
-                raise ValueError("give max_tokens or num_pages for the cache pool")
+        if num_pages is None and max_tokens is not None:
             num_pages = (int(max_tokens) + self.page_size - 1) // self.page_size
+        if num_pages is None:
+            # what the free memory holds, and no more than every slot filled to the limit
+            elem = torch.empty(0, dtype=self.dtype).element_size()
+            page_bytes = sum(2 * n.kv_heads * n.head_dim * self.page_size * elem for n in needs if isinstance(n, PagedKV))
+            free, _ = torch.cuda.mem_get_info(self.device)
+            by_memory = int(free * kv_fraction) // max(page_bytes, 1)
+            by_need = self.max_seqs * ((self.max_model_len + self.page_size - 1) // self.page_size)
+            num_pages = max(1, min(by_memory, by_need))
         self.num_pages = int(num_pages)
         self.groups = [CacheGroup(self.num_pages, self.page_size, w) for w in windows]
         self.cache = CacheManager(self.groups, self.max_seqs)

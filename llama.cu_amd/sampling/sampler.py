@@ -1,0 +1,88 @@
+"""Sampling on the device from rows of float32 logits (kernels: csrc/kernels/sampling.hip).
+
+The uniform number of a draw comes from a counter-based generator keyed by the
+request's seed, its id and the index of the token it draws: a request's tokens do not
+depend on what else is in the batch or on how its prompt was cut.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import List, Sequence, Tuple
+
+import torch
+
+from ..kernels import build
+from ..kernels.ops import KernelError, _check, _gpu, _ptr, _stream
+from .params import SamplingParams
+
+_MASK = (1 << 64) - 1
+
+
+def _splitmix64(x: int) -> int:
+    x = (x + 0x9E3779B97F4A7C15) & _MASK
+    z = x
+    z = ((z ^ (z >> 30)) * 0xBF58476D1CE4E5B9) & _MASK
+    z = ((z ^ (z >> 27)) * 0x94D049BB133111EB) & _MASK
+    return z ^ (z >> 31)
+
+
+def uniform(seed: int, request: int, index: int) -> float:
+    """A number in [0, 1) with 24 random bits, a pure function of its three keys."""
+    h = _splitmix64(seed & _MASK)
+    h = _splitmix64(h ^ (request & _MASK))
+    h = _splitmix64(h ^ (index & _MASK))
+    return (h >> 40) / float(1 << 24)
+
+
+def argmax(logits: torch.Tensor) -> torch.Tensor:
+    """The index of the largest logit of each row (the lowest among equals), int32."""
+    _gpu(logits)
+    if logits.dim() != 2 or logits.dtype != torch.float32 or logits.stride(1) != 1:
+        raise KernelError("argmax: logits must be float32 [rows, vocab] with contiguous rows")
+    out = torch.empty(logits.shape[0], dtype=torch.int32, device=logits.device)
+    lib = build.load("sampling")
+    _check(lib.lcu_argmax(_ptr(logits), logits.stride(0), logits.shape[0], logits.shape[1], _ptr(out), _stream()),
+           "argmax")
+    return out
+
+
+def sample_rows(logits: torch.Tensor, temperature: Sequence[float], top_p: Sequence[float], top_k: Sequence[int],
+                u: Sequence[float]) -> torch.Tensor:
+    """One draw per row with the row's temperature (> 0), top_p, top_k and uniform number."""
+    _gpu(logits)
+    if logits.dim() != 2 or logits.dtype != torch.float32 or logits.stride(1) != 1:
+        raise KernelError("sample: logits must be float32 [rows, vocab] with contiguous rows")
+    rows, vocab = logits.shape
+    if not (len(temperature) == len(top_p) == len(top_k) == len(u) == rows):
+        raise KernelError("sample: one temperature, top_p, top_k and uniform number per row")
+    if any(not t > 0 for t in temperature) or any(not 0 <= x < 1 for x in u):
+        raise KernelError("sample: temperatures must be > 0 and uniform numbers in [0, 1)")
+    dev = logits.device
+    fl = torch.tensor([list(temperature), list(top_p), list(u)], dtype=torch.float32).to(dev)
+    kk = torch.tensor([min(int(k), vocab) for k in top_k], dtype=torch.int32).to(dev)
+    out = torch.empty(rows, dtype=torch.int32, device=dev)
+    lib = build.load("sampling")
+    _check(lib.lcu_sample(_ptr(logits), logits.stride(0), rows, vocab, _ptr(fl[0]), _ptr(fl[1]), _ptr(kk), _ptr(fl[2]),
+                          _ptr(out), _stream()), "sample")
+    return out
+
+
+class Sampler:
+    def sample(self, logits: torch.Tensor, params: Sequence[SamplingParams],
+               keys: Sequence[Tuple[int, int]]) -> List[int]:
+        """A token for every row.  ``keys[i] = (request id, index of the drawn token)``."""
+        rows = logits.shape[0]
+        if rows == 0:
+            return []
+        greedy = argmax(logits)
+        random_rows = [i for i, p in enumerate(params) if not p.is_argmax]
+        if not random_rows:
+            return greedy.tolist()
+        sub = logits if len(random_rows) == rows else logits[torch.tensor(random_rows, device=logits.device)]
+        drawn = sample_rows(sub, [params[i].temperature for i in random_rows], [params[i].top_p for i in random_rows],
+                            [params[i].top_k for i in random_rows],
+                            [uniform(params[i].seed, keys[i][0], keys[i][1]) for i in random_rows]).tolist()
+        out = greedy.tolist()
+        for i, t in zip(random_rows, drawn):
+            out[i] = t
+        return out

@@ -1,0 +1,87 @@
+"""The sampling kernels alone, against the plain sampler, at other sizes than the engine's."""
+import numpy as np
+import pytest
+import torch
+
+import plain
+
+pytestmark = pytest.mark.gpu
+
+
+def _logits(rows, vocab, seed, scale=3.0):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randn(rows, vocab, generator=g) * scale
+
+
+@pytest.mark.parametrize("vocab", [1, 7, 256, 1000, 4097, 128256])
+def test_argmax_lowest_index_among_equals(vocab):
+    from llama_cu_amd.sampling import argmax
+    l = _logits(5, vocab, vocab)
+    if vocab > 6:
+        l[1, 3] = l[1, vocab - 2] = 50.0            # equal maxima: the lower index wins
+        l[2, vocab - 1] = 60.0
+    got = argmax(l.cuda()).tolist()
+    assert got == [plain.sample(r, 0.0, 1.0, 10 ** 9, 0.5) for r in l]
+
+
+@pytest.mark.parametrize("vocab,temperature,top_p,top_k", [
+    (50, 1.0, 1.0, 10 ** 9), (301, 0.8, 1.0, 10 ** 9), (1000, 0.7, 0.9, 10 ** 9), (1000, 1.3, 1.0, 5),
+    (4097, 0.5, 0.5, 40), (128256, 0.8, 0.95, 50), (128256, 1.0, 1.0, 10 ** 9)])
+def test_sample_kernel_matches_plain_sampler(vocab, temperature, top_p, top_k):
+    """The same uniform number gives the same token, except where it falls within rounding
+    of the boundary between two tokens (then either is accepted)."""
+    from llama_cu_amd.sampling import sample_rows
+    rows = 24
+    l = _logits(rows, vocab, 17 + vocab)
+    l[3, 5 % vocab] = l[3, 11 % vocab]              # equal logits inside a row
+    rng = np.random.default_rng(vocab)
+    u = [0.0, 0.999999] + [float(x) for x in rng.random(rows - 2)]
+    got = sample_rows(l.cuda(), [temperature] * rows, [top_p] * rows, [top_k] * rows, u).tolist()
+    for r in range(rows):
+        want = plain.sample(l[r], temperature, top_p, top_k, u[r])
+        if got[r] != want:
+            _assert_draw_within_rounding(l[r], temperature, top_p, top_k, u[r], got[r])
+
+
+def _assert_draw_within_rounding(logits, temperature, top_p, top_k, u, token, tol=2e-6):
+    """``token`` is the right answer for a number within ``tol`` of ``u``: in the sorted
+    order of llama.cu/src/op/random_sample/sample.cuh:186-207 its span of the cumulative
+    weights, widened by ``tol`` of the limit, holds ``u * limit``."""
+    x = logits.double()
+    order = torch.sort(x, descending=True, stable=True).indices
+    w = torch.exp((x[order] - x[order][0]) / temperature)
+    c = torch.cumsum(w, 0)
+    k = min(top_k, x.numel())
+    limit = min(top_p * float(c[-1]), float(c[k - 1]))
+    i = int((order == token).nonzero()[0])
+    lo = float(c[i - 1]) if i else 0.0
+    assert lo - tol * limit <= u * limit <= float(c[i]) + tol * limit, (token, i, u, lo / limit, float(c[i]) / limit)
+
+
+def test_sample_frequencies_follow_the_cut_softmax():
+    from llama_cu_amd.sampling import sample_rows
+    vocab, n = 40, 20000
+    l = _logits(1, vocab, 5, scale=1.5)[0]
+    rng = np.random.default_rng(1)
+    u = [float(x) for x in rng.random(n)]
+    T, k = 0.9, 7
+    got = sample_rows(l.repeat(n, 1).cuda(), [T] * n, [1.0] * n, [k] * n, u).cpu().numpy()
+    p = torch.softmax(l.double() / T, 0).numpy()
+    keep = np.argsort(-p)[:k]
+    q = np.zeros(vocab); q[keep] = p[keep]; q /= q.sum()
+    freq = np.bincount(got, minlength=vocab) / n
+    assert np.abs(freq - q).max() < 0.015
+    assert freq[[i for i in range(vocab) if i not in keep]].sum() == 0
+
+
+def test_per_row_parameters_and_sampler_mix():
+    from llama_cu_amd.sampling import Sampler, SamplingParams, uniform
+    l = _logits(4, 500, 9)
+    params = [SamplingParams(), SamplingParams(temperature=0.8, seed=3), SamplingParams(temperature=1.0, top_k=1),
+              SamplingParams(temperature=1.2, top_p=0.7, top_k=20, seed=5)]
+    keys = [(0, 10), (1, 11), (2, 12), (3, 13)]
+    got = Sampler().sample(l.cuda(), params, keys)
+    for r in range(4):
+        p = params[r]
+        want = plain.sample(l[r], p.temperature, p.top_p, min(p.top_k, 10 ** 9), uniform(p.seed, *keys[r]))
+        assert got[r] == want
