@@ -1,0 +1,416 @@
+// Causal attention over the paged cache on the matrix cores, for bfloat16.
+//
+// Both kernels work on the transposed problem, so that nothing has to move between
+// lanes or through LDS between the two matrix products:
+//   S^T[key, q] = K[key, :] . Q[q, :]      v_mfma_f32_16x16x32_bf16, A = K (a lane holds 8
+//                                          dims of one key: one 16-byte load in the cache's
+//                                          key layout), B = Q (kept in registers)
+//   O^T[dim, q] += V^T[dim, key] . P^T[key, q]   A = V^T (a lane holds tokens of one dim:
+//                                          8-byte loads in the cache's value layout),
+//                                          B = P^T: exactly the lane's own S^T values
+// In S^T a lane owns one query row (lane % 16) and 8 of each 32 keys, so the softmax's
+// maximum and sum run over a lane's registers and two cross-lane steps.  Scores, the
+// running maximum and sum and the output are 32-bit; P is rounded to bfloat16 for the
+// second product.
+//
+// A "row" is one (token, head) pair; 16 rows that share a request and a key/value head
+// form a block: the heads of a group for one token, for several tokens if the group is
+// small.
+//
+//   decode kernel   one token per request.  A workgroup of 4 waves takes one request and
+//                   key/value head and one of `n_splits` equal parts of its keys; the
+//                   waves take 32-key steps in turn and merge through LDS; parts are
+//                   merged by a second kernel.
+//   prefill kernel  any number of tokens per request (also one).  A wave takes QB blocks
+//                   of rows of one request and walks all their keys; no LDS, no barriers.
+#include "common.h"
+#include "kv_layout.h"
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
+
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+    return (uint32_t)from_f32<bf16_t>(lo).bits | ((uint32_t)from_f32<bf16_t>(hi).bits << 16);
+}
+// 2^x by the hardware's instruction (inputs here are <= 0; 2^-inf = 0)
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ f32x4 mfma16(u32x4 a, u32x4 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+}
+
+// What a wave carries through its keys, for QB blocks of 16 rows.
+template <int DH, int QB>
+struct AttnState {
+    f32x4 o[QB][DH / 16];   // O^T: lane = (row lane%16, dims 16*dt + 4*(lane/16) + r)
+    float m[QB];            // running maximum (in units of log2), the same in the 4 lane groups
+    float l[QB];            // running sum over the lane's own keys only
+};
+
+template <int DH, int QB>
+__device__ __forceinline__ void attn_init(AttnState<DH, QB> &st) {
+#pragma unroll
+    for (int b = 0; b < QB; ++b) {
+        st.m[b] = -INFINITY;
+        st.l[b] = 0.f;
+#pragma unroll
+        for (int dt = 0; dt < DH / 16; ++dt) st.o[b][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+}
+
+// One step: the 32 keys k0 .. k0+31 (k0 a multiple of 32) of key/value head kvh.
+// p_row / lo_row: the last and first key each of the lane's rows may see.  MASK: some row
+// of the wave does not see all 32 keys; p_max / lo_min bound what any row sees (values of
+// keys outside are not used at all, whatever the memory holds).
+template <int DH, int QB, bool MASK>
+__device__ __forceinline__ void attn_step(const bf16_t *__restrict__ cache, const int *__restrict__ bt, int max_pages,
+                                          int page, size_t page_elems, int nkvh, int kvh, int k0,
+                                          const u32x4 (&q)[QB][DH / 32], AttnState<DH, QB> &st,
+                                          const int (&p_row)[QB], const int (&lo_row)[QB], int p_max, int lo_min,
+                                          float scale_log2, int l16, int grp) {
+    const bf16_t *pg[2];
+    int tok0[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+        const int j = k0 + 16 * t;
+        int pi = j / page;
+        pi = pi < max_pages ? pi : max_pages - 1;       // a tile beyond the context is masked; keep the read in bounds
+        pg[t] = cache + (size_t)bt[pi] * page_elems;
+        tok0[t] = j % page;
+    }
+    // ---- S^T = K Q^T
+    f32x4 s[QB][2];
+#pragma unroll
+    for (int b = 0; b < QB; ++b) s[b][0] = s[b][1] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+        const bf16_t *kp = pg[t] + ((size_t)kvh * (DH / 8) * page + tok0[t] + l16) * 8;
+#pragma unroll
+        for (int kb = 0; kb < DH / 32; ++kb) {
+            const u32x4 kv = *(const u32x4 *)(kp + (size_t)(4 * kb + grp) * page * 8);
+#pragma unroll
+            for (int b = 0; b < QB; ++b) s[b][t] = mfma16(kv, q[b][kb], s[b][t]);
+        }
+    }
+    // ---- softmax of the step, online
+    u32x4 pb[QB];
+#pragma unroll
+    for (int b = 0; b < QB; ++b) {
+        float v[8];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) { v[r] = s[b][0][r]; v[4 + r] = s[b][1][r]; }
+        if (MASK) {
+#pragma unroll
+            for (int r = 0; r < 8; ++r) {
+                const int j = k0 + 16 * (r / 4) + 4 * grp + (r % 4);
+                if (j > p_row[b] || j < lo_row[b]) v[r] = -INFINITY;
+            }
+        }
+        float mx = v[0];
+#pragma unroll
+        for (int r = 1; r < 8; ++r) mx = fmaxf(mx, v[r]);
+        mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
+        const float m_new = fmaxf(st.m[b], mx * scale_log2);
+        const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+        const float alpha = fast_exp2(st.m[b] - m_safe);
+        float p[8], sum = 0.f;
+#pragma unroll
+        for (int r = 0; r < 8; ++r) {
+            p[r] = fast_exp2(fmaf(v[r], scale_log2, -m_safe));
+            sum += p[r];
+        }
+        st.l[b] = st.l[b] * alpha + sum;
+        st.m[b] = m_new;
+#pragma unroll
+        for (int dt = 0; dt < DH / 16; ++dt) st.o[b][dt] *= alpha;
+        pb[b] = u32x4{pack_bf16(p[0], p[1]), pack_bf16(p[2], p[3]), pack_bf16(p[4], p[5]), pack_bf16(p[6], p[7])};
+    }
+    // ---- O^T += V^T P^T
+    const size_t v_off = (size_t)nkvh * DH * page + (size_t)kvh * DH * page;
+#pragma unroll
+    for (int dt = 0; dt < DH / 16; ++dt) {
+        const size_t row = v_off + (size_t)(16 * dt + l16) * page + 4 * grp;
+        u32x2 v0 = *(const u32x2 *)(pg[0] + row + tok0[0]);
+        u32x2 v1 = *(const u32x2 *)(pg[1] + row + tok0[1]);
+        if (MASK) {
+            // values of keys that no row sees are taken as zero: their memory may hold anything
+            const int j0 = k0 + 4 * grp, j1 = k0 + 16 + 4 * grp;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const uint32_t keep = (r & 1) ? 0x0000ffffu : 0xffff0000u;   // mask that clears element r of its dword
+                if (j0 + r > p_max || j0 + r < lo_min) { if (r < 2) v0.x &= keep; else v0.y &= keep; }
+                if (j1 + r > p_max || j1 + r < lo_min) { if (r < 2) v1.x &= keep; else v1.y &= keep; }
+            }
+        }
+        const u32x4 a = u32x4{v0.x, v0.y, v1.x, v1.y};
+#pragma unroll
+        for (int b = 0; b < QB; ++b) st.o[b][dt] = mfma16(a, pb[b], st.o[b][dt]);
+    }
+}
+
+// The lane's part of the queries of one block of rows: 8 dims of row lane%16 per 32-dim
+// slice, zero for a row that does not exist.
+template <int DH>
+__device__ __forceinline__ void load_q(const bf16_t *__restrict__ qrow, bool valid, u32x4 (&q)[DH / 32], int grp) {
+#pragma unroll
+    for (int kb = 0; kb < DH / 32; ++kb)
+        q[kb] = valid ? *(const u32x4 *)(qrow + 32 * kb + 8 * grp) : u32x4{0u, 0u, 0u, 0u};
+}
+
+// ============================================================================ decode
+constexpr int DEC_WAVES = 4;
+
+template <int DH>
+__global__ void __launch_bounds__(DEC_WAVES *WAVE)
+attention_decode_kernel(const bf16_t *__restrict__ q, int q_stride, bf16_t *__restrict__ out, int out_stride,
+                        const bf16_t *__restrict__ cache, const int *__restrict__ block_table, int max_pages,
+                        const int *__restrict__ q_start, const int *__restrict__ ctx_len, int nh, int nkvh, int page,
+                        float scale_log2, int window, int n_splits, float *__restrict__ part_o,
+                        float *__restrict__ part_ml) {
+    extern __shared__ float lds[];                 // [waves][16][DH] outputs, then [waves][16][2] (m, l)
+    const int g = nh / nkvh;
+    const int chunks = (g + 15) / 16;
+    const int r = blockIdx.x / (nkvh * chunks);
+    const int kvh = (blockIdx.x / chunks) % nkvh;
+    const int chunk = blockIdx.x % chunks;
+    const int split = blockIdx.y;
+    const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
+    const int l16 = lane & 15, grp = lane >> 4;
+    const int rows = (g - 16 * chunk) < 16 ? (g - 16 * chunk) : 16;
+    const int token = q_start[r];
+    const int p = ctx_len[r] - 1;
+    const int lo = window > 0 ? (p - window + 1 > 0 ? p - window + 1 : 0) : 0;
+    const int head0 = kvh * g + 16 * chunk;
+
+    u32x4 qv[1][DH / 32];
+    load_q<DH>(q + (size_t)token * q_stride + (size_t)(head0 + l16) * DH, l16 < rows, qv[0], grp);
+    AttnState<DH, 1> st;
+    attn_init(st);
+    const int p_row[1] = {p}, lo_row[1] = {lo};
+    const int *bt = block_table + (size_t)r * max_pages;
+    const size_t page_elems = kv_page_elems(nkvh, DH, page);
+
+    // this split's share of the 32-key steps, the waves in turn
+    const int first = lo / 32, last = p / 32, nblk = last - first + 1;
+    const int b0 = first + (int)((long long)nblk * split / n_splits);
+    const int b1 = first + (int)((long long)nblk * (split + 1) / n_splits);
+    for (int blk = b0 + wave; blk < b1; blk += DEC_WAVES) {
+        const int k0 = blk * 32;
+        if (k0 + 31 > p || k0 < lo)
+            attn_step<DH, 1, true>(cache, bt, max_pages, page, page_elems, nkvh, kvh, k0, qv, st, p_row, lo_row, p, lo, scale_log2, l16, grp);
+        else
+            attn_step<DH, 1, false>(cache, bt, max_pages, page, page_elems, nkvh, kvh, k0, qv, st, p_row, lo_row, p, lo, scale_log2, l16, grp);
+    }
+    // ---- merge the waves
+    float l_all = st.l[0];
+    l_all += __shfl_xor(l_all, 16, WAVE);
+    l_all += __shfl_xor(l_all, 32, WAVE);
+    float *lds_o = lds;
+    float *lds_ml = lds + DEC_WAVES * 16 * DH;
+#pragma unroll
+    for (int dt = 0; dt < DH / 16; ++dt)
+#pragma unroll
+        for (int rr = 0; rr < 4; ++rr) lds_o[((size_t)wave * 16 + l16) * DH + 16 * dt + 4 * grp + rr] = st.o[0][dt][rr];
+    if (grp == 0) {
+        lds_ml[(wave * 16 + l16) * 2 + 0] = st.m[0];
+        lds_ml[(wave * 16 + l16) * 2 + 1] = l_all;
+    }
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < rows * DH; idx += DEC_WAVES * WAVE) {
+        const int row = idx / DH, d = idx % DH;
+        float M = -INFINITY;
+#pragma unroll
+        for (int w = 0; w < DEC_WAVES; ++w) M = fmaxf(M, lds_ml[(w * 16 + row) * 2]);
+        const float M_safe = M == -INFINITY ? 0.f : M;
+        float L = 0.f, val = 0.f;
+#pragma unroll
+        for (int w = 0; w < DEC_WAVES; ++w) {
+            const float f = exp2f(lds_ml[(w * 16 + row) * 2] - M_safe);
+            L += lds_ml[(w * 16 + row) * 2 + 1] * f;
+            val += lds_o[((size_t)w * 16 + row) * DH + d] * f;
+        }
+        const int head = head0 + row;
+        if (n_splits == 1) {
+            out[(size_t)token * out_stride + (size_t)head * DH + d] = from_f32<bf16_t>(val / L);
+        } else {
+            const size_t slot = ((size_t)token * nh + head) * n_splits + split;
+            part_o[slot * DH + d] = val;
+            if (d == 0) { part_ml[slot * 2] = M; part_ml[slot * 2 + 1] = L; }
+        }
+    }
+}
+
+// Merges the parts of every (token, head): out = sum_s O_s 2^(m_s - M) / sum_s l_s 2^(m_s - M).
+template <int DH>
+__global__ void attention_merge_kernel(bf16_t *__restrict__ out, int out_stride, const float *__restrict__ part_o,
+                                       const float *__restrict__ part_ml, int nh, int n_splits) {
+    const int token = blockIdx.x, head = blockIdx.y;
+    const size_t base = ((size_t)token * nh + head) * n_splits;
+    float M = -INFINITY;
+    for (int s = 0; s < n_splits; ++s) M = fmaxf(M, part_ml[(base + s) * 2]);
+    float L = 0.f;
+    for (int s = 0; s < n_splits; ++s) L += part_ml[(base + s) * 2 + 1] * exp2f(part_ml[(base + s) * 2] - M);
+    for (int d = threadIdx.x; d < DH; d += blockDim.x) {
+        float val = 0.f;
+        for (int s = 0; s < n_splits; ++s) val += part_o[(base + s) * DH + d] * exp2f(part_ml[(base + s) * 2] - M);
+        out[(size_t)token * out_stride + (size_t)head * DH + d] = from_f32<bf16_t>(val / L);
+    }
+}
+
+template <int DH>
+static int launch_decode(const void *q, int q_stride, void *out, int out_stride, const void *cache,
+                         const int *block_table, int max_pages, const int *q_start, const int *ctx_len, int n_req,
+                         int nh, int nkvh, int page, float scale, int window, int n_splits, float *part_o,
+                         float *part_ml, hipStream_t stream) {
+    const int g = nh / nkvh, chunks = (g + 15) / 16;
+    const float scale_log2 = scale * 1.4426950408889634f;
+    const size_t lds_bytes = (size_t)DEC_WAVES * 16 * (DH + 2) * sizeof(float);
+    dim3 grid(n_req * nkvh * chunks, n_splits), block(DEC_WAVES * WAVE);
+    attention_decode_kernel<DH><<<grid, block, lds_bytes, stream>>>(
+        (const bf16_t *)q, q_stride, (bf16_t *)out, out_stride, (const bf16_t *)cache, block_table, max_pages, q_start,
+        ctx_len, nh, nkvh, page, scale_log2, window, n_splits, part_o, part_ml);
+    LCU_LAUNCH_CHECK();
+    if (n_splits > 1) {
+        attention_merge_kernel<DH><<<dim3(n_req, nh), dim3(DH < 64 ? 64 : DH / 2), 0, stream>>>(
+            (bf16_t *)out, out_stride, part_o, part_ml, nh, n_splits);
+        LCU_LAUNCH_CHECK();
+    }
+    return LCU_OK;
+}
+
+// Every request of the batch feeds exactly one token (token r belongs to request r).
+// part_o: [n_req * nh * n_splits * dh] floats, part_ml: [n_req * nh * n_splits * 2] (unused
+// when n_splits == 1).  bfloat16 only; head_dim 64 or 128; page_size a multiple of 16.
+LCU_API int lcu_attention_decode_bf16(const void *q, int q_stride, void *out, int out_stride, const void *cache,
+                                      const int *block_table, int max_pages, const int *q_start, const int *ctx_len,
+                                      int n_req, int nh, int nkvh, int dh, int page, float scale, int window,
+                                      int n_splits, float *part_o, float *part_ml, hipStream_t stream) {
+    if (n_req <= 0) return LCU_OK;
+    if (nh <= 0 || nkvh <= 0 || nh % nkvh || page <= 0 || page % 16 || max_pages <= 0 || window < 0 || n_splits < 1 ||
+        n_splits > 65535 || (n_splits > 1 && (!part_o || !part_ml)) || q_stride % 8 || out_stride % 4)
+        return LCU_BAD_ARGUMENT;
+#define GO(D) return launch_decode<D>(q, q_stride, out, out_stride, cache, block_table, max_pages, q_start, ctx_len, n_req, nh, nkvh, page, scale, window, n_splits, part_o, part_ml, stream)
+    if (dh == 128) GO(128);
+    if (dh == 64) GO(64);
+#undef GO
+    return LCU_UNSUPPORTED;
+}
+
+// ============================================================================ prefill
+constexpr int PRE_WAVES = 4;
+
+// A task is QB blocks of 16 rows of one request: `tokens_per_task` consecutive tokens
+// starting at batch index task_tok0[t], with the `hc` heads of one chunk of a group each.
+template <int DH, int QB>
+__global__ void __launch_bounds__(PRE_WAVES *WAVE)
+attention_prefill_kernel(const bf16_t *__restrict__ q, int q_stride, bf16_t *__restrict__ out, int out_stride,
+                         const bf16_t *__restrict__ cache, const int *__restrict__ block_table, int max_pages,
+                         const int *__restrict__ q_start, const int *__restrict__ ctx_len,
+                         const int *__restrict__ task_req, const int *__restrict__ task_tok0, int n_tasks, int nh,
+                         int nkvh, int page, float scale_log2, int window) {
+    const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
+    const int task = blockIdx.x * PRE_WAVES + wave;
+    if (task >= n_tasks) return;
+    const int l16 = lane & 15, grp = lane >> 4;
+    const int g = nh / nkvh;
+    const int chunks = (g + 15) / 16;
+    const int kvh = blockIdx.y / chunks, chunk = blockIdx.y % chunks;
+    const int hc = (g - 16 * chunk) < 16 ? (g - 16 * chunk) : 16;      // heads of this chunk
+    const int tokens_per_block = 16 / hc;                               // tokens in 16 rows
+    const int r = task_req[task], tok0 = task_tok0[task];
+    const int q_end = q_start[r + 1];
+    const int ctx = ctx_len[r];
+    const int head0 = kvh * g + 16 * chunk;
+
+    u32x4 qv[QB][DH / 32];
+    int p_row[QB], lo_row[QB], tok_row[QB];
+    int p_max = -1, p_min = 0x7fffffff, lo_min = 0x7fffffff, lo_max = 0;
+#pragma unroll
+    for (int b = 0; b < QB; ++b) {
+        const int tok = tok0 + b * tokens_per_block + l16 / hc;
+        const bool valid = l16 < tokens_per_block * hc && tok < q_end;
+        tok_row[b] = valid ? tok : -1;
+        p_row[b] = valid ? ctx - (q_end - tok) : -1;
+        lo_row[b] = valid && window > 0 && p_row[b] - window + 1 > 0 ? p_row[b] - window + 1 : 0;
+        load_q<DH>(q + (size_t)(valid ? tok : tok0) * q_stride + (size_t)(head0 + l16 % hc) * DH, valid, qv[b], grp);
+    }
+    // what the whole wave sees (the same in every lane): first and last token of the task
+    {
+        const int last_tok = (tok0 + QB * tokens_per_block < q_end ? tok0 + QB * tokens_per_block : q_end) - 1;
+        p_max = ctx - (q_end - last_tok);
+        p_min = ctx - (q_end - tok0);
+        lo_min = window > 0 && p_min - window + 1 > 0 ? p_min - window + 1 : 0;
+        lo_max = window > 0 && p_max - window + 1 > 0 ? p_max - window + 1 : 0;
+    }
+    AttnState<DH, QB> st;
+    attn_init(st);
+    const int *bt = block_table + (size_t)r * max_pages;
+    const size_t page_elems = kv_page_elems(nkvh, DH, page);
+    for (int blk = lo_min / 32; blk <= p_max / 32; ++blk) {
+        const int k0 = blk * 32;
+        if (k0 + 31 > p_min || k0 < lo_max)
+            attn_step<DH, QB, true>(cache, bt, max_pages, page, page_elems, nkvh, kvh, k0, qv, st, p_row, lo_row, p_max, lo_min, scale_log2, l16, grp);
+        else
+            attn_step<DH, QB, false>(cache, bt, max_pages, page, page_elems, nkvh, kvh, k0, qv, st, p_row, lo_row, p_max, lo_min, scale_log2, l16, grp);
+    }
+#pragma unroll
+    for (int b = 0; b < QB; ++b) {
+        float l_all = st.l[b];
+        l_all += __shfl_xor(l_all, 16, WAVE);
+        l_all += __shfl_xor(l_all, 32, WAVE);
+        if (tok_row[b] < 0) continue;
+        const float inv = 1.0f / l_all;
+        bf16_t *o = out + (size_t)tok_row[b] * out_stride + (size_t)(head0 + l16 % hc) * DH;
+#pragma unroll
+        for (int dt = 0; dt < DH / 16; ++dt) {
+            u32x2 w;
+            w.x = pack_bf16(st.o[b][dt][0] * inv, st.o[b][dt][1] * inv);
+            w.y = pack_bf16(st.o[b][dt][2] * inv, st.o[b][dt][3] * inv);
+            *(u32x2 *)(o + 16 * dt + 4 * grp) = w;
+        }
+    }
+}
+
+template <int DH, int QB>
+static int launch_prefill(const void *q, int q_stride, void *out, int out_stride, const void *cache,
+                          const int *block_table, int max_pages, const int *q_start, const int *ctx_len,
+                          const int *task_req, const int *task_tok0, int n_tasks, int nh, int nkvh, int page,
+                          float scale, int window, hipStream_t stream) {
+    const int g = nh / nkvh, chunks = (g + 15) / 16;
+    dim3 grid((n_tasks + PRE_WAVES - 1) / PRE_WAVES, nkvh * chunks), block(PRE_WAVES * WAVE);
+    attention_prefill_kernel<DH, QB><<<grid, block, 0, stream>>>(
+        (const bf16_t *)q, q_stride, (bf16_t *)out, out_stride, (const bf16_t *)cache, block_table, max_pages, q_start,
+        ctx_len, task_req, task_tok0, n_tasks, nh, nkvh, page, scale * 1.4426950408889634f, window);
+    LCU_LAUNCH_CHECK();
+    return LCU_OK;
+}
+
+// How many consecutive tokens of one request a task of the prefill kernel covers, for a
+// model with `nh` heads in `nkvh` groups (the host cuts the batch into tasks with it).
+LCU_API int lcu_attention_prefill_tokens_per_task(int nh, int nkvh) {
+    if (nh <= 0 || nkvh <= 0 || nh % nkvh) return 0;
+    const int g = nh / nkvh;
+    if (g > 16 && g % 16) return 0;       // chunks of a group must be equal for one task size
+    const int hc = g < 16 ? g : 16;
+    return 2 * (16 / hc);
+}
+
+// task_req / task_tok0: [n_tasks], tasks cut from the batch with the size above; a
+// request's last task may be shorter.  bfloat16 only; head_dim 64 or 128; page_size a
+// multiple of 16.
+LCU_API int lcu_attention_prefill_bf16(const void *q, int q_stride, void *out, int out_stride, const void *cache,
+                                       const int *block_table, int max_pages, const int *q_start, const int *ctx_len,
+                                       const int *task_req, const int *task_tok0, int n_tasks, int nh, int nkvh,
+                                       int dh, int page, float scale, int window, hipStream_t stream) {
+    if (n_tasks <= 0) return LCU_OK;
+    if (lcu_attention_prefill_tokens_per_task(nh, nkvh) == 0 || page <= 0 || page % 16 || max_pages <= 0 ||
+        window < 0 || q_stride % 8 || out_stride % 4 || nkvh * ((nh / nkvh + 15) / 16) > 65535)
+        return LCU_BAD_ARGUMENT;
+#define GO(D) return launch_prefill<D, 2>(q, q_stride, out, out_stride, cache, block_table, max_pages, q_start, ctx_len, task_req, task_tok0, n_tasks, nh, nkvh, page, scale, window, stream)
+    if (dh == 128) GO(128);
+    if (dh == 64) GO(64);
+#undef GO
+    return LCU_UNSUPPORTED;
+}

@@ -43,6 +43,8 @@ class StepContext:
     q_lens: List[int] = field(default_factory=list)
     ctx_lens: List[int] = field(default_factory=list)
     req_ids: List[int] = field(default_factory=list)
+    attn_splits: Optional[int] = None           # fixed number of key parts for the decode kernel (captured graphs)
+    scratch: dict = field(default_factory=dict)  # what kernels' wrappers derive from the batch once per step
 
     def block_table(self, group: int) -> torch.Tensor:
         return self.block_tables[group]

@@ -30,8 +30,8 @@ HIP_FLAGS = ["-O3", "--offload-arch=gfx950", "-std=c++17", "-shared", "-fPIC",
              "-Wno-unused-command-line-argument"]
 HOST_FLAGS = ["-O2", "-std=c++17", "-shared", "-fPIC", "-Wall"]
 
-KERNEL_LIBRARIES = ["elementwise", "rope_kv", "attention_generic", "attention_decode", "attention_prefill",
-                    "gemm_generic", "gemm_skinny", "sampling"]
+KERNEL_LIBRARIES = ["elementwise", "rope_kv", "attention_generic", "attention_mfma", "gemm_generic", "gemm_skinny",
+                    "sampling"]
 HOST_LIBRARY = "host"
 
 _loaded: Dict[str, ctypes.CDLL] = {}

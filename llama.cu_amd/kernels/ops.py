@@ -269,12 +269,85 @@ def gemm_nt(a: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = None
     return out
 
 
+def mfma_attention_supported(q: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: int, page_size: int) -> bool:
+    """Whether the matrix-core attention kernels take this shape (the generic kernel takes
+    the rest): bfloat16, head_dim 64 or 128, pages of a multiple of 16 tokens, groups of
+    at most 16 heads or of a multiple of 16."""
+    g = n_heads // n_kv_heads
+    return (q.dtype == torch.bfloat16 and head_dim in (64, 128) and page_size % 16 == 0 and (g <= 16 or g % 16 == 0)
+            and q.stride(0) % 8 == 0)
+
+
+def attention_decode(q, out, cache, block_table, q_start, ctx_len, n_req, n_heads, n_kv_heads, head_dim, page_size,
+                     scale, window, n_splits) -> torch.Tensor:
+    """Matrix-core attention for a batch in which every request feeds one token."""
+    part_o = part_ml = None
+    if n_splits > 1:
+        part_o = torch.empty(n_req * n_heads * n_splits * head_dim, dtype=torch.float32, device=q.device)
+        part_ml = torch.empty(n_req * n_heads * n_splits * 2, dtype=torch.float32, device=q.device)
+    lib = build.load("attention_mfma")
+    _check(lib.lcu_attention_decode_bf16(_ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(cache), _ptr(block_table),
+                                         block_table.shape[1], _ptr(q_start), _ptr(ctx_len), n_req, n_heads, n_kv_heads,
+                                         head_dim, page_size, ctypes.c_float(scale), int(window), int(n_splits),
+                                         _ptr(part_o), _ptr(part_ml), _stream()), "attention_decode")
+    return out
+
+
+def prefill_tasks(q_lens, tokens_per_task: int, device):
+    """Cut the batch into the prefill kernel's tasks: (request index, first token) pairs."""
+    reqs, toks = [], []
+    start = 0
+    for r, n in enumerate(q_lens):
+        for t in range(0, n, tokens_per_task):
+            reqs.append(r)
+            toks.append(start + t)
+        start += n
+    both = torch.tensor([reqs, toks], dtype=torch.int32).to(device)
+    return both[0], both[1], len(reqs)
+
+
+def attention_prefill(q, out, cache, block_table, q_start, ctx_len, task_req, task_tok0, n_tasks, n_heads, n_kv_heads,
+                      head_dim, page_size, scale, window) -> torch.Tensor:
+    """Matrix-core attention for any mix of portions and single tokens."""
+    _i32(task_req, "task_req", n_tasks); _i32(task_tok0, "task_tok0", n_tasks)
+    lib = build.load("attention_mfma")
+    _check(lib.lcu_attention_prefill_bf16(_ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(cache), _ptr(block_table),
+                                          block_table.shape[1], _ptr(q_start), _ptr(ctx_len), _ptr(task_req),
+                                          _ptr(task_tok0), n_tasks, n_heads, n_kv_heads, head_dim, page_size,
+                                          ctypes.c_float(scale), int(window), _stream()), "attention_prefill")
+    return out
+
+
+def decode_splits(n_req: int, n_heads: int, n_kv_heads: int, max_ctx_len: int) -> int:
+    """Into how many parts the decode kernel cuts each request's keys: enough workgroups
+    to fill 256 compute units, no part shorter than 128 keys."""
+    base = n_req * n_kv_heads * ((n_heads // n_kv_heads + 15) // 16)
+    return max(1, min(16, 1024 // max(base, 1), (max_ctx_len + 127) // 128))
+
+
 def paged_attention(q: torch.Tensor, out: torch.Tensor, cache: torch.Tensor, step, group: int, n_heads: int,
-                    n_kv_heads: int, head_dim: int, page_size: int, scale: float, window: int = 0) -> torch.Tensor:
+                    n_kv_heads: int, head_dim: int, page_size: int, scale: float, window: int = 0,
+                    force_generic: bool = False) -> torch.Tensor:
     """Attention for the batch ``step`` (an engine.batch.StepContext) over cache group
-    ``group``: picks the kernel for the batch's shape."""
-    return paged_attention_generic(q, out, cache, step.block_table(group), step.q_start, step.ctx_len,
-                                   step.req_of_token, n_heads, n_kv_heads, head_dim, page_size, scale, window)
+    ``group``: picks the kernel for the batch's shape and type."""
+    bt = step.block_table(group)
+    if force_generic or not mfma_attention_supported(q, n_heads, n_kv_heads, head_dim, page_size):
+        return paged_attention_generic(q, out, cache, bt, step.q_start, step.ctx_len, step.req_of_token, n_heads,
+                                       n_kv_heads, head_dim, page_size, scale, window)
+    n = _attention_args(q, out, cache, bt, step.q_start, step.ctx_len, step.req_of_token, n_heads, n_kv_heads, head_dim,
+                        page_size)
+    if step.decode_only:
+        splits = step.attn_splits or decode_splits(step.n_req, n_heads, n_kv_heads, step.max_ctx_len)
+        return attention_decode(q, out, cache, bt, step.q_start, step.ctx_len, step.n_req, n_heads, n_kv_heads, head_dim,
+                                page_size, scale, window, splits)
+    lib = build.load("attention_mfma")
+    tpt = lib.lcu_attention_prefill_tokens_per_task(n_heads, n_kv_heads)
+    key = ("attention_tasks", tpt)
+    if key not in step.scratch:
+        step.scratch[key] = prefill_tasks(step.q_lens, tpt, q.device)
+    task_req, task_tok0, n_tasks = step.scratch[key]
+    return attention_prefill(q, out, cache, bt, step.q_start, step.ctx_len, task_req, task_tok0, n_tasks, n_heads,
+                             n_kv_heads, head_dim, page_size, scale, window)
 
 
 def skinny_supported(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype) -> bool:

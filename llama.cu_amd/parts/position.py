@@ -56,8 +56,9 @@ class Rotary(NoPosition):
 
     def host_tables(self):
         half = self.rot_dim // 2
-        i = np.arange(half, dtype=np.float64)
-        freq = np.power(np.float64(self.theta), -(2.0 * i) / self.rot_dim).astype(np.float32)
+        # 32-bit throughout, as the reference: theta.powf(-((2 * i) as f32 / dh as f32))
+        expo = -(np.float32(2.0) * np.arange(half, dtype=np.float32) / np.float32(self.rot_dim))
+        freq = np.power(np.float32(self.theta), expo.astype(np.float32)).astype(np.float32)
         pos = np.arange(self.max_positions, dtype=np.float32)
         ang = (pos[:, None] * freq[None, :]).astype(np.float32).astype(np.float64)   # the 32-bit product
         return np.cos(ang).astype(np.float32), np.sin(ang).astype(np.float32)

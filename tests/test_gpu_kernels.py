@@ -1,0 +1,322 @@
+"""Each kernel alone against a plain formula, at other sizes than the engine's tiny
+models use: widths and vocabularies that are no power of two, head sizes in steps of 16,
+odd group sizes, pages of several sizes, windows, and inputs made so that a fault shows
+(one key far back that dominates, poisoned memory where nothing may be read)."""
+import math
+import random
+
+import numpy as np
+import pytest
+import torch
+
+import plain
+
+pytestmark = pytest.mark.gpu
+
+DT = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+TOL = {"float32": 2e-5, "bfloat16": 2e-2}
+
+
+def close(got, want, dtype, what=""):
+    want = want.double()
+    scale = float(want.abs().max()) + 1e-30
+    err = float((got.double().cpu() - want).abs().max())
+    assert math.isfinite(err) and err <= TOL[dtype] * scale, f"{what}: error {err:.3e} vs scale {scale:.3e}"
+
+
+def rnd(*shape, seed=0, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randn(*shape, generator=g) * scale
+
+
+# ------------------------------------------------------------------ rows
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("n,d,vocab", [(1, 8, 3), (7, 100, 301), (33, 4096, 1000)])
+def test_embedding_gather(dtype, n, d, vocab):
+    from llama_cu_amd.kernels import ops
+    table = rnd(vocab, d, seed=n).to(DT[dtype])
+    ids = torch.randint(0, vocab, (n,), dtype=torch.int32)
+    out = torch.empty(n, d, dtype=torch.float32, device="cuda")
+    ops.embedding_gather(table.cuda(), ids.cuda(), out)
+    assert torch.equal(out.cpu(), plain.embedding(table.float(), ids.tolist()).float())
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("n,d,eps", [(1, 16, 1e-5), (5, 172, 1e-6), (3, 4096, 1e-5), (2, 5000, 1e-2)])
+@pytest.mark.parametrize("w32", [False, True])
+def test_rmsnorm_with_residual_sum(dtype, n, d, eps, w32):
+    from llama_cu_amd.kernels import ops
+    x = rnd(n, d, seed=1, scale=0.05)
+    delta = rnd(n, d, seed=2, scale=0.05).to(DT[dtype])
+    w = (1 + rnd(d, seed=3, scale=0.1)).to(torch.float32 if w32 else DT[dtype])
+    xg = x.cuda()
+    out = torch.empty(n, d, dtype=DT[dtype], device="cuda")
+    ops.rmsnorm(xg, w.cuda(), eps, out, delta=delta.cuda())
+    xs = x.double() + delta.double()
+    close(xg, xs, "float32", "residual sum")            # the sum is 32-bit on both paths
+    close(out, plain.rms_norm(xs, w, eps), dtype, "norm")
+    out2 = torch.empty_like(out)
+    ops.rmsnorm(xg, w.cuda(), eps, out2)                   # no delta: x unchanged
+    close(out2, plain.rms_norm(xs, w, eps), dtype, "norm without delta")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("n,di", [(1, 8), (3, 172), (17, 14336)])
+def test_swiglu(dtype, n, di):
+    from llama_cu_amd.kernels import ops
+    gu = rnd(n, 2 * di, seed=di, scale=3.0).to(DT[dtype])
+    out = ops.swiglu(gu.cuda())
+    close(out, plain.swiglu(gu[:, :di], gu[:, di:]), dtype)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_gather_rows_and_residual_add(dtype):
+    from llama_cu_amd.kernels import ops
+    x = rnd(9, 70, seed=4).to(DT[dtype])
+    rows = torch.tensor([8, 0, 3, 3], dtype=torch.int32)
+    assert torch.equal(ops.gather_rows(x.cuda(), rows.cuda()).cpu(), x[rows.long()])
+    r = rnd(9, 70, seed=5)
+    rg = r.cuda()
+    ops.residual_add(rg, x.cuda())
+    close(rg, r.double() + x.double(), "float32")
+
+
+# ------------------------------------------------------------------ matrix products
+@pytest.mark.parametrize("a_t,w_t,o_t", [("float32", "float32", "float32"), ("bfloat16", "bfloat16", "bfloat16"),
+                                         ("bfloat16", "bfloat16", "float32"), ("bfloat16", "float32", "bfloat16")])
+@pytest.mark.parametrize("m,n,k", [(1, 1, 1), (3, 172, 64), (65, 301, 100), (130, 64, 352), (2, 1000, 4096)])
+def test_gemm_generic(a_t, w_t, o_t, m, n, k):
+    from llama_cu_amd.kernels import ops
+    a = rnd(m, k, seed=m).to(DT[a_t])
+    w = rnd(n, k, seed=n + 1).to(DT[w_t])
+    out = ops.gemm_nt(a.cuda(), w.cuda(), out_dtype=DT[o_t])
+    close(out, plain.linear(a, w), o_t)
+
+
+def test_gemm_generic_accumulates_in_32_bit_and_rows_are_independent():
+    from llama_cu_amd.kernels import ops
+    a, w = rnd(70, 300, seed=1), rnd(50, 300, seed=2)
+    c = rnd(70, 50, seed=3)
+    cg = c.cuda()
+    ops.gemm_nt(a.cuda(), w.cuda(), out=cg, accumulate=True)
+    close(cg, c.double() + plain.linear(a, w), "float32")
+    # a row's result does not depend on the other rows (bitwise)
+    whole = ops.gemm_nt(a.cuda(), w.cuda())
+    one = ops.gemm_nt(a[17:18].cuda(), w.cuda())
+    assert torch.equal(whole[17:18], one)
+
+
+def test_float32_product_is_a_true_32_bit_product():
+    """Operands 1 + 2^-12: exact in 32-bit, rounded to 1 by any matrix mode with 10 or fewer
+    mantissa bits.  Each of the 256 products is 1 + 2^-11 + 2^-24, so the true sum is
+    256.125; a reduced-precision mode gives 256."""
+    from llama_cu_amd.kernels import ops
+    a = torch.full((4, 256), 1.0 + 2.0 ** -12)
+    w = torch.full((8, 256), 1.0 + 2.0 ** -12)
+    out = ops.gemm_nt(a.cuda(), w.cuda())
+    assert float((out.double().cpu() - 256.125).abs().max()) < 1e-3
+
+
+# ------------------------------------------------------------------ rotation and cache write
+def key_offset(kvh, tok, dim, dh, page):
+    return ((kvh * (dh // 8) + dim // 8) * page + tok) * 8 + dim % 8
+
+
+def value_offset(nkv, kvh, tok, dim, dh, page):
+    return nkv * dh * page + (kvh * dh + dim) * page + tok
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("nh,nkv,dh,page,pairing", [(4, 4, 16, 16, "half"), (6, 2, 48, 8, "adjacent"), (32, 8, 128, 32, "half"),
+                                                     (3, 1, 80, 24, "adjacent")])
+def test_rope_and_cache_write(dtype, nh, nkv, dh, page, pairing):
+    from llama_cu_amd.kernels import ops
+    from llama_cu_amd.parts.position import Rotary
+    n, max_pos, pages = 11, 300, 9
+    theta = 500000.0
+    rot = Rotary(dh, theta, max_pos, interleaved=(pairing == "adjacent"))
+    cos, sin = rot.host_tables()
+    sin_p, cos_p = plain.rope_tables(max_pos, dh, theta)
+    # a frequency may differ in its last bit between two correct implementations of powf
+    bound = max_pos * 2.0 ** -23
+    assert np.abs(cos - cos_p.numpy()).max() < bound and np.abs(sin - sin_p.numpy()).max() < bound
+    qkv = rnd(n, (nh + 2 * nkv) * dh, seed=dh).to(DT[dtype])
+    pos = torch.tensor(random.Random(1).sample(range(max_pos), n), dtype=torch.int32)
+    slots = torch.tensor(random.Random(2).sample(range(pages * page), n), dtype=torch.int32)
+    slots[4] = -1                                              # nothing is stored for this token
+    cache = torch.full((pages, 2, nkv * dh * page), 7.0, dtype=DT[dtype])
+    cg, qg = cache.cuda(), qkv.cuda()
+    ops.rope_kv_store(qg, pos.cuda(), nh, nkv, dh, torch.from_numpy(cos).cuda(), torch.from_numpy(sin).cuda(), dh,
+                      1 if pairing == "adjacent" else 0, cg, slots.cuda(), page)
+    q = qkv[:, :nh * dh].view(n, nh, dh)
+    k = qkv[:, nh * dh:(nh + nkv) * dh].view(n, nkv, dh)
+    v = qkv[:, (nh + nkv) * dh:].view(n, nkv, dh)
+    q_want = plain.rope(q, pos.tolist(), sin_p, cos_p, pairing)
+    k_want = plain.rope(k, pos.tolist(), sin_p, cos_p, pairing)
+    close(qg[:, :nh * dh].reshape(n, nh, dh), q_want, dtype, "q")
+    assert torch.equal(qg[:, nh * dh:].cpu(), qkv[:, nh * dh:])           # k and v in the step's buffer stay
+    flat = cg.cpu().view(pages, -1)
+    expect = torch.full_like(flat, 7.0).double()
+    for t in range(n):
+        if slots[t] < 0:
+            continue
+        pg, tok = int(slots[t]) // page, int(slots[t]) % page
+        for h in range(nkv):
+            for c in range(dh):
+                expect[pg, key_offset(h, tok, c, dh, page)] = k_want[t, h, c]
+                expect[pg, value_offset(nkv, h, tok, c, dh, page)] = v[t, h, c].double()
+    close(flat, expect, dtype, "cache")
+    assert torch.equal(flat == 7.0, expect == 7.0)                        # nothing else was touched
+
+
+def test_rope_partial_rotation_and_no_rotation():
+    from llama_cu_amd.kernels import ops
+    from llama_cu_amd.parts.position import Rotary
+    n, nh, dh, rot_dim = 4, 2, 32, 16
+    rot = Rotary(dh, 10000.0, 64, rot_dim=rot_dim)
+    cos, sin = rot.host_tables()
+    q = rnd(n, nh * dh, seed=3)
+    pos = torch.tensor([0, 5, 17, 63], dtype=torch.int32)
+    qg = q.clone().cuda()
+    ops.rope_kv_store(qg, pos.cuda(), nh, 0, dh, torch.from_numpy(cos).cuda(), torch.from_numpy(sin).cuda(), rot_dim, 0,
+                      None, None, 16)
+    sin_p, cos_p = plain.rope_tables(64, rot_dim, 10000.0)
+    qv = q.view(n, nh, dh)
+    want = qv.clone().double()
+    want[..., :rot_dim] = plain.rope(qv[..., :rot_dim], pos.tolist(), sin_p, cos_p, "half")
+    close(qg.view(n, nh, dh), want, "float32")
+    qg2 = q.clone().cuda()
+    ops.rope_kv_store(qg2, pos.cuda(), nh, 0, dh, None, None, 0, 0, None, None, 16)
+    assert torch.equal(qg2.cpu(), q)
+
+
+# ------------------------------------------------------------------ attention
+class Batch:
+    """The facts of a step that the attention kernels need, made by hand."""
+
+    def __init__(self, q_lens, ctx_lens, tables, max_pages):
+        from llama_cu_amd.engine.batch import StepContext
+        n = sum(q_lens)
+        qs = [0]
+        for x in q_lens:
+            qs.append(qs[-1] + x)
+        rot = [r for r, x in enumerate(q_lens) for _ in range(x)]
+        bt = torch.zeros(len(q_lens), max_pages, dtype=torch.int32)
+        for r, t in enumerate(tables):
+            bt[r, :len(t)] = torch.tensor(t, dtype=torch.int32)
+        i32 = lambda v: torch.tensor(v, dtype=torch.int32).cuda()
+        self.step = StepContext(n=n, n_req=len(q_lens), tokens=i32([0] * n), positions=i32([0] * n), req_of_token=i32(rot),
+                                q_start=i32(qs), ctx_len=i32(ctx_lens), state_slot=i32([0] * len(q_lens)),
+                                logit_rows=i32([]), n_logits=0, block_tables=[bt.cuda()], slot_maps=[i32([0] * n)],
+                                q_lens=list(q_lens), ctx_lens=list(ctx_lens))
+
+
+def paged_case(dtype, nh, nkv, dh, page, q_lens, ctx_lens, window, seed, standout=True, poison=True):
+    """Random keys, values and queries for requests with the given lengths, laid into pages
+    in a random order; returns what the kernels need and the plain answer."""
+    rng = random.Random(seed)
+    tdt = DT[dtype]
+    need = [(c + page - 1) // page for c in ctx_lens]
+    n_pages = sum(need) + 3
+    order = list(range(n_pages))
+    rng.shuffle(order)
+    fill = float("nan") if poison else 0.0
+    cache = torch.full((n_pages, 2 * nkv * dh * page), fill, dtype=torch.float32)
+    tables, outs, qs = [], [], []
+    for r, (ql, cl) in enumerate(zip(q_lens, ctx_lens)):
+        k = rnd(cl, nkv, dh, seed=seed * 100 + r).to(tdt).float()
+        v = rnd(cl, nkv, dh, seed=seed * 100 + r + 50).to(tdt).float()
+        q = rnd(ql, nh, dh, seed=seed * 100 + r + 70).to(tdt).float()
+        if standout and cl > 3:
+            # one key far back that every head's last query points at: it must dominate
+            j = 1 if window == 0 else max(cl - window, 0) + 0
+            j = min(j, cl - 1)
+            for h in range(nh):
+                k[j, h // (nh // nkv)] = (q[-1, h] * 1.5).to(tdt).float() if h % (nh // nkv) == 0 else k[j, h // (nh // nkv)]
+        table = [order.pop() for _ in range(need[r])]
+        if window > 0:
+            # pages that the window of the first query has passed are gone (they hold poison)
+            first_needed = max(cl - ql - window + 1, 0) // page
+        else:
+            first_needed = 0
+        for j in range(cl):
+            pg, tok = table[j // page], j % page
+            if j // page < first_needed:
+                continue
+            for h in range(nkv):
+                for c8 in range(dh // 8):
+                    base = key_offset(h, tok, c8 * 8, dh, page)
+                    cache[pg, base:base + 8] = k[j, h, c8 * 8:c8 * 8 + 8]
+                cache[pg, value_offset(nkv, h, tok, 0, dh, page):value_offset(nkv, h, tok, 0, dh, page) + dh * page:page] = v[j, h]
+        for p in range(first_needed):
+            table[p] = 0 if poison else table[p]
+        tables.append(table)
+        qs.append(q)
+        outs.append(plain.attention(q, k, v, dh ** -0.5, first_pos=cl - ql, window=window or None))
+    q_all = torch.cat(qs).reshape(sum(q_lens), nh * dh).to(tdt)
+    want = torch.cat(outs).reshape(sum(q_lens), nh * dh)
+    cache = cache.to(tdt).view(n_pages, 2, nkv * dh * page)
+    max_pages = max(need) + 2
+    return q_all, cache, Batch(q_lens, ctx_lens, tables, max_pages).step, want
+
+
+SHAPES = [  # nh, nkv, dh, page
+    (4, 4, 16, 16), (4, 1, 32, 32), (6, 2, 48, 8), (8, 2, 64, 16), (32, 8, 128, 16), (6, 2, 128, 48), (32, 2, 64, 32),
+    (5, 5, 256, 16)]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("nh,nkv,dh,page", SHAPES)
+@pytest.mark.parametrize("window", [0, 37])
+def test_attention_mixed_batch(dtype, nh, nkv, dh, page, window):
+    """Portions beside single tokens, from the cache: the kernel the dispatcher picks and
+    the generic kernel both give the plain answer."""
+    from llama_cu_amd.kernels import ops
+    q_lens, ctx_lens = [1, 7, 33, 2, 1], [1, 40, 33, 131, 300]
+    q, cache, step, want = paged_case(dtype, nh, nkv, dh, page, q_lens, ctx_lens, window, seed=nh + dh)
+    for force in (False, True):
+        out = torch.empty(q.shape[0], nh * dh, dtype=DT[dtype], device="cuda")
+        ops.paged_attention(q.cuda(), out, cache.cuda(), step, 0, nh, nkv, dh, page, dh ** -0.5, window, force_generic=force)
+        close(out, want, dtype, f"force_generic={force}")
+
+
+@pytest.mark.parametrize("nh,nkv,dh,page", [(8, 2, 64, 16), (32, 8, 128, 16), (16, 16, 128, 32), (32, 1, 64, 16), (6, 2, 128, 48)])
+@pytest.mark.parametrize("window", [0, 100])
+@pytest.mark.parametrize("splits", [None, 1, 3, 16])
+def test_attention_decode_kernel(nh, nkv, dh, page, window, splits):
+    """Every request feeds one token: the matrix-core decode kernel, with its keys cut
+    into parts or not, against the plain answer; a far key dominates."""
+    from llama_cu_amd.kernels import ops
+    ctx_lens = [1, 31, 32, 33, 500, 2049]
+    q, cache, step, want = paged_case("bfloat16", nh, nkv, dh, page, [1] * len(ctx_lens), ctx_lens, window, seed=dh + page)
+    step.attn_splits = splits
+    assert ops.mfma_attention_supported(q, nh, nkv, dh, page)
+    out = torch.empty(q.shape[0], nh * dh, dtype=torch.bfloat16, device="cuda")
+    ops.paged_attention(q.cuda(), out, cache.cuda(), step, 0, nh, nkv, dh, page, dh ** -0.5, window)
+    close(out, want, "bfloat16")
+
+
+@pytest.mark.parametrize("nh,nkv,dh,page", [(8, 2, 64, 16), (32, 8, 128, 16), (3, 1, 128, 32), (7, 7, 64, 16)])
+def test_attention_prefill_kernel_long(nh, nkv, dh, page):
+    """Whole prompts and portions with history on the matrix cores, long enough that a
+    wave walks many steps and tasks end inside a request."""
+    from llama_cu_amd.kernels import ops
+    q_lens, ctx_lens = [300, 77, 5], [300, 500, 1030]
+    q, cache, step, want = paged_case("bfloat16", nh, nkv, dh, page, q_lens, ctx_lens, 0, seed=page + nh)
+    out = torch.empty(q.shape[0], nh * dh, dtype=torch.bfloat16, device="cuda")
+    ops.paged_attention(q.cuda(), out, cache.cuda(), step, 0, nh, nkv, dh, page, dh ** -0.5, 0)
+    close(out, want, "bfloat16")
+
+
+def test_attention_float32_result_does_not_depend_on_the_batch():
+    from llama_cu_amd.kernels import ops
+    nh, nkv, dh, page = 4, 2, 32, 16
+    q, cache, step, want = paged_case("float32", nh, nkv, dh, page, [9, 1], [100, 64], 0, seed=3)
+    out = torch.empty(q.shape[0], nh * dh, device="cuda")
+    ops.paged_attention(q.cuda(), out, cache.cuda(), step, 0, nh, nkv, dh, page, dh ** -0.5)
+    # the same last token of request 0, alone in a batch of one token
+    q1, cache1, step1, _ = paged_case("float32", nh, nkv, dh, page, [9, 1], [100, 64], 0, seed=3)
+    step1 = Batch([1], [100], [step.block_tables[0][0].tolist()], step.block_tables[0].shape[1]).step
+    out1 = torch.empty(1, nh * dh, device="cuda")
+    ops.paged_attention(q[8:9].cuda(), out1, cache.cuda(), step1, 0, nh, nkv, dh, page, dh ** -0.5)
+    assert torch.equal(out[8:9], out1)
