@@ -1,0 +1,227 @@
+// Y[M, N] = X[M, K] * W[N, K]^T for few rows (decoding: M <= 64), bfloat16 operands,
+// 32-bit accumulation on the matrix cores.  The work is streaming W once from HBM, so
+// the kernel is laid out around W's loads:
+//
+//   * a workgroup of 4 waves owns NT tiles of 16 output features (rows of W) and walks
+//     the whole K: no sum crosses workgroups, results do not depend on the grid, and
+//     the epilogue can be fused;
+//   * K goes in macro-steps of 128; the waves take macro-steps in turn; in a macro-step
+//     lane group g of a wave reads the 64 contiguous bytes k0 + 32g .. k0 + 32g + 31 of
+//     its row as four 16-byte loads, one per matrix instruction (which k a slot of the
+//     instruction holds is free, as long as W and X agree), so the four waves read 1 KB
+//     of a row back to back;
+//   * the next macro-step's loads are issued before the current one is multiplied;
+//   * v_mfma_f32_16x16x32_bf16 with A = W tile, B = X^T: the 16 columns are 16 tokens,
+//     MT such tiles for up to 64 tokens.
+// The four waves' partial sums are added in LDS in a fixed order.
+//
+// Epilogues: store bfloat16; store float32 (logits); add into float32 (the residual
+// stream); SwiGLU, where the workgroup's two tiles are the gate rows n and the up rows
+// n + N/2 of one matrix and silu(gate) * up is stored.
+#include "common.h"
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+
+enum { EPI_BF16 = 0, EPI_F32 = 1, EPI_ADD_F32 = 2, EPI_SWIGLU = 3 };
+constexpr int SK_WAVES = 4;
+
+__device__ __forceinline__ f32x4 mfma16(u32x4 a, u32x4 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+}
+
+template <int NT, int MT>
+struct Frag {
+    u32x4 w[NT][4];
+    u32x4 x[MT][4];
+};
+
+// The lane's loads of macro-step s: k = 128 s + 32 grp + 8 j .. + 7 for j = 0..3.
+template <int NT, int MT>
+__device__ __forceinline__ void load_frag(Frag<NT, MT> &f, const bf16_t *const (&wrow)[NT], const bf16_t *const (&xrow)[MT],
+                                          const bool (&xvalid)[MT], int s, int grp, int K) {
+    const int kb = 128 * s + 32 * grp;
+    const u32x4 zero = u32x4{0u, 0u, 0u, 0u};
+    if (128 * (s + 1) <= K) {
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) f.w[t][j] = *(const u32x4 *)(wrow[t] + kb + 8 * j);
+#pragma unroll
+        for (int m = 0; m < MT; ++m)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) f.x[m][j] = xvalid[m] ? *(const u32x4 *)(xrow[m] + kb + 8 * j) : zero;
+    } else {                                   // the last, partial macro-step (K is a multiple of 8)
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) f.w[t][j] = (kb + 8 * j + 8 <= K) ? *(const u32x4 *)(wrow[t] + kb + 8 * j) : zero;
+#pragma unroll
+        for (int m = 0; m < MT; ++m)
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                f.x[m][j] = (xvalid[m] && kb + 8 * j + 8 <= K) ? *(const u32x4 *)(xrow[m] + kb + 8 * j) : zero;
+    }
+}
+
+template <int NT, int MT>
+__device__ __forceinline__ void mul_frag(const Frag<NT, MT> &f, f32x4 (&acc)[NT][MT]) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+#pragma unroll
+            for (int m = 0; m < MT; ++m) acc[t][m] = mfma16(f.w[t][j], f.x[m][j], acc[t][m]);
+}
+
+template <int NT, int MT, int EPI>
+__global__ void __launch_bounds__(SK_WAVES *WAVE)
+gemm_skinny_kernel(const bf16_t *__restrict__ X, int ldx, const bf16_t *__restrict__ W, int ldw, void *__restrict__ Y,
+                   int ldy, int M, int N, int K) {
+    __shared__ float red[SK_WAVES][NT * MT * 4][WAVE];
+    const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
+    const int l16 = lane & 15, grp = lane >> 4;
+    // the rows of W of tile t: for SwiGLU tile 0 are gate rows, tile 1 the up rows N/2 further
+    const int n_out = EPI == EPI_SWIGLU ? N / 2 : N;                 // width of Y
+    const int n0 = blockIdx.x * 16 * (EPI == EPI_SWIGLU ? 1 : NT);
+    const bf16_t *wrow[NT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+        int row = EPI == EPI_SWIGLU ? n0 + l16 + t * n_out : n0 + 16 * t + l16;
+        const int limit = EPI == EPI_SWIGLU ? (t + 1) * n_out : N;
+        row = row < limit ? row : limit - 1;                          // a row beyond the end is read, not stored
+        wrow[t] = W + (size_t)row * ldw;
+    }
+    const bf16_t *xrow[MT];
+    bool xvalid[MT];
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+        xvalid[m] = 16 * m + l16 < M;
+        xrow[m] = X + (size_t)(xvalid[m] ? 16 * m + l16 : 0) * ldx;
+    }
+    f32x4 acc[NT][MT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int m = 0; m < MT; ++m) acc[t][m] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    const int nsteps = (K + 127) / 128;
+    Frag<NT, MT> fa, fb;
+    int s = wave;
+    if (s < nsteps) load_frag<NT, MT>(fa, wrow, xrow, xvalid, s, grp, K);
+    for (; s < nsteps; s += 2 * SK_WAVES) {
+        const bool has_b = s + SK_WAVES < nsteps;
+        if (has_b) load_frag<NT, MT>(fb, wrow, xrow, xvalid, s + SK_WAVES, grp, K);
+        mul_frag<NT, MT>(fa, acc);
+        if (s + 2 * SK_WAVES < nsteps) load_frag<NT, MT>(fa, wrow, xrow, xvalid, s + 2 * SK_WAVES, grp, K);
+        if (has_b) mul_frag<NT, MT>(fb, acc);
+    }
+    // ---- the four waves' sums, added in the order 0, 1, 2, 3
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int m = 0; m < MT; ++m)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) red[wave][(t * MT + m) * 4 + r][lane] = acc[t][m][r];
+    __syncthreads();
+    if (wave != 0) return;
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int m = 0; m < MT; ++m)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int i = (t * MT + m) * 4 + r;
+                acc[t][m][r] = ((red[0][i][lane] + red[1][i][lane]) + red[2][i][lane]) + red[3][i][lane];
+            }
+    // ---- epilogue: the lane holds, per tile, features 4 grp + r of token 16 m + l16
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+        const int tok = 16 * m + l16;
+        if (tok >= M) continue;
+        if (EPI == EPI_SWIGLU) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int n = n0 + 4 * grp + r;
+                if (n >= n_out) continue;
+                const float gate = acc[0][m][r], up = acc[1][m][r];
+                const float sig = 1.0f / (1.0f + expf(-gate));
+                ((bf16_t *)Y)[(size_t)tok * ldy + n] = from_f32<bf16_t>(gate * sig * up);
+            }
+        } else {
+#pragma unroll
+            for (int t = 0; t < NT; ++t)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int n = n0 + 16 * t + 4 * grp + r;
+                    if (n >= N) continue;
+                    const size_t at = (size_t)tok * ldy + n;
+                    if (EPI == EPI_BF16) ((bf16_t *)Y)[at] = from_f32<bf16_t>(acc[t][m][r]);
+                    else if (EPI == EPI_F32) ((float *)Y)[at] = acc[t][m][r];
+                    else ((float *)Y)[at] += acc[t][m][r];
+                }
+        }
+    }
+}
+
+template <int NT, int MT>
+static int launch_epi(const void *X, int ldx, const void *W, int ldw, void *Y, int ldy, int M, int N, int K, int epi,
+                      hipStream_t stream) {
+    dim3 block(SK_WAVES * WAVE);
+    const dim3 grid((N + 16 * NT - 1) / (16 * NT));
+#define GO(E) gemm_skinny_kernel<NT, MT, E><<<grid, block, 0, stream>>>((const bf16_t *)X, ldx, (const bf16_t *)W, ldw, Y, ldy, M, N, K)
+    switch (epi) {
+    case EPI_BF16: GO(EPI_BF16); break;
+    case EPI_F32: GO(EPI_F32); break;
+    case EPI_ADD_F32: GO(EPI_ADD_F32); break;
+    default: return LCU_BAD_ARGUMENT;
+    }
+#undef GO
+    LCU_LAUNCH_CHECK();
+    return LCU_OK;
+}
+
+template <int MT>
+static int launch_swiglu(const void *X, int ldx, const void *W, int ldw, void *Y, int ldy, int M, int N, int K,
+                         hipStream_t stream) {
+    const int groups = (N / 2 + 15) / 16;
+    gemm_skinny_kernel<2, MT, EPI_SWIGLU><<<dim3(groups), dim3(SK_WAVES * WAVE), 0, stream>>>(
+        (const bf16_t *)X, ldx, (const bf16_t *)W, ldw, Y, ldy, M, N, K);
+    LCU_LAUNCH_CHECK();
+    return LCU_OK;
+}
+
+// X: [M, K] bfloat16 rows ldx apart; W: [N, K] bfloat16 rows ldw apart; Y: [M, N] rows ldy
+// apart (for the SwiGLU epilogue [M, N/2]: W holds N/2 gate rows, then N/2 up rows).
+// M <= 64; K, ldx and ldw multiples of 8 (16-byte loads); tiles: output tiles of 16
+// features per workgroup (1, 2 or 4; more tiles reuse X more, fewer give more workgroups).
+LCU_API int lcu_gemm_skinny_bf16(const void *X, int ldx, const void *W, int ldw, void *Y, int ldy, int M, int N, int K,
+                                 int epilogue, int tiles, hipStream_t stream) {
+    if (M <= 0 || N <= 0) return LCU_OK;
+    if (M > 64 || K <= 0 || K % 8 || ldx % 8 || ldw % 8 || ldx < K || ldw < K) return LCU_BAD_ARGUMENT;
+    const int mt = (M + 15) / 16;
+    if (epilogue == EPI_SWIGLU) {
+        if (N % 2 || ldy < N / 2) return LCU_BAD_ARGUMENT;
+        switch (mt) {
+        case 1: return launch_swiglu<1>(X, ldx, W, ldw, Y, ldy, M, N, K, stream);
+        case 2: return launch_swiglu<2>(X, ldx, W, ldw, Y, ldy, M, N, K, stream);
+        case 3: return launch_swiglu<3>(X, ldx, W, ldw, Y, ldy, M, N, K, stream);
+        default: return launch_swiglu<4>(X, ldx, W, ldw, Y, ldy, M, N, K, stream);
+        }
+    }
+    if (ldy < N) return LCU_BAD_ARGUMENT;
+#define PICK(NT)                                                                                   \
+    switch (mt) {                                                                                  \
+    case 1: return launch_epi<NT, 1>(X, ldx, W, ldw, Y, ldy, M, N, K, epilogue, stream);           \
+    case 2: return launch_epi<NT, 2>(X, ldx, W, ldw, Y, ldy, M, N, K, epilogue, stream);           \
+    case 3: return launch_epi<NT, 3>(X, ldx, W, ldw, Y, ldy, M, N, K, epilogue, stream);           \
+    default: return launch_epi<NT, 4>(X, ldx, W, ldw, Y, ldy, M, N, K, epilogue, stream);          \
+    }
+    if (tiles == 4 && mt > 2) tiles = 2;      // 4 x 4 tiles of accumulators and operands do not fit the registers
+    if (tiles == 1) { PICK(1) }
+    if (tiles == 2) { PICK(2) }
+    if (tiles == 4) { PICK(4) }
+#undef PICK
+    return LCU_BAD_ARGUMENT;
+}

@@ -350,10 +350,56 @@ def paged_attention(q: torch.Tensor, out: torch.Tensor, cache: torch.Tensor, ste
                              n_kv_heads, head_dim, page_size, scale, window)
 
 
+SKINNY_MAX_ROWS = 64
+_EPILOGUES = {"bf16": 0, "f32": 1, "add_f32": 2, "swiglu": 3}
+
+
 def skinny_supported(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype) -> bool:
-    """Whether the weight-streaming kernel for few rows takes this product."""
-    return False
+    """Whether the weight-streaming kernel for few rows takes this product: bfloat16
+    operands, at most 64 rows, K a multiple of 8 (16-byte loads)."""
+    return (x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and x.dim() == 2 and w.dim() == 2
+            and 0 < x.shape[0] <= SKINNY_MAX_ROWS and x.shape[1] % 8 == 0 and x.stride(1) == 1 and w.stride(1) == 1
+            and x.stride(0) % 8 == 0 and w.stride(0) % 8 == 0 and out_dtype in (torch.bfloat16, torch.float32)
+            and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
 
 
-def gemm_skinny(x, w, out=None, out_dtype=None, accumulate=False):
-    raise KernelError("gemm_skinny: not available")
+def _skinny_tiles(n_features: int, m: int) -> int:
+    """Output tiles of 16 features per workgroup: as many as still leave about four
+    workgroups for each of the 256 compute units."""
+    for tiles in (4, 2):
+        if n_features // (16 * tiles) >= 1024 and (tiles < 4 or m <= 32):
+            return tiles
+    return 1
+
+
+def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = None,
+                out_dtype: Optional[torch.dtype] = None, accumulate: bool = False, swiglu: bool = False,
+                tiles: Optional[int] = None) -> torch.Tensor:
+    """``out (+)= x @ w.T`` for at most 64 rows of bfloat16 ``x`` by streaming ``w`` once.
+    ``swiglu``: ``w`` holds gate rows, then up rows; ``out = silu(x @ gate.T) * (x @ up.T)``."""
+    _gpu(x, w, out)
+    _rows(x, "skinny x"); _rows(w, "skinny w")
+    m, k = x.shape
+    n = w.shape[0]
+    out_dtype = out.dtype if out is not None else (out_dtype or torch.bfloat16)
+    if w.shape[1] != k or not skinny_supported(x, w, out_dtype):
+        raise KernelError(f"gemm_skinny: x {tuple(x.shape)} {x.dtype} with w {tuple(w.shape)} {w.dtype} is not supported")
+    if swiglu:
+        if n % 2 or out_dtype != torch.bfloat16 or accumulate:
+            raise KernelError("gemm_skinny: the SwiGLU epilogue needs an even number of rows of w and a bfloat16 output")
+        epi, width = "swiglu", n // 2
+    elif accumulate:
+        if out is None or out.dtype != torch.float32:
+            raise KernelError("gemm_skinny: accumulate needs a float32 output to add to")
+        epi, width = "add_f32", n
+    else:
+        epi, width = ("f32" if out_dtype == torch.float32 else "bf16"), n
+    if out is None:
+        out = torch.empty((m, width), dtype=out_dtype, device=x.device)
+    _rows(out, "skinny out")
+    if out.shape != (m, width):
+        raise KernelError(f"gemm_skinny out: shape {tuple(out.shape)}, expected {(m, width)}")
+    lib = build.load("gemm_skinny")
+    _check(lib.lcu_gemm_skinny_bf16(_ptr(x), x.stride(0), _ptr(w), w.stride(0), _ptr(out), out.stride(0), m, n, k,
+                                    _EPILOGUES[epi], tiles or _skinny_tiles(width, m), _stream()), "gemm_skinny")
+    return out

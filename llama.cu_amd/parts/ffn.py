@@ -35,8 +35,12 @@ class SwiGLU(Part):
         self.dtype = build.dtype
 
     def forward(self, h: torch.Tensor) -> torch.Tensor:
-        gu = linear(h, self.w_gate_up, out_dtype=self.dtype)
-        act = ops.swiglu(gu)
+        if ops.skinny_supported(h, self.w_gate_up, self.dtype) and self.dtype == torch.bfloat16:
+            # few rows: one pass over the weights, the activation in the product's epilogue
+            act = ops.gemm_skinny(h, self.w_gate_up, swiglu=True)
+        else:
+            gu = linear(h, self.w_gate_up, out_dtype=self.dtype)
+            act = ops.swiglu(gu)
         return linear(act, self.w_down, out_dtype=self.dtype)
 
 

@@ -190,10 +190,16 @@ def run_trace_program(folder: str, dtype: str, steps, max_tokens: int, vocab: in
     return outputs
 
 
-# tolerances, as a fraction of the largest logit of the sequence (set from the formats'
-# precision, not from what passes): float32 rounds at 6e-8 and sums a few hundred terms;
-# bfloat16 activations round at 4e-3 about ten times per layer.
-REL_TOL = {"float32": 1e-4, "bfloat16": 5e-2}
+# Tolerances, as a fraction of the largest logit of the sequence, from the formats'
+# precision: float32 rounds at 6e-8 and sums a few hundred terms.  bfloat16 activations
+# round at 2^-8 = 4e-3 some forty times on the way through a tiny model; as independent
+# errors that is 4e-3 * sqrt(40) = 2.5e-2.  That model of the error holds while the softmax
+# is not sharp, so bfloat16 folders are made with a smaller weight scale (BF16_STD) than
+# float32 ones: with sharp scores a rounding of a score by 4e-3 * |score| moves the
+# softmax by several percent, and the comparison would measure the model's sensitivity,
+# not the engine.  Sharp scores are covered in 32-bit and by the kernels' own tests.
+REL_TOL = {"float32": 1e-4, "bfloat16": 2.5e-2}
+BF16_STD = 0.06
 
 
 def assert_matches_plain(got: Dict[str, Dict[int, np.ndarray]], want: Dict[str, torch.Tensor], dtype: str, what: str):

@@ -320,3 +320,48 @@ def test_attention_float32_result_does_not_depend_on_the_batch():
     out1 = torch.empty(1, nh * dh, device="cuda")
     ops.paged_attention(q[8:9].cuda(), out1, cache.cuda(), step1, 0, nh, nkv, dh, page, dh ** -0.5)
     assert torch.equal(out[8:9], out1)
+
+
+# ------------------------------------------------------------------ weight-streaming product for few rows
+@pytest.mark.parametrize("m", [1, 8, 16, 17, 40, 64])
+@pytest.mark.parametrize("n,k", [(16, 8), (100, 64), (301, 136), (1000, 4096), (4096, 1000)])
+@pytest.mark.parametrize("tiles", [1, 2, 4])
+def test_gemm_skinny(m, n, k, tiles):
+    from llama_cu_amd.kernels import ops
+    x = rnd(m, k, seed=m + k).to(torch.bfloat16)
+    w = rnd(n, k, seed=n).to(torch.bfloat16)
+    want = plain.linear(x, w)
+    close(ops.gemm_skinny(x.cuda(), w.cuda(), tiles=tiles), want, "bfloat16", "bf16 out")
+    close(ops.gemm_skinny(x.cuda(), w.cuda(), out_dtype=torch.float32, tiles=tiles), want, "float32", "f32 out")
+    c = rnd(m, n, seed=5)
+    cg = c.cuda()
+    ops.gemm_skinny(x.cuda(), w.cuda(), out=cg, accumulate=True, tiles=tiles)
+    close(cg, c.double() + want, "float32", "accumulate")
+
+
+@pytest.mark.parametrize("m,di,k", [(1, 8, 16), (8, 172, 64), (33, 1000, 128), (64, 14336, 256)])
+def test_gemm_skinny_swiglu(m, di, k):
+    from llama_cu_amd.kernels import ops
+    x = rnd(m, k, seed=m).to(torch.bfloat16)
+    w = rnd(2 * di, k, seed=di, scale=0.3).to(torch.bfloat16)
+    gu = plain.linear(x, w)
+    close(ops.gemm_skinny(x.cuda(), w.cuda(), swiglu=True), plain.swiglu(gu[:, :di], gu[:, di:]), "bfloat16")
+
+
+def test_gemm_skinny_result_does_not_depend_on_the_batch():
+    from llama_cu_amd.kernels import ops
+    x = rnd(40, 512, seed=1).to(torch.bfloat16).cuda()
+    w = rnd(300, 512, seed=2).to(torch.bfloat16).cuda()
+    whole = ops.gemm_skinny(x, w, out_dtype=torch.float32)
+    one = ops.gemm_skinny(x[23:24], w, out_dtype=torch.float32)
+    assert torch.equal(whole[23:24], one)
+
+
+def test_gemm_skinny_refuses_what_it_cannot_take():
+    from llama_cu_amd.kernels import ops
+    x = rnd(4, 172).to(torch.bfloat16).cuda()        # K no multiple of 8
+    w = rnd(16, 172).to(torch.bfloat16).cuda()
+    assert not ops.skinny_supported(x, w, torch.bfloat16)
+    with pytest.raises(ops.KernelError):
+        ops.gemm_skinny(x, w)
+    assert not ops.skinny_supported(rnd(65, 64).to(torch.bfloat16).cuda(), rnd(16, 64).to(torch.bfloat16).cuda(), torch.bfloat16)

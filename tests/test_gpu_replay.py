@@ -17,7 +17,8 @@ def models():
     out = {}
     for name, cfg in common.TINY.items():
         for dtype, tdt in (("float32", torch.float32), ("bfloat16", torch.bfloat16)):
-            folder = common.make_folder(cfg, seed=11 + len(out), dtype=tdt)
+            folder = common.make_folder(cfg, seed=11 + len(out), dtype=tdt,
+                                        std=common.BF16_STD if dtype == "bfloat16" else 0.15)
             reqs = common.random_requests(cfg["vocab_size"], LENGTHS[name], seed=5)
             out[(name, dtype)] = (folder, reqs, common.plain_logits(folder, reqs))
     return out
