@@ -59,40 +59,53 @@ __device__ __forceinline__ void attn_init(AttnState<DH, QB> &st) {
     }
 }
 
-// One step: the 32 keys k0 .. k0+31 (k0 a multiple of 32) of key/value head kvh.
-// p_row / lo_row: the last and first key each of the lane's rows may see.  MASK: some row
-// of the wave does not see all 32 keys; p_max / lo_min bound what any row sees (values of
-// keys outside are not used at all, whatever the memory holds).
-template <int DH, int QB, bool MASK>
-__device__ __forceinline__ void attn_step(const bf16_t *__restrict__ cache, const int *__restrict__ bt, int max_pages,
-                                          int page, size_t page_elems, int nkvh, int kvh, int k0,
-                                          const u32x4 (&q)[QB][DH / 32], AttnState<DH, QB> &st,
-                                          const int (&p_row)[QB], const int (&lo_row)[QB], int p_max, int lo_min,
-                                          float scale_log2, int l16, int grp) {
-    const bf16_t *pg[2];
-    int tok0[2];
+// The lane's share of the keys and values of one step: the 32 keys k0 .. k0+31 (k0 a
+// multiple of 32) of key/value head kvh, as two tiles of 16 keys.
+template <int DH>
+struct KVFrag {
+    u32x4 k[2][DH / 32];    // tile t, dims 32*kb + 8*grp .. + 7 of key 16*t + lane%16
+    u32x2 v[DH / 16][2];    // dim 16*dt + lane%16, keys 16*t + 4*grp .. + 3
+};
+
+template <int DH>
+__device__ __forceinline__ void load_kv(KVFrag<DH> &f, const bf16_t *__restrict__ cache, const int *__restrict__ bt,
+                                        int max_pages, int page, size_t page_elems, int nkvh, int kvh, int k0, int l16,
+                                        int grp) {
+    const size_t v_off = (size_t)nkvh * DH * page + (size_t)kvh * DH * page + 4 * grp;
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
         const int j = k0 + 16 * t;
         int pi = j / page;
         pi = pi < max_pages ? pi : max_pages - 1;       // a tile beyond the context is masked; keep the read in bounds
-        pg[t] = cache + (size_t)bt[pi] * page_elems;
-        tok0[t] = j % page;
+        const bf16_t *pg = cache + (size_t)bt[pi] * page_elems;
+        const int tok0 = j % page;
+        const bf16_t *kp = pg + ((size_t)kvh * (DH / 8) * page + tok0 + l16) * 8;
+#pragma unroll
+        for (int kb = 0; kb < DH / 32; ++kb) f.k[t][kb] = *(const u32x4 *)(kp + (size_t)(4 * kb + grp) * page * 8);
+        const bf16_t *vp = pg + v_off + tok0;
+#pragma unroll
+        for (int dt = 0; dt < DH / 16; ++dt) f.v[dt][t] = *(const u32x2 *)(vp + (size_t)(16 * dt + l16) * page);
     }
+}
+
+// One step of the online softmax on loaded keys and values.  p_row / lo_row: the last and
+// first key each of the lane's rows may see.  MASK: some row of the wave does not see all
+// 32 keys; p_max / lo_min bound what any row sees (values of keys outside are not used at
+// all, whatever the memory holds).
+template <int DH, int QB, bool MASK>
+__device__ __forceinline__ void attn_compute(const KVFrag<DH> &f, int k0, const u32x4 (&q)[QB][DH / 32],
+                                             AttnState<DH, QB> &st, const int (&p_row)[QB], const int (&lo_row)[QB],
+                                             int p_max, int lo_min, float scale_log2, int grp) {
     // ---- S^T = K Q^T
     f32x4 s[QB][2];
 #pragma unroll
     for (int b = 0; b < QB; ++b) s[b][0] = s[b][1] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
-        const bf16_t *kp = pg[t] + ((size_t)kvh * (DH / 8) * page + tok0[t] + l16) * 8;
+    for (int t = 0; t < 2; ++t)
 #pragma unroll
-        for (int kb = 0; kb < DH / 32; ++kb) {
-            const u32x4 kv = *(const u32x4 *)(kp + (size_t)(4 * kb + grp) * page * 8);
+        for (int kb = 0; kb < DH / 32; ++kb)
 #pragma unroll
-            for (int b = 0; b < QB; ++b) s[b][t] = mfma16(kv, q[b][kb], s[b][t]);
-        }
-    }
+            for (int b = 0; b < QB; ++b) s[b][t] = mfma16(f.k[t][kb], q[b][kb], s[b][t]);
     // ---- softmax of the step, online
     u32x4 pb[QB];
 #pragma unroll
@@ -128,18 +141,15 @@ __device__ __forceinline__ void attn_step(const bf16_t *__restrict__ cache, cons
         pb[b] = u32x4{pack_bf16(p[0], p[1]), pack_bf16(p[2], p[3]), pack_bf16(p[4], p[5]), pack_bf16(p[6], p[7])};
     }
     // ---- O^T += V^T P^T
-    const size_t v_off = (size_t)nkvh * DH * page + (size_t)kvh * DH * page;
 #pragma unroll
     for (int dt = 0; dt < DH / 16; ++dt) {
-        const size_t row = v_off + (size_t)(16 * dt + l16) * page + 4 * grp;
-        u32x2 v0 = *(const u32x2 *)(pg[0] + row + tok0[0]);
-        u32x2 v1 = *(const u32x2 *)(pg[1] + row + tok0[1]);
+        u32x2 v0 = f.v[dt][0], v1 = f.v[dt][1];
         if (MASK) {
             // values of keys that no row sees are taken as zero: their memory may hold anything
             const int j0 = k0 + 4 * grp, j1 = k0 + 16 + 4 * grp;
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                const uint32_t keep = (r & 1) ? 0x0000ffffu : 0xffff0000u;   // mask that clears element r of its dword
+                const uint32_t keep = (r & 1) ? 0x0000ffffu : 0xffff0000u;   // clears element r of its dword
                 if (j0 + r > p_max || j0 + r < lo_min) { if (r < 2) v0.x &= keep; else v0.y &= keep; }
                 if (j1 + r > p_max || j1 + r < lo_min) { if (r < 2) v1.x &= keep; else v1.y &= keep; }
             }
@@ -148,6 +158,15 @@ __device__ __forceinline__ void attn_step(const bf16_t *__restrict__ cache, cons
 #pragma unroll
         for (int b = 0; b < QB; ++b) st.o[b][dt] = mfma16(a, pb[b], st.o[b][dt]);
     }
+}
+
+// Masks only where a row needs them (the choice is the same for the whole wave).
+template <int DH, int QB>
+__device__ __forceinline__ void attn_block(const KVFrag<DH> &f, int k0, bool mask, const u32x4 (&q)[QB][DH / 32],
+                                           AttnState<DH, QB> &st, const int (&p_row)[QB], const int (&lo_row)[QB],
+                                           int p_max, int lo_min, float scale_log2, int grp) {
+    if (mask) attn_compute<DH, QB, true>(f, k0, q, st, p_row, lo_row, p_max, lo_min, scale_log2, grp);
+    else attn_compute<DH, QB, false>(f, k0, q, st, p_row, lo_row, p_max, lo_min, scale_log2, grp);
 }
 
 // The lane's part of the queries of one block of rows: 8 dims of row lane%16 per 32-dim
@@ -196,12 +215,17 @@ attention_decode_kernel(const bf16_t *__restrict__ q, int q_stride, bf16_t *__re
     const int first = lo / 32, last = p / 32, nblk = last - first + 1;
     const int b0 = first + (int)((long long)nblk * split / n_splits);
     const int b1 = first + (int)((long long)nblk * (split + 1) / n_splits);
-    for (int blk = b0 + wave; blk < b1; blk += DEC_WAVES) {
-        const int k0 = blk * 32;
-        if (k0 + 31 > p || k0 < lo)
-            attn_step<DH, 1, true>(cache, bt, max_pages, page, page_elems, nkvh, kvh, k0, qv, st, p_row, lo_row, p, lo, scale_log2, l16, grp);
-        else
-            attn_step<DH, 1, false>(cache, bt, max_pages, page, page_elems, nkvh, kvh, k0, qv, st, p_row, lo_row, p, lo, scale_log2, l16, grp);
+    // the wave's steps are blk, blk + 4, ...; the next step's loads are in flight while one is computed
+    KVFrag<DH> fa, fb;
+    int blk = b0 + wave;
+    if (blk < b1) load_kv<DH>(fa, cache, bt, max_pages, page, page_elems, nkvh, kvh, blk * 32, l16, grp);
+    for (; blk < b1; blk += 2 * DEC_WAVES) {
+        const int nb = blk + DEC_WAVES, nb2 = blk + 2 * DEC_WAVES;
+        if (nb < b1) load_kv<DH>(fb, cache, bt, max_pages, page, page_elems, nkvh, kvh, nb * 32, l16, grp);
+        attn_block<DH, 1>(fa, blk * 32, blk * 32 + 31 > p || blk * 32 < lo, qv, st, p_row, lo_row, p, lo, scale_log2, grp);
+        if (nb2 < b1) load_kv<DH>(fa, cache, bt, max_pages, page, page_elems, nkvh, kvh, nb2 * 32, l16, grp);
+        if (nb < b1)
+            attn_block<DH, 1>(fb, nb * 32, nb * 32 + 31 > p || nb * 32 < lo, qv, st, p_row, lo_row, p, lo, scale_log2, grp);
     }
     // ---- merge the waves
     float l_all = st.l[0];
@@ -243,6 +267,9 @@ attention_decode_kernel(const bf16_t *__restrict__ q, int q_stride, bf16_t *__re
 }
 
 // Merges the parts of every (token, head): out = sum_s O_s 2^(m_s - M) / sum_s l_s 2^(m_s - M).
+// (A merge inside the decode kernel by the workgroup that finishes last needs a
+// device-wide fence per workgroup, which writes back and invalidates the whole L2: measured
+// several times slower than this second launch.)
 template <int DH>
 __global__ void attention_merge_kernel(bf16_t *__restrict__ out, int out_stride, const float *__restrict__ part_o,
                                        const float *__restrict__ part_ml, int nh, int n_splits) {
@@ -252,10 +279,11 @@ __global__ void attention_merge_kernel(bf16_t *__restrict__ out, int out_stride,
     for (int s = 0; s < n_splits; ++s) M = fmaxf(M, part_ml[(base + s) * 2]);
     float L = 0.f;
     for (int s = 0; s < n_splits; ++s) L += part_ml[(base + s) * 2 + 1] * exp2f(part_ml[(base + s) * 2] - M);
+    const float inv = 1.0f / L;
     for (int d = threadIdx.x; d < DH; d += blockDim.x) {
         float val = 0.f;
         for (int s = 0; s < n_splits; ++s) val += part_o[(base + s) * DH + d] * exp2f(part_ml[(base + s) * 2] - M);
-        out[(size_t)token * out_stride + (size_t)head * DH + d] = from_f32<bf16_t>(val / L);
+        out[(size_t)token * out_stride + (size_t)head * DH + d] = from_f32<bf16_t>(val * inv);
     }
 }
 
@@ -273,8 +301,8 @@ static int launch_decode(const void *q, int q_stride, void *out, int out_stride,
         ctx_len, nh, nkvh, page, scale_log2, window, n_splits, part_o, part_ml);
     LCU_LAUNCH_CHECK();
     if (n_splits > 1) {
-        attention_merge_kernel<DH><<<dim3(n_req, nh), dim3(DH < 64 ? 64 : DH / 2), 0, stream>>>(
-            (bf16_t *)out, out_stride, part_o, part_ml, nh, n_splits);
+        attention_merge_kernel<DH><<<dim3(n_req, nh), dim3(WAVE), 0, stream>>>((bf16_t *)out, out_stride, part_o, part_ml,
+                                                                                nh, n_splits);
         LCU_LAUNCH_CHECK();
     }
     return LCU_OK;
@@ -348,12 +376,16 @@ attention_prefill_kernel(const bf16_t *__restrict__ q, int q_stride, bf16_t *__r
     attn_init(st);
     const int *bt = block_table + (size_t)r * max_pages;
     const size_t page_elems = kv_page_elems(nkvh, DH, page);
-    for (int blk = lo_min / 32; blk <= p_max / 32; ++blk) {
-        const int k0 = blk * 32;
-        if (k0 + 31 > p_min || k0 < lo_max)
-            attn_step<DH, QB, true>(cache, bt, max_pages, page, page_elems, nkvh, kvh, k0, qv, st, p_row, lo_row, p_max, lo_min, scale_log2, l16, grp);
-        else
-            attn_step<DH, QB, false>(cache, bt, max_pages, page, page_elems, nkvh, kvh, k0, qv, st, p_row, lo_row, p_max, lo_min, scale_log2, l16, grp);
+    KVFrag<DH> fa, fb;
+    const int blk_end = p_max / 32 + 1;
+    int blk = lo_min / 32;
+    load_kv<DH>(fa, cache, bt, max_pages, page, page_elems, nkvh, kvh, blk * 32, l16, grp);
+    for (; blk < blk_end; blk += 2) {
+        if (blk + 1 < blk_end) load_kv<DH>(fb, cache, bt, max_pages, page, page_elems, nkvh, kvh, (blk + 1) * 32, l16, grp);
+        attn_block<DH, QB>(fa, blk * 32, blk * 32 + 31 > p_min || blk * 32 < lo_max, qv, st, p_row, lo_row, p_max, lo_min, scale_log2, grp);
+        if (blk + 2 < blk_end) load_kv<DH>(fa, cache, bt, max_pages, page, page_elems, nkvh, kvh, (blk + 2) * 32, l16, grp);
+        if (blk + 1 < blk_end)
+            attn_block<DH, QB>(fb, (blk + 1) * 32, (blk + 1) * 32 + 31 > p_min || (blk + 1) * 32 < lo_max, qv, st, p_row, lo_row, p_max, lo_min, scale_log2, grp);
     }
 #pragma unroll
     for (int b = 0; b < QB; ++b) {

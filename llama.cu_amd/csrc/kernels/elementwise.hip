@@ -92,10 +92,70 @@ __global__ void rmsnorm_kernel(TX *__restrict__ x, const TD *__restrict__ delta,
     }
 }
 
+// The same for rows of up to 8192 elements whose width is a multiple of 4: one read of
+// the row (four elements per thread and load), the row kept in registers between the sum
+// and the scaling.  The order of the sum depends on d only.
+constexpr int NORM_THREADS = 256, NORM_ITEMS = 8;
+
+template <class T> struct alignas(4 * sizeof(T)) Vec4 { T v[4]; };
+
+template <class TX, class TD, class TW, class TO>
+__global__ void __launch_bounds__(NORM_THREADS)
+rmsnorm_fast_kernel(TX *__restrict__ x, const TD *__restrict__ delta, const TW *__restrict__ w, TO *__restrict__ out,
+                    int d, float eps, int write_back) {
+    __shared__ float scratch[16];
+    TX *xr = x + (size_t)blockIdx.x * d;
+    const TD *dr = delta ? delta + (size_t)blockIdx.x * d : nullptr;
+    float v[NORM_ITEMS][4];
+    float acc = 0.f;
+#pragma unroll
+    for (int i = 0; i < NORM_ITEMS; ++i) {
+        const int c = (i * NORM_THREADS + threadIdx.x) * 4;
+        if (c < d) {
+            const Vec4<TX> xv = *(const Vec4<TX> *)(xr + c);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[i][e] = to_f32(xv.v[e]);
+            if (dr) {
+                const Vec4<TD> dv = *(const Vec4<TD> *)(dr + c);
+                Vec4<TX> back;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) { v[i][e] += to_f32(dv.v[e]); back.v[e] = from_f32<TX>(v[i][e]); }
+                if (write_back) *(Vec4<TX> *)(xr + c) = back;
+            }
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc += v[i][e] * v[i][e];
+        }
+    }
+    const float total = block_sum(acc, scratch);
+    const float rms = rsqrtf(total / (float)d + eps);
+    TO *o = out + (size_t)blockIdx.x * d;
+#pragma unroll
+    for (int i = 0; i < NORM_ITEMS; ++i) {
+        const int c = (i * NORM_THREADS + threadIdx.x) * 4;
+        if (c < d) {
+            const Vec4<TW> wv = *(const Vec4<TW> *)(w + c);
+            Vec4<TO> ov;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) ov.v[e] = from_f32<TO>(rms * v[i][e] * to_f32(wv.v[e]));
+            *(Vec4<TO> *)(o + c) = ov;
+        }
+    }
+}
+
 template <class TX, class TD, class TO>
 static int rmsnorm_w(void *x, const void *delta, const void *w, int w_type, void *out, int n, int d, float eps,
                      int write_back, hipStream_t stream) {
     dim3 grid(n), block(d >= 2048 ? 512 : 256);
+    if (d % 4 == 0 && d <= NORM_THREADS * NORM_ITEMS * 4) {
+        if (w_type == LCU_F32)
+            rmsnorm_fast_kernel<TX, TD, float, TO><<<grid, dim3(NORM_THREADS), 0, stream>>>((TX *)x, (const TD *)delta, (const float *)w, (TO *)out, d, eps, write_back);
+        else if (w_type == LCU_BF16)
+            rmsnorm_fast_kernel<TX, TD, bf16_t, TO><<<grid, dim3(NORM_THREADS), 0, stream>>>((TX *)x, (const TD *)delta, (const bf16_t *)w, (TO *)out, d, eps, write_back);
+        else
+            return LCU_BAD_ARGUMENT;
+        LCU_LAUNCH_CHECK();
+        return LCU_OK;
+    }
     if (w_type == LCU_F32)
         rmsnorm_kernel<TX, TD, float, TO><<<grid, block, 0, stream>>>((TX *)x, (const TD *)delta, (const float *)w, (TO *)out, d, eps, write_back);
     else if (w_type == LCU_BF16)

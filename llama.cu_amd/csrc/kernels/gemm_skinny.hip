@@ -2,7 +2,7 @@
 // 32-bit accumulation on the matrix cores.  The work is streaming W once from HBM, so
 // the kernel is laid out around W's loads:
 //
-//   * a workgroup of 4 waves owns NT tiles of 16 output features (rows of W) and walks
+//   * a workgroup of 4 or 8 waves owns NT tiles of 16 output features (rows of W) and walks
 //     the whole K: no sum crosses workgroups, results do not depend on the grid, and
 //     the epilogue can be fused;
 //   * K goes in macro-steps of 128; the waves take macro-steps in turn; in a macro-step
@@ -13,7 +13,7 @@
 //   * the next macro-step's loads are issued before the current one is multiplied;
 //   * v_mfma_f32_16x16x32_bf16 with A = W tile, B = X^T: the 16 columns are 16 tokens,
 //     MT such tiles for up to 64 tokens.
-// The four waves' partial sums are added in LDS in a fixed order.
+// The waves' partial sums are added in LDS in a fixed order.
 //
 // Epilogues: store bfloat16; store float32 (logits); add into float32 (the residual
 // stream); SwiGLU, where the workgroup's two tiles are the gate rows n and the up rows
@@ -25,7 +25,6 @@ typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 
 enum { EPI_BF16 = 0, EPI_F32 = 1, EPI_ADD_F32 = 2, EPI_SWIGLU = 3 };
-constexpr int SK_WAVES = 4;
 
 __device__ __forceinline__ f32x4 mfma16(u32x4 a, u32x4 b, f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
@@ -75,7 +74,7 @@ __device__ __forceinline__ void mul_frag(const Frag<NT, MT> &f, f32x4 (&acc)[NT]
             for (int m = 0; m < MT; ++m) acc[t][m] = mfma16(f.w[t][j], f.x[m][j], acc[t][m]);
 }
 
-template <int NT, int MT, int EPI>
+template <int NT, int MT, int EPI, int SK_WAVES>
 __global__ void __launch_bounds__(SK_WAVES *WAVE)
 gemm_skinny_kernel(const bf16_t *__restrict__ X, int ldx, const bf16_t *__restrict__ W, int ldw, void *__restrict__ Y,
                    int ldy, int M, int N, int K) {
@@ -117,7 +116,7 @@ gemm_skinny_kernel(const bf16_t *__restrict__ X, int ldx, const bf16_t *__restri
         if (s + 2 * SK_WAVES < nsteps) load_frag<NT, MT>(fa, wrow, xrow, xvalid, s + 2 * SK_WAVES, grp, K);
         if (has_b) mul_frag<NT, MT>(fb, acc);
     }
-    // ---- the four waves' sums, added in the order 0, 1, 2, 3
+    // ---- the waves' sums, added in the order 0, 1, 2, ...
 #pragma unroll
     for (int t = 0; t < NT; ++t)
 #pragma unroll
@@ -133,7 +132,10 @@ gemm_skinny_kernel(const bf16_t *__restrict__ X, int ldx, const bf16_t *__restri
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int i = (t * MT + m) * 4 + r;
-                acc[t][m][r] = ((red[0][i][lane] + red[1][i][lane]) + red[2][i][lane]) + red[3][i][lane];
+                float sum = red[0][i][lane];
+#pragma unroll
+                for (int w = 1; w < SK_WAVES; ++w) sum += red[w][i][lane];
+                acc[t][m][r] = sum;
             }
     // ---- epilogue: the lane holds, per tile, features 4 grp + r of token 16 m + l16
 #pragma unroll
@@ -165,12 +167,12 @@ gemm_skinny_kernel(const bf16_t *__restrict__ X, int ldx, const bf16_t *__restri
     }
 }
 
-template <int NT, int MT>
+template <int NT, int MT, int WAVES>
 static int launch_epi(const void *X, int ldx, const void *W, int ldw, void *Y, int ldy, int M, int N, int K, int epi,
                       hipStream_t stream) {
-    dim3 block(SK_WAVES * WAVE);
+    dim3 block(WAVES * WAVE);
     const dim3 grid((N + 16 * NT - 1) / (16 * NT));
-#define GO(E) gemm_skinny_kernel<NT, MT, E><<<grid, block, 0, stream>>>((const bf16_t *)X, ldx, (const bf16_t *)W, ldw, Y, ldy, M, N, K)
+#define GO(E) gemm_skinny_kernel<NT, MT, E, WAVES><<<grid, block, 0, stream>>>((const bf16_t *)X, ldx, (const bf16_t *)W, ldw, Y, ldy, M, N, K)
     switch (epi) {
     case EPI_BF16: GO(EPI_BF16); break;
     case EPI_F32: GO(EPI_F32); break;
@@ -182,11 +184,11 @@ static int launch_epi(const void *X, int ldx, const void *W, int ldw, void *Y, i
     return LCU_OK;
 }
 
-template <int MT>
+template <int MT, int WAVES>
 static int launch_swiglu(const void *X, int ldx, const void *W, int ldw, void *Y, int ldy, int M, int N, int K,
                          hipStream_t stream) {
     const int groups = (N / 2 + 15) / 16;
-    gemm_skinny_kernel<2, MT, EPI_SWIGLU><<<dim3(groups), dim3(SK_WAVES * WAVE), 0, stream>>>(
+    gemm_skinny_kernel<2, MT, EPI_SWIGLU, WAVES><<<dim3(groups), dim3(WAVES * WAVE), 0, stream>>>(
         (const bf16_t *)X, ldx, (const bf16_t *)W, ldw, Y, ldy, M, N, K);
     LCU_LAUNCH_CHECK();
     return LCU_OK;
@@ -195,33 +197,41 @@ static int launch_swiglu(const void *X, int ldx, const void *W, int ldw, void *Y
 // X: [M, K] bfloat16 rows ldx apart; W: [N, K] bfloat16 rows ldw apart; Y: [M, N] rows ldy
 // apart (for the SwiGLU epilogue [M, N/2]: W holds N/2 gate rows, then N/2 up rows).
 // M <= 64; K, ldx and ldw multiples of 8 (16-byte loads); tiles: output tiles of 16
-// features per workgroup (1, 2 or 4; more tiles reuse X more, fewer give more workgroups).
+// features per workgroup (1, 2 or 4; more tiles reuse X more, fewer give more workgroups);
+// waves: 4 or 8 waves share a workgroup's K.
 LCU_API int lcu_gemm_skinny_bf16(const void *X, int ldx, const void *W, int ldw, void *Y, int ldy, int M, int N, int K,
-                                 int epilogue, int tiles, hipStream_t stream) {
+                                 int epilogue, int tiles, int waves, hipStream_t stream) {
     if (M <= 0 || N <= 0) return LCU_OK;
     if (M > 64 || K <= 0 || K % 8 || ldx % 8 || ldw % 8 || ldx < K || ldw < K) return LCU_BAD_ARGUMENT;
+    if (waves != 4 && waves != 8) return LCU_BAD_ARGUMENT;
     const int mt = (M + 15) / 16;
     if (epilogue == EPI_SWIGLU) {
         if (N % 2 || ldy < N / 2) return LCU_BAD_ARGUMENT;
+#define SW(MT_) return waves == 8 ? launch_swiglu<MT_, 8>(X, ldx, W, ldw, Y, ldy, M, N, K, stream) \
+                                  : launch_swiglu<MT_, 4>(X, ldx, W, ldw, Y, ldy, M, N, K, stream)
         switch (mt) {
-        case 1: return launch_swiglu<1>(X, ldx, W, ldw, Y, ldy, M, N, K, stream);
-        case 2: return launch_swiglu<2>(X, ldx, W, ldw, Y, ldy, M, N, K, stream);
-        case 3: return launch_swiglu<3>(X, ldx, W, ldw, Y, ldy, M, N, K, stream);
-        default: return launch_swiglu<4>(X, ldx, W, ldw, Y, ldy, M, N, K, stream);
+        case 1: SW(1);
+        case 2: SW(2);
+        case 3: SW(3);
+        default: SW(4);
         }
+#undef SW
     }
     if (ldy < N) return LCU_BAD_ARGUMENT;
-#define PICK(NT)                                                                                   \
-    switch (mt) {                                                                                  \
-    case 1: return launch_epi<NT, 1>(X, ldx, W, ldw, Y, ldy, M, N, K, epilogue, stream);           \
-    case 2: return launch_epi<NT, 2>(X, ldx, W, ldw, Y, ldy, M, N, K, epilogue, stream);           \
-    case 3: return launch_epi<NT, 3>(X, ldx, W, ldw, Y, ldy, M, N, K, epilogue, stream);           \
-    default: return launch_epi<NT, 4>(X, ldx, W, ldw, Y, ldy, M, N, K, epilogue, stream);          \
-    }
     if (tiles == 4 && mt > 2) tiles = 2;      // 4 x 4 tiles of accumulators and operands do not fit the registers
+#define EP(NT_, MT_) return waves == 8 ? launch_epi<NT_, MT_, 8>(X, ldx, W, ldw, Y, ldy, M, N, K, epilogue, stream) \
+                                       : launch_epi<NT_, MT_, 4>(X, ldx, W, ldw, Y, ldy, M, N, K, epilogue, stream)
+#define PICK(NT_)          \
+    switch (mt) {          \
+    case 1: EP(NT_, 1);    \
+    case 2: EP(NT_, 2);    \
+    case 3: EP(NT_, 3);    \
+    default: EP(NT_, 4);   \
+    }
     if (tiles == 1) { PICK(1) }
     if (tiles == 2) { PICK(2) }
     if (tiles == 4) { PICK(4) }
 #undef PICK
+#undef EP
     return LCU_BAD_ARGUMENT;
 }

@@ -9,14 +9,16 @@
 #include "common.h"
 #include "kv_layout.h"
 
+// One block per (token, head): query heads are rotated in place, key heads are rotated into
+// the cache, value heads are copied into the cache.
 template <class T>
 __global__ void rope_kv_store_kernel(T *__restrict__ qkv, int row_stride, const int *__restrict__ positions,
                                      const int *__restrict__ slots, const float *__restrict__ cos_t,
                                      const float *__restrict__ sin_t, int max_pos, T *__restrict__ cache,
                                      int nh, int nkvh, int dh, int rot_dim, int pairing, int page,
                                      int store_kv) {
-    const int t = blockIdx.x;
-    T *row = qkv + (size_t)t * row_stride;
+    const int t = blockIdx.x, head = blockIdx.y;
+    T *x = qkv + (size_t)t * row_stride + (size_t)head * dh;
     const int pos = positions[t];
     const int half = rot_dim / 2;
     const bool in_table = pos >= 0 && pos < max_pos;
@@ -30,12 +32,16 @@ __global__ void rope_kv_store_kernel(T *__restrict__ qkv, int row_stride, const 
         pg = cache + (size_t)(slot / page) * kv_page_elems(nkvh, dh, page);
         tok = slot % page;
     }
-    const int rot_heads = store_kv ? nh + nkvh : nh;
-    const int pairs_per_head = dh / 2;
-    // queries and keys: one work item per pair of dims
-    for (int w = threadIdx.x; w < rot_heads * pairs_per_head; w += blockDim.x) {
-        const int head = w / pairs_per_head, i = w % pairs_per_head;
-        T *x = row + (size_t)head * dh;
+    if (head >= nh + nkvh) {                    // a value head: copied as it is
+        if (!pg) return;
+        const int kvh = head - nh - nkvh;
+        for (int c = threadIdx.x; c < dh; c += blockDim.x) pg[kv_value_offset(nkvh, kvh, tok, c, dh, page)] = x[c];
+        return;
+    }
+    const bool is_key = head >= nh;
+    if (is_key && !pg) return;
+    if (!is_key && !rotate && !poison) return;  // a query head that is not rotated stays as it is
+    for (int i = threadIdx.x; i < dh / 2; i += blockDim.x) {
         int ia, ib;
         const bool rot = rotate && i < half;
         if (i < half) {                // a rotated pair
@@ -51,20 +57,12 @@ __global__ void rope_kv_store_kernel(T *__restrict__ qkv, int row_stride, const 
         }
         if (poison && i < half) a = b = __uint_as_float(0x7fc00000u);
         const T va = from_f32<T>(a), vb = from_f32<T>(b);
-        if (head < nh) {
+        if (!is_key) {
             if (rot || poison) { x[ia] = va; x[ib] = vb; }
-        } else if (pg) {
+        } else {
             const int kvh = head - nh;
             pg[kv_key_offset(kvh, tok, ia, dh, page)] = va;
             pg[kv_key_offset(kvh, tok, ib, dh, page)] = vb;
-        }
-    }
-    // values: copied as they are
-    if (pg) {
-        const T *v = row + (size_t)(nh + nkvh) * dh;
-        for (int w = threadIdx.x; w < nkvh * dh; w += blockDim.x) {
-            const int kvh = w / dh, c = w % dh;
-            pg[kv_value_offset(nkvh, kvh, tok, c, dh, page)] = v[w];
         }
     }
 }
@@ -81,7 +79,8 @@ LCU_API int lcu_rope_kv_store(void *qkv, int type, int n, int row_stride, const 
         return LCU_BAD_ARGUMENT;
     if (store_kv && (!cache || !slots || nkvh <= 0)) return LCU_BAD_ARGUMENT;
     if (row_stride < (store_kv ? (nh + 2 * nkvh) : nh) * dh) return LCU_BAD_ARGUMENT;
-    dim3 grid(n), block(256);
+    if (nh + 2 * nkvh > 65535) return LCU_BAD_ARGUMENT;
+    dim3 grid(n, store_kv ? nh + 2 * nkvh : nh), block(dh / 2 >= 64 ? 64 : 32);
     if (type == LCU_F32)
         rope_kv_store_kernel<float><<<grid, block, 0, stream>>>((float *)qkv, row_stride, positions, slots, cos_t, sin_t, max_pos, (float *)cache, nh, nkvh, dh, rot_dim, pairing, page, store_kv);
     else if (type == LCU_BF16)

@@ -49,7 +49,7 @@ class ModelRunner:
     def __init__(self, spec: ModelSpec, tensors: Dict[str, torch.Tensor], dtype, device="cuda:0",
                  page_size: int = 16, max_tokens: Optional[int] = None, num_pages: Optional[int] = None,
                  max_seqs: int = 8, max_batch_tokens: int = 2048, max_model_len: Optional[int] = None,
-                 kv_fraction: float = 0.85):
+                 kv_fraction: float = 0.85, use_graphs: bool = True):
         self.device = require_gpu(device)
         self.dtype = DTYPES[dtype]
         self.spec = spec
@@ -97,6 +97,10 @@ class ModelRunner:
                 raise ValueError(f"run order entry {i}: unknown cache need {need!r}")
         max_pages = [(self.max_model_len + self.page_size - 1) // self.page_size for _ in self.groups]
         self.builder = BatchBuilder(self.cache, self.max_batch_tokens, self.max_seqs, max_pages, self.device)
+        # captured decode steps, by batch size: (graph, its logits tensor)
+        self.use_graphs = bool(use_graphs)
+        self._graphs: Dict[int, Any] = {}
+        self._seen: Dict[int, int] = {}
 
     # ------------------------------------------------------------ construction helpers
     @classmethod
@@ -150,8 +154,43 @@ class ModelRunner:
             raise
         return self.builder.build(req_ids, tokens, want, self.spec.vocab_size)
 
+    GRAPH_AFTER = 2          # a batch size is captured when it comes for the third time
+    GRAPH_MAX_BATCH = 256
+
     def run(self, step: StepContext) -> torch.Tensor:
-        return self.model.forward(step, self.caches)
+        """The model on the batch.  A step in which every request decodes one token and
+        wants its logits is launch-bound, so such steps are captured per batch size into a
+        HIP graph and replayed: the batch arrays live at fixed device addresses (the
+        builder's buffer), so a replay reads the new step's tokens, positions and block
+        tables.  (The reference captures everything between two attentions per token-count
+        bucket, llama.cu/src/exec/step.rs:82-96; here the whole step is one graph.)"""
+        b = step.n_req
+        if not (self.use_graphs and step.decode_only and step.n_logits == b and b <= self.GRAPH_MAX_BATCH):
+            return self.model.forward(step, self.caches)
+        # the number of key parts of the decode attention must not change between replays
+        step.attn_splits = self._decode_splits(b)
+        entry = self._graphs.get(b)
+        if entry is None:
+            self._seen[b] = self._seen.get(b, 0) + 1
+            if self._seen[b] <= self.GRAPH_AFTER:
+                return self.model.forward(step, self.caches)
+            torch.cuda.synchronize(self.device)
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                logits = self.model.forward(step, self.caches)
+            entry = self._graphs[b] = (graph, logits)
+        graph, logits = entry
+        graph.replay()
+        return logits
+
+    def _decode_splits(self, batch: int) -> int:
+        from ..kernels.ops import decode_splits
+        best = 1
+        for need in self.model.cache_needs():
+            if isinstance(need, PagedKV):
+                heads = getattr(self.model.layers[0].mixer, "heads", need.kv_heads)
+                best = max(best, decode_splits(batch, heads, need.kv_heads, self.max_model_len))
+        return best
 
     def step(self, req_ids: Sequence[int], tokens: Sequence[Sequence[int]],
              want: Optional[Sequence[Sequence[int]]] = None) -> torch.Tensor:

@@ -29,6 +29,8 @@ HIP_FLAGS = ["-O3", "--offload-arch=gfx950", "-std=c++17", "-shared", "-fPIC",
              "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
              "-Wno-unused-command-line-argument"]
 HOST_FLAGS = ["-O2", "-std=c++17", "-shared", "-fPIC", "-Wall"]
+# extra flags for experiments (they enter the hash in the libraries' names)
+HIP_FLAGS += os.environ.get("LCU_HIP_FLAGS", "").split()
 
 KERNEL_LIBRARIES = ["elementwise", "rope_kv", "attention_generic", "attention_mfma", "gemm_generic", "gemm_skinny",
                     "sampling"]

@@ -319,10 +319,11 @@ def attention_prefill(q, out, cache, block_table, q_start, ctx_len, task_req, ta
 
 
 def decode_splits(n_req: int, n_heads: int, n_kv_heads: int, max_ctx_len: int) -> int:
-    """Into how many parts the decode kernel cuts each request's keys: enough workgroups
-    to fill 256 compute units, no part shorter than 128 keys."""
+    """Into how many parts the decode kernel cuts each request's keys: about one workgroup
+    for each of the 256 compute units, no part shorter than 256 keys (measured: more parts
+    cost more in the merge than they gain)."""
     base = n_req * n_kv_heads * ((n_heads // n_kv_heads + 15) // 16)
-    return max(1, min(16, 1024 // max(base, 1), (max_ctx_len + 127) // 128))
+    return max(1, min(8, 256 // max(base, 1), (max_ctx_len + 255) // 256))
 
 
 def paged_attention(q: torch.Tensor, out: torch.Tensor, cache: torch.Tensor, step, group: int, n_heads: int,
@@ -350,7 +351,8 @@ def paged_attention(q: torch.Tensor, out: torch.Tensor, cache: torch.Tensor, ste
                              n_kv_heads, head_dim, page_size, scale, window)
 
 
-SKINNY_MAX_ROWS = 64
+SKINNY_MAX_ROWS = 64      # what the kernel takes
+SKINNY_ROWS = 16          # up to here it beats the library's product (measured on the Llama-3-8B shapes)
 _EPILOGUES = {"bf16": 0, "f32": 1, "add_f32": 2, "swiglu": 3}
 
 
@@ -374,7 +376,7 @@ def _skinny_tiles(n_features: int, m: int) -> int:
 
 def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = None,
                 out_dtype: Optional[torch.dtype] = None, accumulate: bool = False, swiglu: bool = False,
-                tiles: Optional[int] = None) -> torch.Tensor:
+                tiles: Optional[int] = None, waves: Optional[int] = None) -> torch.Tensor:
     """``out (+)= x @ w.T`` for at most 64 rows of bfloat16 ``x`` by streaming ``w`` once.
     ``swiglu``: ``w`` holds gate rows, then up rows; ``out = silu(x @ gate.T) * (x @ up.T)``."""
     _gpu(x, w, out)
@@ -401,5 +403,6 @@ def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = 
         raise KernelError(f"gemm_skinny out: shape {tuple(out.shape)}, expected {(m, width)}")
     lib = build.load("gemm_skinny")
     _check(lib.lcu_gemm_skinny_bf16(_ptr(x), x.stride(0), _ptr(w), w.stride(0), _ptr(out), out.stride(0), m, n, k,
-                                    _EPILOGUES[epi], tiles or _skinny_tiles(width, m), _stream()), "gemm_skinny")
+                                    _EPILOGUES[epi], tiles or _skinny_tiles(width, m), waves or 4, _stream()),
+           "gemm_skinny")
     return out

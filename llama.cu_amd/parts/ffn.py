@@ -35,7 +35,7 @@ class SwiGLU(Part):
         self.dtype = build.dtype
 
     def forward(self, h: torch.Tensor) -> torch.Tensor:
-        if ops.skinny_supported(h, self.w_gate_up, self.dtype) and self.dtype == torch.bfloat16:
+        if self.dtype == torch.bfloat16 and h.shape[0] <= ops.SKINNY_ROWS and ops.skinny_supported(h, self.w_gate_up, self.dtype):
             # few rows: one pass over the weights, the activation in the product's epilogue
             act = ops.gemm_skinny(h, self.w_gate_up, swiglu=True)
         else:

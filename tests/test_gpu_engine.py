@@ -130,3 +130,32 @@ def test_smoke_entry():
     sys.path.insert(0, common.ROOT)
     import __graft_entry__
     __graft_entry__.smoke()
+
+
+def test_captured_decode_steps_equal_eager_ones():
+    """Decode steps replayed from a captured graph give the logits of eager steps, on
+    every replay, with eager work and synchronisations between the replays, and when the
+    batch's requests change places and lengths."""
+    from llama_cu_amd.engine.runner import ModelRunner
+    folder = common.make_folder(common.TINY_B, seed=31, dtype=torch.bfloat16, std=common.BF16_STD)
+    reqs = list(common.random_requests(384, [9, 40, 33], seed=8).values())
+
+    def decode(use_graphs):
+        runner = ModelRunner.from_folder(folder, dtype="bfloat16", max_tokens=1024, max_seqs=4, use_graphs=use_graphs)
+        runner.step([0, 1, 2], reqs)
+        outs = []
+        rng = np.random.default_rng(0)
+        for i in range(12):
+            toks = [[int(rng.integers(384))] for _ in range(3)]
+            outs.append(runner.step([0, 1, 2], toks).float().cpu())
+            if i == 6:                                    # eager work between replays: a prompt portion of another request
+                runner.step([3], [[1, 2, 3, 4, 5]])
+                runner.end(3)
+            torch.cuda.synchronize()
+        return outs, runner
+
+    eager, _ = decode(False)
+    graphed, runner = decode(True)
+    assert 3 in runner._graphs                              # the batch size was captured and replayed
+    for i, (a, b) in enumerate(zip(eager, graphed)):
+        assert torch.equal(a, b), f"decode step {i} differs between eager and captured"
