@@ -80,6 +80,7 @@ void Scheduler::preempt_last(std::vector<PlanEntry> &plan) {
     v.computed = 0;
     v.preemptions++;
     preemptions_++;
+    preempted_now_ = true;
     waiting_.push_front(victim);
 }
 
@@ -106,6 +107,7 @@ bool Scheduler::reserve_or_preempt(SchedRequest &r, int new_len, bool may_preemp
 
 std::vector<PlanEntry> Scheduler::plan() {
     std::vector<PlanEntry> plan;
+    preempted_now_ = false;
     for (;;) {
         plan.clear();
         int budget = cfg_.max_batch_tokens;
@@ -136,8 +138,9 @@ std::vector<PlanEntry> Scheduler::plan() {
             plan.push_back({r.id, r.computed, n, r.computed + n == (int)r.tokens.size()});
             budget -= n;
         }
-        // 3. admission, first come first served
-        while (!waiting_.empty() && budget > 0 && (int)running_.size() < cfg_.max_num_seqs) {
+        // 3. admission, first come first served; not in a round that had to preempt (the pages
+        //    that the victim gave back would go straight to it again)
+        while (!preempted_now_ && !waiting_.empty() && budget > 0 && (int)running_.size() < cfg_.max_num_seqs) {
             SchedRequest &r = reqs_.at(waiting_.front());
             if ((int)r.tokens.size() > cfg_.max_model_len) {
                 finish(r, FINISH_LENGTH);

@@ -91,6 +91,7 @@ class Scheduler {
     std::vector<int64_t> running_;     // in admission order
     std::vector<int64_t> finished_;
     int64_t preemptions_ = 0;
+    bool preempted_now_ = false;       // the plan being made has preempted a request
 };
 
 }  // namespace lcu

@@ -43,6 +43,7 @@ class StepContext:
     q_lens: List[int] = field(default_factory=list)
     ctx_lens: List[int] = field(default_factory=list)
     req_ids: List[int] = field(default_factory=list)
+    state_slots: List[int] = field(default_factory=list)    # ``state_slot`` on the host
     attn_splits: Optional[int] = None           # fixed number of key parts for the decode kernel (captured graphs)
     scratch: dict = field(default_factory=dict)  # what kernels' wrappers derive from the batch once per step
 
@@ -144,4 +145,5 @@ class BatchBuilder:
             logit_rows=self._d("logit_rows", len(rows)), n_logits=len(rows),
             block_tables=[self._d(f"block_table{g}", n_req * mp).view(n_req, mp) for g, mp in enumerate(self.max_pages)],
             slot_maps=[self._d(f"slots{g}", n) for g in range(len(self.max_pages))],
-            q_lens=n_new, ctx_lens=ctx_lens, req_ids=list(req_ids))
+            q_lens=n_new, ctx_lens=ctx_lens, req_ids=list(req_ids),
+            state_slots=self._h("state_slot")[:n_req].tolist())

@@ -98,7 +98,7 @@ class ModelRunner:
         max_pages = [(self.max_model_len + self.page_size - 1) // self.page_size for _ in self.groups]
         self.builder = BatchBuilder(self.cache, self.max_batch_tokens, self.max_seqs, max_pages, self.device)
         # captured decode steps, by batch size: (graph, its logits tensor)
-        self.use_graphs = bool(use_graphs)
+        self.use_graphs = bool(use_graphs) and self.model.graph_safe
         self._graphs: Dict[int, Any] = {}
         self._seen: Dict[int, int] = {}
 

@@ -19,6 +19,7 @@ from .linear import linear
 
 
 class Attention(Part):
+
     def __init__(self, hidden_size: int, heads: int, kv_heads: int, head_dim: int, scale: Optional[float] = None,
                  window: int = 0, position: Optional[PartSpec] = None, shares_kv: bool = False):
         if heads % kv_heads:
@@ -31,6 +32,7 @@ class Attention(Part):
         self.window = int(window or 0)
         self.shares_kv = bool(shares_kv)          # reads another layer's keys and values: has q and o only
         self.position = make_part("position", position or PartSpec("none"))
+        self.graph_safe = self.position.graph_safe
         self.w_qkv = self.w_o = None
         self.page_size = 0
 

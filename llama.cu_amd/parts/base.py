@@ -15,8 +15,8 @@ the registry of its category:
   ``position``  ``tables(...)``/``apply(...)``         see parts.position
   ``block``     ``forward(x, pending, step, cache) -> pending``   the arrangement of the four above
 
-Every part also has ``tensors() -> {relative name: TensorSpec}`` and
-``load(tensors, build)``.  No part knows which model it is in: sizes and constants
+Every part also has ``tensors() -> {relative name: TensorSpec}``,
+``load(tensors, build)`` and the flag ``graph_safe`` (see Part).  No part knows which model it is in: sizes and constants
 arrive as parameters.
 """
 from __future__ import annotations
@@ -35,7 +35,8 @@ class TensorSpec:
     shape: Tuple[int, ...]
     init: str = "normal"
     integer: bool = False
-    optional: bool = False
+    optional: bool = False        # a file may lack it
+    random: bool = True           # the random-weights mode makes it
 
 
 @dataclass
@@ -99,6 +100,11 @@ class BuildContext:
 
 
 class Part:
+    # Whether a step through this part may be captured into a graph and replayed: true only
+    # if all it does is launch work on the current stream whose shape depends on the batch's
+    # sizes alone, never on values it reads on the host (lengths, positions, slots).
+    graph_safe = False
+
     def tensors(self) -> Dict[str, TensorSpec]:
         return {}
 

@@ -23,6 +23,7 @@ class PreNormBlock(Part):
         self.mixer = make_part("mixer", mixer)
         self.norm2 = make_part("norm", norm2)
         self.ffn = make_part("ffn", ffn)
+        self.graph_safe = all(p.graph_safe for p in (self.norm1, self.mixer, self.norm2, self.ffn))
 
     def _children(self):
         return [(self.specs[k].name, getattr(self, k)) for k in ("norm1", "mixer", "norm2", "ffn")]

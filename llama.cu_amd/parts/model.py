@@ -20,6 +20,8 @@ from .linear import linear
 
 
 class TokenEmbedding(Part):
+    graph_safe = True
+
     def __init__(self, vocab_size: int, hidden_size: int):
         self.vocab_size, self.hidden_size = int(vocab_size), int(hidden_size)
         self.weight = None
@@ -37,6 +39,8 @@ class TokenEmbedding(Part):
 
 
 class OutputHead(Part):
+    graph_safe = True
+
     """``logits = y @ W.T``; ``tied``: W is the embedding table."""
 
     def __init__(self, vocab_size: int, hidden_size: int, tied: bool = False):
@@ -46,7 +50,7 @@ class OutputHead(Part):
     def tensors(self):
         # a file may hold the matrix although the model ties it (then it is not used), or
         # hold none although it does not (then the table is used: the reference's rule)
-        return {"weight": TensorSpec((self.vocab_size, self.hidden_size), optional=True)}
+        return {"weight": TensorSpec((self.vocab_size, self.hidden_size), optional=True, random=not self.tied)}
 
     def load(self, tensors, build: BuildContext, table: Optional[torch.Tensor] = None) -> None:
         own = tensors.get("weight")
@@ -67,6 +71,7 @@ class DecoderModel:
         self.layers: List[Part] = [make_part("block", s) for s in spec.layers]
         self.final_norm = make_part("norm", spec.final_norm)
         self.head = make_part("head", spec.head)
+        self.graph_safe = all(p.graph_safe for p in [self.embedding, self.final_norm, self.head] + self.layers)
         n = len(self.layers)
         for i, e in enumerate(spec.run_order):
             if not 0 <= e.layer < n:

@@ -15,6 +15,8 @@ from .base import BuildContext, Part, TensorSpec, register_part
 
 
 class RMSNorm(Part):
+    graph_safe = True
+
     def __init__(self, size: int, eps: float):
         self.size = int(size)
         self.eps = float(eps)

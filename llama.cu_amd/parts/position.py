@@ -20,6 +20,8 @@ from .base import BuildContext, Part, register_part
 
 
 class NoPosition(Part):
+    graph_safe = True
+
     """Queries and keys are used as they are."""
 
     def load(self, tensors, build: BuildContext) -> None:

@@ -22,12 +22,13 @@ def _stream_seed(seed: int, name: str) -> int:
 
 def random_tensors(expected: Dict[str, TensorSpec], seed: int, dtype: torch.dtype = torch.bfloat16,
                    std: float = 0.02, device="cpu", vector_dtype=None) -> Dict[str, torch.Tensor]:
-    """A tensor for every non-optional expected name.  ``vector_dtype`` (default: ``dtype``)
+    """A tensor for every expected name that the random mode makes (a tied model gets no
+    output matrix).  ``vector_dtype`` (default: ``dtype``)
     is the type of 1-d tensors (norm weights)."""
     out = {}
     dev = torch.device(device)
     for name, spec in expected.items():
-        if spec.optional:
+        if not spec.random:
             continue
         g = torch.Generator(device=dev).manual_seed(_stream_seed(seed, name))
         if spec.integer:

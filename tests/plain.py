@@ -178,7 +178,7 @@ class PlainConfig:
 
 
 def attention_block(cfg: PlainConfig, w: Dict[str, torch.Tensor], prefix: str, x1: torch.Tensor,
-                    pos: Sequence[int], sin, cos) -> torch.Tensor:
+                    pos: Sequence[int], sin, cos, shared_kv=None, keep_kv: Optional[list] = None) -> torch.Tensor:
     """q, k, v projections, rotation of q and k, causal attention, output projection,
 for one whole sequence: ``pos`` (the positions the rotation uses) may start anywhere,
 the mask only counts places in the sequence.
@@ -190,10 +190,15 @@ the mask only counts places in the sequence.
     n = x1.shape[0]
     nh, nkvh, dh = cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim
     q = linear(x1, w[prefix + "self_attn.q_proj.weight"]).view(n, nh, dh)
-    k = linear(x1, w[prefix + "self_attn.k_proj.weight"]).view(n, nkvh, dh)
-    v = linear(x1, w[prefix + "self_attn.v_proj.weight"]).view(n, nkvh, dh)
     q = rope(q, pos, sin, cos, cfg.rope_pairing)
-    k = rope(k, pos, sin, cos, cfg.rope_pairing)
+    if shared_kv is not None:          # not Llama's: a layer that reads the keys and values another one made
+        k, v = shared_kv
+    else:
+        k = linear(x1, w[prefix + "self_attn.k_proj.weight"]).view(n, nkvh, dh)
+        v = linear(x1, w[prefix + "self_attn.v_proj.weight"]).view(n, nkvh, dh)
+        k = rope(k, pos, sin, cos, cfg.rope_pairing)
+    if keep_kv is not None:
+        keep_kv.append((k, v))
     o = attention(q, k, v, dh ** -0.5, first_pos=0, window=cfg.window)
     return linear(o.reshape(n, nh * dh), w[prefix + "self_attn.o_proj.weight"])
 
@@ -219,11 +224,18 @@ def forward(cfg: PlainConfig, w: Dict[str, torch.Tensor], tokens: Sequence[int])
     pos = list(range(n))
     sin, cos = rope_tables(max(n, 1), cfg.head_dim, cfg.rope_theta)
     x = embedding(w["model.embed_tokens.weight"], tokens)
+    # Llama runs its layers once each, in order; tests of the parts' generality may name a
+    # layer twice, or as (layer, j) let it read the keys and values that entry j made
     order = cfg.run_order if cfg.run_order is not None else list(range(cfg.num_hidden_layers))
-    for layer in order:
+    kept = []
+    for entry in order:
+        layer, cache_of = entry if isinstance(entry, tuple) else (entry, None)
         p = f"model.layers.{layer}."
         x1 = rms_norm(x, w[p + "input_layernorm.weight"], cfg.rms_norm_eps)
-        x = x + attention_block(cfg, w, p, x1, pos, sin, cos)
+        made = []
+        x = x + attention_block(cfg, w, p, x1, pos, sin, cos,
+                                shared_kv=kept[cache_of] if cache_of is not None else None, keep_kv=made)
+        kept.append(made[0] if cache_of is None else None)
         x2 = rms_norm(x, w[p + "post_attention_layernorm.weight"], cfg.rms_norm_eps)
         x = x + feed_forward(w, p, x2)
     y = rms_norm(x, w["model.norm.weight"], cfg.rms_norm_eps)

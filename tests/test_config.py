@@ -1,0 +1,130 @@
+"""Configuration and registry: every size and constant comes from config.json's keys,
+errors name the key, and the architecture's name picks the model."""
+import json
+import os
+
+import pytest
+
+import common
+import llama_cu_amd
+from llama_cu_amd.config import (ConfigError, LlamaConfig, architecture_of, load_config, register_architecture,
+                                 registered_architectures)
+from llama_cu_amd.models.llama import llama_spec
+
+
+def test_all_keys_are_read():
+    cfg = LlamaConfig.from_dict(common.TINY_C)
+    assert (cfg.num_hidden_layers, cfg.hidden_size, cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim,
+            cfg.intermediate_size, cfg.vocab_size, cfg.max_position_embeddings) == (1, 80, 6, 2, 48, 100, 301, 200)
+    assert (cfg.rope_theta, cfg.rms_norm_eps, cfg.tie_word_embeddings, cfg.rope_interleaved) == (777.0, 1e-3, False, True)
+
+
+def test_defaults_are_the_reference_s():
+    """llama.cu/src/model/mod.rs:73-77: kv heads = heads, head size = width / heads,
+    epsilon 1e-5, rotation base 1e4."""
+    d = dict(architectures=["LlamaForCausalLM"], num_hidden_layers=1, hidden_size=96, num_attention_heads=6,
+             intermediate_size=10, vocab_size=11, max_position_embeddings=12)
+    cfg = LlamaConfig.from_dict(d)
+    assert cfg.num_key_value_heads == 6 and cfg.head_dim == 16
+    assert cfg.rope_theta == 1e4 and cfg.rms_norm_eps == 1e-5 and cfg.tie_word_embeddings is False
+
+
+@pytest.mark.parametrize("key", ["num_hidden_layers", "hidden_size", "num_attention_heads", "intermediate_size",
+                                 "vocab_size", "max_position_embeddings"])
+def test_missing_required_key_is_named(key):
+    d = dict(common.TINY_A)
+    del d[key]
+    with pytest.raises(ConfigError, match=key):
+        LlamaConfig.from_dict(d)
+
+
+@pytest.mark.parametrize("key,value", [("hidden_size", 0), ("num_hidden_layers", -1), ("vocab_size", 3.5),
+                                       ("rms_norm_eps", 0), ("rope_theta", -2.0), ("tie_word_embeddings", "yes"),
+                                       ("num_attention_heads", True)])
+def test_bad_value_is_named(key, value):
+    d = dict(common.TINY_A)
+    d[key] = value
+    with pytest.raises(ConfigError, match=key):
+        LlamaConfig.from_dict(d)
+
+
+def test_inconsistent_sizes():
+    with pytest.raises(ConfigError, match="num_key_value_heads"):
+        LlamaConfig.from_dict(dict(common.TINY_A, num_key_value_heads=3))
+    with pytest.raises(ConfigError, match="head_dim"):
+        LlamaConfig.from_dict(dict(common.TINY_A, head_dim=15))
+    d = dict(common.TINY_A, hidden_size=66)
+    del d["head_dim"]
+    with pytest.raises(ConfigError, match="head_dim"):
+        LlamaConfig.from_dict(d)
+
+
+@pytest.mark.parametrize("key,value", [("rope_scaling", {"rope_type": "llama3", "factor": 8.0}), ("hidden_act", "gelu"),
+                                       ("attention_bias", True), ("mlp_bias", True), ("sliding_window", 4096)])
+def test_keys_that_would_change_the_computation_are_refused(key, value):
+    with pytest.raises(ConfigError, match=key):
+        LlamaConfig.from_dict(dict(common.TINY_A, **{key: value}))
+    # the harmless spellings are accepted
+    LlamaConfig.from_dict(dict(common.TINY_A, rope_scaling=None, hidden_act="silu", attention_bias=False,
+                               sliding_window=None, model_type="llama", torch_dtype="bfloat16", use_cache=True))
+
+
+def test_eos_ids():
+    assert LlamaConfig.from_dict(dict(common.TINY_A, eos_token_id=7)).eos_token_ids == (7,)
+    assert LlamaConfig.from_dict(dict(common.TINY_A, eos_token_id=[7, 9])).eos_token_ids == (7, 9)
+    assert LlamaConfig.from_dict(common.TINY_A).eos_token_ids == ()
+
+
+def test_round_trip_through_config_json(tmp_path):
+    cfg = LlamaConfig.from_dict(dict(common.TINY_B, eos_token_id=[3, 4], bos_token_id=1))
+    (tmp_path / "config.json").write_text(json.dumps(cfg.to_dict()))
+    arch, back = load_config(str(tmp_path))
+    assert arch.name == "LlamaForCausalLM" and back == cfg
+
+
+def test_registry_picks_by_name_and_lists_what_it_knows(tmp_path):
+    assert "LlamaForCausalLM" in registered_architectures()
+    with pytest.raises(ConfigError, match="NoSuchModel.*LlamaForCausalLM"):
+        architecture_of({"architectures": ["NoSuchModel"]})
+    with pytest.raises(ConfigError, match="architectures"):
+        architecture_of({"hidden_size": 3})
+    with pytest.raises(ConfigError, match="config.json"):
+        load_config(str(tmp_path))
+    (tmp_path / "config.json").write_text("{ not json")
+    with pytest.raises(ConfigError, match="JSON"):
+        load_config(str(tmp_path))
+
+
+def test_another_architecture_can_be_registered():
+    seen = {}
+
+    def from_dict(d):
+        seen["dict"] = d
+        return LlamaConfig.from_dict(dict(d, architectures=["LlamaForCausalLM"]))
+
+    register_architecture("ToyForTesting", from_dict, llama_spec, replace=True)
+    arch = architecture_of({"architectures": ["ToyForTesting"]})
+    cfg = arch.config_from_dict(dict(common.TINY_A, architectures=["ToyForTesting"]))
+    assert arch.build_spec(cfg).hidden_size == 64
+    with pytest.raises(ValueError):
+        register_architecture("ToyForTesting", from_dict, llama_spec)
+
+
+def test_the_model_s_layout_holds_the_configuration_s_values_and_nothing_else():
+    """Every size and constant of the parts comes from the configuration: two
+    configurations that differ everywhere give layouts that differ everywhere."""
+    for d in (common.TINY_A, common.TINY_B, common.TINY_C):
+        cfg = LlamaConfig.from_dict(d)
+        spec = llama_spec(cfg)
+        assert (spec.hidden_size, spec.vocab_size, spec.max_positions) == (cfg.hidden_size, cfg.vocab_size, cfg.max_position_embeddings)
+        assert len(spec.layers) == cfg.num_hidden_layers == len(spec.run_order)
+        blk = spec.layers[-1].params
+        assert blk["norm1"].params == {"size": cfg.hidden_size, "eps": cfg.rms_norm_eps} == blk["norm2"].params
+        m = blk["mixer"].params
+        assert (m["heads"], m["kv_heads"], m["head_dim"], m["hidden_size"]) == (cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim, cfg.hidden_size)
+        assert m["scale"] == cfg.head_dim ** -0.5 and m["window"] == 0
+        assert m["position"].params == {"head_dim": cfg.head_dim, "theta": cfg.rope_theta,
+                                        "max_positions": cfg.max_position_embeddings, "interleaved": cfg.rope_interleaved}
+        assert blk["ffn"].params == {"hidden_size": cfg.hidden_size, "intermediate_size": cfg.intermediate_size}
+        assert spec.head.params["tied"] == cfg.tie_word_embeddings
+        assert spec.final_norm.params["eps"] == cfg.rms_norm_eps

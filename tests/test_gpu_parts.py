@@ -1,0 +1,287 @@
+"""Each part of a layer alone against its plain formula, and the generality of the
+composition: a run order that names a layer twice and lets a layer read another's cache,
+a window with pages of its own, and a toy mixer with per-request state that is defined
+here, registered, built and stepped without a change to the framework."""
+import copy
+
+import numpy as np
+import pytest
+import torch
+
+import common
+import plain
+from test_gpu_kernels import Batch, close, rnd
+
+pytestmark = pytest.mark.gpu
+
+DT = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+
+
+def build_ctx(dtype, page=16, max_pos=512):
+    from llama_cu_amd.parts import BuildContext
+    return BuildContext(DT[dtype], torch.device("cuda:0"), max_pos, page)
+
+
+def random_part_tensors(part, seed, dtype, std=0.2):
+    from llama_cu_amd.weights import random_tensors
+    return random_tensors(part.tensors(), seed, dtype=DT[dtype], std=std, device="cuda")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_norm_part(dtype):
+    from llama_cu_amd.parts import PartSpec, make_part
+    part = make_part("norm", PartSpec("rmsnorm", {"size": 100, "eps": 1e-3}))
+    t = random_part_tensors(part, 1, dtype)
+    part.load(t, build_ctx(dtype))
+    x = rnd(7, 100, seed=1, scale=0.02)
+    delta = rnd(7, 100, seed=2, scale=0.02).to(DT[dtype])
+    xg = x.cuda()
+    y = part.forward(xg, delta.cuda())
+    want_x = x.double() + delta.double()
+    close(xg, want_x, "float32")
+    close(y, plain.rms_norm(want_x, t["weight"].cpu(), 1e-3), dtype)
+    assert y.dtype == DT[dtype]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_feed_forward_part(dtype):
+    from llama_cu_amd.parts import PartSpec, make_part
+    for n in (3, 70):                                   # few rows (the fused kernel) and many
+        part = make_part("ffn", PartSpec("swiglu", {"hidden_size": 48, "intermediate_size": 100}))
+        t = random_part_tensors(part, 2, dtype)
+        part.load(dict(t), build_ctx(dtype))
+        h = rnd(n, 48, seed=3).to(DT[dtype])
+        w = {"L.mlp." + k: v.cpu() for k, v in t.items()}
+        close(part.forward(h.cuda()), plain.feed_forward(w, "L.", h), dtype)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("interleaved", [False, True])
+def test_attention_mixer_part_whole_prompt_then_decode(dtype, interleaved):
+    """The mixer alone: a whole prompt, then two single tokens from its cache, against the
+    plain attention block on the whole sequence."""
+    from llama_cu_amd.engine.runner import LayerCache
+    from llama_cu_amd.parts import PartSpec, make_part
+    d, nh, nkv, dh, page = 80, 6, 2, 32, 16
+    pos_spec = PartSpec("rotary", {"head_dim": dh, "theta": 777.0, "max_positions": 64, "interleaved": interleaved})
+    part = make_part("mixer", PartSpec("attention", {"hidden_size": d, "heads": nh, "kv_heads": nkv, "head_dim": dh,
+                                                     "position": pos_spec}))
+    t = random_part_tensors(part, 3, dtype)
+    part.load(dict(t), build_ctx(dtype, page, 64))
+    cfg = plain.PlainConfig(1, d, nh, nkv, dh, 1, 1, 64, rope_theta=777.0, rope_pairing="adjacent" if interleaved else "half")
+    w = {"L.self_attn." + k: v.cpu() for k, v in t.items()}
+    n = 21
+    h = rnd(n, d, seed=4).to(DT[dtype])
+    sin, cos = plain.rope_tables(64, dh, 777.0)
+    want = plain.attention_block(cfg, w, "L.", h, list(range(n)), sin, cos)
+    cache = LayerCache(group=0, pages=torch.zeros(4, 2, nkv * dh * page, dtype=DT[dtype], device="cuda"))
+    table = [2, 0, 3]
+
+    def step(q_len, ctx_len):
+        s = Batch([q_len], [ctx_len], [table], 4).step
+        first = ctx_len - q_len
+        s.positions = torch.arange(first, ctx_len, dtype=torch.int32).cuda()
+        s.slot_maps = [torch.tensor([table[p // page] * page + p % page for p in range(first, ctx_len)], dtype=torch.int32).cuda()]
+        return s
+
+    got = [part.forward(h[:n - 2].cuda(), step(n - 2, n - 2), cache)]
+    got.append(part.forward(h[n - 2:n - 1].cuda(), step(1, n - 1), cache))
+    got.append(part.forward(h[n - 1:].cuda(), step(1, n), cache))
+    close(torch.cat(got), want, dtype)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_embedding_and_output_parts(dtype):
+    from llama_cu_amd.parts import PartSpec, make_part
+    emb = make_part("embedding", PartSpec("tokens", {"vocab_size": 301, "hidden_size": 40}))
+    t = random_part_tensors(emb, 5, dtype)
+    emb.load(dict(t), build_ctx(dtype))
+    ids = torch.tensor([300, 0, 17], dtype=torch.int32)
+    x = emb.forward(ids.cuda())
+    assert x.dtype == torch.float32 and torch.equal(x.cpu(), t["weight"].cpu().float()[ids.long()])
+    for tied in (True, False):
+        head = make_part("head", PartSpec("linear", {"vocab_size": 301, "hidden_size": 40, "tied": tied}))
+        own = random_part_tensors(emb, 6, dtype)
+        head.load({} if tied else {"weight": own["weight"]}, build_ctx(dtype), table=emb.weight)
+        y = rnd(3, 40, seed=7).to(DT[dtype])
+        logits = head.forward(y.cuda())
+        assert logits.dtype == torch.float32
+        close(logits, plain.linear(y, (t if tied else own)["weight"].cpu()), dtype)
+
+
+# ----------------------------------------------------------------------------- whole models from custom layouts
+def runner_for(spec, seed, dtype, std=0.15, **kw):
+    from llama_cu_amd.engine.runner import ModelRunner
+    from llama_cu_amd.parts import DecoderModel
+    from llama_cu_amd.weights import random_tensors
+    tensors = random_tensors(DecoderModel(spec).tensors(), seed, dtype=DT[dtype], std=std, device="cuda")
+    kw.setdefault("max_tokens", 1024)
+    return ModelRunner(spec, dict(tensors), dtype, **kw), {k: v.cpu() for k, v in tensors.items()}
+
+
+def run_cut(runner, toks, sizes, rid=0):
+    """Feed ``toks`` in portions of the given sizes; logits at every position."""
+    out, fed, i = [], 0, 0
+    while fed < len(toks):
+        n = min(sizes[i % len(sizes)], len(toks) - fed)
+        i += 1
+        out.append(runner.step([rid], [toks[fed:fed + n]], [list(range(n))]).cpu())
+        fed += n
+    runner.end(rid)
+    return torch.cat(out)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_run_order_names_a_layer_twice_and_shares_a_cache(dtype):
+    """Run order: layer 0, layer 1, layer 0 again (with a cache of its own), then layer 2,
+    which has no key and value projections and reads the cache of the second entry."""
+    from llama_cu_amd.config import LlamaConfig
+    from llama_cu_amd.models.llama import llama_spec
+    from llama_cu_amd.parts import RunEntry
+    cfg_d = dict(common.TINY_A, num_hidden_layers=3)
+    spec = llama_spec(LlamaConfig.from_dict(cfg_d))
+    spec.layers[2].params["mixer"].params["shares_kv"] = True
+    spec.run_order = [RunEntry(0), RunEntry(1), RunEntry(0), RunEntry(2, cache_of=1)]
+    std = 0.15 if dtype == "float32" else common.BF16_STD
+    runner, w = runner_for(spec, 3, dtype, std=std)
+    assert "model.layers.2.self_attn.k_proj.weight" not in w
+    assert runner.caches[3].pages is runner.caches[1].pages and not runner.caches[3].writes
+    assert runner.caches[2].pages is not runner.caches[0].pages
+    toks = common.random_requests(256, [90], 4)["r0"]
+    pcfg = plain.PlainConfig.from_dict(cfg_d)
+    pcfg.run_order = [0, 1, 0, (2, 1)]
+    want = plain.forward(pcfg, w, toks)
+    for sizes in ([90], [58, 1, 1, 7, 2, 16]):
+        got = run_cut(runner, toks, sizes)
+        err = float((got.double() - want).abs().max()) / float(want.abs().max())
+        assert err <= common.REL_TOL[dtype], (sizes, err)
+    with pytest.raises(ValueError, match="before"):
+        from llama_cu_amd.parts import DecoderModel
+        bad = copy.copy(spec)
+        bad.run_order = [RunEntry(0, cache_of=1), RunEntry(1)]
+        DecoderModel(bad)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_window_with_pages_of_its_own(dtype):
+    """Layer 0 attends to all keys, layer 1 to the last 24: two groups of pages; the
+    window's group gives pages back as the window passes them, and the logits are those of
+    the plain implementation with the same window."""
+    from llama_cu_amd.config import LlamaConfig
+    from llama_cu_amd.models.llama import llama_spec
+    cfg_d = dict(common.TINY_B, num_hidden_layers=2, head_dim=64, num_attention_heads=2, num_key_value_heads=1)
+    spec = llama_spec(LlamaConfig.from_dict(cfg_d))
+    spec.layers[1].params["mixer"].params["window"] = 24
+    std = 0.15 if dtype == "float32" else common.BF16_STD
+    runner, w = runner_for(spec, 5, dtype, std=std, max_tokens=256)
+    assert [g.window for g in runner.groups] == [0, 24]
+    assert runner.caches[0].group == 0 and runner.caches[1].group == 1
+    toks = common.random_requests(384, [150], 6)["r0"]
+    # the plain model with a window in layer 1 only
+    pcfg = plain.PlainConfig.from_dict(cfg_d)
+    sin, cos = plain.rope_tables(150, pcfg.head_dim, pcfg.rope_theta)
+    x = plain.embedding(w["model.embed_tokens.weight"], toks)
+    for layer, window in ((0, None), (1, 24)):
+        p = f"model.layers.{layer}."
+        pcfg.window = window
+        x = x + plain.attention_block(pcfg, w, p, plain.rms_norm(x, w[p + "input_layernorm.weight"], pcfg.rms_norm_eps),
+                                      list(range(150)), sin, cos)
+        x = x + plain.feed_forward(w, p, plain.rms_norm(x, w[p + "post_attention_layernorm.weight"], pcfg.rms_norm_eps))
+    want = plain.linear(plain.rms_norm(x, w["model.norm.weight"], pcfg.rms_norm_eps), w["model.embed_tokens.weight"])
+    for sizes in ([150], [100, 1, 1, 1, 30, 2], [1]):
+        out, fed, i = [], 0, 0
+        while fed < len(toks):
+            n = min(sizes[i % len(sizes)], len(toks) - fed)
+            i += 1
+            out.append(runner.step([7], [toks[fed:fed + n]], [list(range(n))]).cpu())
+            fed += n
+            held = [p for p in runner.cache.table(7, 1) if p >= 0]
+            assert len(held) <= (24 + 15) // 16 + 1             # the window's group holds a window's worth of pages
+            assert all(p >= 0 for p in runner.cache.table(7, 0))
+        runner.end(7)
+        got = torch.cat(out)
+        err = float((got.double() - want).abs().max()) / float(want.abs().max())
+        assert err <= common.REL_TOL[dtype], (sizes, err)
+    runner.cache.check()
+
+
+# ----------------------------------------------------------------------------- a toy mixer with state of its own
+def test_a_toy_mixer_with_state_is_registered_built_and_stepped():
+    """The mixer ``running_mean`` is defined here: its output at a token is a matrix times
+    the mean of its inputs up to that token.  Its state per request (the running sum, of
+    fixed size) lives in the engine's state slots.  It is registered, laid into a model
+    beside an attention layer, and stepped whole, in portions, token by token and mixed
+    with other requests whose slots are used again; all agree with a direct computation."""
+    import llama_cu_amd
+    from llama_cu_amd.config import LlamaConfig
+    from llama_cu_amd.models.llama import llama_spec
+    from llama_cu_amd.parts import Part, PartSpec, SlotState, TensorSpec, register_part
+
+    class RunningMean(Part):
+        def __init__(self, hidden_size):
+            self.d = hidden_size
+
+        def tensors(self):
+            return {"mix.weight": TensorSpec((self.d, self.d))}
+
+        def cache_need(self):
+            return SlotState((self.d,), torch.float32)
+
+        def load(self, tensors, build):
+            self.w = tensors["mix.weight"].float()
+            self.dtype = build.dtype
+
+        def forward(self, h, step, cache):
+            out = torch.empty_like(h)
+            start = 0
+            for r, n in enumerate(step.q_lens):
+                slot = step.state_slots[r]
+                first = step.ctx_lens[r] - n
+                if first == 0:
+                    cache.state[slot].zero_()                     # a new request in this slot
+                sums = cache.state[slot] + torch.cumsum(h[start:start + n].float(), 0)
+                counts = torch.arange(first + 1, first + n + 1, device=h.device, dtype=torch.float32)[:, None]
+                out[start:start + n] = ((sums / counts) @ self.w.T).to(h.dtype)
+                cache.state[slot] = sums[-1]
+                start += n
+            return out
+
+    register_part("mixer", "running_mean", RunningMean, replace=True)
+    cfg_d = dict(common.TINY_A)
+    cfg = LlamaConfig.from_dict(cfg_d)
+    spec = llama_spec(cfg)
+    spec.layers[1].params["mixer"] = PartSpec("running_mean", {"hidden_size": 64}, "toy")
+    runner, w = runner_for(spec, 9, "float32", max_tokens=512, max_seqs=3)
+    assert "model.layers.1.toy.mix.weight" in w and "model.layers.1.self_attn.q_proj.weight" not in w
+    assert runner.caches[1].state.shape == (3, 64) and runner.caches[1].pages is None
+    assert not runner.use_graphs                # the toy reads lengths on the host: its steps are not captured
+
+    def direct(toks):
+        pcfg = plain.PlainConfig.from_dict(cfg_d)
+        sin, cos = plain.rope_tables(len(toks), 16, pcfg.rope_theta)
+        x = plain.embedding(w["model.embed_tokens.weight"], toks)
+        p = "model.layers.0."
+        x = x + plain.attention_block(pcfg, w, p, plain.rms_norm(x, w[p + "input_layernorm.weight"], 1e-5), list(range(len(toks))), sin, cos)
+        x = x + plain.feed_forward(w, p, plain.rms_norm(x, w[p + "post_attention_layernorm.weight"], 1e-5))
+        p = "model.layers.1."
+        h = plain.rms_norm(x, w[p + "input_layernorm.weight"], 1e-5)
+        mean = torch.cumsum(h, 0) / torch.arange(1, len(toks) + 1, dtype=torch.float64)[:, None]
+        x = x + mean @ w[p + "toy.mix.weight"].double().T
+        x = x + plain.feed_forward(w, p, plain.rms_norm(x, w[p + "post_attention_layernorm.weight"], 1e-5))
+        return plain.linear(plain.rms_norm(x, w["model.norm.weight"], 1e-5), w["lm_head.weight"])
+
+    reqs = common.random_requests(256, [40, 9, 77, 30, 5], 12)
+    want = {k: direct(v) for k, v in reqs.items()}
+    for mode in (common.trace_whole, common.trace_portions, common.trace_tail_decode, lambda r: common.trace_mixed(r, max_live=3)):
+        steps, _ = mode(reqs)
+        ids, outputs = {}, {}
+        for st in steps:
+            es = st["entries"]
+            logits = runner.step([ids.setdefault(e["id"], len(ids)) for e in es], [e["tokens"] for e in es], [e["want"] for e in es])
+            outputs[st["step"]] = logits.cpu().numpy()
+            for name in st["end"]:
+                runner.end(ids[name])
+        got = common.collect(steps, outputs, 256)
+        common.assert_matches_plain(got, want, "float32", "toy mixer")
+    runner.cache.check()
+    assert runner.cache.free_slots() == 3

@@ -1,0 +1,156 @@
+"""Weights: the safetensors container, the check of a folder against what the model
+expects (one error that lists everything), the type policy, and the random-weights mode."""
+import json
+import os
+import struct
+
+import pytest
+import torch
+
+import common
+import llama_cu_amd
+from llama_cu_amd.config import LlamaConfig
+from llama_cu_amd.models.llama import llama_spec
+from llama_cu_amd.parts import DecoderModel, TensorSpec
+from llama_cu_amd.weights import (SafetensorsError, WeightError, check_tensors, load_weights, open_safetensors,
+                                  random_tensors, write_random_model, write_safetensors)
+from llama_cu_amd.weights.loader import convert
+
+
+def expected(cfg_dict):
+    return DecoderModel(llama_spec(LlamaConfig.from_dict(cfg_dict))).tensors()
+
+
+def test_expected_tensor_names_and_shapes():
+    e = expected(common.TINY_B)            # 3 layers, d 128, 4 heads of 32, 1 kv head, di 352, vocab 384, tied
+    assert e["model.embed_tokens.weight"].shape == (384, 128)
+    assert e["model.layers.2.self_attn.q_proj.weight"].shape == (128, 128)
+    assert e["model.layers.0.self_attn.k_proj.weight"].shape == (32, 128)
+    assert e["model.layers.0.self_attn.v_proj.weight"].shape == (32, 128)
+    assert e["model.layers.1.self_attn.o_proj.weight"].shape == (128, 128)
+    assert e["model.layers.1.mlp.gate_proj.weight"].shape == (352, 128)
+    assert e["model.layers.1.mlp.up_proj.weight"].shape == (352, 128)
+    assert e["model.layers.1.mlp.down_proj.weight"].shape == (128, 352)
+    assert e["model.layers.1.input_layernorm.weight"].shape == (128,)
+    assert e["model.layers.1.post_attention_layernorm.weight"].shape == (128,)
+    assert e["model.norm.weight"].shape == (128,)
+    assert e["lm_head.weight"].optional
+    assert len(e) == 3 * 9 + 3
+
+
+def test_container_round_trip_and_agreement_with_the_safetensors_package(tmp_path):
+    tensors = {"a": torch.randn(3, 5), "b": torch.randn(7).to(torch.bfloat16), "c": torch.arange(6, dtype=torch.int32).view(2, 3),
+               "empty": torch.zeros(0, 4)}
+    path = str(tmp_path / "x.safetensors")
+    write_safetensors(path, tensors)
+    from llama_cu_amd.weights.safetensors_io import SafetensorsFile
+    f = SafetensorsFile(path)
+    assert sorted(f.names()) == sorted(tensors)
+    for k, v in tensors.items():
+        assert f.dtype(k) == v.dtype and f.shape(k) == tuple(v.shape) and torch.equal(f.tensor(k), v)
+    from safetensors.torch import load_file, save_file
+    theirs = load_file(path)                                   # their reader reads our file
+    assert all(torch.equal(theirs[k], v) for k, v in tensors.items())
+    path2 = str(tmp_path / "y.safetensors")
+    save_file({k: v for k, v in tensors.items() if v.numel()}, path2)
+    g = SafetensorsFile(path2)                                 # our reader reads their file
+    assert all(torch.equal(g.tensor(k), tensors[k]) for k in g.names())
+
+
+def test_broken_files_are_refused(tmp_path):
+    path = str(tmp_path / "model.safetensors")
+    write_safetensors(path, {"a": torch.randn(4, 4)})
+    raw = open(path, "rb").read()
+    open(path, "wb").write(raw[:-8])                           # truncated
+    with pytest.raises(SafetensorsError, match="outside the file"):
+        open_safetensors(str(tmp_path))
+    open(path, "wb").write(struct.pack("<Q", 10 ** 9) + b"{}")
+    with pytest.raises(SafetensorsError, match="header length"):
+        open_safetensors(str(tmp_path))
+    open(path, "wb").write(struct.pack("<Q", 5) + b"{oops")
+    with pytest.raises(SafetensorsError, match="JSON"):
+        open_safetensors(str(tmp_path))
+    os.remove(path)
+    with pytest.raises(SafetensorsError, match="no model.safetensors"):
+        open_safetensors(str(tmp_path))
+
+
+def test_one_error_lists_missing_unexpected_and_wrong_shapes(tmp_path):
+    folder = common.make_folder(common.TINY_A, seed=1, dtype=torch.float32, folder=str(tmp_path))
+    from llama_cu_amd.weights.safetensors_io import SafetensorsFile
+    w = {n: SafetensorsFile(os.path.join(folder, "model.safetensors")).tensor(n).clone()
+         for n in SafetensorsFile(os.path.join(folder, "model.safetensors")).names()}
+    del w["model.layers.1.mlp.up_proj.weight"]
+    del w["model.norm.weight"]
+    w["model.layers.0.self_attn.q_proj.weight"] = torch.zeros(64, 63)
+    w["model.layers.7.extra.weight"] = torch.zeros(2)
+    w["model.layers.0.self_attn.rotary_emb.inv_freq"] = torch.zeros(8)      # carried by some files, holds no weight
+    write_safetensors(os.path.join(folder, "model.safetensors"), w)
+    with pytest.raises(WeightError) as err:
+        load_weights(open_safetensors(folder), expected(common.TINY_A), torch.float32, torch.device("cpu"))
+    msg = str(err.value)
+    assert "missing tensors (2)" in msg and "model.layers.1.mlp.up_proj.weight" in msg and "model.norm.weight" in msg
+    assert "unexpected tensors (1)" in msg and "model.layers.7.extra.weight" in msg and "inv_freq" not in msg
+    assert "wrong shapes (1)" in msg and "found [64, 63], expected [64, 64]" in msg
+
+
+def test_tied_and_untied_output_matrix(tmp_path):
+    # tied model: no lm_head.weight needed; present but unused is fine too
+    folder = common.make_folder(common.TINY_B, seed=1, dtype=torch.float32, folder=str(tmp_path))
+    t = load_weights(open_safetensors(folder), expected(common.TINY_B), torch.float32, torch.device("cpu"))
+    assert "lm_head.weight" not in t
+    # an untied configuration whose file holds no output matrix falls back to the table
+    # (the reference's rule, llama.cu/src/model/mod.rs:83-88): no error at load
+    check_tensors(expected(dict(common.TINY_B, tie_word_embeddings=False)), {n: tuple(v.shape) for n, v in t.items()})
+
+
+def test_type_policy():
+    spec = TensorSpec((2, 2))
+    f32, bf16, f16 = torch.ones(2, 2), torch.ones(2, 2, dtype=torch.bfloat16), torch.ones(2, 2, dtype=torch.float16)
+    # bfloat16 engine: bfloat16 stays, 16-bit float becomes bfloat16, what is stored in 32-bit stays 32-bit
+    assert convert(bf16, spec, torch.bfloat16).dtype == torch.bfloat16
+    assert convert(f16, spec, torch.bfloat16).dtype == torch.bfloat16
+    assert convert(f32, spec, torch.bfloat16).dtype == torch.float32
+    # float32 engine: everything 32-bit, exactly
+    x = torch.randn(2, 2).to(torch.bfloat16)
+    assert torch.equal(convert(x, spec, torch.float32), x.float())
+    assert convert(f32, spec, torch.float32).dtype == torch.float32
+    # integer tables are int32
+    ispec = TensorSpec((2, 2), integer=True)
+    assert convert(torch.ones(2, 2, dtype=torch.int64), ispec, torch.bfloat16).dtype == torch.int32
+    with pytest.raises(WeightError):
+        convert(f32, ispec, torch.bfloat16)
+    with pytest.raises(WeightError):
+        convert(torch.ones(2, 2, dtype=torch.int32), spec, torch.bfloat16)
+
+
+def test_random_weights_mode(tmp_path):
+    cfg = LlamaConfig.from_dict(common.TINY_B)
+    a = write_random_model(str(tmp_path / "a"), cfg, seed=5, dtype=torch.bfloat16)
+    b = write_random_model(str(tmp_path / "b"), cfg, seed=5, dtype=torch.bfloat16)
+    c = write_random_model(str(tmp_path / "c"), cfg, seed=6, dtype=torch.bfloat16)
+    ra, rb, rc = (open(os.path.join(d, "model.safetensors"), "rb").read() for d in (a, b, c))
+    assert ra == rb and ra != rc                                   # the seed decides
+    assert LlamaConfig.from_dict(json.load(open(os.path.join(a, "config.json")))) == cfg
+    t = load_weights(open_safetensors(a), expected(common.TINY_B), torch.bfloat16, torch.device("cpu"))
+    assert "lm_head.weight" not in t                               # tied: none written
+    q0, q1 = t["model.layers.0.self_attn.q_proj.weight"].float(), t["model.layers.1.self_attn.q_proj.weight"].float()
+    assert not torch.equal(q0, q1)                                 # each tensor its own stream
+    assert abs(float(q0.std()) - 0.02) < 0.002 and abs(float(q0.mean())) < 0.002
+    n = t["model.norm.weight"].float()
+    assert abs(float(n.mean()) - 1.0) < 0.01 and 0.01 < float(n.std()) < 0.03
+    # a tensor's values do not depend on which other tensors the model has
+    small = random_tensors({"model.norm.weight": TensorSpec((128,), init="one_plus_normal")}, 5, dtype=torch.bfloat16)
+    assert torch.equal(small["model.norm.weight"], t["model.norm.weight"])
+    # the plain implementation reads the folder too
+    import plain
+    pcfg, pw = plain.load_folder(a)
+    assert plain.forward(pcfg, pw, [1, 2, 3]).shape == (3, 384)
+
+
+def test_random_weights_of_an_untied_model_hold_an_output_matrix(tmp_path):
+    cfg = LlamaConfig.from_dict(common.TINY_A)
+    d = write_random_model(str(tmp_path / "a"), cfg, seed=1, dtype=torch.float32)
+    t = load_weights(open_safetensors(d), expected(common.TINY_A), torch.float32, torch.device("cpu"))
+    assert t["lm_head.weight"].shape == (256, 64)
+    assert not torch.equal(t["lm_head.weight"], t["model.embed_tokens.weight"])
