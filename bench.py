@@ -108,6 +108,7 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the shape has (named in config)")
     ap.add_argument("--dtype", choices=["bfloat16", "float32"], default="bfloat16")
     ap.add_argument("--no-points", action="store_true", help="skip decoding at batch 1 and 64 and the prefill")
+    ap.add_argument("--only-prefill", action="store_true", help="time the 2048-token prefill alone (for profiles)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported (no multi-GPU path)")
@@ -128,13 +129,18 @@ def main() -> int:
     rng = random.Random(0)
     sync = torch.cuda.synchronize
     page = 16
-    biggest = max(args.batch, 1 if args.no_points else 64)
+    biggest = max(args.batch, 1 if (args.no_points or args.only_prefill) else 64)
     # a request decodes while later ones still prefill: room for that too
     per_req = PROMPT_LEN + args.steps + args.warmup + 2 * biggest + 64
     engine = Engine.from_config(cfg, seed=0, dtype=args.dtype, page_size=page,
                                 max_tokens=biggest * ((per_req + page - 1) // page * page) + PREFILL_TOKENS + page,
                                 max_seqs=biggest + 2, max_batch_tokens=max(PREFILL_TOKENS, biggest), prefill_chunk=PREFILL_TOKENS)
 
+    if args.only_prefill:
+        pt = run_prefill(engine, cfg, rng, sync, repeats=args.steps)
+        print(json.dumps({"prefill": {"value": round(PREFILL_TOKENS / pt, 1), "tokens": PREFILL_TOKENS, "ms": round(pt * 1e3, 3),
+                                      "frac": round(prefill_flops(cfg, PREFILL_TOKENS) / pt / MATRIX_PEAK[dt_name], 4)}}))
+        return 0
     seconds, produced, mean_ctx = run_decode(engine, cfg, args.batch, args.steps, args.warmup, rng, sync)
     ms_per_step = seconds / args.steps * 1e3
     value = produced / seconds

@@ -21,8 +21,9 @@
 //                   key/value head and one of `n_splits` equal parts of its keys; the
 //                   waves take 32-key steps in turn and merge through LDS; parts are
 //                   merged by a second kernel.
-//   prefill kernel  any number of tokens per request (also one).  A wave takes QB blocks
-//                   of rows of one request and walks all their keys; no LDS, no barriers.
+//   prefill kernel  any number of tokens per request (also one).  A workgroup of 4 waves
+//                   takes consecutive tokens of one request; the keys and values of a step
+//                   are copied to LDS once and shared by the waves.
 #include "common.h"
 #include "kv_layout.h"
 
@@ -180,9 +181,12 @@ __device__ __forceinline__ void load_q(const bf16_t *__restrict__ qrow, bool val
 
 // ============================================================================ decode
 constexpr int DEC_WAVES = 4;
+#ifndef LCU_DEC_MIN_WAVES
+#define LCU_DEC_MIN_WAVES 2      // two waves per SIMD: measured faster than one with more registers
+#endif
 
 template <int DH>
-__global__ void __launch_bounds__(DEC_WAVES *WAVE)
+__global__ void __launch_bounds__(DEC_WAVES *WAVE, LCU_DEC_MIN_WAVES)
 attention_decode_kernel(const bf16_t *__restrict__ q, int q_stride, bf16_t *__restrict__ out, int out_stride,
                         const bf16_t *__restrict__ cache, const int *__restrict__ block_table, int max_pages,
                         const int *__restrict__ q_start, const int *__restrict__ ctx_len, int nh, int nkvh, int page,
@@ -327,34 +331,94 @@ LCU_API int lcu_attention_decode_bf16(const void *q, int q_stride, void *out, in
 }
 
 // ============================================================================ prefill
+#ifndef LCU_PRE_QB
+#define LCU_PRE_QB 1
+#endif
+#ifndef LCU_PRE_MIN_WAVES
+#define LCU_PRE_MIN_WAVES 2
+#endif
 constexpr int PRE_WAVES = 4;
+constexpr int PRE_QB = LCU_PRE_QB;
 
-// A task is QB blocks of 16 rows of one request: `tokens_per_task` consecutive tokens
-// starting at batch index task_tok0[t], with the `hc` heads of one chunk of a group each.
+// The 32 keys of one step, copied into LDS as they lie in their pages: per tile of 16 keys
+// first the keys [dim/8][token][8], then (after both key tiles) the values [dim][token].
+// In units of 16 bytes a buffer holds 8*DH chunks: [K tile 0 | K tile 1 | V tile 0 | V tile 1],
+// 2*DH chunks each.  A thread of the workgroup copies chunks tid, tid + 256, ...
+template <int DH>
+struct StageRegs {
+    u32x4 c[DH / 32];
+};
+
+template <int DH>
+__device__ __forceinline__ void stage_load(StageRegs<DH> &r, const bf16_t *__restrict__ cache, const int *__restrict__ bt,
+                                           int max_pages, int page, size_t page_elems, int nkvh, int kvh, int k0) {
+    const size_t v_off = (size_t)nkvh * DH * page + (size_t)kvh * DH * page;
+#pragma unroll
+    for (int i = 0; i < DH / 32; ++i) {
+        const int c = threadIdx.x + 256 * i;
+        const int region = c / (2 * DH), w = c % (2 * DH), t = region & 1;
+        const int j = k0 + 16 * t;
+        int pi = j / page;
+        pi = pi < max_pages ? pi : max_pages - 1;
+        const bf16_t *pg = cache + (size_t)bt[pi] * page_elems;
+        const int tok0 = j % page;
+        const bf16_t *src = region < 2
+            ? pg + ((size_t)(kvh * (DH / 8) + w / 16) * page + tok0 + (w % 16)) * 8
+            : pg + v_off + (size_t)(w / 2) * page + tok0 + (w % 2) * 8;
+        r.c[i] = *(const u32x4 *)src;
+    }
+}
+
+template <int DH>
+__device__ __forceinline__ void stage_store(const StageRegs<DH> &r, u32x4 *__restrict__ buf) {
+#pragma unroll
+    for (int i = 0; i < DH / 32; ++i) buf[threadIdx.x + 256 * i] = r.c[i];
+}
+
+// A wave's operands of the step, read from the LDS copy.
+template <int DH>
+__device__ __forceinline__ void frag_from_lds(KVFrag<DH> &f, const u32x4 *__restrict__ buf, int l16, int grp) {
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+#pragma unroll
+        for (int kb = 0; kb < DH / 32; ++kb) f.k[t][kb] = buf[t * 2 * DH + (4 * kb + grp) * 16 + l16];
+        const u32x2 *vb = (const u32x2 *)(buf + 4 * DH + t * 2 * DH);
+#pragma unroll
+        for (int dt = 0; dt < DH / 16; ++dt) f.v[dt][t] = vb[(16 * dt + l16) * 4 + grp];
+    }
+}
+
+// A task is a block of consecutive tokens of one request: every wave of the workgroup takes
+// QB blocks of 16 rows (tokens x the heads of one chunk of a group), so a task covers
+// 4 * QB * (16 / heads per chunk) tokens, starting at batch index task_tok0[t].  The
+// workgroup walks the keys that any of its rows sees, 32 at a time; the keys and values of a
+// step are copied to LDS once (double buffered: the next step's loads are in flight while
+// one is computed) and every wave takes its operands from there.
 template <int DH, int QB>
-__global__ void __launch_bounds__(PRE_WAVES *WAVE)
+__global__ void __launch_bounds__(PRE_WAVES *WAVE, LCU_PRE_MIN_WAVES)
 attention_prefill_kernel(const bf16_t *__restrict__ q, int q_stride, bf16_t *__restrict__ out, int out_stride,
                          const bf16_t *__restrict__ cache, const int *__restrict__ block_table, int max_pages,
                          const int *__restrict__ q_start, const int *__restrict__ ctx_len,
-                         const int *__restrict__ task_req, const int *__restrict__ task_tok0, int n_tasks, int nh,
-                         int nkvh, int page, float scale_log2, int window) {
+                         const int *__restrict__ task_req, const int *__restrict__ task_tok0, int nh, int nkvh,
+                         int page, float scale_log2, int window) {
+    __shared__ u32x4 lds[2][8 * DH];
     const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
-    const int task = blockIdx.x * PRE_WAVES + wave;
-    if (task >= n_tasks) return;
+    const int task = blockIdx.x;
     const int l16 = lane & 15, grp = lane >> 4;
     const int g = nh / nkvh;
     const int chunks = (g + 15) / 16;
     const int kvh = blockIdx.y / chunks, chunk = blockIdx.y % chunks;
     const int hc = (g - 16 * chunk) < 16 ? (g - 16 * chunk) : 16;      // heads of this chunk
     const int tokens_per_block = 16 / hc;                               // tokens in 16 rows
-    const int r = task_req[task], tok0 = task_tok0[task];
+    const int tokens_per_wave = QB * tokens_per_block;
+    const int r = task_req[task], task_tok = task_tok0[task];
     const int q_end = q_start[r + 1];
     const int ctx = ctx_len[r];
     const int head0 = kvh * g + 16 * chunk;
+    const int tok0 = task_tok + wave * tokens_per_wave;                 // this wave's first token
 
     u32x4 qv[QB][DH / 32];
     int p_row[QB], lo_row[QB], tok_row[QB];
-    int p_max = -1, p_min = 0x7fffffff, lo_min = 0x7fffffff, lo_max = 0;
 #pragma unroll
     for (int b = 0; b < QB; ++b) {
         const int tok = tok0 + b * tokens_per_block + l16 / hc;
@@ -362,30 +426,43 @@ attention_prefill_kernel(const bf16_t *__restrict__ q, int q_stride, bf16_t *__r
         tok_row[b] = valid ? tok : -1;
         p_row[b] = valid ? ctx - (q_end - tok) : -1;
         lo_row[b] = valid && window > 0 && p_row[b] - window + 1 > 0 ? p_row[b] - window + 1 : 0;
-        load_q<DH>(q + (size_t)(valid ? tok : tok0) * q_stride + (size_t)(head0 + l16 % hc) * DH, valid, qv[b], grp);
+        load_q<DH>(q + (size_t)(valid ? tok : task_tok) * q_stride + (size_t)(head0 + l16 % hc) * DH, valid, qv[b], grp);
     }
-    // what the whole wave sees (the same in every lane): first and last token of the task
-    {
-        const int last_tok = (tok0 + QB * tokens_per_block < q_end ? tok0 + QB * tokens_per_block : q_end) - 1;
+    // what this wave sees (the same in all its lanes), and what the workgroup sees
+    const bool wave_has = tok0 < q_end;
+    int p_max = -1, p_min = -1, lo_min = 0, lo_max = 0;
+    if (wave_has) {
+        const int last_tok = (tok0 + tokens_per_wave < q_end ? tok0 + tokens_per_wave : q_end) - 1;
         p_max = ctx - (q_end - last_tok);
         p_min = ctx - (q_end - tok0);
         lo_min = window > 0 && p_min - window + 1 > 0 ? p_min - window + 1 : 0;
         lo_max = window > 0 && p_max - window + 1 > 0 ? p_max - window + 1 : 0;
     }
+    const int wg_last_tok = (task_tok + PRE_WAVES * tokens_per_wave < q_end ? task_tok + PRE_WAVES * tokens_per_wave : q_end) - 1;
+    const int wg_p_max = ctx - (q_end - wg_last_tok);
+    const int wg_p_min = ctx - (q_end - task_tok);
+    const int wg_lo_min = window > 0 && wg_p_min - window + 1 > 0 ? wg_p_min - window + 1 : 0;
+
     AttnState<DH, QB> st;
     attn_init(st);
     const int *bt = block_table + (size_t)r * max_pages;
     const size_t page_elems = kv_page_elems(nkvh, DH, page);
-    KVFrag<DH> fa, fb;
-    const int blk_end = p_max / 32 + 1;
-    int blk = lo_min / 32;
-    load_kv<DH>(fa, cache, bt, max_pages, page, page_elems, nkvh, kvh, blk * 32, l16, grp);
-    for (; blk < blk_end; blk += 2) {
-        if (blk + 1 < blk_end) load_kv<DH>(fb, cache, bt, max_pages, page, page_elems, nkvh, kvh, (blk + 1) * 32, l16, grp);
-        attn_block<DH, QB>(fa, blk * 32, blk * 32 + 31 > p_min || blk * 32 < lo_max, qv, st, p_row, lo_row, p_max, lo_min, scale_log2, grp);
-        if (blk + 2 < blk_end) load_kv<DH>(fa, cache, bt, max_pages, page, page_elems, nkvh, kvh, (blk + 2) * 32, l16, grp);
-        if (blk + 1 < blk_end)
-            attn_block<DH, QB>(fb, (blk + 1) * 32, (blk + 1) * 32 + 31 > p_min || (blk + 1) * 32 < lo_max, qv, st, p_row, lo_row, p_max, lo_min, scale_log2, grp);
+    const int blk0 = wg_lo_min / 32, blk_end = wg_p_max / 32 + 1;
+    StageRegs<DH> regs;
+    stage_load<DH>(regs, cache, bt, max_pages, page, page_elems, nkvh, kvh, blk0 * 32);
+    stage_store<DH>(regs, lds[0]);
+    __syncthreads();
+    for (int blk = blk0; blk < blk_end; ++blk) {
+        const int cur = (blk - blk0) & 1;
+        if (blk + 1 < blk_end) stage_load<DH>(regs, cache, bt, max_pages, page, page_elems, nkvh, kvh, (blk + 1) * 32);
+        const int k0 = blk * 32;
+        if (wave_has && k0 <= p_max && k0 + 31 >= lo_min) {
+            KVFrag<DH> f;
+            frag_from_lds<DH>(f, lds[cur], l16, grp);
+            attn_block<DH, QB>(f, k0, k0 + 31 > p_min || k0 < lo_max, qv, st, p_row, lo_row, p_max, lo_min, scale_log2, grp);
+        }
+        if (blk + 1 < blk_end) stage_store<DH>(regs, lds[cur ^ 1]);
+        __syncthreads();
     }
 #pragma unroll
     for (int b = 0; b < QB; ++b) {
@@ -411,10 +488,10 @@ static int launch_prefill(const void *q, int q_stride, void *out, int out_stride
                           const int *task_req, const int *task_tok0, int n_tasks, int nh, int nkvh, int page,
                           float scale, int window, hipStream_t stream) {
     const int g = nh / nkvh, chunks = (g + 15) / 16;
-    dim3 grid((n_tasks + PRE_WAVES - 1) / PRE_WAVES, nkvh * chunks), block(PRE_WAVES * WAVE);
+    dim3 grid(n_tasks, nkvh * chunks), block(PRE_WAVES * WAVE);
     attention_prefill_kernel<DH, QB><<<grid, block, 0, stream>>>(
         (const bf16_t *)q, q_stride, (bf16_t *)out, out_stride, (const bf16_t *)cache, block_table, max_pages, q_start,
-        ctx_len, task_req, task_tok0, n_tasks, nh, nkvh, page, scale * 1.4426950408889634f, window);
+        ctx_len, task_req, task_tok0, nh, nkvh, page, scale * 1.4426950408889634f, window);
     LCU_LAUNCH_CHECK();
     return LCU_OK;
 }
@@ -426,7 +503,7 @@ LCU_API int lcu_attention_prefill_tokens_per_task(int nh, int nkvh) {
     const int g = nh / nkvh;
     if (g > 16 && g % 16) return 0;       // chunks of a group must be equal for one task size
     const int hc = g < 16 ? g : 16;
-    return 2 * (16 / hc);
+    return PRE_WAVES * PRE_QB * (16 / hc);
 }
 
 // task_req / task_tok0: [n_tasks], tasks cut from the batch with the size above; a
@@ -440,7 +517,7 @@ LCU_API int lcu_attention_prefill_bf16(const void *q, int q_stride, void *out, i
     if (lcu_attention_prefill_tokens_per_task(nh, nkvh) == 0 || page <= 0 || page % 16 || max_pages <= 0 ||
         window < 0 || q_stride % 8 || out_stride % 4 || nkvh * ((nh / nkvh + 15) / 16) > 65535)
         return LCU_BAD_ARGUMENT;
-#define GO(D) return launch_prefill<D, 2>(q, q_stride, out, out_stride, cache, block_table, max_pages, q_start, ctx_len, task_req, task_tok0, n_tasks, nh, nkvh, page, scale, window, stream)
+#define GO(D) return launch_prefill<D, PRE_QB>(q, q_stride, out, out_stride, cache, block_table, max_pages, q_start, ctx_len, task_req, task_tok0, n_tasks, nh, nkvh, page, scale, window, stream)
     if (dh == 128) GO(128);
     if (dh == 64) GO(64);
 #undef GO

@@ -208,6 +208,26 @@ __global__ void swiglu_kernel(T *__restrict__ out, const T *__restrict__ gu, int
     out[r * di + c] = from_f32<T>(gate * sig * up);
 }
 
+// The same, eight neighbouring columns per thread (16-byte loads of bfloat16, 32-byte of
+// float32); for widths that are multiples of 8.
+template <class T> struct alignas(8 * sizeof(T)) Vec8 { T v[8]; };
+
+template <class T>
+__global__ void swiglu_vec8_kernel(T *__restrict__ out, const T *__restrict__ gu, int di) {
+    const int c = (blockIdx.x * blockDim.x + threadIdx.x) * 8;
+    if (c >= di) return;
+    const size_t r = blockIdx.y;
+    const Vec8<T> g = *(const Vec8<T> *)(gu + r * 2 * di + c);
+    const Vec8<T> u = *(const Vec8<T> *)(gu + r * 2 * di + di + c);
+    Vec8<T> o;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        const float gate = to_f32(g.v[e]);
+        o.v[e] = from_f32<T>(gate * (1.0f / (1.0f + expf(-gate))) * to_f32(u.v[e]));
+    }
+    *(Vec8<T> *)(out + r * di + c) = o;
+}
+
 LCU_API int lcu_swiglu(void *out, const void *gate_up, int type, int n, int di, hipStream_t stream) {
     if (n <= 0) return LCU_OK;
     if (di <= 0) return LCU_BAD_ARGUMENT;
@@ -216,6 +236,16 @@ LCU_API int lcu_swiglu(void *out, const void *gate_up, int type, int n, int di, 
     for (int r0 = 0; r0 < n; r0 += 65535) {
         const int rows = (n - r0) < 65535 ? (n - r0) : 65535;
         dim3 grid((di + 255) / 256, rows);
+        if (di % 8 == 0) {
+            dim3 vgrid((di / 8 + 255) / 256, rows);
+            if (type == LCU_F32)
+                swiglu_vec8_kernel<float><<<vgrid, block, 0, stream>>>((float *)out + (size_t)r0 * di, (const float *)gate_up + (size_t)r0 * 2 * di, di);
+            else if (type == LCU_BF16)
+                swiglu_vec8_kernel<bf16_t><<<vgrid, block, 0, stream>>>((bf16_t *)out + (size_t)r0 * di, (const bf16_t *)gate_up + (size_t)r0 * 2 * di, di);
+            else
+                return LCU_BAD_ARGUMENT;
+            continue;
+        }
         if (type == LCU_F32)
             swiglu_kernel<float><<<grid, block, 0, stream>>>((float *)out + (size_t)r0 * di, (const float *)gate_up + (size_t)r0 * 2 * di, di);
         else if (type == LCU_BF16)

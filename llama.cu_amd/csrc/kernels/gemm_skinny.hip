@@ -10,7 +10,7 @@
 //     its row as four 16-byte loads, one per matrix instruction (which k a slot of the
 //     instruction holds is free, as long as W and X agree), so the four waves read 1 KB
 //     of a row back to back;
-//   * the next macro-step's loads are issued before the current one is multiplied;
+//   * a wave keeps the loads of several macro-steps in flight while it multiplies one;
 //   * v_mfma_f32_16x16x32_bf16 with A = W tile, B = X^T: the 16 columns are 16 tokens,
 //     MT such tiles for up to 64 tokens.
 // The waves' partial sums are added in LDS in a fixed order.
@@ -105,16 +105,25 @@ gemm_skinny_kernel(const bf16_t *__restrict__ X, int ldx, const bf16_t *__restri
 #pragma unroll
         for (int m = 0; m < MT; ++m) acc[t][m] = f32x4{0.f, 0.f, 0.f, 0.f};
 
+    // A ring of STAGES macro-steps in flight per wave: with few workgroups per compute unit
+    // (small N) this is what keeps enough bytes on their way from HBM.
+    constexpr int STAGES = NT * MT == 1 ? 4 : (NT * MT == 2 ? 3 : 2);
     const int nsteps = (K + 127) / 128;
-    Frag<NT, MT> fa, fb;
+    Frag<NT, MT> f[STAGES];
     int s = wave;
-    if (s < nsteps) load_frag<NT, MT>(fa, wrow, xrow, xvalid, s, grp, K);
-    for (; s < nsteps; s += 2 * SK_WAVES) {
-        const bool has_b = s + SK_WAVES < nsteps;
-        if (has_b) load_frag<NT, MT>(fb, wrow, xrow, xvalid, s + SK_WAVES, grp, K);
-        mul_frag<NT, MT>(fa, acc);
-        if (s + 2 * SK_WAVES < nsteps) load_frag<NT, MT>(fa, wrow, xrow, xvalid, s + 2 * SK_WAVES, grp, K);
-        if (has_b) mul_frag<NT, MT>(fb, acc);
+#pragma unroll
+    for (int i = 0; i < STAGES; ++i)
+        if (s + i * SK_WAVES < nsteps) load_frag<NT, MT>(f[i], wrow, xrow, xvalid, s + i * SK_WAVES, grp, K);
+    for (; s < nsteps; s += STAGES * SK_WAVES) {
+#pragma unroll
+        for (int i = 0; i < STAGES; ++i) {
+            const int cur = s + i * SK_WAVES;
+            if (cur < nsteps) {
+                mul_frag<NT, MT>(f[i], acc);
+                if (cur + STAGES * SK_WAVES < nsteps)
+                    load_frag<NT, MT>(f[i], wrow, xrow, xvalid, cur + STAGES * SK_WAVES, grp, K);
+            }
+        }
     }
     // ---- the waves' sums, added in the order 0, 1, 2, ...
 #pragma unroll

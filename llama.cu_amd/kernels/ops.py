@@ -403,6 +403,7 @@ def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = 
         raise KernelError(f"gemm_skinny out: shape {tuple(out.shape)}, expected {(m, width)}")
     lib = build.load("gemm_skinny")
     _check(lib.lcu_gemm_skinny_bf16(_ptr(x), x.stride(0), _ptr(w), w.stride(0), _ptr(out), out.stride(0), m, n, k,
-                                    _EPILOGUES[epi], tiles or _skinny_tiles(width, m), waves or 4, _stream()),
+                                    _EPILOGUES[epi], tiles or _skinny_tiles(width, m),
+                                    waves or (8 if width <= 8192 else 4), _stream()),
            "gemm_skinny")
     return out
