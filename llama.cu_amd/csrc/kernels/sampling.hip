@@ -36,7 +36,18 @@ argmax_kernel(const float *__restrict__ logits, int ld, int vocab, int *__restri
     const float *row = logits + (size_t)blockIdx.x * ld;
     float best = -INFINITY;
     int bi = 0x7fffffff;
-    for (int i = threadIdx.x; i < vocab; i += blockDim.x) {
+    // four neighbouring logits per load where the row allows it (many loads in flight: a
+    // row is read by one workgroup, so latency, not bandwidth, is what counts)
+    const int vec_end = (((size_t)row % 16) == 0) ? (vocab / 4) * 4 : 0;
+#pragma unroll 4
+    for (int i = threadIdx.x * 4; i < vec_end; i += blockDim.x * 4) {
+        const float4 v = *(const float4 *)(row + i);
+        const float e[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+            if (e[k] > best || (e[k] == best && i + k < bi)) { best = e[k]; bi = i + k; }
+    }
+    for (int i = vec_end + threadIdx.x; i < vocab; i += blockDim.x) {
         const float v = row[i];
         if (v > best || (v == best && i < bi)) { best = v; bi = i; }
     }

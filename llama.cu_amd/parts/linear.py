@@ -2,10 +2,10 @@
 
 Which routine multiplies is decided here and nowhere else:
 
-* bfloat16 activations and weights, bfloat16 out: few rows (decoding) go to the
-  hand-written weight-streaming kernel, many rows to the library's matrix product
-  (hipBLASLt through torch), as the reference's engine calls its vendor library
-  (llama.cu/src/op/linear.rs:91-118);
+* bfloat16 activations and weights: few rows (decoding) go to the hand-written
+  weight-streaming kernel, many rows to the library's matrix product (hipBLASLt through
+  torch, with bfloat16 or, for logits, float32 output), as the reference's engine calls
+  its vendor library (llama.cu/src/op/linear.rs:91-118);
 * everything else (float32 anywhere: the true 32-bit path, a weight that its file
   stores in 32-bit, float32 logits): the hand-written kernel with 32-bit
   multiply-adds.
@@ -32,4 +32,6 @@ def linear(x: torch.Tensor, weight: torch.Tensor, out_dtype: Optional[torch.dtyp
         if out is None:
             return torch.matmul(x, weight.t())
         return torch.matmul(x, weight.t(), out=out)
+    if all_bf16 and out_dtype == torch.float32 and not accumulate and out is None and x.shape[0] > ops.SKINNY_ROWS:
+        return torch.mm(x, weight.t(), out_dtype=torch.float32)      # 32-bit accumulation, stored unrounded (logits)
     return ops.gemm_nt(x, weight, out=out, out_dtype=out_dtype, accumulate=accumulate)
