@@ -32,9 +32,7 @@ typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
 
-__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
-    return (uint32_t)from_f32<bf16_t>(lo).bits | ((uint32_t)from_f32<bf16_t>(hi).bits << 16);
-}
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) { return pack2_bf16(lo, hi); }
 // 2^x by the hardware's instruction (inputs here are <= 0; 2^-inf = 0)
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ f32x4 mfma16(u32x4 a, u32x4 b, f32x4 c) {
@@ -137,8 +135,11 @@ __device__ __forceinline__ void attn_compute(const KVFrag<DH> &f, int k0, const 
         }
         st.l[b] = st.l[b] * alpha + sum;
         st.m[b] = m_new;
+        // the output is rescaled only when some row's maximum has moved (the same test in all lanes)
+        if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
 #pragma unroll
-        for (int dt = 0; dt < DH / 16; ++dt) st.o[b][dt] *= alpha;
+            for (int dt = 0; dt < DH / 16; ++dt) st.o[b][dt] *= alpha;
+        }
         pb[b] = u32x4{pack_bf16(p[0], p[1]), pack_bf16(p[2], p[3]), pack_bf16(p[4], p[5]), pack_bf16(p[6], p[7])};
     }
     // ---- O^T += V^T P^T
@@ -332,21 +333,25 @@ LCU_API int lcu_attention_decode_bf16(const void *q, int q_stride, void *out, in
 
 // ============================================================================ prefill
 #ifndef LCU_PRE_QB
-#define LCU_PRE_QB 1
+#define LCU_PRE_QB 2
 #endif
 #ifndef LCU_PRE_MIN_WAVES
 #define LCU_PRE_MIN_WAVES 2
 #endif
+#ifndef LCU_PRE_SUB
+#define LCU_PRE_SUB 2
+#endif
 constexpr int PRE_WAVES = 4;
 constexpr int PRE_QB = LCU_PRE_QB;
+constexpr int PRE_SUB = LCU_PRE_SUB;      // 32-key steps that one copy to LDS (one barrier) brings
 
-// The 32 keys of one step, copied into LDS as they lie in their pages: per tile of 16 keys
+// The keys of PRE_SUB steps of 32, copied into LDS as they lie in their pages: per step, per tile of 16 keys
 // first the keys [dim/8][token][8], then (after both key tiles) the values [dim][token].
 // In units of 16 bytes a buffer holds 8*DH chunks: [K tile 0 | K tile 1 | V tile 0 | V tile 1],
 // 2*DH chunks each.  A thread of the workgroup copies chunks tid, tid + 256, ...
 template <int DH>
 struct StageRegs {
-    u32x4 c[DH / 32];
+    u32x4 c[PRE_SUB][DH / 32];
 };
 
 template <int DH>
@@ -354,10 +359,12 @@ __device__ __forceinline__ void stage_load(StageRegs<DH> &r, const bf16_t *__res
                                            int max_pages, int page, size_t page_elems, int nkvh, int kvh, int k0) {
     const size_t v_off = (size_t)nkvh * DH * page + (size_t)kvh * DH * page;
 #pragma unroll
+    for (int sub = 0; sub < PRE_SUB; ++sub)
+#pragma unroll
     for (int i = 0; i < DH / 32; ++i) {
         const int c = threadIdx.x + 256 * i;
         const int region = c / (2 * DH), w = c % (2 * DH), t = region & 1;
-        const int j = k0 + 16 * t;
+        const int j = k0 + 32 * sub + 16 * t;
         int pi = j / page;
         pi = pi < max_pages ? pi : max_pages - 1;
         const bf16_t *pg = cache + (size_t)bt[pi] * page_elems;
@@ -365,14 +372,16 @@ __device__ __forceinline__ void stage_load(StageRegs<DH> &r, const bf16_t *__res
         const bf16_t *src = region < 2
             ? pg + ((size_t)(kvh * (DH / 8) + w / 16) * page + tok0 + (w % 16)) * 8
             : pg + v_off + (size_t)(w / 2) * page + tok0 + (w % 2) * 8;
-        r.c[i] = *(const u32x4 *)src;
+        r.c[sub][i] = *(const u32x4 *)src;
     }
 }
 
 template <int DH>
 __device__ __forceinline__ void stage_store(const StageRegs<DH> &r, u32x4 *__restrict__ buf) {
 #pragma unroll
-    for (int i = 0; i < DH / 32; ++i) buf[threadIdx.x + 256 * i] = r.c[i];
+    for (int sub = 0; sub < PRE_SUB; ++sub)
+#pragma unroll
+        for (int i = 0; i < DH / 32; ++i) buf[sub * 8 * DH + threadIdx.x + 256 * i] = r.c[sub][i];
 }
 
 // A wave's operands of the step, read from the LDS copy.
@@ -401,7 +410,7 @@ attention_prefill_kernel(const bf16_t *__restrict__ q, int q_stride, bf16_t *__r
                          const int *__restrict__ q_start, const int *__restrict__ ctx_len,
                          const int *__restrict__ task_req, const int *__restrict__ task_tok0, int nh, int nkvh,
                          int page, float scale_log2, int window) {
-    __shared__ u32x4 lds[2][8 * DH];
+    __shared__ u32x4 lds[2][PRE_SUB * 8 * DH];
     const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
     const int task = blockIdx.x;
     const int l16 = lane & 15, grp = lane >> 4;
@@ -452,16 +461,20 @@ attention_prefill_kernel(const bf16_t *__restrict__ q, int q_stride, bf16_t *__r
     stage_load<DH>(regs, cache, bt, max_pages, page, page_elems, nkvh, kvh, blk0 * 32);
     stage_store<DH>(regs, lds[0]);
     __syncthreads();
-    for (int blk = blk0; blk < blk_end; ++blk) {
-        const int cur = (blk - blk0) & 1;
-        if (blk + 1 < blk_end) stage_load<DH>(regs, cache, bt, max_pages, page, page_elems, nkvh, kvh, (blk + 1) * 32);
-        const int k0 = blk * 32;
-        if (wave_has && k0 <= p_max && k0 + 31 >= lo_min) {
-            KVFrag<DH> f;
-            frag_from_lds<DH>(f, lds[cur], l16, grp);
-            attn_block<DH, QB>(f, k0, k0 + 31 > p_min || k0 < lo_max, qv, st, p_row, lo_row, p_max, lo_min, scale_log2, grp);
+    int cur = 0;
+    for (int blk = blk0; blk < blk_end; blk += PRE_SUB, cur ^= 1) {
+        const bool more = blk + PRE_SUB < blk_end;
+        if (more) stage_load<DH>(regs, cache, bt, max_pages, page, page_elems, nkvh, kvh, (blk + PRE_SUB) * 32);
+#pragma unroll
+        for (int sub = 0; sub < PRE_SUB; ++sub) {
+            const int k0 = (blk + sub) * 32;
+            if (wave_has && blk + sub < blk_end && k0 <= p_max && k0 + 31 >= lo_min) {
+                KVFrag<DH> f;
+                frag_from_lds<DH>(f, lds[cur] + sub * 8 * DH, l16, grp);
+                attn_block<DH, QB>(f, k0, k0 + 31 > p_min || k0 < lo_max, qv, st, p_row, lo_row, p_max, lo_min, scale_log2, grp);
+            }
         }
-        if (blk + 1 < blk_end) stage_store<DH>(regs, lds[cur ^ 1]);
+        if (more) stage_store<DH>(regs, lds[cur ^ 1]);
         __syncthreads();
     }
 #pragma unroll

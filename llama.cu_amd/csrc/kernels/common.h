@@ -21,17 +21,19 @@ __device__ __forceinline__ float to_f32(bf16_t x) { return __uint_as_float(((uin
 
 template <class T> __device__ __forceinline__ T from_f32(float x);
 template <> __device__ __forceinline__ float from_f32<float>(float x) { return x; }
-// round to nearest, ties to even; NaN stays NaN
+// round to nearest, ties to even; NaN stays NaN (the hardware's v_cvt_pk_bf16_f32)
 template <> __device__ __forceinline__ bf16_t from_f32<bf16_t>(float x) {
-    uint32_t u = __float_as_uint(x);
+    const __bf16 b = (__bf16)x;
     bf16_t r;
-    if ((u & 0x7fffffffu) > 0x7f800000u) {
-        r.bits = (uint16_t)((u >> 16) | 0x0040u);
-    } else {
-        u += 0x7fffu + ((u >> 16) & 1u);
-        r.bits = (uint16_t)(u >> 16);
-    }
+    r.bits = __builtin_bit_cast(uint16_t, b);
     return r;
+}
+// two at once, packed into 32 bits (lo in the low half)
+__device__ __forceinline__ uint32_t pack2_bf16(float lo, float hi) {
+    typedef __attribute__((ext_vector_type(2))) float f32x2_t;
+    typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
+    const f32x2_t v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
 }
 
 constexpr int WAVE = 64;
