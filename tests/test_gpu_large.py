@@ -1,0 +1,53 @@
+"""Two layers with the layer sizes of the Llama-3-8B shape (width 4096, 32 heads in 8
+groups of head size 128, feed-forward 14336, vocabulary 128256): the kernels that serve
+that shape (matrix-core attention for prefill and decode, the weight-streaming product,
+the library product, captured decode steps) inside the whole model, against the plain
+implementation, in 32-bit and in bfloat16."""
+import numpy as np
+import pytest
+import torch
+
+import common
+import plain
+
+pytestmark = pytest.mark.gpu
+
+SHAPE = dict(architectures=["LlamaForCausalLM"], num_hidden_layers=2, hidden_size=4096, num_attention_heads=32,
+             num_key_value_heads=8, head_dim=128, intermediate_size=14336, vocab_size=128256,
+             max_position_embeddings=8192, rope_theta=500000.0, rms_norm_eps=1e-5, tie_word_embeddings=False)
+
+
+@pytest.fixture(scope="module")
+def big():
+    out = {}
+    reqs = common.random_requests(SHAPE["vocab_size"], [70, 33], seed=3)
+    for dtype, tdt, std in (("float32", torch.float32, 0.02), ("bfloat16", torch.bfloat16, 0.02)):
+        folder = common.make_folder(SHAPE, seed=41, dtype=tdt, std=std)
+        out[dtype] = (folder, reqs, common.plain_logits(folder, reqs))
+    return out
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_whole_portions_and_decoding_at_full_layer_sizes(big, dtype):
+    from llama_cu_amd.engine.runner import ModelRunner
+    folder, reqs, want = big[dtype]
+    runner = ModelRunner.from_folder(folder, dtype=dtype, max_tokens=512, max_seqs=4)
+    names = list(reqs)
+    ids = {n: i for i, n in enumerate(names)}
+    got = {n: {} for n in names}
+    # both requests: most of the prompt in one step (together, a mixed batch), ...
+    head = {n: len(reqs[n]) - 12 for n in names}
+    logits = runner.step([ids[n] for n in names], [reqs[n][:head[n]] for n in names],
+                         [list(range(head[n])) for n in names]).cpu().numpy()
+    row = 0
+    for n in names:
+        for p in range(head[n]):
+            got[n][p] = logits[row]; row += 1
+    # ... then the last 12 tokens one by one, both requests in every step (captured after two)
+    for k in range(12):
+        logits = runner.step([ids[n] for n in names], [[reqs[n][head[n] + k]] for n in names]).cpu().numpy()
+        for i, n in enumerate(names):
+            got[n][head[n] + k] = logits[i]
+    if dtype == "bfloat16":
+        assert 2 in runner._graphs
+    common.assert_matches_plain(got, want, dtype, f"8B-sized layers/{dtype}")
