@@ -293,17 +293,20 @@ def attention_decode(q, out, cache, block_table, q_start, ctx_len, n_req, n_head
     return out
 
 
-def prefill_tasks(q_lens, tokens_per_task: int, device):
-    """Cut the batch into the prefill kernel's tasks: (request index, first token) pairs."""
-    reqs, toks = [], []
+def prefill_tasks(q_lens, ctx_lens, tokens_per_task: int, device):
+    """Cut the batch into the prefill kernel's tasks: (request index, first token) pairs, the
+    tasks that walk the most keys first (workgroups start in this order, so the long ones
+    do not start last and leave the other compute units waiting for them)."""
+    tasks = []
     start = 0
     for r, n in enumerate(q_lens):
         for t in range(0, n, tokens_per_task):
-            reqs.append(r)
-            toks.append(start + t)
+            keys = ctx_lens[r] - n + min(t + tokens_per_task, n)        # keys the task's last token sees
+            tasks.append((-keys, r, start + t))
         start += n
-    both = torch.tensor([reqs, toks], dtype=torch.int32).to(device)
-    return both[0], both[1], len(reqs)
+    tasks.sort()
+    both = torch.tensor([[t[1] for t in tasks], [t[2] for t in tasks]], dtype=torch.int32).to(device)
+    return both[0], both[1], len(tasks)
 
 
 def attention_prefill(q, out, cache, block_table, q_start, ctx_len, task_req, task_tok0, n_tasks, n_heads, n_kv_heads,
@@ -345,7 +348,7 @@ def paged_attention(q: torch.Tensor, out: torch.Tensor, cache: torch.Tensor, ste
     tpt = lib.lcu_attention_prefill_tokens_per_task(n_heads, n_kv_heads)
     key = ("attention_tasks", tpt)
     if key not in step.scratch:
-        step.scratch[key] = prefill_tasks(step.q_lens, tpt, q.device)
+        step.scratch[key] = prefill_tasks(step.q_lens, step.ctx_lens, tpt, q.device)
     task_req, task_tok0, n_tasks = step.scratch[key]
     return attention_prefill(q, out, cache, bt, step.q_start, step.ctx_len, task_req, task_tok0, n_tasks, n_heads,
                              n_kv_heads, head_dim, page_size, scale, window)
