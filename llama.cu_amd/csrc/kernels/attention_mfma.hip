@@ -408,11 +408,14 @@ __global__ void __launch_bounds__(PRE_WAVES *WAVE, LCU_PRE_MIN_WAVES)
 attention_prefill_kernel(const bf16_t *__restrict__ q, int q_stride, bf16_t *__restrict__ out, int out_stride,
                          const bf16_t *__restrict__ cache, const int *__restrict__ block_table, int max_pages,
                          const int *__restrict__ q_start, const int *__restrict__ ctx_len,
-                         const int *__restrict__ task_req, const int *__restrict__ task_tok0, int nh, int nkvh,
-                         int page, float scale_log2, int window) {
+                         const int *__restrict__ task_req, const int *__restrict__ task_tok0, int n_tasks,
+                         int tasks_per_wg, int nh, int nkvh, int page, float scale_log2, int window) {
     __shared__ u32x4 lds[2][PRE_SUB * 8 * DH];
     const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
-    const int task = blockIdx.x;
+    // a workgroup takes tasks_per_wg tasks one after the other (the host pairs a long one with
+    // a short one, so that workgroups take about equally long)
+    for (int task = blockIdx.x * tasks_per_wg; task < (blockIdx.x + 1) * tasks_per_wg && task < n_tasks; ++task) {
+    __syncthreads();                               // the last task's reads of LDS are over
     const int l16 = lane & 15, grp = lane >> 4;
     const int g = nh / nkvh;
     const int chunks = (g + 15) / 16;
@@ -493,18 +496,19 @@ attention_prefill_kernel(const bf16_t *__restrict__ q, int q_stride, bf16_t *__r
             *(u32x2 *)(o + 16 * dt + 4 * grp) = w;
         }
     }
+    }
 }
 
 template <int DH, int QB>
 static int launch_prefill(const void *q, int q_stride, void *out, int out_stride, const void *cache,
                           const int *block_table, int max_pages, const int *q_start, const int *ctx_len,
-                          const int *task_req, const int *task_tok0, int n_tasks, int nh, int nkvh, int page,
-                          float scale, int window, hipStream_t stream) {
+                          const int *task_req, const int *task_tok0, int n_tasks, int tasks_per_wg, int nh, int nkvh,
+                          int page, float scale, int window, hipStream_t stream) {
     const int g = nh / nkvh, chunks = (g + 15) / 16;
-    dim3 grid(n_tasks, nkvh * chunks), block(PRE_WAVES * WAVE);
+    dim3 grid((n_tasks + tasks_per_wg - 1) / tasks_per_wg, nkvh * chunks), block(PRE_WAVES * WAVE);
     attention_prefill_kernel<DH, QB><<<grid, block, 0, stream>>>(
         (const bf16_t *)q, q_stride, (bf16_t *)out, out_stride, (const bf16_t *)cache, block_table, max_pages, q_start,
-        ctx_len, task_req, task_tok0, nh, nkvh, page, scale * 1.4426950408889634f, window);
+        ctx_len, task_req, task_tok0, n_tasks, tasks_per_wg, nh, nkvh, page, scale * 1.4426950408889634f, window);
     LCU_LAUNCH_CHECK();
     return LCU_OK;
 }
@@ -520,17 +524,18 @@ LCU_API int lcu_attention_prefill_tokens_per_task(int nh, int nkvh) {
 }
 
 // task_req / task_tok0: [n_tasks], tasks cut from the batch with the size above; a
-// request's last task may be shorter.  bfloat16 only; head_dim 64 or 128; page_size a
+// request's last task may be shorter.  Workgroup i takes tasks i*tasks_per_wg .. + tasks_per_wg-1.  bfloat16 only; head_dim 64 or 128; page_size a
 // multiple of 16.
 LCU_API int lcu_attention_prefill_bf16(const void *q, int q_stride, void *out, int out_stride, const void *cache,
                                        const int *block_table, int max_pages, const int *q_start, const int *ctx_len,
-                                       const int *task_req, const int *task_tok0, int n_tasks, int nh, int nkvh,
-                                       int dh, int page, float scale, int window, hipStream_t stream) {
+                                       const int *task_req, const int *task_tok0, int n_tasks, int tasks_per_wg,
+                                       int nh, int nkvh, int dh, int page, float scale, int window,
+                                       hipStream_t stream) {
     if (n_tasks <= 0) return LCU_OK;
-    if (lcu_attention_prefill_tokens_per_task(nh, nkvh) == 0 || page <= 0 || page % 16 || max_pages <= 0 ||
+    if (tasks_per_wg < 1 || lcu_attention_prefill_tokens_per_task(nh, nkvh) == 0 || page <= 0 || page % 16 || max_pages <= 0 ||
         window < 0 || q_stride % 8 || out_stride % 4 || nkvh * ((nh / nkvh + 15) / 16) > 65535)
         return LCU_BAD_ARGUMENT;
-#define GO(D) return launch_prefill<D, PRE_QB>(q, q_stride, out, out_stride, cache, block_table, max_pages, q_start, ctx_len, task_req, task_tok0, n_tasks, nh, nkvh, page, scale, window, stream)
+#define GO(D) return launch_prefill<D, PRE_QB>(q, q_stride, out, out_stride, cache, block_table, max_pages, q_start, ctx_len, task_req, task_tok0, n_tasks, tasks_per_wg, nh, nkvh, page, scale, window, stream)
     if (dh == 128) GO(128);
     if (dh == 64) GO(64);
 #undef GO

@@ -293,7 +293,7 @@ def attention_decode(q, out, cache, block_table, q_start, ctx_len, n_req, n_head
     return out
 
 
-def prefill_tasks(q_lens, ctx_lens, tokens_per_task: int, device):
+def prefill_tasks(q_lens, ctx_lens, tokens_per_task: int, device, pair: Optional[bool] = None):
     """Cut the batch into the prefill kernel's tasks: (request index, first token) pairs, the
     tasks that walk the most keys first (workgroups start in this order, so the long ones
     do not start last and leave the other compute units waiting for them)."""
@@ -305,18 +305,39 @@ def prefill_tasks(q_lens, ctx_lens, tokens_per_task: int, device):
             tasks.append((-keys, r, start + t))
         start += n
     tasks.sort()
+    per_wg = 1
+    if pair is None:
+        # Tasks of very unequal length (a whole prompt: the last block walks all keys, the first
+        # none) leave compute units idle, since all workgroups are resident at once; then a
+        # workgroup takes a long and a short task.  Equal tasks run better one per workgroup
+        # (measured on the Llama-3-8B shape).
+        keys = [-t[0] for t in tasks]
+        pair = len(tasks) >= 2 and max(keys) >= 1.5 * (sum(keys) / len(keys))
+    if pair:
+        # the longest with the shortest, the second longest with the second shortest, ...
+        half = (len(tasks) + 1) // 2
+        paired = []
+        for i in range(half):
+            paired.append(tasks[i])
+            if len(tasks) - 1 - i > i:
+                paired.append(tasks[len(tasks) - 1 - i])
+            else:
+                paired.append(tasks[i])            # an odd one out: placeholder, removed below
+        if len(tasks) % 2:
+            paired.pop()
+        tasks, per_wg = paired, 2
     both = torch.tensor([[t[1] for t in tasks], [t[2] for t in tasks]], dtype=torch.int32).to(device)
-    return both[0], both[1], len(tasks)
+    return both[0], both[1], len(tasks), per_wg
 
 
-def attention_prefill(q, out, cache, block_table, q_start, ctx_len, task_req, task_tok0, n_tasks, n_heads, n_kv_heads,
-                      head_dim, page_size, scale, window) -> torch.Tensor:
+def attention_prefill(q, out, cache, block_table, q_start, ctx_len, task_req, task_tok0, n_tasks, tasks_per_wg, n_heads,
+                      n_kv_heads, head_dim, page_size, scale, window) -> torch.Tensor:
     """Matrix-core attention for any mix of portions and single tokens."""
     _i32(task_req, "task_req", n_tasks); _i32(task_tok0, "task_tok0", n_tasks)
     lib = build.load("attention_mfma")
     _check(lib.lcu_attention_prefill_bf16(_ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(cache), _ptr(block_table),
                                           block_table.shape[1], _ptr(q_start), _ptr(ctx_len), _ptr(task_req),
-                                          _ptr(task_tok0), n_tasks, n_heads, n_kv_heads, head_dim, page_size,
+                                          _ptr(task_tok0), n_tasks, tasks_per_wg, n_heads, n_kv_heads, head_dim, page_size,
                                           ctypes.c_float(scale), int(window), _stream()), "attention_prefill")
     return out
 
@@ -349,8 +370,8 @@ def paged_attention(q: torch.Tensor, out: torch.Tensor, cache: torch.Tensor, ste
     key = ("attention_tasks", tpt)
     if key not in step.scratch:
         step.scratch[key] = prefill_tasks(step.q_lens, step.ctx_lens, tpt, q.device)
-    task_req, task_tok0, n_tasks = step.scratch[key]
-    return attention_prefill(q, out, cache, bt, step.q_start, step.ctx_len, task_req, task_tok0, n_tasks, n_heads,
+    task_req, task_tok0, n_tasks, per_wg = step.scratch[key]
+    return attention_prefill(q, out, cache, bt, step.q_start, step.ctx_len, task_req, task_tok0, n_tasks, per_wg, n_heads,
                              n_kv_heads, head_dim, page_size, scale, window)
 
 
