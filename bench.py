@@ -27,7 +27,7 @@ sys.path.insert(0, ROOT)
 HBM_PEAK = 8.0e12
 MATRIX_PEAK = {"bf16": 2.5e15, "f32": 157.3e12}
 
-# BASELINE.json configs[2]: the Llama-3-8B shape
+# the Llama-3-8B shape
 SHAPE = dict(architectures=["LlamaForCausalLM"], num_hidden_layers=32, hidden_size=4096, num_attention_heads=32,
              num_key_value_heads=8, head_dim=128, intermediate_size=14336, vocab_size=128256,
              max_position_embeddings=8192, rope_theta=500000.0, rms_norm_eps=1e-5, tie_word_embeddings=False)
