@@ -244,3 +244,118 @@ LCU_API int lcu_gemm_skinny_bf16(const void *X, int ldx, const void *W, int ldw,
 #undef EP
     return LCU_BAD_ARGUMENT;
 }
+
+
+// ============================================================================ float32
+// The same weight-streaming layout for float32 operands, with v_mfma_f32_16x16x4_f32: a true
+// 32-bit matrix product (32-bit multiplies and adds; no reduced-precision mode).  A lane's
+// 16-byte load holds four k of its row, one per instruction.  K goes in macro-steps of 64; the
+// waves of a workgroup take macro-steps in turn and their sums are added in a fixed order, so
+// a token's result depends on K and the number of waves only: not on M, not on which tile of
+// 64 tokens (grid.y) it is in, not on the other tokens.
+constexpr int F32_WAVES = 8;
+
+template <int MT>
+struct FragF32 {
+    f32x4 w[4];
+    f32x4 x[MT][4];
+};
+
+template <int MT>
+__device__ __forceinline__ void load_frag_f32(FragF32<MT> &f, const float *wrow, const float *const (&xrow)[MT],
+                                              const bool (&xvalid)[MT], int s, int grp, int K) {
+    const int kb = 64 * s + 16 * grp;
+    const f32x4 zero = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const bool in = kb + 4 * j + 4 <= K;                // K is a multiple of 4
+        f.w[j] = in ? *(const f32x4 *)(wrow + kb + 4 * j) : zero;
+#pragma unroll
+        for (int m = 0; m < MT; ++m) f.x[m][j] = (in && xvalid[m]) ? *(const f32x4 *)(xrow[m] + kb + 4 * j) : zero;
+    }
+}
+
+template <int MT>
+__global__ void __launch_bounds__(F32_WAVES *WAVE)
+gemm_skinny_f32_kernel(const float *__restrict__ X, int ldx, const float *__restrict__ W, int ldw, float *__restrict__ Y,
+                       int ldy, int M, int N, int K, int accumulate) {
+    __shared__ float red[F32_WAVES][MT * 4][WAVE];
+    const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
+    const int l16 = lane & 15, grp = lane >> 4;
+    const int n0 = blockIdx.x * 16, m0 = blockIdx.y * 16 * MT;
+    int row = n0 + l16;
+    row = row < N ? row : N - 1;                            // a row beyond the end is read, not stored
+    const float *wrow = W + (size_t)row * ldw;
+    const float *xrow[MT];
+    bool xvalid[MT];
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+        xvalid[m] = m0 + 16 * m + l16 < M;
+        xrow[m] = X + (size_t)(xvalid[m] ? m0 + 16 * m + l16 : 0) * ldx;
+    }
+    f32x4 acc[MT];
+#pragma unroll
+    for (int m = 0; m < MT; ++m) acc[m] = f32x4{0.f, 0.f, 0.f, 0.f};
+    const int nsteps = (K + 63) / 64;
+    FragF32<MT> fa, fb;
+    int s = wave;
+    if (s < nsteps) load_frag_f32<MT>(fa, wrow, xrow, xvalid, s, grp, K);
+    for (; s < nsteps; s += 2 * F32_WAVES) {
+        const bool has_b = s + F32_WAVES < nsteps;
+        if (has_b) load_frag_f32<MT>(fb, wrow, xrow, xvalid, s + F32_WAVES, grp, K);
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+#pragma unroll
+                for (int m = 0; m < MT; ++m) acc[m] = __builtin_amdgcn_mfma_f32_16x16x4f32(fa.w[j][e], fa.x[m][j][e], acc[m], 0, 0, 0);
+        if (s + 2 * F32_WAVES < nsteps) load_frag_f32<MT>(fa, wrow, xrow, xvalid, s + 2 * F32_WAVES, grp, K);
+        if (has_b) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+#pragma unroll
+                    for (int m = 0; m < MT; ++m) acc[m] = __builtin_amdgcn_mfma_f32_16x16x4f32(fb.w[j][e], fb.x[m][j][e], acc[m], 0, 0, 0);
+        }
+    }
+#pragma unroll
+    for (int m = 0; m < MT; ++m)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) red[wave][m * 4 + r][lane] = acc[m][r];
+    __syncthreads();
+    if (wave != 0) return;
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+        const int tok = m0 + 16 * m + l16;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            float sum = red[0][m * 4 + r][lane];
+#pragma unroll
+            for (int w = 1; w < F32_WAVES; ++w) sum += red[w][m * 4 + r][lane];
+            const int n = n0 + 4 * grp + r;
+            if (tok < M && n < N) {
+                float *y = Y + (size_t)tok * ldy + n;
+                *y = accumulate ? *y + sum : sum;
+            }
+        }
+    }
+}
+
+// X: [M, K] float32, W: [N, K] float32, Y: [M, N] float32 (accumulate: Y += X W^T).  Any M
+// (tiles of 64 tokens; W is read once per tile); K, ldx, ldw multiples of 4.
+LCU_API int lcu_gemm_skinny_f32(const float *X, int ldx, const float *W, int ldw, float *Y, int ldy, int M, int N,
+                                int K, int accumulate, hipStream_t stream) {
+    if (M <= 0 || N <= 0) return LCU_OK;
+    if (K <= 0 || K % 4 || ldx % 4 || ldw % 4 || ldx < K || ldw < K || ldy < N) return LCU_BAD_ARGUMENT;
+    const dim3 block(F32_WAVES * WAVE);
+    if (M <= 16) {
+        gemm_skinny_f32_kernel<1><<<dim3((N + 15) / 16, 1), block, 0, stream>>>(X, ldx, W, ldw, Y, ldy, M, N, K, accumulate);
+    } else {
+        const int tiles = (M + 63) / 64;
+        if (tiles > 65535) return LCU_BAD_ARGUMENT;
+        gemm_skinny_f32_kernel<4><<<dim3((N + 15) / 16, tiles), block, 0, stream>>>(X, ldx, W, ldw, Y, ldy, M, N, K, accumulate);
+    }
+    LCU_LAUNCH_CHECK();
+    return LCU_OK;
+}

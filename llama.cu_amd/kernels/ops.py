@@ -431,3 +431,34 @@ def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = 
                                     waves or (8 if width <= 8192 else 4), _stream()),
            "gemm_skinny")
     return out
+
+
+def skinny_f32_supported(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype) -> bool:
+    """Whether the float32 weight-streaming kernel takes this product: all float32, K a
+    multiple of 4 (16-byte loads)."""
+    return (x.dtype == torch.float32 and w.dtype == torch.float32 and out_dtype == torch.float32 and x.dim() == 2
+            and w.dim() == 2 and x.shape[0] > 0 and x.shape[1] % 4 == 0 and x.stride(1) == 1 and w.stride(1) == 1
+            and x.stride(0) % 4 == 0 and w.stride(0) % 4 == 0 and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
+
+
+def gemm_skinny_f32(x: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = None,
+                    accumulate: bool = False) -> torch.Tensor:
+    """``out (+)= x @ w.T`` in true 32-bit on the matrix cores (v_mfma_f32_16x16x4_f32), any
+    number of rows; a row's result does not depend on the other rows."""
+    _gpu(x, w, out)
+    _rows(x, "skinny x"); _rows(w, "skinny w")
+    m, k = x.shape
+    n = w.shape[0]
+    if w.shape[1] != k or not skinny_f32_supported(x, w, torch.float32):
+        raise KernelError(f"gemm_skinny_f32: x {tuple(x.shape)} {x.dtype} with w {tuple(w.shape)} {w.dtype} is not supported")
+    if out is None:
+        if accumulate:
+            raise KernelError("gemm_skinny_f32: accumulate needs an output to add to")
+        out = torch.empty((m, n), dtype=torch.float32, device=x.device)
+    _rows(out, "skinny out")
+    if out.shape != (m, n) or out.dtype != torch.float32:
+        raise KernelError("gemm_skinny_f32 out: wrong shape or type")
+    lib = build.load("gemm_skinny")
+    _check(lib.lcu_gemm_skinny_f32(_ptr(x), x.stride(0), _ptr(w), w.stride(0), _ptr(out), out.stride(0), m, n, k,
+                                   int(bool(accumulate)), _stream()), "gemm_skinny_f32")
+    return out

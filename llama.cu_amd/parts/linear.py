@@ -6,9 +6,11 @@ Which routine multiplies is decided here and nowhere else:
   weight-streaming kernel, many rows to the library's matrix product (hipBLASLt through
   torch, with bfloat16 or, for logits, float32 output), as the reference's engine calls
   its vendor library (llama.cu/src/op/linear.rs:91-118);
-* everything else (float32 anywhere: the true 32-bit path, a weight that its file
-  stores in 32-bit, float32 logits): the hand-written kernel with 32-bit
-  multiply-adds.
+* all float32 (the true 32-bit path): the hand-written weight-streaming kernel on the
+  32-bit matrix instruction, for any number of rows;
+* everything else (mixed types: a weight that its file stores in 32-bit beside
+  bfloat16 activations; widths the others refuse): the generic hand-written kernel with
+  32-bit multiply-adds.
 """
 from __future__ import annotations
 
@@ -34,4 +36,6 @@ def linear(x: torch.Tensor, weight: torch.Tensor, out_dtype: Optional[torch.dtyp
         return torch.matmul(x, weight.t(), out=out)
     if all_bf16 and out_dtype == torch.float32 and not accumulate and out is None and x.shape[0] > ops.SKINNY_ROWS:
         return torch.mm(x, weight.t(), out_dtype=torch.float32)      # 32-bit accumulation, stored unrounded (logits)
+    if ops.skinny_f32_supported(x, weight, out_dtype):
+        return ops.gemm_skinny_f32(x, weight, out=out, accumulate=accumulate)
     return ops.gemm_nt(x, weight, out=out, out_dtype=out_dtype, accumulate=accumulate)

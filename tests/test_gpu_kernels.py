@@ -365,3 +365,28 @@ def test_gemm_skinny_refuses_what_it_cannot_take():
     with pytest.raises(ops.KernelError):
         ops.gemm_skinny(x, w)
     assert not ops.skinny_supported(rnd(65, 64).to(torch.bfloat16).cuda(), rnd(16, 64).to(torch.bfloat16).cuda(), torch.bfloat16)
+
+
+@pytest.mark.parametrize("m,n,k", [(1, 16, 4), (8, 301, 172), (17, 100, 64), (70, 4096, 352), (300, 1000, 4096)])
+def test_gemm_skinny_f32(m, n, k):
+    from llama_cu_amd.kernels import ops
+    x, w = rnd(m, k, seed=m), rnd(n, k, seed=n + 3)
+    want = plain.linear(x, w)
+    close(ops.gemm_skinny_f32(x.cuda(), w.cuda()), want, "float32")
+    c = rnd(m, n, seed=9)
+    cg = c.cuda()
+    ops.gemm_skinny_f32(x.cuda(), w.cuda(), out=cg, accumulate=True)
+    close(cg, c.double() + want, "float32", "accumulate")
+
+
+def test_gemm_skinny_f32_is_true_32_bit_and_rows_are_independent():
+    from llama_cu_amd.kernels import ops
+    a = torch.full((4, 256), 1.0 + 2.0 ** -12)
+    w = torch.full((20, 256), 1.0 + 2.0 ** -12)
+    out = ops.gemm_skinny_f32(a.cuda(), w.cuda())
+    assert float((out.double().cpu() - 256.125).abs().max()) < 1e-3          # a reduced-precision mode gives 256
+    x, w = rnd(150, 512, seed=1).cuda(), rnd(77, 512, seed=2).cuda()
+    whole = ops.gemm_skinny_f32(x, w)
+    for r in (0, 15, 16, 63, 64, 149):                                        # alone, in a batch of few, in any tile of 64
+        assert torch.equal(whole[r:r + 1], ops.gemm_skinny_f32(x[r:r + 1], w))
+    assert torch.equal(whole[60:70], ops.gemm_skinny_f32(x[60:70], w))
