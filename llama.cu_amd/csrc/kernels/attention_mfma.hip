@@ -190,13 +190,14 @@ template <int DH>
 __global__ void __launch_bounds__(DEC_WAVES *WAVE, LCU_DEC_MIN_WAVES)
 attention_decode_kernel(const bf16_t *__restrict__ q, int q_stride, bf16_t *__restrict__ out, int out_stride,
                         const bf16_t *__restrict__ cache, const int *__restrict__ block_table, int max_pages,
-                        const int *__restrict__ q_start, const int *__restrict__ ctx_len, int nh, int nkvh, int page,
-                        float scale_log2, int window, int n_splits, float *__restrict__ part_o,
-                        float *__restrict__ part_ml) {
+                        const int *__restrict__ q_start, const int *__restrict__ ctx_len,
+                        const int *__restrict__ req_list, int nh, int nkvh, int page, float scale_log2, int window,
+                        int n_splits, float *__restrict__ part_o, float *__restrict__ part_ml) {
     extern __shared__ float lds[];                 // [waves][16][DH] outputs, then [waves][16][2] (m, l)
     const int g = nh / nkvh;
     const int chunks = (g + 15) / 16;
-    const int r = blockIdx.x / (nkvh * chunks);
+    const int ri = blockIdx.x / (nkvh * chunks);
+    const int r = req_list ? req_list[ri] : ri;         // the batch's decoding requests, or all of them
     const int kvh = (blockIdx.x / chunks) % nkvh;
     const int chunk = blockIdx.x % chunks;
     const int split = blockIdx.y;
@@ -264,7 +265,7 @@ attention_decode_kernel(const bf16_t *__restrict__ q, int q_stride, bf16_t *__re
         if (n_splits == 1) {
             out[(size_t)token * out_stride + (size_t)head * DH + d] = from_f32<bf16_t>(val / L);
         } else {
-            const size_t slot = ((size_t)token * nh + head) * n_splits + split;
+            const size_t slot = ((size_t)ri * nh + head) * n_splits + split;
             part_o[slot * DH + d] = val;
             if (d == 0) { part_ml[slot * 2] = M; part_ml[slot * 2 + 1] = L; }
         }
@@ -277,9 +278,11 @@ attention_decode_kernel(const bf16_t *__restrict__ q, int q_stride, bf16_t *__re
 // several times slower than this second launch.)
 template <int DH>
 __global__ void attention_merge_kernel(bf16_t *__restrict__ out, int out_stride, const float *__restrict__ part_o,
-                                       const float *__restrict__ part_ml, int nh, int n_splits) {
-    const int token = blockIdx.x, head = blockIdx.y;
-    const size_t base = ((size_t)token * nh + head) * n_splits;
+                                       const float *__restrict__ part_ml, const int *__restrict__ q_start,
+                                       const int *__restrict__ req_list, int nh, int n_splits) {
+    const int ri = blockIdx.x, head = blockIdx.y;
+    const int token = q_start[req_list ? req_list[ri] : ri];
+    const size_t base = ((size_t)ri * nh + head) * n_splits;
     float M = -INFINITY;
     for (int s = 0; s < n_splits; ++s) M = fmaxf(M, part_ml[(base + s) * 2]);
     float L = 0.f;
@@ -294,37 +297,38 @@ __global__ void attention_merge_kernel(bf16_t *__restrict__ out, int out_stride,
 
 template <int DH>
 static int launch_decode(const void *q, int q_stride, void *out, int out_stride, const void *cache,
-                         const int *block_table, int max_pages, const int *q_start, const int *ctx_len, int n_req,
-                         int nh, int nkvh, int page, float scale, int window, int n_splits, float *part_o,
-                         float *part_ml, hipStream_t stream) {
+                         const int *block_table, int max_pages, const int *q_start, const int *ctx_len,
+                         const int *req_list, int n_req, int nh, int nkvh, int page, float scale, int window,
+                         int n_splits, float *part_o, float *part_ml, hipStream_t stream) {
     const int g = nh / nkvh, chunks = (g + 15) / 16;
     const float scale_log2 = scale * 1.4426950408889634f;
     const size_t lds_bytes = (size_t)DEC_WAVES * 16 * (DH + 2) * sizeof(float);
     dim3 grid(n_req * nkvh * chunks, n_splits), block(DEC_WAVES * WAVE);
     attention_decode_kernel<DH><<<grid, block, lds_bytes, stream>>>(
         (const bf16_t *)q, q_stride, (bf16_t *)out, out_stride, (const bf16_t *)cache, block_table, max_pages, q_start,
-        ctx_len, nh, nkvh, page, scale_log2, window, n_splits, part_o, part_ml);
+        ctx_len, req_list, nh, nkvh, page, scale_log2, window, n_splits, part_o, part_ml);
     LCU_LAUNCH_CHECK();
     if (n_splits > 1) {
         attention_merge_kernel<DH><<<dim3(n_req, nh), dim3(WAVE), 0, stream>>>((bf16_t *)out, out_stride, part_o, part_ml,
-                                                                                nh, n_splits);
+                                                                                q_start, req_list, nh, n_splits);
         LCU_LAUNCH_CHECK();
     }
     return LCU_OK;
 }
 
-// Every request of the batch feeds exactly one token (token r belongs to request r).
+// The n_req requests req_list[0..n_req) of the batch (all of the batch's requests in order
+// if req_list is null) feed exactly one token each.
 // part_o: [n_req * nh * n_splits * dh] floats, part_ml: [n_req * nh * n_splits * 2] (unused
 // when n_splits == 1).  bfloat16 only; head_dim 64 or 128; page_size a multiple of 16.
 LCU_API int lcu_attention_decode_bf16(const void *q, int q_stride, void *out, int out_stride, const void *cache,
                                       const int *block_table, int max_pages, const int *q_start, const int *ctx_len,
-                                      int n_req, int nh, int nkvh, int dh, int page, float scale, int window,
-                                      int n_splits, float *part_o, float *part_ml, hipStream_t stream) {
+                                      const int *req_list, int n_req, int nh, int nkvh, int dh, int page, float scale,
+                                      int window, int n_splits, float *part_o, float *part_ml, hipStream_t stream) {
     if (n_req <= 0) return LCU_OK;
     if (nh <= 0 || nkvh <= 0 || nh % nkvh || page <= 0 || page % 16 || max_pages <= 0 || window < 0 || n_splits < 1 ||
         n_splits > 65535 || (n_splits > 1 && (!part_o || !part_ml)) || q_stride % 8 || out_stride % 4)
         return LCU_BAD_ARGUMENT;
-#define GO(D) return launch_decode<D>(q, q_stride, out, out_stride, cache, block_table, max_pages, q_start, ctx_len, n_req, nh, nkvh, page, scale, window, n_splits, part_o, part_ml, stream)
+#define GO(D) return launch_decode<D>(q, q_stride, out, out_stride, cache, block_table, max_pages, q_start, ctx_len, req_list, n_req, nh, nkvh, page, scale, window, n_splits, part_o, part_ml, stream)
     if (dh == 128) GO(128);
     if (dh == 64) GO(64);
 #undef GO

@@ -279,28 +279,32 @@ def mfma_attention_supported(q: torch.Tensor, n_heads: int, n_kv_heads: int, hea
 
 
 def attention_decode(q, out, cache, block_table, q_start, ctx_len, n_req, n_heads, n_kv_heads, head_dim, page_size,
-                     scale, window, n_splits) -> torch.Tensor:
-    """Matrix-core attention for a batch in which every request feeds one token."""
+                     scale, window, n_splits, req_list: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Matrix-core attention for requests that feed one token each: all ``n_req`` requests of
+    the batch, or the ``n_req`` whose indices ``req_list`` holds."""
+    if req_list is not None:
+        _i32(req_list, "req_list", n_req)
     part_o = part_ml = None
     if n_splits > 1:
         part_o = torch.empty(n_req * n_heads * n_splits * head_dim, dtype=torch.float32, device=q.device)
         part_ml = torch.empty(n_req * n_heads * n_splits * 2, dtype=torch.float32, device=q.device)
     lib = build.load("attention_mfma")
     _check(lib.lcu_attention_decode_bf16(_ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(cache), _ptr(block_table),
-                                         block_table.shape[1], _ptr(q_start), _ptr(ctx_len), n_req, n_heads, n_kv_heads,
+                                         block_table.shape[1], _ptr(q_start), _ptr(ctx_len), _ptr(req_list), n_req, n_heads,
+                                         n_kv_heads,
                                          head_dim, page_size, ctypes.c_float(scale), int(window), int(n_splits),
                                          _ptr(part_o), _ptr(part_ml), _stream()), "attention_decode")
     return out
 
 
-def prefill_tasks(q_lens, ctx_lens, tokens_per_task: int, device, pair: Optional[bool] = None):
+def prefill_tasks(q_lens, ctx_lens, tokens_per_task: int, device, pair: Optional[bool] = None, skip_single: bool = False):
     """Cut the batch into the prefill kernel's tasks: (request index, first token) pairs, the
     tasks that walk the most keys first (workgroups start in this order, so the long ones
     do not start last and leave the other compute units waiting for them)."""
     tasks = []
     start = 0
     for r, n in enumerate(q_lens):
-        for t in range(0, n, tokens_per_task):
+        for t in range(0, n if not (skip_single and n == 1) else 0, tokens_per_task):
             keys = ctx_lens[r] - n + min(t + tokens_per_task, n)        # keys the task's last token sees
             tasks.append((-keys, r, start + t))
         start += n
@@ -326,6 +330,8 @@ def prefill_tasks(q_lens, ctx_lens, tokens_per_task: int, device, pair: Optional
         if len(tasks) % 2:
             paired.pop()
         tasks, per_wg = paired, 2
+    if not tasks:
+        return None, None, 0, 1
     both = torch.tensor([[t[1] for t in tasks], [t[2] for t in tasks]], dtype=torch.int32).to(device)
     return both[0], both[1], len(tasks), per_wg
 
@@ -365,14 +371,26 @@ def paged_attention(q: torch.Tensor, out: torch.Tensor, cache: torch.Tensor, ste
         splits = step.attn_splits or decode_splits(step.n_req, n_heads, n_kv_heads, step.max_ctx_len)
         return attention_decode(q, out, cache, bt, step.q_start, step.ctx_len, step.n_req, n_heads, n_kv_heads, head_dim,
                                 page_size, scale, window, splits)
+    # a mixed batch: the requests that decode one token go to the decode kernel, the portions
+    # to the prefill kernel (each would be slow at the other's work)
     lib = build.load("attention_mfma")
     tpt = lib.lcu_attention_prefill_tokens_per_task(n_heads, n_kv_heads)
     key = ("attention_tasks", tpt)
     if key not in step.scratch:
-        step.scratch[key] = prefill_tasks(step.q_lens, step.ctx_lens, tpt, q.device)
-    task_req, task_tok0, n_tasks, per_wg = step.scratch[key]
-    return attention_prefill(q, out, cache, bt, step.q_start, step.ctx_len, task_req, task_tok0, n_tasks, per_wg, n_heads,
-                             n_kv_heads, head_dim, page_size, scale, window)
+        singles = [r for r, n in enumerate(step.q_lens) if n == 1]
+        use_decode = len(singles) >= 1
+        tasks = prefill_tasks(step.q_lens, step.ctx_lens, tpt, q.device, skip_single=use_decode)
+        req_list = torch.tensor(singles, dtype=torch.int32).to(q.device) if use_decode else None
+        max_ctx = max([step.ctx_lens[r] for r in singles], default=0)
+        step.scratch[key] = (tasks, req_list, len(singles) if use_decode else 0, max_ctx)
+    (task_req, task_tok0, n_tasks, per_wg), req_list, n_single, max_ctx = step.scratch[key]
+    if n_single:
+        attention_decode(q, out, cache, bt, step.q_start, step.ctx_len, n_single, n_heads, n_kv_heads, head_dim, page_size,
+                         scale, window, decode_splits(n_single, n_heads, n_kv_heads, max_ctx), req_list=req_list)
+    if n_tasks:
+        attention_prefill(q, out, cache, bt, step.q_start, step.ctx_len, task_req, task_tok0, n_tasks, per_wg, n_heads,
+                          n_kv_heads, head_dim, page_size, scale, window)
+    return out
 
 
 SKINNY_MAX_ROWS = 64      # what the kernel takes
