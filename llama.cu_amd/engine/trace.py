@@ -42,7 +42,7 @@ class TraceReplayer:
     def step(self, obj: Dict[str, Any]) -> Optional[np.ndarray]:
         """Run one step; returns the wanted logits ``[wanted, vocab]`` (float32) or None if
         nothing was wanted."""
-        entries = obj.get("entries", [])
+        entries = [e for e in obj.get("entries", []) if len(e.get("tokens", [])) > 0]
         out = None
         if entries:
             names = [e["id"] for e in entries]

@@ -407,6 +407,16 @@ def skinny_supported(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype) -
             and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
 
 
+def skinny_preferred(m: int, n: int, k: int, out_dtype: torch.dtype) -> bool:
+    """Whether the weight-streaming kernel is the faster choice for a plain bfloat16 product
+    of ``m`` rows with an ``[n, k]`` weight (measured against the library on the Llama-3-8B
+    shapes): always for very few rows and for float32 output; for 5 to 16 rows only for small
+    weights (the library's split over K wins on the large ones)."""
+    if m > SKINNY_ROWS:
+        return False
+    return m <= 4 or out_dtype == torch.float32 or n * k <= (1 << 24)
+
+
 def _skinny_tiles(n_features: int, m: int) -> int:
     """Output tiles of 16 features per workgroup: as many as still leave about four
     workgroups for each of the 256 compute units."""

@@ -28,7 +28,8 @@ def linear(x: torch.Tensor, weight: torch.Tensor, out_dtype: Optional[torch.dtyp
         raise ops.KernelError("linear: operands must be on the GPU (there is no CPU path)")
     out_dtype = out.dtype if out is not None else (out_dtype or x.dtype)
     all_bf16 = x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
-    if all_bf16 and x.shape[0] <= ops.SKINNY_ROWS and ops.skinny_supported(x, weight, out_dtype):
+    if all_bf16 and ops.skinny_supported(x, weight, out_dtype) and (
+            accumulate or ops.skinny_preferred(x.shape[0], weight.shape[0], weight.shape[1], out_dtype)):
         return ops.gemm_skinny(x, weight, out=out, out_dtype=out_dtype, accumulate=accumulate)
     if all_bf16 and out_dtype == torch.bfloat16 and not accumulate:
         if out is None:
