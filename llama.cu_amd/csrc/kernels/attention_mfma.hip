@@ -319,7 +319,7 @@ static int launch_decode(const void *q, int q_stride, void *out, int out_stride,
 // The n_req requests req_list[0..n_req) of the batch (all of the batch's requests in order
 // if req_list is null) feed exactly one token each.
 // part_o: [n_req * nh * n_splits * dh] floats, part_ml: [n_req * nh * n_splits * 2] (unused
-// when n_splits == 1).  bfloat16 only; head_dim 64 or 128; page_size a multiple of 16.
+// when n_splits == 1).  bfloat16 only; head_dim 32, 64, 96 or 128; page_size a multiple of 16.
 LCU_API int lcu_attention_decode_bf16(const void *q, int q_stride, void *out, int out_stride, const void *cache,
                                       const int *block_table, int max_pages, const int *q_start, const int *ctx_len,
                                       const int *req_list, int n_req, int nh, int nkvh, int dh, int page, float scale,
@@ -331,6 +331,8 @@ LCU_API int lcu_attention_decode_bf16(const void *q, int q_stride, void *out, in
 #define GO(D) return launch_decode<D>(q, q_stride, out, out_stride, cache, block_table, max_pages, q_start, ctx_len, req_list, n_req, nh, nkvh, page, scale, window, n_splits, part_o, part_ml, stream)
     if (dh == 128) GO(128);
     if (dh == 64) GO(64);
+    if (dh == 96) GO(96);
+    if (dh == 32) GO(32);
 #undef GO
     return LCU_UNSUPPORTED;
 }
@@ -528,8 +530,8 @@ LCU_API int lcu_attention_prefill_tokens_per_task(int nh, int nkvh) {
 }
 
 // task_req / task_tok0: [n_tasks], tasks cut from the batch with the size above; a
-// request's last task may be shorter.  Workgroup i takes tasks i*tasks_per_wg .. + tasks_per_wg-1.  bfloat16 only; head_dim 64 or 128; page_size a
-// multiple of 16.
+// request's last task may be shorter.  Workgroup i takes tasks i*tasks_per_wg .. + tasks_per_wg-1.
+// bfloat16 only; head_dim 32, 64, 96 or 128; page_size a multiple of 16.
 LCU_API int lcu_attention_prefill_bf16(const void *q, int q_stride, void *out, int out_stride, const void *cache,
                                        const int *block_table, int max_pages, const int *q_start, const int *ctx_len,
                                        const int *task_req, const int *task_tok0, int n_tasks, int tasks_per_wg,
@@ -542,6 +544,8 @@ LCU_API int lcu_attention_prefill_bf16(const void *q, int q_stride, void *out, i
 #define GO(D) return launch_prefill<D, PRE_QB>(q, q_stride, out, out_stride, cache, block_table, max_pages, q_start, ctx_len, task_req, task_tok0, n_tasks, tasks_per_wg, nh, nkvh, page, scale, window, stream)
     if (dh == 128) GO(128);
     if (dh == 64) GO(64);
+    if (dh == 96) GO(96);
+    if (dh == 32) GO(32);
 #undef GO
     return LCU_UNSUPPORTED;
 }

@@ -83,12 +83,14 @@ gemm_skinny_kernel(const bf16_t *__restrict__ X, int ldx, const bf16_t *__restri
     const int l16 = lane & 15, grp = lane >> 4;
     // the rows of W of tile t: for SwiGLU tile 0 are gate rows, tile 1 the up rows N/2 further
     const int n_out = EPI == EPI_SWIGLU ? N / 2 : N;                 // width of Y
-    const int n0 = blockIdx.x * 16 * (EPI == EPI_SWIGLU ? 1 : NT);
+    // SwiGLU: the first NT/2 tiles are gate rows, the other NT/2 the up rows N/2 further
+    const int n0 = blockIdx.x * 16 * (EPI == EPI_SWIGLU ? NT / 2 : NT);
     const bf16_t *wrow[NT];
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
-        int row = EPI == EPI_SWIGLU ? n0 + l16 + t * n_out : n0 + 16 * t + l16;
-        const int limit = EPI == EPI_SWIGLU ? (t + 1) * n_out : N;
+        const int half = t / (NT / 2 > 0 ? NT / 2 : 1);              // 0: gate tiles, 1: up tiles (SwiGLU)
+        int row = EPI == EPI_SWIGLU ? n0 + 16 * (t % (NT / 2 > 0 ? NT / 2 : 1)) + l16 + half * n_out : n0 + 16 * t + l16;
+        const int limit = EPI == EPI_SWIGLU ? (half + 1) * n_out : N;
         row = row < limit ? row : limit - 1;                          // a row beyond the end is read, not stored
         wrow[t] = W + (size_t)row * ldw;
     }
@@ -153,13 +155,15 @@ gemm_skinny_kernel(const bf16_t *__restrict__ X, int ldx, const bf16_t *__restri
         if (tok >= M) continue;
         if (EPI == EPI_SWIGLU) {
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const int n = n0 + 4 * grp + r;
-                if (n >= n_out) continue;
-                const float gate = acc[0][m][r], up = acc[1][m][r];
-                const float sig = 1.0f / (1.0f + expf(-gate));
-                ((bf16_t *)Y)[(size_t)tok * ldy + n] = from_f32<bf16_t>(gate * sig * up);
-            }
+            for (int t = 0; t < NT / 2; ++t)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int n = n0 + 16 * t + 4 * grp + r;
+                    if (n >= n_out) continue;
+                    const float gate = acc[t][m][r], up = acc[t + NT / 2][m][r];
+                    const float sig = 1.0f / (1.0f + expf(-gate));
+                    ((bf16_t *)Y)[(size_t)tok * ldy + n] = from_f32<bf16_t>(gate * sig * up);
+                }
         } else {
 #pragma unroll
             for (int t = 0; t < NT; ++t)
@@ -193,11 +197,11 @@ static int launch_epi(const void *X, int ldx, const void *W, int ldw, void *Y, i
     return LCU_OK;
 }
 
-template <int MT, int WAVES>
+template <int NT, int MT, int WAVES>
 static int launch_swiglu(const void *X, int ldx, const void *W, int ldw, void *Y, int ldy, int M, int N, int K,
                          hipStream_t stream) {
-    const int groups = (N / 2 + 15) / 16;
-    gemm_skinny_kernel<2, MT, EPI_SWIGLU, WAVES><<<dim3(groups), dim3(WAVES * WAVE), 0, stream>>>(
+    const int groups = (N / 2 + 8 * NT - 1) / (8 * NT);
+    gemm_skinny_kernel<NT, MT, EPI_SWIGLU, WAVES><<<dim3(groups), dim3(WAVES * WAVE), 0, stream>>>(
         (const bf16_t *)X, ldx, (const bf16_t *)W, ldw, Y, ldy, M, N, K);
     LCU_LAUNCH_CHECK();
     return LCU_OK;
@@ -216,13 +220,18 @@ LCU_API int lcu_gemm_skinny_bf16(const void *X, int ldx, const void *W, int ldw,
     const int mt = (M + 15) / 16;
     if (epilogue == EPI_SWIGLU) {
         if (N % 2 || ldy < N / 2) return LCU_BAD_ARGUMENT;
-#define SW(MT_) return waves == 8 ? launch_swiglu<MT_, 8>(X, ldx, W, ldw, Y, ldy, M, N, K, stream) \
-                                  : launch_swiglu<MT_, 4>(X, ldx, W, ldw, Y, ldy, M, N, K, stream)
+        // tiles: gate and up tiles together (2: one of each, 4: two of each)
+#define SW(NT_, MT_) return waves == 8 ? launch_swiglu<NT_, MT_, 8>(X, ldx, W, ldw, Y, ldy, M, N, K, stream) \
+                                       : launch_swiglu<NT_, MT_, 4>(X, ldx, W, ldw, Y, ldy, M, N, K, stream)
+        if (tiles == 4 && mt <= 2) {
+            if (mt == 1) SW(4, 1);
+            SW(4, 2);
+        }
         switch (mt) {
-        case 1: SW(1);
-        case 2: SW(2);
-        case 3: SW(3);
-        default: SW(4);
+        case 1: SW(2, 1);
+        case 2: SW(2, 2);
+        case 3: SW(2, 3);
+        default: SW(2, 4);
         }
 #undef SW
     }

@@ -271,10 +271,10 @@ def gemm_nt(a: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = None
 
 def mfma_attention_supported(q: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: int, page_size: int) -> bool:
     """Whether the matrix-core attention kernels take this shape (the generic kernel takes
-    the rest): bfloat16, head_dim 64 or 128, pages of a multiple of 16 tokens, groups of
+    the rest): bfloat16, head_dim 32, 64, 96 or 128, pages of a multiple of 16 tokens, groups of
     at most 16 heads or of a multiple of 16."""
     g = n_heads // n_kv_heads
-    return (q.dtype == torch.bfloat16 and head_dim in (64, 128) and page_size % 16 == 0 and (g <= 16 or g % 16 == 0)
+    return (q.dtype == torch.bfloat16 and head_dim in (32, 64, 96, 128) and page_size % 16 == 0 and (g <= 16 or g % 16 == 0)
             and q.stride(0) % 8 == 0)
 
 
@@ -455,7 +455,7 @@ def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = 
         raise KernelError(f"gemm_skinny out: shape {tuple(out.shape)}, expected {(m, width)}")
     lib = build.load("gemm_skinny")
     _check(lib.lcu_gemm_skinny_bf16(_ptr(x), x.stride(0), _ptr(w), w.stride(0), _ptr(out), out.stride(0), m, n, k,
-                                    _EPILOGUES[epi], tiles or _skinny_tiles(width, m),
+                                    _EPILOGUES[epi], tiles or ((4 if m > 8 else 2) if swiglu else _skinny_tiles(width, m)),
                                     waves or (8 if width <= 8192 else 4), _stream()),
            "gemm_skinny")
     return out

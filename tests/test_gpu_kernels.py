@@ -262,7 +262,7 @@ def paged_case(dtype, nh, nkv, dh, page, q_lens, ctx_lens, window, seed, standou
 
 SHAPES = [  # nh, nkv, dh, page
     (4, 4, 16, 16), (4, 1, 32, 32), (6, 2, 48, 8), (8, 2, 64, 16), (32, 8, 128, 16), (6, 2, 128, 48), (32, 2, 64, 32),
-    (5, 5, 256, 16)]
+    (5, 5, 256, 16), (6, 3, 96, 16)]
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -280,7 +280,8 @@ def test_attention_mixed_batch(dtype, nh, nkv, dh, page, window):
         close(out, want, dtype, f"force_generic={force}")
 
 
-@pytest.mark.parametrize("nh,nkv,dh,page", [(8, 2, 64, 16), (32, 8, 128, 16), (16, 16, 128, 32), (32, 1, 64, 16), (6, 2, 128, 48)])
+@pytest.mark.parametrize("nh,nkv,dh,page", [(8, 2, 64, 16), (32, 8, 128, 16), (16, 16, 128, 32), (32, 1, 64, 16), (6, 2, 128, 48),
+                                            (4, 1, 32, 32), (6, 3, 96, 16)])
 @pytest.mark.parametrize("window", [0, 100])
 @pytest.mark.parametrize("splits", [None, 1, 3, 16])
 def test_attention_decode_kernel(nh, nkv, dh, page, window, splits):
@@ -296,7 +297,7 @@ def test_attention_decode_kernel(nh, nkv, dh, page, window, splits):
     close(out, want, "bfloat16")
 
 
-@pytest.mark.parametrize("nh,nkv,dh,page", [(8, 2, 64, 16), (32, 8, 128, 16), (3, 1, 128, 32), (7, 7, 64, 16)])
+@pytest.mark.parametrize("nh,nkv,dh,page", [(8, 2, 64, 16), (32, 8, 128, 16), (3, 1, 128, 32), (7, 7, 64, 16), (4, 1, 32, 32), (6, 3, 96, 16)])
 def test_attention_prefill_kernel_long(nh, nkv, dh, page):
     """Whole prompts and portions with history on the matrix cores, long enough that a
     wave walks many steps and tasks end inside a request."""
