@@ -111,6 +111,12 @@ API void lcu_sched_commit(void *h) {
 API int lcu_sched_append(void *h, long long id, int token, int is_eos) {
     return ((SchedHandle *)h)->sched.append(id, token, is_eos);
 }
+API int lcu_sched_set_token(void *h, long long id, int index, int token) {
+    return ((SchedHandle *)h)->sched.set_token(id, index, token);
+}
+API int lcu_sched_finish(void *h, long long id, int reason, int n_tokens) {
+    return ((SchedHandle *)h)->sched.finish_now(id, reason, n_tokens);
+}
 API int lcu_sched_n_waiting(void *h) { return ((SchedHandle *)h)->sched.n_waiting(); }
 API int lcu_sched_n_running(void *h) { return ((SchedHandle *)h)->sched.n_running(); }
 API long long lcu_sched_preemptions(void *h) { return ((SchedHandle *)h)->sched.total_preemptions(); }

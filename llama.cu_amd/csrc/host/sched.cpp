@@ -201,3 +201,34 @@ int Scheduler::append(int64_t id, int token, int is_eos) {
 }
 
 }  // namespace lcu
+
+namespace lcu {
+
+int Scheduler::set_token(int64_t id, int index, int token) {
+    auto it = reqs_.find(id);
+    if (it == reqs_.end()) return CACHE_UNKNOWN_REQUEST;
+    if (index < 0 || index >= (int)it->second.tokens.size()) return CACHE_BAD_ARGUMENT;
+    it->second.tokens[index] = token;
+    return CACHE_OK;
+}
+
+int Scheduler::finish_now(int64_t id, int reason, int n_tokens) {
+    auto it = reqs_.find(id);
+    if (it == reqs_.end()) return CACHE_UNKNOWN_REQUEST;
+    SchedRequest &r = it->second;
+    if (n_tokens > (int)r.tokens.size() || n_tokens == 0) return CACHE_BAD_ARGUMENT;
+    if (r.reason == FINISH_ABORTED) return r.reason;
+    if (n_tokens > 0) {
+        r.generated -= (int)r.tokens.size() - n_tokens;
+        r.tokens.resize(n_tokens);
+        if (r.computed > n_tokens - 1) {
+            r.computed = n_tokens - 1;
+            if (cache_->has(id) && cache_->get(id)->len > r.computed) cache_->truncate(id, r.computed);
+        }
+    }
+    if (r.reason == NOT_FINISHED) finish(r, reason);
+    else r.reason = reason;
+    return r.reason;
+}
+
+}  // namespace lcu

@@ -70,6 +70,14 @@ class Scheduler {
     // A sampled token for a request whose portion wanted logits; `is_eos` ends it.
     // Returns the finish reason (NOT_FINISHED = 0 if it goes on).
     int append(int64_t id, int token, int is_eos);
+    // The value of a token that was appended before it was known (the engine runs ahead of
+    // its sampler's results).
+    int set_token(int64_t id, int index, int token);
+    // End a request from outside (an end-of-sequence token learned late): its tokens are cut to
+    // n_tokens (if that is not negative) and a kept cache to what precedes the last of them, as if
+    // the request had ended when that token was appended.  A request that ended by count at the
+    // same token takes the new reason.
+    int finish_now(int64_t id, int reason, int n_tokens);
 
     const SchedRequest *get(int64_t id) const;
     int n_waiting() const { return (int)waiting_.size(); }

@@ -256,3 +256,24 @@ LCU_API int lcu_swiglu(void *out, const void *gate_up, int type, int n, int di, 
     LCU_LAUNCH_CHECK();
     return LCU_OK;
 }
+
+// ---------------------------------------------------------------- token feedback
+// tokens[dst[i]] = sampled[src[i]]: the ids that the last step sampled become this step's
+// inputs on the device, so the host need not wait for them before it launches
+// (llama.cu/src/op/fast_embedding.cuh:1-15 does the same from its sampled pairs).
+__global__ void feed_tokens_kernel(int *__restrict__ tokens, const int *__restrict__ sampled,
+                                   const int *__restrict__ src, const int *__restrict__ dst, int n, int n_tokens,
+                                   int n_sampled) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const int s = src[i], d = dst[i];
+    if (s >= 0 && s < n_sampled && d >= 0 && d < n_tokens) tokens[d] = sampled[s];
+}
+
+LCU_API int lcu_feed_tokens(int *tokens, int n_tokens, const int *sampled, int n_sampled, const int *src, const int *dst,
+                            int n, hipStream_t stream) {
+    if (n <= 0) return LCU_OK;
+    feed_tokens_kernel<<<dim3((n + 255) / 256), dim3(256), 0, stream>>>(tokens, sampled, src, dst, n, n_tokens, n_sampled);
+    LCU_LAUNCH_CHECK();
+    return LCU_OK;
+}

@@ -46,6 +46,10 @@ class StepContext:
     state_slots: List[int] = field(default_factory=list)    # ``state_slot`` on the host
     attn_splits: Optional[int] = None           # fixed number of key parts for the decode kernel (captured graphs)
     scratch: dict = field(default_factory=dict)  # what kernels' wrappers derive from the batch once per step
+    # tokens that the step before sampled and the host does not know yet: tokens[feed_dst[i]] is
+    # to be taken from row feed_src[i] of that step's sampled ids, on the device
+    feed_src: Optional[torch.Tensor] = None
+    feed_dst: Optional[torch.Tensor] = None
 
     def block_table(self, group: int) -> torch.Tensor:
         return self.block_tables[group]
@@ -79,7 +83,7 @@ class BatchBuilder:
         self.device = device
         n, r = self.max_tokens, self.max_reqs
         sizes = [("tokens", n), ("positions", n), ("req_of_token", n), ("logit_rows", n),
-                 ("q_start", r + 1), ("ctx_len", r), ("state_slot", r)]
+                 ("q_start", r + 1), ("ctx_len", r), ("state_slot", r), ("feed_src", r), ("feed_dst", r)]
         for g, mp in enumerate(self.max_pages):
             sizes += [(f"slots{g}", n), (f"block_table{g}", r * mp)]
         self.offsets = {}
@@ -101,9 +105,11 @@ class BatchBuilder:
         return self.dev[o:o + count]
 
     def build(self, req_ids: Sequence[int], tokens: Sequence[Sequence[int]], want: Sequence[Sequence[int]],
-              vocab_size: int) -> StepContext:
+              vocab_size: int, feed: Sequence[tuple] = ()) -> StepContext:
         """The batch in which request ``req_ids[i]`` feeds ``tokens[i]`` and wants the logits
-        at the places ``want[i]`` among them.  The requests' pages must be reserved."""
+        at the places ``want[i]`` among them.  The requests' pages must be reserved.
+        ``feed``: pairs (row of the last step's sampled ids, request index here) for requests
+        whose last token here is a placeholder that the device fills in."""
         n_req = len(req_ids)
         n_new = [len(t) for t in tokens]
         n = sum(n_new)
@@ -129,6 +135,15 @@ class BatchBuilder:
             start += n_new[i]
         if rows:
             self._h("logit_rows")[:len(rows)] = torch.tensor(rows, dtype=torch.int32)
+        if feed:
+            if len(feed) > self.max_reqs:
+                raise ValueError(f"{len(feed)} fed tokens exceed the builder's capacity of {self.max_reqs}")
+            ends, at = [], 0
+            for c in n_new:
+                at += c
+                ends.append(at - 1)
+            self._h("feed_src")[:len(feed)] = torch.tensor([f[0] for f in feed], dtype=torch.int32)
+            self._h("feed_dst")[:len(feed)] = torch.tensor([ends[f[1]] for f in feed], dtype=torch.int32)
         ptr = lambda name: self._h(name).data_ptr()
         self.cache.fill_batch(req_ids, n_new, ptr("positions"), ptr("req_of_token"), ptr("q_start"), ptr("ctx_len"),
                               ptr("state_slot"), [ptr(f"block_table{g}") for g in range(len(self.max_pages))],
@@ -146,4 +161,6 @@ class BatchBuilder:
             block_tables=[self._d(f"block_table{g}", n_req * mp).view(n_req, mp) for g, mp in enumerate(self.max_pages)],
             slot_maps=[self._d(f"slots{g}", n) for g in range(len(self.max_pages))],
             q_lens=n_new, ctx_lens=ctx_lens, req_ids=list(req_ids),
-            state_slots=self._h("state_slot")[:n_req].tolist())
+            state_slots=self._h("state_slot")[:n_req].tolist(),
+            feed_src=self._d("feed_src", len(feed)) if feed else None,
+            feed_dst=self._d("feed_dst", len(feed)) if feed else None)

@@ -3,8 +3,13 @@ through the runner's step function, sample where a request's known tokens end, h
 the tokens back to the scheduler, report what finished.
 
 The reference's loop (llama.cu/src/exec/engine.rs:217-295) runs ahead of its caller and
-learns of an end-of-sequence token a round or two late (llama.cu/src/lib.rs:175-184); this
-one samples and checks for the end before it plans the next round.
+learns of an end-of-sequence token a round or two late (llama.cu/src/lib.rs:175-184).  So
+does this one by default (``run_ahead``): a round's sampled ids stay on the device, the next
+round is planned with placeholders for them and takes them from there
+(llama.cu/src/op/fast_embedding.cuh:1-15), and the host reads a round's ids while the next
+one runs, so the GPU does not wait for the host between rounds.  What a request computed
+beyond an end-of-sequence token that was learned late is cut away again.  With
+``run_ahead=False`` every round is sampled and read before the next is planned.
 """
 from __future__ import annotations
 
@@ -14,6 +19,7 @@ from typing import Callable, Dict, List, Optional, Sequence, Tuple, Union
 
 import torch
 
+from ..kernels import ops
 from ..sampling import GREEDY, Sampler, SamplingParams
 from .runner import ModelRunner
 from .scheduler import PlanEntry, Scheduler
@@ -32,11 +38,31 @@ class _Request:
     params: SamplingParams
     prompt_len: int
     ignore_eos: bool = False
+    unknown: Optional[int] = None     # index of a token that is sampled but not read yet
+    done: bool = False                # its end has been reported (or it was aborted)
+    turn: int = 0                     # counts continuations: a row of an earlier turn is stale
+
+
+@dataclass
+class _Flight:
+    """A launched round whose sampled ids the host has not read."""
+    rows: List[int]                   # the request of each sampled row
+    index: List[int]                  # where the id goes in that request's tokens
+    reasons: List[Optional[str]]      # an end by count, known at launch
+    turns: List[int]                  # the request's turn at launch
+    owners: List["_Request"]          # and the request itself (an id may come again after a drop)
+    sampled: torch.Tensor             # the ids on the device
+    host: torch.Tensor                # and where the copy to the host lands
+    copied: torch.cuda.Event
 
 
 class Engine:
-    def __init__(self, runner: ModelRunner, prefill_chunk: Optional[int] = None, eos_token_ids: Sequence[int] = ()):
+    def __init__(self, runner: ModelRunner, prefill_chunk: Optional[int] = None, eos_token_ids: Sequence[int] = (),
+                 run_ahead: bool = True):
         self.runner = runner
+        self.run_ahead = bool(run_ahead)
+        self._flight: Optional[_Flight] = None
+        self._awaiting: set = set()    # ended by count at launch, token not read yet
         self.sched = Scheduler(runner.cache, runner.max_seqs, runner.max_batch_tokens,
                                prefill_chunk or runner.max_batch_tokens, runner.max_model_len)
         self.sampler = Sampler()
@@ -47,13 +73,15 @@ class Engine:
 
     @classmethod
     def from_folder(cls, folder: str, dtype: str = "bfloat16", device: str = "cuda:0",
-                    prefill_chunk: Optional[int] = None, **runner_kw) -> "Engine":
-        return cls(ModelRunner.from_folder(folder, dtype=dtype, device=device, **runner_kw), prefill_chunk)
+                    prefill_chunk: Optional[int] = None, run_ahead: bool = True, **runner_kw) -> "Engine":
+        return cls(ModelRunner.from_folder(folder, dtype=dtype, device=device, **runner_kw), prefill_chunk,
+                   run_ahead=run_ahead)
 
     @classmethod
     def from_config(cls, cfg, seed: int, dtype: str = "bfloat16", device: str = "cuda:0",
-                    prefill_chunk: Optional[int] = None, **runner_kw) -> "Engine":
-        return cls(ModelRunner.from_config(cfg, seed, dtype=dtype, device=device, **runner_kw), prefill_chunk)
+                    prefill_chunk: Optional[int] = None, run_ahead: bool = True, **runner_kw) -> "Engine":
+        return cls(ModelRunner.from_config(cfg, seed, dtype=dtype, device=device, **runner_kw), prefill_chunk,
+                   run_ahead=run_ahead)
 
     # ---------------------------------------------------------------- requests
     def add_request(self, tokens: Sequence[int], params: SamplingParams = GREEDY, max_steps: int = 1000,
@@ -81,21 +109,118 @@ class Engine:
         r = self.requests[rid]
         r.tokens.extend(tokens)
         r.prompt_len = len(r.tokens)
+        r.done = False
+        r.turn += 1
 
     def abort(self, rid: int) -> None:
         self.sched.abort(rid)
+        r = self.requests.get(rid)
+        if r is not None:
+            r.done = True
+        self._awaiting.discard(rid)
 
     def drop(self, rid: int) -> None:
         """Forget a finished request and give back a cache it kept."""
         self.sched.drop(rid)
         self.requests.pop(rid, None)
+        self._awaiting.discard(rid)
 
     @property
     def idle(self) -> bool:
-        return self.sched.idle
+        return self.sched.idle and self._flight is None
 
     # ---------------------------------------------------------------- one round
     def step(self) -> List[StepOutput]:
+        """Run one round; returns the tokens that became known and the requests that ended.
+        Running ahead, these are the tokens of the round before the one launched here."""
+        if not self.run_ahead:
+            return self._step_in_turn()
+        launched = self._launch()
+        outputs = self._collect(self._flight) if self._flight is not None else []
+        self._flight = launched
+        reported = {o.req for o in outputs if o.finished}
+        for rid in self.sched.take_finished():
+            if rid not in reported and rid not in self._awaiting:
+                outputs.append(StepOutput(rid, None, self.sched.info(rid).reason))
+        return outputs
+
+    def _launch(self) -> Optional[_Flight]:
+        """Plan and launch a round; the ids it samples stay on the device, and the requests
+        get placeholders for them."""
+        plan = self.sched.plan()
+        if not plan:
+            return None
+        before = self._flight
+        row_of = {rid: i for i, rid in enumerate(before.rows)} if before is not None else {}
+        ids, toks, want, feed = [], [], [], []
+        for j, e in enumerate(plan):
+            r = self.requests[e.req]
+            have = self.runner.cache.length(e.req)
+            if have != e.start:
+                raise RuntimeError(f"request {e.req}: the cache holds {have} tokens, the plan starts at {e.start}")
+            last = e.start + e.count - 1
+            if r.unknown is not None and e.start <= r.unknown <= last:
+                if r.unknown != last or e.req not in row_of:
+                    raise RuntimeError(f"request {e.req}: token {r.unknown} is not known and the round before does not give it")
+                feed.append((row_of[e.req], j))
+            ids.append(e.req)
+            toks.append(r.tokens[e.start:e.start + e.count])
+            want.append([e.count - 1] if e.want_logits else [])
+        step = self.runner.prepare(ids, toks, want, feed)
+        if feed:
+            ops.feed_tokens(step.tokens, before.sampled, step.feed_src, step.feed_dst)
+        logits = self.runner.run(step)
+        self.sched.commit()
+        self.steps += 1
+        rows = [e for e in plan if e.want_logits]
+        if not rows:
+            return None
+        params = [self.requests[e.req].params for e in rows]
+        keys = [(e.req, len(self.requests[e.req].tokens)) for e in rows]
+        sampled = self.sampler.sample_device(logits, params, keys)
+        host = torch.empty(len(rows), dtype=torch.int32, pin_memory=True)
+        host.copy_(sampled, non_blocking=True)
+        copied = torch.cuda.Event()
+        copied.record()
+        flight = _Flight([e.req for e in rows], [], [], [], [], sampled, host, copied)
+        for e in rows:
+            r = self.requests[e.req]
+            r.unknown = len(r.tokens)
+            flight.index.append(r.unknown)
+            flight.turns.append(r.turn)
+            flight.owners.append(r)
+            r.tokens.append(0)
+            reason = self.sched.append(e.req, 0, False)
+            flight.reasons.append(reason)
+            if reason:
+                self._awaiting.add(e.req)
+        return flight
+
+    def _collect(self, flight: _Flight) -> List[StepOutput]:
+        """Read a round's ids, put them where the placeholders stand, and end the requests that
+        an end-of-sequence token ends."""
+        flight.copied.synchronize()
+        outputs: List[StepOutput] = []
+        for rid, index, reason, turn, owner, tok in zip(flight.rows, flight.index, flight.reasons, flight.turns,
+                                                        flight.owners, flight.host.tolist()):
+            r = self.requests.get(rid)
+            if r is not owner or r.done or r.turn != turn:
+                continue                                    # ended earlier; this row ran for nothing
+            r.tokens[index] = tok
+            if r.unknown == index:
+                r.unknown = None
+            self.sched.set_token(rid, index, tok)
+            if tok in self.eos and not r.ignore_eos:
+                reason = self.sched.finish(rid, "eos", index + 1)
+                del r.tokens[index + 1:]
+                r.unknown = None
+            if reason:
+                r.done = True
+                self._awaiting.discard(rid)
+            outputs.append(StepOutput(rid, tok, reason))
+        return outputs
+
+    def _step_in_turn(self) -> List[StepOutput]:
         plan = self.sched.plan()
         outputs: List[StepOutput] = []
         if plan:

@@ -129,7 +129,8 @@ class ModelRunner:
         return runner
 
     # ------------------------------------------------------------ the step function
-    def prepare(self, req_ids: Sequence[int], tokens: Sequence[Sequence[int]], want: Sequence[Sequence[int]]) -> StepContext:
+    def prepare(self, req_ids: Sequence[int], tokens: Sequence[Sequence[int]], want: Sequence[Sequence[int]],
+                feed: Sequence[tuple] = ()) -> StepContext:
         """Give the requests their pages (new requests get a slot) and build the batch."""
         added = []
         reserved = []
@@ -152,7 +153,7 @@ class ModelRunner:
             for rid in added:
                 self.cache.release(rid)
             raise
-        return self.builder.build(req_ids, tokens, want, self.spec.vocab_size)
+        return self.builder.build(req_ids, tokens, want, self.spec.vocab_size, feed)
 
     GRAPH_AFTER = 2          # a batch size is captured when it comes for the third time
     GRAPH_MAX_BATCH = 256

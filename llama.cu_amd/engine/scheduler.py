@@ -84,6 +84,20 @@ class Scheduler:
             self._st(r, f"append to request {req}")
         return REASONS[r]
 
+    def set_token(self, req: int, index: int, token: int) -> None:
+        """The value of a token that was appended before it was known."""
+        self._st(self._lib.lcu_sched_set_token(self._h, ctypes.c_longlong(req), int(index), int(token)),
+                 f"set token {index} of request {req}")
+
+    def finish(self, req: int, reason: str, n_tokens: int = -1):
+        """End a request from outside, its tokens cut to ``n_tokens`` (an end of sequence
+        learned after more was appended); returns the reason it now has."""
+        code = {v: k for k, v in REASONS.items()}[reason]
+        r = self._lib.lcu_sched_finish(self._h, ctypes.c_longlong(req), code, int(n_tokens))
+        if r < 0:
+            self._st(r, f"finish request {req}")
+        return REASONS[r]
+
     def take_finished(self) -> List[int]:
         buf = (ctypes.c_longlong * 1024)()
         n = self._lib.lcu_sched_take_finished(self._h, buf, 1024)

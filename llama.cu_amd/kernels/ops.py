@@ -165,6 +165,15 @@ def swiglu(gate_up: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.T
     return out
 
 
+def feed_tokens(tokens: torch.Tensor, sampled: torch.Tensor, src: torch.Tensor, dst: torch.Tensor) -> None:
+    """``tokens[dst[i]] = sampled[src[i]]`` on the device."""
+    _gpu(tokens, sampled, src, dst)
+    _i32(tokens, "tokens"); _i32(sampled, "sampled"); _i32(src, "src"); _i32(dst, "dst", src.numel())
+    lib = build.load("elementwise")
+    _check(lib.lcu_feed_tokens(_ptr(tokens), tokens.numel(), _ptr(sampled), sampled.numel(), _ptr(src), _ptr(dst),
+                               src.numel(), _stream()), "feed_tokens")
+
+
 # ------------------------------------------------------------------ rotation and cache write
 
 

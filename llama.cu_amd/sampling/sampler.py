@@ -68,6 +68,20 @@ def sample_rows(logits: torch.Tensor, temperature: Sequence[float], top_p: Seque
 
 
 class Sampler:
+    def sample_device(self, logits: torch.Tensor, params: Sequence[SamplingParams],
+                      keys: Sequence[Tuple[int, int]]) -> torch.Tensor:
+        """A token for every row, left on the device (int32)."""
+        out = argmax(logits)
+        random_rows = [i for i, p in enumerate(params) if not p.is_argmax]
+        if random_rows:
+            idx = torch.tensor(random_rows, dtype=torch.long).to(logits.device)
+            sub = logits if len(random_rows) == logits.shape[0] else logits[idx]
+            drawn = sample_rows(sub, [params[i].temperature for i in random_rows], [params[i].top_p for i in random_rows],
+                                [params[i].top_k for i in random_rows],
+                                [uniform(params[i].seed, keys[i][0], keys[i][1]) for i in random_rows])
+            out[idx] = drawn
+        return out
+
     def sample(self, logits: torch.Tensor, params: Sequence[SamplingParams],
                keys: Sequence[Tuple[int, int]]) -> List[int]:
         """A token for every row.  ``keys[i] = (request id, index of the drawn token)``."""

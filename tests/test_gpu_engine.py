@@ -159,3 +159,81 @@ def test_captured_decode_steps_equal_eager_ones():
     assert 3 in runner._graphs                              # the batch size was captured and replayed
     for i, (a, b) in enumerate(zip(eager, graphed)):
         assert torch.equal(a, b), f"decode step {i} differs between eager and captured"
+
+
+def _run(engine, prompts, params=None, max_steps=20, ignore_eos=False, keep=False):
+    """Tokens and finish reasons per request, through ``step()`` until idle."""
+    from llama_cu_amd.sampling import GREEDY
+    ids = [engine.add_request(p, params or GREEDY, max_steps, keep=keep, ignore_eos=ignore_eos) for p in prompts]
+    toks = {i: [] for i in ids}
+    why = {}
+    while not engine.idle:
+        for o in engine.step():
+            if o.token is not None:
+                toks[o.req].append(o.token)
+            if o.finished:
+                assert o.req not in why, "a request's end is reported once"
+                why[o.req] = o.finished
+    return ids, [toks[i] for i in ids], [why.get(i) for i in ids]
+
+
+def test_running_ahead_changes_no_token_and_no_reason(folder_b):
+    """The engine that launches a round before it has read the round before gives the
+    tokens and finish reasons of the engine that works in turn: greedy and seeded, with
+    portions, and with an end-of-sequence token that is learned a round late (what was
+    computed beyond it is cut away; every page comes back)."""
+    from llama_cu_amd.engine.engine import Engine
+    from llama_cu_amd.sampling import SamplingParams
+    prompts = list(common.random_requests(384, [3, 40, 77, 21], seed=5).values())
+    kw = dict(dtype="float32", max_tokens=1024, max_seqs=4, max_batch_tokens=64, prefill_chunk=32)
+    for params in (None, SamplingParams(temperature=0.9, top_p=0.95, top_k=50, seed=7)):
+        in_turn = Engine.from_folder(folder_b, run_ahead=False, **kw)
+        _, want, why = _run(in_turn, prompts, params, max_steps=20, ignore_eos=True)
+        assert why == ["max_steps"] * 4
+        ahead = Engine.from_folder(folder_b, run_ahead=True, **kw)
+        _, got, why2 = _run(ahead, prompts, params, max_steps=20, ignore_eos=True)
+        assert got == want and why2 == why
+        # tokens that the requests generate at different steps become end-of-sequence tokens
+        eos = {want[0][4], want[1][9], want[2][0]}
+        a = Engine.from_folder(folder_b, run_ahead=False, **kw); a.eos = set(eos)
+        b = Engine.from_folder(folder_b, run_ahead=True, **kw); b.eos = set(eos)
+        _, ta, wa = _run(a, prompts, params, max_steps=20)
+        _, tb, wb = _run(b, prompts, params, max_steps=20)
+        assert "eos" in wa and tb == ta and wb == wa
+        for e in (a, b):
+            e.runner.cache.check()
+            assert e.runner.cache.free_pages(0) == e.runner.num_pages
+
+
+def test_a_kept_request_goes_on_after_a_late_end_of_sequence(folder_b):
+    """Chat turns: a request that keeps its cache ends with an end-of-sequence token (learned
+    late when running ahead) and goes on with more tokens; both engines give the same."""
+    from llama_cu_amd.engine.engine import Engine
+    prompt = list(common.random_requests(384, [25], seed=6).values())[0]
+    kw = dict(dtype="float32", max_tokens=512, max_seqs=2)
+    probe = Engine.from_folder(folder_b, run_ahead=False, **kw)
+    _, first, _ = _run(probe, [prompt], max_steps=12, ignore_eos=True)
+    outs = []
+    for ahead in (False, True):
+        e = Engine.from_folder(folder_b, run_ahead=ahead, **kw)
+        e.eos = {first[0][6]}
+        ids, t1, w1 = _run(e, [prompt], max_steps=12, keep=True)
+        assert w1 == ["eos"] and t1[0] == first[0][:first[0].index(first[0][6]) + 1]
+        assert e.runner.cache.length(ids[0]) == len(prompt) + len(t1[0]) - 1
+        e.continue_request(ids[0], [11, 12, 13], max_steps=8)
+        t2, w2 = [], None
+        while not e.idle:
+            for o in e.step():
+                if o.token is not None:
+                    t2.append(o.token)
+                w2 = o.finished or w2
+        outs.append((t1, t2, w2))
+        e.drop(ids[0])
+        e.runner.cache.check()
+        assert e.runner.cache.free_pages(0) == e.runner.num_pages
+    assert outs[0] == outs[1]
+    # and the continuation is what the plain implementation generates from the whole context
+    cfg, w = plain.load_folder(folder_b)
+    t1, t2, _ = outs[0]
+    whole = plain.greedy_generate(cfg, w, prompt + t1[0] + [11, 12, 13], len(t2))
+    assert t2 == whole[:len(t2)]

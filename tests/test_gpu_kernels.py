@@ -391,3 +391,22 @@ def test_gemm_skinny_f32_is_true_32_bit_and_rows_are_independent():
     for r in (0, 15, 16, 63, 64, 149):                                        # alone, in a batch of few, in any tile of 64
         assert torch.equal(whole[r:r + 1], ops.gemm_skinny_f32(x[r:r + 1], w))
     assert torch.equal(whole[60:70], ops.gemm_skinny_f32(x[60:70], w))
+
+
+def test_feed_tokens():
+    """tokens[dst[i]] = sampled[src[i]]; pairs outside either array are left out."""
+    from llama_cu_amd.kernels import ops
+    g = torch.Generator().manual_seed(0)
+    tokens = torch.randint(0, 1000, (37,), generator=g, dtype=torch.int32)
+    sampled = torch.randint(0, 1000, (9,), generator=g, dtype=torch.int32)
+    src = torch.tensor([8, 0, 3, 5], dtype=torch.int32)
+    dst = torch.tensor([36, 1, 20, 7], dtype=torch.int32)
+    want = tokens.clone()
+    want[dst.long()] = sampled[src.long()]
+    got = tokens.cuda()
+    ops.feed_tokens(got, sampled.cuda(), src.cuda(), dst.cuda())
+    assert torch.equal(got.cpu(), want)
+    got2 = tokens.cuda()
+    ops.feed_tokens(got2, sampled.cuda(), torch.tensor([9, -1, 2], dtype=torch.int32).cuda(),
+                    torch.tensor([0, 1, 37], dtype=torch.int32).cuda())
+    assert torch.equal(got2.cpu(), tokens)
