@@ -210,3 +210,53 @@ def test_random_load_every_request_ends_and_nothing_is_lost(seed):
             assert info.reason == "length"
             assert info.n_tokens >= 96 or (n + 15) // 16 + 0 >= 0
     assert cache.live_requests() == 0
+
+
+def test_a_token_appended_before_it_is_known_gets_its_value_later():
+    cache, s = make()
+    s.add(0, [1, 2, 3], 4)
+    run_round(s, next_token=lambda req, n: 0)            # a placeholder stands for the sampled token
+    assert s.tokens(0) == [1, 2, 3, 0]
+    s.set_token(0, 3, 77)
+    assert s.tokens(0) == [1, 2, 3, 77]
+    with pytest.raises(Exception):
+        s.set_token(0, 4, 5)
+    with pytest.raises(Exception):
+        s.set_token(9, 0, 5)
+
+
+def test_an_end_learned_late_cuts_what_was_appended_and_computed_beyond_it():
+    """Two rounds ran with placeholders; the first round's token turns out to end the sequence.
+    The tokens are cut after it, a kept cache to what precedes it, and the pages beyond come back."""
+    cache, s = make(page=4, pages=16)
+    s.add(0, list(range(7)), 10, keep=True)
+    run_round(s, next_token=lambda req, n: 0)            # prompt, first placeholder (index 7)
+    run_round(s, next_token=lambda req, n: 0)            # computes index 7, second placeholder (index 8)
+    run_round(s, next_token=lambda req, n: 0)            # computes index 8 (a third page), third placeholder
+    assert s.info(0).n_tokens == 10 and cache.length(0) == 9
+    assert s.finish(0, "eos", 8) == "eos"
+    info = s.info(0)
+    assert (info.n_tokens, info.generated, info.reason) == (8, 1, "eos")
+    assert cache.length(0) == 7                            # the end-of-sequence token itself is not in the cache
+    assert s.take_finished() == [0]
+    assert s.plan() == []
+    cache.check()
+    # it goes on from there
+    s.extend(0, [5, 6], 3)
+    plan = s.plan()
+    assert [(e.req, e.start, e.count) for e in plan] == [(0, 7, 3)]
+    s.commit()
+    s.abort(0)
+    s.drop(0)
+    cache.check()
+    assert cache.free_pages(0) == 16
+
+
+def test_an_end_by_count_at_the_same_token_takes_the_late_reason():
+    cache, s = make()
+    s.add(0, [1, 2, 3], 1)
+    _, done = run_round(s, next_token=lambda req, n: 0)
+    assert done == {0: "max_steps"}
+    assert s.finish(0, "eos", 4) == "eos" and s.info(0).reason == "eos"
+    cache.check()
+    assert cache.free_pages(0) == 64
