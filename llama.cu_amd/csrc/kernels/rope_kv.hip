@@ -11,6 +11,16 @@
 
 // One block per (token, head): query heads are rotated in place, key heads are rotated into
 // the cache, value heads are copied into the cache.
+// One rotation, rounded the same way in every kernel of this file: one product rounded, the
+// other fused into the sum, written out so that the compiler has no choice of its own.  A
+// token's rotated values then do not depend on which kernel its batch was given to.
+__device__ inline void rotate_pair(float a, float b, float c, float s, float &ra, float &rb) {
+#pragma clang fp contract(off)
+    const float bs = b * s, bc = b * c;
+    ra = __builtin_fmaf(a, c, -bs);
+    rb = __builtin_fmaf(a, s, bc);
+}
+
 template <class T>
 __global__ void rope_kv_store_kernel(T *__restrict__ qkv, int row_stride, const int *__restrict__ positions,
                                      const int *__restrict__ slots, const float *__restrict__ cos_t,
@@ -52,7 +62,8 @@ __global__ void rope_kv_store_kernel(T *__restrict__ qkv, int row_stride, const 
         float a = to_f32(x[ia]), b = to_f32(x[ib]);
         if (rot) {
             const float c = cos_t[(size_t)pos * half + i], s = sin_t[(size_t)pos * half + i];
-            const float ra = a * c - b * s, rb = a * s + b * c;
+            float ra, rb;
+            rotate_pair(a, b, c, s, ra, rb);
             a = ra; b = rb;
         }
         if (poison && i < half) a = b = __uint_as_float(0x7fc00000u);
@@ -106,8 +117,10 @@ rope_kv_store_half_kernel(T *__restrict__ qkv, int row_stride, const int *__rest
                 const float fa = to_f32(a.v[e]), fb = to_f32(b.v[e]);
                 float c = __uint_as_float(0x7fc00000u), s = c;      // a position outside the table gives NaN
                 if (in_table) { c = cos_t[(size_t)pos * half + i0 + e]; s = sin_t[(size_t)pos * half + i0 + e]; }
-                ra.v[e] = from_f32<T>(fa * c - fb * s);
-                rb.v[e] = from_f32<T>(fa * s + fb * c);
+                float xa, xb;
+                rotate_pair(fa, fb, c, s, xa, xb);
+                ra.v[e] = from_f32<T>(xa);
+                rb.v[e] = from_f32<T>(xb);
             }
             if (head < nh) {
                 *(Row8<T> *)(x + i0) = ra;
@@ -122,6 +135,90 @@ rope_kv_store_half_kernel(T *__restrict__ qkv, int row_stride, const int *__rest
             const Row8<T> val = *(const Row8<T> *)(row + (size_t)(nh + nkvh) * dh + (size_t)kvh * dh + c0);
 #pragma unroll
             for (int e = 0; e < 8; ++e) pg[kv_value_offset(nkvh, kvh, tok, c0 + e, dh, page)] = val.v[e];
+        }
+    }
+}
+
+// The same for many tokens: a block takes eight neighbouring tokens of the batch, so that the
+// values of one dim, which lie along the tokens in a page, leave as one 16- or 32-byte store
+// when the eight tokens stand in a row in one page (a prompt's portion that starts at a
+// multiple of eight); otherwise element by element.
+template <class T>
+__global__ void __launch_bounds__(256)
+rope_kv_store_half_tokens8_kernel(T *__restrict__ qkv, int row_stride, int n, const int *__restrict__ positions,
+                                  const int *__restrict__ slots, const float *__restrict__ cos_t,
+                                  const float *__restrict__ sin_t, int max_pos, T *__restrict__ cache, int nh, int nkvh,
+                                  int dh, int page) {
+    const int t0 = blockIdx.x * 8;
+    const int nt = min(8, n - t0);
+    const int half = dh / 2;
+    const int per_head = half / 8;
+    const int n_rot = (nh + nkvh) * per_head;               // per token
+    const int n_val = nkvh * dh;                            // per group of eight tokens
+    const int w = blockIdx.y * blockDim.x + threadIdx.x;
+    if (w < 8 * n_rot) {
+        const int e_t = w / n_rot, item = w % n_rot;
+        if (e_t >= nt) return;
+        const int t = t0 + e_t;
+        T *row = qkv + (size_t)t * row_stride;
+        const int pos = positions[t];
+        const bool in_table = pos >= 0 && pos < max_pos;
+        const int head = item / per_head, i0 = (item % per_head) * 8;
+        T *x = row + (size_t)head * dh;
+        const Row8<T> a = *(const Row8<T> *)(x + i0), b = *(const Row8<T> *)(x + half + i0);
+        float c[8], sn[8];
+        if (in_table) {
+            const float4 *cp = (const float4 *)(cos_t + (size_t)pos * half + i0), *sp = (const float4 *)(sin_t + (size_t)pos * half + i0);
+            const float4 c0 = cp[0], c1 = cp[1], s0 = sp[0], s1 = sp[1];
+            c[0] = c0.x; c[1] = c0.y; c[2] = c0.z; c[3] = c0.w; c[4] = c1.x; c[5] = c1.y; c[6] = c1.z; c[7] = c1.w;
+            sn[0] = s0.x; sn[1] = s0.y; sn[2] = s0.z; sn[3] = s0.w; sn[4] = s1.x; sn[5] = s1.y; sn[6] = s1.z; sn[7] = s1.w;
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) c[e] = sn[e] = __uint_as_float(0x7fc00000u);   // a position outside the table gives NaN
+        }
+        Row8<T> ra, rb;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const float fa = to_f32(a.v[e]), fb = to_f32(b.v[e]);
+            float xa, xb;
+            rotate_pair(fa, fb, c[e], sn[e], xa, xb);
+            ra.v[e] = from_f32<T>(xa);
+            rb.v[e] = from_f32<T>(xb);
+        }
+        if (head < nh) {
+            *(Row8<T> *)(x + i0) = ra;
+            *(Row8<T> *)(x + half + i0) = rb;
+        } else {
+            const int slot = slots[t];
+            if (slot >= 0) {
+                T *pg = cache + (size_t)(slot / page) * kv_page_elems(nkvh, dh, page);
+                const int kvh = head - nh, tok = slot % page;
+                *(Row8<T> *)(pg + kv_key_offset(kvh, tok, i0, dh, page)) = ra;
+                *(Row8<T> *)(pg + kv_key_offset(kvh, tok, half + i0, dh, page)) = rb;
+            }
+        }
+        return;
+    }
+    const int v = w - 8 * n_rot;
+    if (v >= n_val) return;
+    const int kvh = v / dh, dim = v % dh;
+    const T *src = qkv + (size_t)t0 * row_stride + (size_t)(nh + nkvh) * dh + (size_t)kvh * dh + dim;
+    const int slot0 = slots[t0];
+    bool row8 = nt == 8 && slot0 >= 0 && slot0 % 8 == 0;     // page sizes are multiples of 8: such a run stays in its page
+#pragma unroll
+    for (int e = 1; e < 8; ++e) row8 = row8 && (e >= nt || slots[t0 + e] == slot0 + e);
+    if (row8) {
+        Row8<T> val;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) val.v[e] = src[(size_t)e * row_stride];
+        T *pg = cache + (size_t)(slot0 / page) * kv_page_elems(nkvh, dh, page);
+        *(Row8<T> *)(pg + kv_value_offset(nkvh, kvh, slot0 % page, dim, dh, page)) = val;
+    } else {
+        for (int e = 0; e < nt; ++e) {
+            const int slot = slots[t0 + e];
+            if (slot < 0) continue;
+            T *pg = cache + (size_t)(slot / page) * kv_page_elems(nkvh, dh, page);
+            pg[kv_value_offset(nkvh, kvh, slot % page, dim, dh, page)] = src[(size_t)e * row_stride];
         }
     }
 }
@@ -142,6 +239,16 @@ LCU_API int lcu_rope_kv_store(void *qkv, int type, int n, int row_stride, const 
     const int elem = type == LCU_F32 ? 4 : 2;
     if (cos_t && pairing == 0 && rot_dim == dh && dh % 16 == 0 && (row_stride * elem) % (8 * elem) == 0 &&
         ((size_t)qkv % (8 * elem)) == 0 && (type == LCU_F32 || type == LCU_BF16)) {
+        if (store_kv && n >= 64 && (size_t)cos_t % 16 == 0 && (size_t)sin_t % 16 == 0) {
+            const int items8 = 8 * (nh + nkvh) * (dh / 16) + nkvh * dh;
+            const dim3 g8((n + 7) / 8, (items8 + 255) / 256);
+            if (type == LCU_F32)
+                rope_kv_store_half_tokens8_kernel<float><<<g8, dim3(256), 0, stream>>>((float *)qkv, row_stride, n, positions, slots, cos_t, sin_t, max_pos, (float *)cache, nh, nkvh, dh, page);
+            else
+                rope_kv_store_half_tokens8_kernel<bf16_t><<<g8, dim3(256), 0, stream>>>((bf16_t *)qkv, row_stride, n, positions, slots, cos_t, sin_t, max_pos, (bf16_t *)cache, nh, nkvh, dh, page);
+            LCU_LAUNCH_CHECK();
+            return LCU_OK;
+        }
         const int items = (nh + (store_kv ? nkvh : 0)) * (dh / 16) + (store_kv ? nkvh * dh / 8 : 0);
         const dim3 hgrid(n, (items + 255) / 256);
         if (type == LCU_F32)

@@ -169,6 +169,71 @@ def test_rope_and_cache_write(dtype, nh, nkv, dh, page, pairing):
     assert torch.equal(flat == 7.0, expect == 7.0)                        # nothing else was touched
 
 
+@pytest.mark.parametrize("dtype,nh,nkv,dh,page", [("bfloat16", 4, 2, 128, 16), ("float32", 3, 1, 32, 32),
+                                                   ("bfloat16", 2, 2, 16, 8)])
+def test_rope_and_cache_write_many_tokens(dtype, nh, nkv, dh, page):
+    """The kernel for many tokens takes eight tokens a block: runs of places in a page that
+    start at a multiple of eight, runs that do not, places in no order, tokens that store
+    nothing, and a last block that is not full."""
+    from llama_cu_amd.kernels import ops
+    from llama_cu_amd.parts.position import Rotary
+    max_pos, pages, theta = 400, 40, 10000.0
+    rot = Rotary(dh, theta, max_pos)
+    cos, sin = rot.host_tables()
+    sin_p, cos_p = plain.rope_tables(max_pos, dh, theta)
+    rng = random.Random(5)
+    free = list(range(pages))
+    rng.shuffle(free)
+    slots, pos = [], []
+
+    def run(start_place, length, first_pos):
+        """A request's portion: consecutive positions, places that go on through its pages."""
+        place = start_place
+        pg = free.pop()
+        for i in range(length):
+            if place == page:
+                pg, place = free.pop(), 0
+            slots.append(pg * page + place)
+            pos.append(first_pos + i)
+            place += 1
+
+    run(0, 5 * page // 2 + 8, 0)            # starts a page: rows of eight all along (batch offset 0)
+    run(3, 29, 100)                         # starts in the middle of a page: no row of eight fits
+    n_run = len(slots)
+    rest = [pg * page + k for pg in free[:3] for k in range(page)]
+    rng.shuffle(rest)
+    extra = 64 + 13
+    slots += rest[:extra] if len(rest) >= extra else (rest + [-1] * (extra - len(rest)))
+    pos += [rng.randrange(max_pos) for _ in range(len(slots) - n_run)]
+    for i in (2, n_run + 5):
+        slots[i] = -1
+    n = len(slots)
+    assert n >= 64 and n % 8 != 0
+    qkv = rnd(n, (nh + 2 * nkv) * dh, seed=dh + 1).to(DT[dtype])
+    cache = torch.full((pages, 2, nkv * dh * page), 7.0, dtype=DT[dtype])
+    cg, qg = cache.cuda(), qkv.cuda()
+    ops.rope_kv_store(qg, torch.tensor(pos, dtype=torch.int32).cuda(), nh, nkv, dh, torch.from_numpy(cos).cuda(),
+                      torch.from_numpy(sin).cuda(), dh, 0, cg, torch.tensor(slots, dtype=torch.int32).cuda(), page)
+    q = qkv[:, :nh * dh].view(n, nh, dh)
+    k = qkv[:, nh * dh:(nh + nkv) * dh].view(n, nkv, dh)
+    v = qkv[:, (nh + nkv) * dh:].view(n, nkv, dh)
+    close(qg[:, :nh * dh].reshape(n, nh, dh), plain.rope(q, pos, sin_p, cos_p, "half"), dtype, "q")
+    assert torch.equal(qg[:, nh * dh:].cpu(), qkv[:, nh * dh:])
+    k_want = plain.rope(k, pos, sin_p, cos_p, "half")
+    flat = cg.cpu().view(pages, -1)
+    expect = torch.full_like(flat, 7.0).double()
+    for t in range(n):
+        if slots[t] < 0:
+            continue
+        pg, tok = slots[t] // page, slots[t] % page
+        for h in range(nkv):
+            for c in range(dh):
+                expect[pg, key_offset(h, tok, c, dh, page)] = k_want[t, h, c]
+                expect[pg, value_offset(nkv, h, tok, c, dh, page)] = v[t, h, c].double()
+    close(flat, expect, dtype, "cache")
+    assert torch.equal(flat == 7.0, expect == 7.0)
+
+
 def test_rope_partial_rotation_and_no_rotation():
     from llama_cu_amd.kernels import ops
     from llama_cu_amd.parts.position import Rotary
