@@ -87,26 +87,33 @@ __device__ __forceinline__ void load_kv(KVFrag<DH> &f, const bf16_t *__restrict_
     }
 }
 
-// One step of the online softmax on loaded keys and values.  p_row / lo_row: the last and
-// first key each of the lane's rows may see.  MASK: some row of the wave does not see all
-// 32 keys; p_max / lo_min bound what any row sees (values of keys outside are not used at
-// all, whatever the memory holds).
-template <int DH, int QB, bool MASK>
-__device__ __forceinline__ void attn_compute(const KVFrag<DH> &f, int k0, const u32x4 (&q)[QB][DH / 32],
-                                             AttnState<DH, QB> &st, const int (&p_row)[QB], const int (&lo_row)[QB],
-                                             int p_max, int lo_min, float scale_log2, int grp) {
-    // ---- S^T = K Q^T
-    f32x4 s[QB][2];
+// One step of the online softmax on loaded keys and values, in three parts.  p_row / lo_row:
+// the last and first key each of the lane's rows may see.  MASK: some row of the wave does
+// not see all 32 keys; p_max / lo_min bound what any row sees (values of keys outside are not
+// used at all, whatever the memory holds).
+//
+// S^T = K Q^T.  The four sums (two key tiles, QB blocks of rows) are independent chains of
+// DH/32 dependent matrix instructions; they are issued in turn, so that an instruction's
+// result (ready after about three instructions' time) is there when its chain goes on.
+template <int DH, int QB>
+__device__ __forceinline__ void attn_scores(const u32x4 (&k)[2][DH / 32], const u32x4 (&q)[QB][DH / 32], f32x4 (&s)[QB][2]) {
 #pragma unroll
     for (int b = 0; b < QB; ++b) s[b][0] = s[b][1] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int t = 0; t < 2; ++t)
+    for (int kb = 0; kb < DH / 32; ++kb)
 #pragma unroll
-        for (int kb = 0; kb < DH / 32; ++kb)
+        for (int t = 0; t < 2; ++t)
 #pragma unroll
-            for (int b = 0; b < QB; ++b) s[b][t] = mfma16(f.k[t][kb], q[b][kb], s[b][t]);
-    // ---- softmax of the step, online
-    u32x4 pb[QB];
+            for (int b = 0; b < QB; ++b) s[b][t] = mfma16(k[t][kb], q[b][kb], s[b][t]);
+}
+
+constexpr float RESCALE_SLACK = 6.0f;
+
+// The softmax of the step, online: new maxima and sums, the output rescaled, the weights as
+// bfloat16 operands.
+template <int DH, int QB, bool MASK>
+__device__ __forceinline__ void attn_softmax(const f32x4 (&s)[QB][2], int k0, AttnState<DH, QB> &st, const int (&p_row)[QB],
+                                             const int (&lo_row)[QB], float scale_log2, int grp, u32x4 (&pb)[QB]) {
 #pragma unroll
     for (int b = 0; b < QB; ++b) {
         float v[8];
@@ -124,7 +131,11 @@ __device__ __forceinline__ void attn_compute(const KVFrag<DH> &f, int k0, const 
         for (int r = 1; r < 8; ++r) mx = fmaxf(mx, v[r]);
         mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
         mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
-        const float m_new = fmaxf(st.m[b], mx * scale_log2);
+        // The reference point of the exponentials need not be the exact maximum: it moves only
+        // when the maximum has grown by more than 2^RESCALE_SLACK, so the weights stay below
+        // that and the output is rarely rescaled (the result is the same up to rounding).
+        const float m_true = fmaxf(st.m[b], mx * scale_log2);
+        const float m_new = m_true - st.m[b] <= RESCALE_SLACK ? st.m[b] : m_true;   // false for the first keys (-inf)
         const float m_safe = m_new == -INFINITY ? 0.f : m_new;
         const float alpha = fast_exp2(st.m[b] - m_safe);
         float p[8], sum = 0.f;
@@ -142,10 +153,15 @@ __device__ __forceinline__ void attn_compute(const KVFrag<DH> &f, int k0, const 
         }
         pb[b] = u32x4{pack_bf16(p[0], p[1]), pack_bf16(p[2], p[3]), pack_bf16(p[4], p[5]), pack_bf16(p[6], p[7])};
     }
-    // ---- O^T += V^T P^T
+}
+
+// O^T += V^T P^T
+template <int DH, int QB, bool MASK>
+__device__ __forceinline__ void attn_mix(const u32x2 (&v)[DH / 16][2], const u32x4 (&pb)[QB], int k0, int p_max, int lo_min,
+                                         int grp, AttnState<DH, QB> &st) {
 #pragma unroll
     for (int dt = 0; dt < DH / 16; ++dt) {
-        u32x2 v0 = f.v[dt][0], v1 = f.v[dt][1];
+        u32x2 v0 = v[dt][0], v1 = v[dt][1];
         if (MASK) {
             // values of keys that no row sees are taken as zero: their memory may hold anything
             const int j0 = k0 + 4 * grp, j1 = k0 + 16 + 4 * grp;
@@ -160,6 +176,46 @@ __device__ __forceinline__ void attn_compute(const KVFrag<DH> &f, int k0, const 
 #pragma unroll
         for (int b = 0; b < QB; ++b) st.o[b][dt] = mfma16(a, pb[b], st.o[b][dt]);
     }
+}
+
+template <int DH, int QB, bool MASK>
+__device__ __forceinline__ void attn_compute(const KVFrag<DH> &f, int k0, const u32x4 (&q)[QB][DH / 32],
+                                             AttnState<DH, QB> &st, const int (&p_row)[QB], const int (&lo_row)[QB],
+                                             int p_max, int lo_min, float scale_log2, int grp) {
+    f32x4 s[QB][2];
+    attn_scores<DH, QB>(f.k, q, s);
+    u32x4 pb[QB];
+    attn_softmax<DH, QB, MASK>(s, k0, st, p_row, lo_row, scale_log2, grp, pb);
+    attn_mix<DH, QB, MASK>(f.v, pb, k0, p_max, lo_min, grp, st);
+}
+
+// The same step with the operands taken from a copy in LDS (the layout that stage_issue
+// makes): first the keys alone, so that the values do not hold registers while the scores
+// are made; the values are asked for before the softmax's arithmetic and are there after it.
+template <int DH, int QB, bool MASK>
+__device__ __forceinline__ void attn_compute_lds(const u32x4 *__restrict__ buf, int k0, const u32x4 (&q)[QB][DH / 32],
+                                                 AttnState<DH, QB> &st, const int (&p_row)[QB], const int (&lo_row)[QB],
+                                                 int p_max, int lo_min, float scale_log2, int l16, int grp) {
+    f32x4 s[QB][2];
+    {
+        u32x4 k[2][DH / 32];
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int kb = 0; kb < DH / 32; ++kb) k[t][kb] = buf[t * 2 * DH + (4 * kb + grp) * 16 + l16];
+        attn_scores<DH, QB>(k, q, s);
+    }
+    __builtin_amdgcn_sched_barrier(0);             // the values' reads stay below the scores
+    u32x2 v[DH / 16][2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+        const u32x2 *vb = (const u32x2 *)(buf + 4 * DH + t * 2 * DH);
+#pragma unroll
+        for (int dt = 0; dt < DH / 16; ++dt) v[dt][t] = vb[(16 * dt + l16) * 4 + grp];
+    }
+    u32x4 pb[QB];
+    attn_softmax<DH, QB, MASK>(s, k0, st, p_row, lo_row, scale_log2, grp, pb);
+    attn_mix<DH, QB, MASK>(v, pb, k0, p_max, lo_min, grp, st);
 }
 
 // Masks only where a row needs them (the choice is the same for the whole wave).
@@ -344,71 +400,106 @@ LCU_API int lcu_attention_decode_bf16(const void *q, int q_stride, void *out, in
 #ifndef LCU_PRE_MIN_WAVES
 #define LCU_PRE_MIN_WAVES 2
 #endif
-#ifndef LCU_PRE_SUB
-#define LCU_PRE_SUB 2
-#endif
-constexpr int PRE_WAVES = 4;
+constexpr int PRE_QWAVES = 4;             // waves of a workgroup that hold different rows
+constexpr int PRE_HALVES = 2;             // wave groups that share the rows and take every second step of 32 keys
+constexpr int PRE_WAVES = PRE_QWAVES * PRE_HALVES;
 constexpr int PRE_QB = LCU_PRE_QB;
-constexpr int PRE_SUB = LCU_PRE_SUB;      // 32-key steps that one copy to LDS (one barrier) brings
+constexpr int PRE_RING = 3;               // buffers of 64 keys in LDS: one is read, two are on their way
 
-// The keys of PRE_SUB steps of 32, copied into LDS as they lie in their pages: per step, per tile of 16 keys
-// first the keys [dim/8][token][8], then (after both key tiles) the values [dim][token].
-// In units of 16 bytes a buffer holds 8*DH chunks: [K tile 0 | K tile 1 | V tile 0 | V tile 1],
-// 2*DH chunks each.  A thread of the workgroup copies chunks tid, tid + 256, ...
+// The keys and values of two steps of 32, copied into LDS as they lie in their pages: per step
+// and tile of 16 keys first the keys [dim/8][token][8], then (after both key tiles) the values
+// [dim][token].  In units of 16 bytes a step holds 8*DH chunks: [K tile 0 | K tile 1 | V tile 0
+// | V tile 1], 2*DH chunks each; a buffer holds two steps.  A thread of the workgroup copies
+// chunks tid, tid + 512, ...
+//
+// The copy goes from memory straight into LDS (global_load_lds_dwordx4: no registers hold the
+// data on its way, lane l of a wave writes the 16 bytes l of the wave's 1 KB), so the loads of
+// two buffers can be in flight while one is computed.  The page of a chunk is the same for a
+// whole wave (2*DH chunks of a region are a multiple of 64), so the block table is read with
+// scalar loads, which do not make the wave wait for the vector loads in flight.
+// Steps beyond the end of the keys are copied all the same, from the pages that the clamped
+// block table names (valid memory), into a buffer that nobody reads: no branch around a load.
+// The address of a chunk is a wave-uniform base (page, token) plus a small per-lane offset.
+// A page holds less than 4 GiB (the host checks).
 template <int DH>
-struct StageRegs {
-    u32x4 c[PRE_SUB][DH / 32];
-};
-
-template <int DH>
-__device__ __forceinline__ void stage_load(StageRegs<DH> &r, const bf16_t *__restrict__ cache, const int *__restrict__ bt,
-                                           int max_pages, int page, size_t page_elems, int nkvh, int kvh, int k0) {
-    const size_t v_off = (size_t)nkvh * DH * page + (size_t)kvh * DH * page;
-#pragma unroll
-    for (int sub = 0; sub < PRE_SUB; ++sub)
+__device__ __forceinline__ void stage_issue(u32x4 *__restrict__ buf, const bf16_t *__restrict__ cache,
+                                            const int *__restrict__ bt, int max_pages, int page, size_t page_elems,
+                                            int nkvh, int kvh, int k0) {
+    const uint32_t v_off = (uint32_t)(nkvh + kvh) * DH * page;
+    const int wave = threadIdx.x / WAVE;
 #pragma unroll
     for (int i = 0; i < DH / 32; ++i) {
-        const int c = threadIdx.x + 256 * i;
+        const int c2 = threadIdx.x + 512 * i;
+        const int sub = c2 / (8 * DH), c = c2 % (8 * DH);
         const int region = c / (2 * DH), w = c % (2 * DH), t = region & 1;
         const int j = k0 + 32 * sub + 16 * t;
         int pi = j / page;
         pi = pi < max_pages ? pi : max_pages - 1;
-        const bf16_t *pg = cache + (size_t)bt[pi] * page_elems;
+        const int page_id = bt[__builtin_amdgcn_readfirstlane(pi)];
         const int tok0 = j % page;
-        const bf16_t *src = region < 2
-            ? pg + ((size_t)(kvh * (DH / 8) + w / 16) * page + tok0 + (w % 16)) * 8
-            : pg + v_off + (size_t)(w / 2) * page + tok0 + (w % 2) * 8;
-        r.c[sub][i] = *(const u32x4 *)src;
+        // within the page, in elements: keys [dim/8][token][8], values [dim][token]
+        const uint32_t lane_off = region < 2 ? ((uint32_t)(kvh * (DH / 8) + w / 16) * page + (w % 16)) * 8
+                                             : v_off + (uint32_t)(w / 2) * page + (w % 2) * 8;
+        const uint32_t tok_off = __builtin_amdgcn_readfirstlane(region < 2 ? tok0 * 8 : tok0);
+        // a buffer load whose buffer is the page: all of the address but the lane's offset is scalar
+        const __amdgpu_buffer_rsrc_t pg = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<bf16_t *>(cache + (size_t)page_id * page_elems), 0, (uint32_t)(page_elems * sizeof(bf16_t)), 0x00020000);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(pg, (__attribute__((address_space(3))) void *)(buf + 512 * i + WAVE * wave), 16,
+                                                 lane_off * (uint32_t)sizeof(bf16_t), tok_off * (uint32_t)sizeof(bf16_t), 0, 0);
     }
 }
 
-template <int DH>
-__device__ __forceinline__ void stage_store(const StageRegs<DH> &r, u32x4 *__restrict__ buf) {
-#pragma unroll
-    for (int sub = 0; sub < PRE_SUB; ++sub)
-#pragma unroll
-        for (int i = 0; i < DH / 32; ++i) buf[sub * 8 * DH + threadIdx.x + 256 * i] = r.c[sub][i];
+// Wait until at most `left` of this wave's vector memory operations are outstanding.
+template <int LEFT>
+__device__ __forceinline__ void wait_loads() {
+    static_assert(LEFT >= 0 && LEFT < 64, "vmcnt has six bits");
+    __builtin_amdgcn_s_waitcnt((LEFT & 15) | ((LEFT >> 4) << 14) | (7 << 4) | (15 << 8));
 }
 
-// A wave's operands of the step, read from the LDS copy.
-template <int DH>
-__device__ __forceinline__ void frag_from_lds(KVFrag<DH> &f, const u32x4 *__restrict__ buf, int l16, int grp) {
+// One turn of the ring: this wave's step of 32 keys from the buffer `src`, and the workgroup's
+// copy of a later double step into the buffer `dst`.  The two are different buffers of the
+// ring, which the qualifiers say: a read from LDS otherwise waits for every copy in flight,
+// the one into `dst` included, as if it read what that copy writes.
+template <int DH, int QB>
+__device__ __forceinline__ void ring_step(const u32x4 *__restrict__ src, u32x4 *__restrict__ dst,
+                                          const bf16_t *__restrict__ cache, const int *__restrict__ bt, int max_pages, int page,
+                                          size_t page_elems, int nkvh, int kvh, int k0_copy, int blk, int blk_end,
+                                          bool wave_has, int p_max, int p_min, int lo_min, int lo_max,
+                                          const int (&tok_row)[QB], int pos_of_tok, int window, const u32x4 (&qv)[QB][DH / 32],
+                                          AttnState<DH, QB> &st, float scale_log2) {
+    stage_issue<DH>(dst, cache, bt, max_pages, page, page_elems, nkvh, kvh, k0_copy);
+    const int k0 = blk * 32;
+    // the lane's coordinates are made anew in every step: kept across the loop they would
+    // be spilled, and a reload from scratch waits for all the copies in flight
+    int tid = threadIdx.x;
+    asm volatile("" : "+v"(tid));
+    const int l16 = tid & 15, grp = (tid >> 4) & 3;
+    if (wave_has && blk < blk_end && k0 <= p_max && k0 + 31 >= lo_min) {
+        if (k0 + 31 > p_min || k0 < lo_max) {
+            // the rows' limits are made here, where a step needs them, not kept in registers
+            int p_row[QB], lo_row[QB];
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
-#pragma unroll
-        for (int kb = 0; kb < DH / 32; ++kb) f.k[t][kb] = buf[t * 2 * DH + (4 * kb + grp) * 16 + l16];
-        const u32x2 *vb = (const u32x2 *)(buf + 4 * DH + t * 2 * DH);
-#pragma unroll
-        for (int dt = 0; dt < DH / 16; ++dt) f.v[dt][t] = vb[(16 * dt + l16) * 4 + grp];
+            for (int b = 0; b < QB; ++b) {
+                p_row[b] = tok_row[b] < 0 ? -1 : tok_row[b] + pos_of_tok;
+                lo_row[b] = tok_row[b] >= 0 && window > 0 && p_row[b] - window + 1 > 0 ? p_row[b] - window + 1 : 0;
+            }
+            attn_compute_lds<DH, QB, true>(src, k0, qv, st, p_row, lo_row, p_max, lo_min, scale_log2, l16, grp);
+        } else {
+            const int none[QB] = {};
+            attn_compute_lds<DH, QB, false>(src, k0, qv, st, none, none, p_max, lo_min, scale_log2, l16, grp);
+        }
     }
 }
 
-// A task is a block of consecutive tokens of one request: every wave of the workgroup takes
-// QB blocks of 16 rows (tokens x the heads of one chunk of a group), so a task covers
-// 4 * QB * (16 / heads per chunk) tokens, starting at batch index task_tok0[t].  The
-// workgroup walks the keys that any of its rows sees, 32 at a time; the keys and values of a
-// step are copied to LDS once (double buffered: the next step's loads are in flight while
-// one is computed) and every wave takes its operands from there.
+// A task is a block of consecutive tokens of one request: a workgroup has PRE_QWAVES x 2 waves;
+// wave q of either half takes QB blocks of 16 rows (tokens x the heads of one chunk of a
+// group), so a task covers 4 * QB * (16 / heads per chunk) tokens, starting at batch index
+// task_tok0[t].  The workgroup walks the keys that any of its rows sees, 64 at a time: the
+// first half of the waves takes the first 32 of them, the second half the other 32, each
+// with an online softmax of its own, and the two are merged at the end.  So a compute unit
+// holds two waves per SIMD that work on one task (while one waits for the softmax's
+// arithmetic the other feeds the matrix cores), however few tasks there are.  The keys and
+// values are copied to LDS once per workgroup, two buffers ahead of the one that is read.
 template <int DH, int QB>
 __global__ void __launch_bounds__(PRE_WAVES *WAVE, LCU_PRE_MIN_WAVES)
 attention_prefill_kernel(const bf16_t *__restrict__ q, int q_stride, bf16_t *__restrict__ out, int out_stride,
@@ -416,12 +507,14 @@ attention_prefill_kernel(const bf16_t *__restrict__ q, int q_stride, bf16_t *__r
                          const int *__restrict__ q_start, const int *__restrict__ ctx_len,
                          const int *__restrict__ task_req, const int *__restrict__ task_tok0, int n_tasks,
                          int tasks_per_wg, int nh, int nkvh, int page, float scale_log2, int window) {
-    __shared__ u32x4 lds[2][PRE_SUB * 8 * DH];
-    const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
+    extern __shared__ u32x4 lds_ring[];            // [PRE_RING][16 * DH]; at the end the halves' states
+    // the wave's number as a scalar: what follows from it (its rows' limits) then lives in scalar registers
+    const int wave_id = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
+    const int lane = threadIdx.x & (WAVE - 1), wave = wave_id % PRE_QWAVES, half = wave_id / PRE_QWAVES;
     // a workgroup takes tasks_per_wg tasks one after the other (the host pairs a long one with
     // a short one, so that workgroups take about equally long)
     for (int task = blockIdx.x * tasks_per_wg; task < (blockIdx.x + 1) * tasks_per_wg && task < n_tasks; ++task) {
-    __syncthreads();                               // the last task's reads of LDS are over
+    __syncthreads();                               // the last task's use of LDS is over (and its copies have landed)
     const int l16 = lane & 15, grp = lane >> 4;
     const int g = nh / nkvh;
     const int chunks = (g + 15) / 16;
@@ -436,14 +529,13 @@ attention_prefill_kernel(const bf16_t *__restrict__ q, int q_stride, bf16_t *__r
     const int tok0 = task_tok + wave * tokens_per_wave;                 // this wave's first token
 
     u32x4 qv[QB][DH / 32];
-    int p_row[QB], lo_row[QB], tok_row[QB];
+    int tok_row[QB];
+    const int pos_of_tok = ctx - q_end;                                 // a token's position = its batch index + this
 #pragma unroll
     for (int b = 0; b < QB; ++b) {
         const int tok = tok0 + b * tokens_per_block + l16 / hc;
         const bool valid = l16 < tokens_per_block * hc && tok < q_end;
         tok_row[b] = valid ? tok : -1;
-        p_row[b] = valid ? ctx - (q_end - tok) : -1;
-        lo_row[b] = valid && window > 0 && p_row[b] - window + 1 > 0 ? p_row[b] - window + 1 : 0;
         load_q<DH>(q + (size_t)(valid ? tok : task_tok) * q_stride + (size_t)(head0 + l16 % hc) * DH, valid, qv[b], grp);
     }
     // what this wave sees (the same in all its lanes), and what the workgroup sees
@@ -456,7 +548,7 @@ attention_prefill_kernel(const bf16_t *__restrict__ q, int q_stride, bf16_t *__r
         lo_min = window > 0 && p_min - window + 1 > 0 ? p_min - window + 1 : 0;
         lo_max = window > 0 && p_max - window + 1 > 0 ? p_max - window + 1 : 0;
     }
-    const int wg_last_tok = (task_tok + PRE_WAVES * tokens_per_wave < q_end ? task_tok + PRE_WAVES * tokens_per_wave : q_end) - 1;
+    const int wg_last_tok = (task_tok + PRE_QWAVES * tokens_per_wave < q_end ? task_tok + PRE_QWAVES * tokens_per_wave : q_end) - 1;
     const int wg_p_max = ctx - (q_end - wg_last_tok);
     const int wg_p_min = ctx - (q_end - task_tok);
     const int wg_lo_min = window > 0 && wg_p_min - window + 1 > 0 ? wg_p_min - window + 1 : 0;
@@ -466,41 +558,70 @@ attention_prefill_kernel(const bf16_t *__restrict__ q, int q_stride, bf16_t *__r
     const int *bt = block_table + (size_t)r * max_pages;
     const size_t page_elems = kv_page_elems(nkvh, DH, page);
     const int blk0 = wg_lo_min / 32, blk_end = wg_p_max / 32 + 1;
-    StageRegs<DH> regs;
-    stage_load<DH>(regs, cache, bt, max_pages, page, page_elems, nkvh, kvh, blk0 * 32);
-    stage_store<DH>(regs, lds[0]);
-    __syncthreads();
-    int cur = 0;
-    for (int blk = blk0; blk < blk_end; blk += PRE_SUB, cur ^= 1) {
-        const bool more = blk + PRE_SUB < blk_end;
-        if (more) stage_load<DH>(regs, cache, bt, max_pages, page, page_elems, nkvh, kvh, (blk + PRE_SUB) * 32);
+    // Double steps of 64 keys; double step d is read from buffer d % PRE_RING while the loads of the
+    // next two are on their way.  Before one, every wave waits for its own part of its copy, then
+    // the barrier makes the whole copy visible and says that the buffer of the double step before
+    // is free for the one two ahead.
+    const int n_dsteps = (blk_end - blk0 + 1) / 2;
 #pragma unroll
-        for (int sub = 0; sub < PRE_SUB; ++sub) {
-            const int k0 = (blk + sub) * 32;
-            if (wave_has && blk + sub < blk_end && k0 <= p_max && k0 + 31 >= lo_min) {
-                KVFrag<DH> f;
-                frag_from_lds<DH>(f, lds[cur] + sub * 8 * DH, l16, grp);
-                attn_block<DH, QB>(f, k0, k0 + 31 > p_min || k0 < lo_max, qv, st, p_row, lo_row, p_max, lo_min, scale_log2, grp);
+    for (int d = 0; d < PRE_RING - 1; ++d)
+        stage_issue<DH>(lds_ring + d * 16 * DH, cache, bt, max_pages, page, page_elems, nkvh, kvh, (blk0 + 2 * d) * 32);
+    int slot = 0, fill = PRE_RING - 1;
+    for (int d = 0; d < n_dsteps; ++d) {
+        wait_loads<(PRE_RING - 2) * (DH / 32)>();
+        lds_barrier();
+        ring_step<DH, QB>(lds_ring + slot * 16 * DH + half * 8 * DH, lds_ring + fill * 16 * DH, cache, bt, max_pages, page,
+                          page_elems, nkvh, kvh, (blk0 + 2 * (d + PRE_RING - 1)) * 32, blk0 + 2 * d + half, blk_end, wave_has,
+                          p_max, p_min, lo_min, lo_max, tok_row, pos_of_tok, window, qv, st, scale_log2);
+        slot = slot + 1 == PRE_RING ? 0 : slot + 1;
+        fill = fill + 1 == PRE_RING ? 0 : fill + 1;
+    }
+    // ---- the second half hands its state to the first, which merges and writes
+    __syncthreads();                               // every copy has landed, every wave is done with the buffers
+    float *xch = (float *)lds_ring;                // [value][query wave][lane]
+    constexpr int NV = QB * (2 + (DH / 16) * 4);
+    if (half == 1) {
+        int v = 0;
+#pragma unroll
+        for (int b = 0; b < QB; ++b) {
+            xch[((v++) * PRE_QWAVES + wave) * WAVE + lane] = st.m[b];
+            xch[((v++) * PRE_QWAVES + wave) * WAVE + lane] = st.l[b];
+#pragma unroll
+            for (int dt = 0; dt < DH / 16; ++dt)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) xch[((v++) * PRE_QWAVES + wave) * WAVE + lane] = st.o[b][dt][e];
+        }
+    }
+    __syncthreads();
+    if (half == 0) {
+        int v = 0;
+#pragma unroll
+        for (int b = 0; b < QB; ++b) {
+            const float m1 = xch[((v++) * PRE_QWAVES + wave) * WAVE + lane];
+            const float l1 = xch[((v++) * PRE_QWAVES + wave) * WAVE + lane];
+            const float m = fmaxf(st.m[b], m1);
+            const float m_safe = m == -INFINITY ? 0.f : m;
+            const float a0 = fast_exp2(st.m[b] - m_safe), a1 = fast_exp2(m1 - m_safe);
+            float l_all = st.l[b] * a0 + l1 * a1;
+            l_all += __shfl_xor(l_all, 16, WAVE);
+            l_all += __shfl_xor(l_all, 32, WAVE);
+            const float inv = 1.0f / l_all;
+            bf16_t *o = tok_row[b] < 0 ? nullptr : out + (size_t)tok_row[b] * out_stride + (size_t)(head0 + l16 % hc) * DH;
+#pragma unroll
+            for (int dt = 0; dt < DH / 16; ++dt) {
+                float e4[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    e4[e] = (st.o[b][dt][e] * a0 + xch[((v++) * PRE_QWAVES + wave) * WAVE + lane] * a1) * inv;
+                if (o) {
+                    u32x2 w;
+                    w.x = pack_bf16(e4[0], e4[1]);
+                    w.y = pack_bf16(e4[2], e4[3]);
+                    *(u32x2 *)(o + 16 * dt + 4 * grp) = w;
+                }
             }
         }
-        if (more) stage_store<DH>(regs, lds[cur ^ 1]);
-        __syncthreads();
-    }
-#pragma unroll
-    for (int b = 0; b < QB; ++b) {
-        float l_all = st.l[b];
-        l_all += __shfl_xor(l_all, 16, WAVE);
-        l_all += __shfl_xor(l_all, 32, WAVE);
-        if (tok_row[b] < 0) continue;
-        const float inv = 1.0f / l_all;
-        bf16_t *o = out + (size_t)tok_row[b] * out_stride + (size_t)(head0 + l16 % hc) * DH;
-#pragma unroll
-        for (int dt = 0; dt < DH / 16; ++dt) {
-            u32x2 w;
-            w.x = pack_bf16(st.o[b][dt][0] * inv, st.o[b][dt][1] * inv);
-            w.y = pack_bf16(st.o[b][dt][2] * inv, st.o[b][dt][3] * inv);
-            *(u32x2 *)(o + 16 * dt + 4 * grp) = w;
-        }
+        static_assert(NV * PRE_QWAVES * WAVE * 4 <= PRE_RING * 16 * DH * 16, "the halves' states fit the ring");
     }
     }
 }
@@ -512,7 +633,15 @@ static int launch_prefill(const void *q, int q_stride, void *out, int out_stride
                           int page, float scale, int window, hipStream_t stream) {
     const int g = nh / nkvh, chunks = (g + 15) / 16;
     dim3 grid((n_tasks + tasks_per_wg - 1) / tasks_per_wg, nkvh * chunks), block(PRE_WAVES * WAVE);
-    attention_prefill_kernel<DH, QB><<<grid, block, 0, stream>>>(
+    constexpr size_t lds_bytes = (size_t)PRE_RING * 16 * DH * sizeof(u32x4);
+    static bool allowed = false;                   // more than 64 KB of LDS must be asked for once
+    if (!allowed) {
+        const hipError_t e = hipFuncSetAttribute((const void *)attention_prefill_kernel<DH, QB>,
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+        if (e != hipSuccess) return (int)e;
+        allowed = true;
+    }
+    attention_prefill_kernel<DH, QB><<<grid, block, lds_bytes, stream>>>(
         (const bf16_t *)q, q_stride, (bf16_t *)out, out_stride, (const bf16_t *)cache, block_table, max_pages, q_start,
         ctx_len, task_req, task_tok0, n_tasks, tasks_per_wg, nh, nkvh, page, scale * 1.4426950408889634f, window);
     LCU_LAUNCH_CHECK();
@@ -526,7 +655,7 @@ LCU_API int lcu_attention_prefill_tokens_per_task(int nh, int nkvh) {
     const int g = nh / nkvh;
     if (g > 16 && g % 16) return 0;       // chunks of a group must be equal for one task size
     const int hc = g < 16 ? g : 16;
-    return PRE_WAVES * PRE_QB * (16 / hc);
+    return PRE_QWAVES * PRE_QB * (16 / hc);
 }
 
 // task_req / task_tok0: [n_tasks], tasks cut from the batch with the size above; a
@@ -538,6 +667,7 @@ LCU_API int lcu_attention_prefill_bf16(const void *q, int q_stride, void *out, i
                                        int nh, int nkvh, int dh, int page, float scale, int window,
                                        hipStream_t stream) {
     if (n_tasks <= 0) return LCU_OK;
+    if ((unsigned long long)kv_page_elems(nkvh, dh, page) * 2ull >= (1ull << 31)) return LCU_UNSUPPORTED;
     if (tasks_per_wg < 1 || lcu_attention_prefill_tokens_per_task(nh, nkvh) == 0 || page <= 0 || page % 16 || max_pages <= 0 ||
         window < 0 || q_stride % 8 || out_stride % 4 || nkvh * ((nh / nkvh + 15) / 16) > 65535)
         return LCU_BAD_ARGUMENT;

@@ -64,6 +64,14 @@ __device__ __forceinline__ float block_sum(float v, float *scratch) {
     return t;
 }
 
+// A workgroup barrier that waits for this wave's LDS accesses only.  __syncthreads() also
+// waits until every global load of the wave has come back, which empties a software
+// pipeline that keeps loads of later steps in flight across the barrier.  Use it where the
+// waves exchange data through LDS only.
+__device__ __forceinline__ void lds_barrier() {
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
 #define LCU_LAUNCH_CHECK()                                   \
     do {                                                     \
         hipError_t e_ = hipGetLastError();                   \
