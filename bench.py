@@ -99,6 +99,37 @@ def run_prefill(engine, cfg, rng, sync, repeats=3):
     return best
 
 
+def kernel_summary(db: str, steps: int) -> int:
+    """Per-step table of kernels from the database that ``rocprofv3 --kernel-trace`` wrote for a
+    run of this program: the kernels between two embedding gathers are one step of the model;
+    the last ``steps`` steps are averaged."""
+    import re
+    import sqlite3
+    con = sqlite3.connect(db)
+    rows = con.execute("select name, start, end from kernels order by start").fetchall()
+    marks = [i for i, r in enumerate(rows) if "embedding_gather" in r[0]]
+    if len(marks) < steps + 1:
+        print(f"bench.py: {db} holds {len(marks)} steps, fewer than the {steps + 1} needed")
+        return 1
+    sel = marks[-(steps + 1):]
+    agg = {}
+    for a, b in zip(sel[:-1], sel[1:]):
+        for name, t0, t1 in rows[a:b]:
+            short = re.sub(r"\(.*", "", name).replace("void ", "")
+            short = re.sub(r"_SN_LDSB.*", "", short)[:70]
+            item = agg.setdefault(short, [0, 0.0])
+            item[0] += 1
+            item[1] += (t1 - t0) / 1e3
+    wall = (rows[sel[-1]][1] - rows[sel[0]][1]) / 1e3 / steps
+    busy = sum(v[1] for v in agg.values()) / steps
+    print(f"steps averaged: {steps}; wall {wall:.1f} us/step, kernels busy {busy:.1f} us/step\n")
+    print("| kernel | launches/step | us/step | avg us | % of busy |")
+    print("|---|---|---|---|---|")
+    for name, (n, t) in sorted(agg.items(), key=lambda kv: -kv[1][1]):
+        print(f"| `{name}` | {n / steps:.0f} | {t / steps:.1f} | {t / n:.1f} | {100 * t / steps / busy:.1f} |")
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -109,7 +140,11 @@ def main() -> int:
     ap.add_argument("--dtype", choices=["bfloat16", "float32"], default="bfloat16")
     ap.add_argument("--no-points", action="store_true", help="skip decoding at batch 1 and 64 and the prefill")
     ap.add_argument("--only-prefill", action="store_true", help="time the 2048-token prefill alone (for profiles)")
+    ap.add_argument("--kernel-summary", metavar="DB", help="print the per-step kernel table of a rocprofv3 database and exit")
+    ap.add_argument("--summary-steps", type=int, default=8)
     args = ap.parse_args()
+    if args.kernel_summary:
+        return kernel_summary(args.kernel_summary, args.summary_steps)
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported (no multi-GPU path)")
         return 2
