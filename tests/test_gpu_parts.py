@@ -285,3 +285,122 @@ def test_a_toy_mixer_with_state_is_registered_built_and_stepped():
         common.assert_matches_plain(got, want, "float32", "toy mixer")
     runner.cache.check()
     assert runner.cache.free_slots() == 3
+
+
+def test_a_toy_routed_feed_forward_and_a_toy_position_encoding_are_registered_and_stepped():
+    """Two more parts defined here and not in the package.  ``pick_one``: a feed-forward that
+    routes each token to the one of its experts whose router score is largest (the score in
+    32-bit) and scales the expert's output by the softmax weight of that score.  ``key_shift``:
+    a position encoding that is no rotation: it adds ``sin(pos / 7)`` times a learned vector to
+    every query and key head before the cache write.  Layer 0 gets the position encoding and
+    keeps SwiGLU, layer 1 keeps the rotation and gets the routed feed-forward; the model is
+    stepped whole, in portions, token by token and mixed, and agrees with a direct computation."""
+    import llama_cu_amd
+    from llama_cu_amd.config import LlamaConfig
+    from llama_cu_amd.models.llama import llama_spec
+    from llama_cu_amd.parts import Part, PartSpec, TensorSpec, register_part
+
+    class PickOne(Part):
+        graph_safe = True
+
+        def __init__(self, hidden_size, inner, experts):
+            self.d, self.di, self.e = hidden_size, inner, experts
+
+        def tensors(self):
+            return {"router.weight": TensorSpec((self.e, self.d)), "w_in": TensorSpec((self.e * self.di, self.d)),
+                    "w_out": TensorSpec((self.e * self.d, self.di))}
+
+        def load(self, tensors, build):
+            self.router = tensors["router.weight"].float()
+            self.w_in = tensors["w_in"].float().view(self.e, self.di, self.d)
+            self.w_out = tensors["w_out"].float().view(self.e, self.d, self.di)
+            self.dtype = build.dtype
+
+        def forward(self, h):
+            x = h.float()
+            scores = torch.softmax(x @ self.router.T, dim=-1)                    # router in 32-bit
+            weight, which = scores.max(dim=-1)
+            inner = torch.relu(torch.einsum("nd,nid->ni", x, self.w_in[which]))
+            return (torch.einsum("ni,ndi->nd", inner, self.w_out[which]) * weight[:, None]).to(self.dtype)
+
+    class KeyShift(Part):
+        graph_safe = True
+
+        def __init__(self, head_dim):
+            self.dh = head_dim
+
+        def tensors(self):
+            return {}
+
+        def load(self, tensors, build):
+            g = torch.Generator().manual_seed(77)
+            self.vec = (torch.randn(self.dh, generator=g) * 0.5).to(build.device)
+
+        def rotary_tables(self):
+            return None
+
+        def apply(self, qkv, positions, heads, kv_heads, head_dim):
+            n = qkv.shape[0]
+            shift = torch.sin(positions.float() / 7.0)[:, None, None] * self.vec[None, None, :]
+            qk = qkv[:, :(heads + kv_heads) * head_dim].view(n, heads + kv_heads, head_dim)
+            qk += shift.to(qkv.dtype)
+
+    register_part("ffn", "pick_one", PickOne, replace=True)
+    register_part("position", "key_shift", KeyShift, replace=True)
+    cfg_d = dict(common.TINY_A)
+    cfg = LlamaConfig.from_dict(cfg_d)
+    spec = llama_spec(cfg)
+    spec.layers[0].params["mixer"].params["position"] = PartSpec("key_shift", {"head_dim": 16})
+    spec.layers[1].params["ffn"] = PartSpec("pick_one", {"hidden_size": 64, "inner": 40, "experts": 3}, "moe")
+    runner, w = runner_for(spec, 13, "float32", max_tokens=512, max_seqs=3)
+    assert "model.layers.1.moe.router.weight" in w and "model.layers.1.mlp.gate_proj.weight" not in w
+    vec = runner.model.layers[0].mixer.position.vec.double().cpu()
+
+    def direct(toks):
+        pcfg = plain.PlainConfig.from_dict(cfg_d)
+        n = len(toks)
+        pos = list(range(n))
+        sin, cos = plain.rope_tables(n, 16, pcfg.rope_theta)
+        x = plain.embedding(w["model.embed_tokens.weight"], toks)
+        # layer 0: attention whose queries and keys are shifted, not rotated
+        p = "model.layers.0."
+        h = plain.rms_norm(x, w[p + "input_layernorm.weight"], 1e-5)
+        shift = torch.sin(torch.tensor(pos, dtype=torch.float32) / 7.0).double()[:, None, None] * vec[None, None, :]
+        q = plain.linear(h, w[p + "self_attn.q_proj.weight"]).view(n, 4, 16) + shift
+        k = plain.linear(h, w[p + "self_attn.k_proj.weight"]).view(n, 4, 16) + shift
+        v = plain.linear(h, w[p + "self_attn.v_proj.weight"]).view(n, 4, 16)
+        o = plain.attention(q, k, v, 16 ** -0.5, first_pos=0, window=None)
+        x = x + plain.linear(o.reshape(n, 64), w[p + "self_attn.o_proj.weight"])
+        x = x + plain.feed_forward(w, p, plain.rms_norm(x, w[p + "post_attention_layernorm.weight"], 1e-5))
+        # layer 1: Llama's attention, then the routed feed-forward
+        p = "model.layers.1."
+        x = x + plain.attention_block(pcfg, w, p, plain.rms_norm(x, w[p + "input_layernorm.weight"], 1e-5), pos, sin, cos)
+        h = plain.rms_norm(x, w[p + "post_attention_layernorm.weight"], 1e-5)
+        scores = torch.softmax(h @ w[p + "moe.router.weight"].double().T, dim=-1)
+        weight, which = scores.max(dim=-1)
+        w_in = w[p + "moe.w_in"].double().view(3, 40, 64)
+        w_out = w[p + "moe.w_out"].double().view(3, 64, 40)
+        out = torch.stack([w_out[e] @ torch.relu(w_in[e] @ h[t]) * weight[t] for t, e in enumerate(which.tolist())])
+        x = x + out
+        return plain.linear(plain.rms_norm(x, w["model.norm.weight"], 1e-5), w["lm_head.weight"]), scores
+
+    reqs = common.random_requests(256, [40, 9, 77, 30], 14)
+    want = {}
+    for name, toks in reqs.items():
+        logits, scores = direct(toks)
+        top2 = scores.topk(2, dim=-1).values
+        # a token whose two best experts are nearly tied may go either way in 32-bit: none here
+        assert float((top2[:, 0] - top2[:, 1]).min()) > 1e-4, "choose another seed: a routing tie"
+        want[name] = logits
+    for mode in (common.trace_whole, common.trace_portions, common.trace_tail_decode, lambda r: common.trace_mixed(r, max_live=3)):
+        steps, _ = mode(reqs)
+        ids, outputs = {}, {}
+        for st in steps:
+            es = st["entries"]
+            logits = runner.step([ids.setdefault(e["id"], len(ids)) for e in es], [e["tokens"] for e in es], [e["want"] for e in es])
+            outputs[st["step"]] = logits.cpu().numpy()
+            for name in st["end"]:
+                runner.end(ids[name])
+        got = common.collect(steps, outputs, 256)
+        common.assert_matches_plain(got, want, "float32", "toy parts")
+    runner.cache.check()
