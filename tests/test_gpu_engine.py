@@ -237,3 +237,66 @@ def test_a_kept_request_goes_on_after_a_late_end_of_sequence(folder_b):
     t1, t2, _ = outs[0]
     whole = plain.greedy_generate(cfg, w, prompt + t1[0] + [11, 12, 13], len(t2))
     assert t2 == whole[:len(t2)]
+
+
+def test_a_random_serving_session_changes_no_token(folder_b):
+    """Requests arrive at random rounds, with random lengths, budgets and sampling, some are
+    aborted on the way, the pool is so small that requests are preempted and recomputed, and
+    the engine runs ahead.  Every request that was not aborted gets exactly the tokens it gets
+    alone in turn with an ample pool (32-bit logits do not depend on the batch, and the random
+    numbers depend on the request and the token's index only); no page or slot is lost."""
+    import random
+    from llama_cu_amd.engine.engine import Engine
+    from llama_cu_amd.sampling import GREEDY, SamplingParams
+    rng = random.Random(11)
+    n_req = 14
+    plan = []
+    for i in range(n_req):
+        prompt = [rng.randrange(384) for _ in range(rng.choice([1, 2, 17, 33, 48, 60, 60]))]
+        params = GREEDY if rng.random() < 0.4 else SamplingParams(temperature=rng.choice([0.7, 1.0]), top_p=rng.choice([1.0, 0.9]),
+                                                                 top_k=rng.choice([1000, 20]), seed=rng.randrange(1 << 30))
+        plan.append(dict(prompt=prompt, params=params, max_steps=rng.randrange(1, 40), arrive=rng.randrange(0, 12),
+                         abort_after=rng.choice([None, None, None, rng.randrange(1, 10)])))
+    # alone, in turn, ample pool
+    alone = Engine.from_folder(folder_b, dtype="float32", max_tokens=1024, max_seqs=1, run_ahead=False)
+    want = []
+    for i, r in enumerate(plan):
+        rid = alone.add_request(r["prompt"], r["params"], r["max_steps"], req_id=i, ignore_eos=True)
+        out = []
+        while not alone.idle:
+            out += [o.token for o in alone.step() if o.token is not None]
+        alone.drop(rid)
+        want.append(out)
+    # the session: ten pages of 16 tokens; a request needs up to seven, four may be live
+    eng = Engine.from_folder(folder_b, dtype="float32", max_tokens=160, max_seqs=4, max_batch_tokens=40, prefill_chunk=24,
+                             run_ahead=True)
+    got = {i: [] for i in range(n_req)}
+    why, aborted = {}, set()
+    rounds = 0
+    while rounds < 12 or not eng.idle:
+        for i, r in enumerate(plan):
+            if r["arrive"] == rounds:
+                eng.add_request(r["prompt"], r["params"], r["max_steps"], req_id=i, ignore_eos=True)
+        for o in eng.step():
+            if o.token is not None:
+                got[o.req].append(o.token)
+                r = plan[o.req]
+                if r["abort_after"] is not None and len(got[o.req]) == r["abort_after"] and o.finished is None:
+                    eng.abort(o.req)
+                    aborted.add(o.req)
+            if o.finished:
+                assert o.req not in why, "a request's end is reported once"
+                why[o.req] = o.finished
+        rounds += 1
+        assert rounds < 3000, "the session does not end"
+    assert eng.sched.preemptions > 0, "the pool was meant to be too small"
+    for i in range(n_req):
+        if i in aborted:
+            assert why[i] == "aborted" and got[i] == want[i][:len(got[i])]
+        else:
+            assert got[i] == want[i], f"request {i}"
+            assert why[i] == "max_steps"
+    for i in range(n_req):
+        eng.drop(i)
+    eng.runner.cache.check()
+    assert eng.runner.cache.free_pages(0) == eng.runner.num_pages and eng.runner.cache.free_slots() == 4
