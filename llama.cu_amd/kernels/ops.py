@@ -60,7 +60,29 @@ def _i32(t: torch.Tensor, what: str, n: Optional[int] = None) -> None:
         raise KernelError(f"{what}: expected {n} entries, got {t.numel()}")
 
 
+_scoped_stream: Optional[ctypes.c_void_p] = None
+
+
+class stream_scope:
+    """Within the scope the kernels are launched on the stream that is torch's current one at
+    its entry.  Asking torch for its current stream at every launch costs more host time than
+    the launch itself; a model's forward pass asks once."""
+
+    def __enter__(self):
+        global _scoped_stream
+        self._before = _scoped_stream
+        _scoped_stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        return self
+
+    def __exit__(self, *exc):
+        global _scoped_stream
+        _scoped_stream = self._before
+        return False
+
+
 def _stream() -> ctypes.c_void_p:
+    if _scoped_stream is not None:
+        return _scoped_stream
     return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
 
 

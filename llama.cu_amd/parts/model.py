@@ -119,13 +119,14 @@ class DecoderModel:
     def forward(self, step, caches) -> torch.Tensor:
         """Logits ``[len(step.logit_rows), vocab]`` (float32) for the batch ``step``;
         ``caches[i]`` is the cache of run-order entry ``i``."""
-        x = self.embedding.forward(step.tokens)
-        pending = None
-        for i, e in enumerate(self.spec.run_order):
-            pending = self.layers[e.layer].forward(x, pending, step, caches[i])
-        if step.n_logits == 0:
-            return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=x.device)
-        xs = ops.gather_rows(x, step.logit_rows)
-        ps = ops.gather_rows(pending, step.logit_rows) if pending is not None else None
-        y = self.final_norm.forward(xs, ps)
-        return self.head.forward(y)
+        with ops.stream_scope():                  # the whole pass goes to one stream, asked for once
+            x = self.embedding.forward(step.tokens)
+            pending = None
+            for i, e in enumerate(self.spec.run_order):
+                pending = self.layers[e.layer].forward(x, pending, step, caches[i])
+            if step.n_logits == 0:
+                return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=x.device)
+            xs = ops.gather_rows(x, step.logit_rows)
+            ps = ops.gather_rows(pending, step.logit_rows) if pending is not None else None
+            y = self.final_norm.forward(xs, ps)
+            return self.head.forward(y)
