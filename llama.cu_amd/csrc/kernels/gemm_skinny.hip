@@ -24,7 +24,28 @@ typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 
-enum { EPI_BF16 = 0, EPI_F32 = 1, EPI_ADD_F32 = 2, EPI_SWIGLU = 3 };
+enum { EPI_BF16 = 0, EPI_F32 = 1, EPI_ADD_F32 = 2, EPI_SWIGLU = 3, EPI_ADD_NORM = 4 };
+
+// What two epilogues need beside Y, so that no kernel stands between a projection that ends
+// a branch and the product that follows the next norm:
+//   EPI_ADD_NORM: Y is the float32 residual stream and takes the product in; the new rows times
+//     the norm's weight go to h_out as bfloat16, *not yet normalised*, and the workgroup's
+//     share of each row's sum of squares goes to sumsq_out[row][workgroup].
+//   row scale (any other epilogue, sumsq_in not null): the rows of X are such rows; a row of
+//     the product is multiplied by rsqrt(sum of its shares / norm_width + eps) before the
+//     epilogue (the normalisation is a factor per row, so it commutes with the product).
+// The shares are added in a fixed order: no atomics, results do not depend on timing.
+struct SkinnyExtra {
+    const void *norm_w;        // [N] norm weight of EPI_ADD_NORM
+    int norm_w_type;           // LCU_F32 or LCU_BF16
+    bf16_t *h_out;             // [M, N] rows ldh apart
+    int ldh;
+    float *sumsq_out;          // [M][gridDim.x]
+    const float *sumsq_in;     // [M][n_in] or null
+    int n_in;
+    int norm_width;
+    float eps;
+};
 
 __device__ __forceinline__ f32x4 mfma16(u32x4 a, u32x4 b, f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
@@ -77,8 +98,9 @@ __device__ __forceinline__ void mul_frag(const Frag<NT, MT> &f, f32x4 (&acc)[NT]
 template <int NT, int MT, int EPI, int SK_WAVES>
 __global__ void __launch_bounds__(SK_WAVES *WAVE)
 gemm_skinny_kernel(const bf16_t *__restrict__ X, int ldx, const bf16_t *__restrict__ W, int ldw, void *__restrict__ Y,
-                   int ldy, int M, int N, int K) {
+                   int ldy, int M, int N, int K, SkinnyExtra ex) {
     __shared__ float red[SK_WAVES][NT * MT * 4][WAVE];
+    __shared__ float row_scale[16 * MT];
     const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
     const int l16 = lane & 15, grp = lane >> 4;
     // the rows of W of tile t: for SwiGLU tile 0 are gate rows, tile 1 the up rows N/2 further
@@ -106,6 +128,36 @@ gemm_skinny_kernel(const bf16_t *__restrict__ X, int ldx, const bf16_t *__restri
     for (int t = 0; t < NT; ++t)
 #pragma unroll
         for (int m = 0; m < MT; ++m) acc[t][m] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    // The rows' factors, by the last wave before it starts on its share of K.  Lane group g adds
+    // the g-th quarter of a row's shares, eight 16-byte loads in flight at a time (one load after
+    // the other would hold the wave back for tens of microseconds); the quarters' sums are added
+    // in the order of the shuffles.  Always the same order: no dependence on timing.
+    if (EPI != EPI_ADD_NORM && ex.sumsq_in != nullptr && wave == SK_WAVES - 1) {
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+            const int tok = 16 * m + l16;
+            const float *p = ex.sumsq_in + (size_t)(tok < M ? tok : 0) * ex.n_in;
+            float ss = 0.f;
+            if ((ex.n_in & 15) == 0) {
+                const int q4 = ex.n_in / 16;                       // float4s in a quarter
+                const f32x4 *p4 = (const f32x4 *)p + grp * q4;
+                for (int i = 0; i < q4; i += 8) {
+                    f32x4 v[8];
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) v[e] = p4[i + e < q4 ? i + e : q4 - 1];
+#pragma unroll
+                    for (int e = 0; e < 8; ++e)
+                        if (i + e < q4) ss += (v[e][0] + v[e][1]) + (v[e][2] + v[e][3]);
+                }
+            } else {
+                for (int i = grp; i < ex.n_in; i += 4) ss += p[i];
+            }
+            ss += __shfl_xor(ss, 16, WAVE);
+            ss += __shfl_xor(ss, 32, WAVE);
+            if (grp == 0) row_scale[tok] = rsqrtf(ss / (float)ex.norm_width + ex.eps);
+        }
+    }
 
     // A ring of STAGES macro-steps in flight per wave: with few workgroups per compute unit
     // (small N) this is what keeps enough bytes on their way from HBM.
@@ -149,6 +201,40 @@ gemm_skinny_kernel(const bf16_t *__restrict__ X, int ldx, const bf16_t *__restri
                 acc[t][m][r] = sum;
             }
     // ---- epilogue: the lane holds, per tile, features 4 grp + r of token 16 m + l16
+    if (EPI != EPI_ADD_NORM && ex.sumsq_in != nullptr) {
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+            const float rs = row_scale[16 * m + l16];
+#pragma unroll
+            for (int t = 0; t < NT; ++t)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) acc[t][m][r] *= rs;
+        }
+    }
+    if (EPI == EPI_ADD_NORM) {
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+            const int tok = 16 * m + l16;
+            float ss = 0.f;
+#pragma unroll
+            for (int t = 0; t < NT; ++t)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int n = n0 + 16 * t + 4 * grp + r;
+                    if (tok >= M || n >= N) continue;
+                    float *res = (float *)Y + (size_t)tok * ldy + n;
+                    const float xn = *res + acc[t][m][r];
+                    *res = xn;
+                    ss += xn * xn;
+                    const float wn = ex.norm_w_type == LCU_F32 ? ((const float *)ex.norm_w)[n] : to_f32(((const bf16_t *)ex.norm_w)[n]);
+                    ex.h_out[(size_t)tok * ex.ldh + n] = from_f32<bf16_t>(xn * wn);
+                }
+            ss += __shfl_xor(ss, 16, WAVE);               // every lane takes part: the others bring zero
+            ss += __shfl_xor(ss, 32, WAVE);
+            if (grp == 0 && tok < M) ex.sumsq_out[(size_t)tok * gridDim.x + blockIdx.x] = ss;
+        }
+        return;
+    }
 #pragma unroll
     for (int m = 0; m < MT; ++m) {
         const int tok = 16 * m + l16;
@@ -182,14 +268,17 @@ gemm_skinny_kernel(const bf16_t *__restrict__ X, int ldx, const bf16_t *__restri
 
 template <int NT, int MT, int WAVES>
 static int launch_epi(const void *X, int ldx, const void *W, int ldw, void *Y, int ldy, int M, int N, int K, int epi,
-                      hipStream_t stream) {
+                      const SkinnyExtra &ex, hipStream_t stream) {
     dim3 block(WAVES * WAVE);
     const dim3 grid((N + 16 * NT - 1) / (16 * NT));
-#define GO(E) gemm_skinny_kernel<NT, MT, E, WAVES><<<grid, block, 0, stream>>>((const bf16_t *)X, ldx, (const bf16_t *)W, ldw, Y, ldy, M, N, K)
+#define GO(E) gemm_skinny_kernel<NT, MT, E, WAVES><<<grid, block, 0, stream>>>((const bf16_t *)X, ldx, (const bf16_t *)W, ldw, Y, ldy, M, N, K, ex)
     switch (epi) {
     case EPI_BF16: GO(EPI_BF16); break;
     case EPI_F32: GO(EPI_F32); break;
     case EPI_ADD_F32: GO(EPI_ADD_F32); break;
+    case EPI_ADD_NORM:
+        if constexpr (MT == 1 && NT <= 2) { GO(EPI_ADD_NORM); break; }      // made for decoding: at most 16 rows
+        return LCU_UNSUPPORTED;
     default: return LCU_BAD_ARGUMENT;
     }
 #undef GO
@@ -199,10 +288,10 @@ static int launch_epi(const void *X, int ldx, const void *W, int ldw, void *Y, i
 
 template <int NT, int MT, int WAVES>
 static int launch_swiglu(const void *X, int ldx, const void *W, int ldw, void *Y, int ldy, int M, int N, int K,
-                         hipStream_t stream) {
+                         const SkinnyExtra &ex, hipStream_t stream) {
     const int groups = (N / 2 + 8 * NT - 1) / (8 * NT);
     gemm_skinny_kernel<NT, MT, EPI_SWIGLU, WAVES><<<dim3(groups), dim3(WAVES * WAVE), 0, stream>>>(
-        (const bf16_t *)X, ldx, (const bf16_t *)W, ldw, Y, ldy, M, N, K);
+        (const bf16_t *)X, ldx, (const bf16_t *)W, ldw, Y, ldy, M, N, K, ex);
     LCU_LAUNCH_CHECK();
     return LCU_OK;
 }
@@ -212,8 +301,8 @@ static int launch_swiglu(const void *X, int ldx, const void *W, int ldw, void *Y
 // M <= 64; K, ldx and ldw multiples of 8 (16-byte loads); tiles: output tiles of 16
 // features per workgroup (1, 2 or 4; more tiles reuse X more, fewer give more workgroups);
 // waves: 4 or 8 waves share a workgroup's K.
-LCU_API int lcu_gemm_skinny_bf16(const void *X, int ldx, const void *W, int ldw, void *Y, int ldy, int M, int N, int K,
-                                 int epilogue, int tiles, int waves, hipStream_t stream) {
+static int skinny_bf16(const void *X, int ldx, const void *W, int ldw, void *Y, int ldy, int M, int N, int K, int epilogue,
+                       int tiles, int waves, const SkinnyExtra &ex, hipStream_t stream) {
     if (M <= 0 || N <= 0) return LCU_OK;
     if (M > 64 || K <= 0 || K % 8 || ldx % 8 || ldw % 8 || ldx < K || ldw < K) return LCU_BAD_ARGUMENT;
     if (waves != 4 && waves != 8) return LCU_BAD_ARGUMENT;
@@ -221,8 +310,8 @@ LCU_API int lcu_gemm_skinny_bf16(const void *X, int ldx, const void *W, int ldw,
     if (epilogue == EPI_SWIGLU) {
         if (N % 2 || ldy < N / 2) return LCU_BAD_ARGUMENT;
         // tiles: gate and up tiles together (2: one of each, 4: two of each)
-#define SW(NT_, MT_) return waves == 8 ? launch_swiglu<NT_, MT_, 8>(X, ldx, W, ldw, Y, ldy, M, N, K, stream) \
-                                       : launch_swiglu<NT_, MT_, 4>(X, ldx, W, ldw, Y, ldy, M, N, K, stream)
+#define SW(NT_, MT_) return waves == 8 ? launch_swiglu<NT_, MT_, 8>(X, ldx, W, ldw, Y, ldy, M, N, K, ex, stream) \
+                                       : launch_swiglu<NT_, MT_, 4>(X, ldx, W, ldw, Y, ldy, M, N, K, ex, stream)
         if (tiles == 4 && mt <= 2) {
             if (mt == 1) SW(4, 1);
             SW(4, 2);
@@ -237,8 +326,8 @@ LCU_API int lcu_gemm_skinny_bf16(const void *X, int ldx, const void *W, int ldw,
     }
     if (ldy < N) return LCU_BAD_ARGUMENT;
     if (tiles == 4 && mt > 2) tiles = 2;      // 4 x 4 tiles of accumulators and operands do not fit the registers
-#define EP(NT_, MT_) return waves == 8 ? launch_epi<NT_, MT_, 8>(X, ldx, W, ldw, Y, ldy, M, N, K, epilogue, stream) \
-                                       : launch_epi<NT_, MT_, 4>(X, ldx, W, ldw, Y, ldy, M, N, K, epilogue, stream)
+#define EP(NT_, MT_) return waves == 8 ? launch_epi<NT_, MT_, 8>(X, ldx, W, ldw, Y, ldy, M, N, K, epilogue, ex, stream) \
+                                       : launch_epi<NT_, MT_, 4>(X, ldx, W, ldw, Y, ldy, M, N, K, epilogue, ex, stream)
 #define PICK(NT_)          \
     switch (mt) {          \
     case 1: EP(NT_, 1);    \
@@ -252,6 +341,39 @@ LCU_API int lcu_gemm_skinny_bf16(const void *X, int ldx, const void *W, int ldw,
 #undef PICK
 #undef EP
     return LCU_BAD_ARGUMENT;
+}
+
+LCU_API int lcu_gemm_skinny_bf16(const void *X, int ldx, const void *W, int ldw, void *Y, int ldy, int M, int N, int K,
+                                 int epilogue, int tiles, int waves, hipStream_t stream) {
+    if (epilogue == EPI_ADD_NORM) return LCU_BAD_ARGUMENT;
+    const SkinnyExtra none = {};
+    return skinny_bf16(X, ldx, W, ldw, Y, ldy, M, N, K, epilogue, tiles, waves, none, stream);
+}
+
+// The product that ends a branch, the residual sum and the next norm's weight in one kernel:
+// res[M, N] (float32, rows ldres apart) += X W^T; h_out[M, N] = bfloat16(res * norm_w), not yet
+// normalised; sumsq_out[M][ceil(N / (16 tiles))] = each workgroup's share of the rows' sums of
+// squares.  At most 16 rows, tiles 1 or 2.
+LCU_API int lcu_gemm_skinny_bf16_add_norm(const void *X, int ldx, const void *W, int ldw, float *res, int ldres, int M, int N,
+                                          int K, const void *norm_w, int norm_w_type, void *h_out, int ldh, float *sumsq_out,
+                                          int sumsq_cols, int tiles, int waves, hipStream_t stream) {
+    if (M > 16 || (tiles != 1 && tiles != 2) || !res || !norm_w || !h_out || !sumsq_out || ldh < N || ldres < N ||
+        (norm_w_type != LCU_F32 && norm_w_type != LCU_BF16) || sumsq_cols != (N + 16 * tiles - 1) / (16 * tiles))
+        return LCU_BAD_ARGUMENT;
+    SkinnyExtra ex = {};
+    ex.norm_w = norm_w; ex.norm_w_type = norm_w_type; ex.h_out = (bf16_t *)h_out; ex.ldh = ldh; ex.sumsq_out = sumsq_out;
+    return skinny_bf16(X, ldx, W, ldw, res, ldres, M, N, K, EPI_ADD_NORM, tiles, waves, ex, stream);
+}
+
+// A product whose rows of X wait for their normalisation: row i of the product is multiplied by
+// rsqrt(sum(sumsq_in[i][0 .. n_in)) / norm_width + eps) before the epilogue (not EPI_ADD_NORM).
+LCU_API int lcu_gemm_skinny_bf16_scaled(const void *X, int ldx, const void *W, int ldw, void *Y, int ldy, int M, int N, int K,
+                                        int epilogue, int tiles, int waves, const float *sumsq_in, int n_in, int norm_width,
+                                        float eps, hipStream_t stream) {
+    if (epilogue == EPI_ADD_NORM || !sumsq_in || n_in <= 0 || norm_width <= 0) return LCU_BAD_ARGUMENT;
+    SkinnyExtra ex = {};
+    ex.sumsq_in = sumsq_in; ex.n_in = n_in; ex.norm_width = norm_width; ex.eps = eps;
+    return skinny_bf16(X, ldx, W, ldw, Y, ldy, M, N, K, epilogue, tiles, waves, ex, stream);
 }
 
 

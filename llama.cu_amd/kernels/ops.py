@@ -459,10 +459,14 @@ def _skinny_tiles(n_features: int, m: int) -> int:
 
 def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = None,
                 out_dtype: Optional[torch.dtype] = None, accumulate: bool = False, swiglu: bool = False,
-                tiles: Optional[int] = None, waves: Optional[int] = None) -> torch.Tensor:
+                tiles: Optional[int] = None, waves: Optional[int] = None,
+                row_sumsq: Optional[torch.Tensor] = None, norm_width: int = 0, eps: float = 0.0) -> torch.Tensor:
     """``out (+)= x @ w.T`` for at most 64 rows of bfloat16 ``x`` by streaming ``w`` once.
-    ``swiglu``: ``w`` holds gate rows, then up rows; ``out = silu(x @ gate.T) * (x @ up.T)``."""
-    _gpu(x, w, out)
+    ``swiglu``: ``w`` holds gate rows, then up rows; ``out = silu(x @ gate.T) * (x @ up.T)``.
+    ``row_sumsq [m, parts]``: the rows of ``x`` wait for their normalisation (see
+    ``gemm_skinny_add_norm``); row ``i`` of the product is multiplied by
+    ``rsqrt(sum(row_sumsq[i]) / norm_width + eps)`` before the epilogue."""
+    _gpu(x, w, out, row_sumsq)
     _rows(x, "skinny x"); _rows(w, "skinny w")
     m, k = x.shape
     n = w.shape[0]
@@ -484,12 +488,54 @@ def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = 
     _rows(out, "skinny out")
     if out.shape != (m, width):
         raise KernelError(f"gemm_skinny out: shape {tuple(out.shape)}, expected {(m, width)}")
+    tiles = tiles or ((4 if m > 8 else 2) if swiglu else _skinny_tiles(width, m))
+    waves = waves or (8 if width <= 8192 else 4)
     lib = build.load("gemm_skinny")
+    if row_sumsq is not None:
+        if row_sumsq.dtype != torch.float32 or row_sumsq.dim() != 2 or row_sumsq.shape[0] != m or not row_sumsq.is_contiguous() \
+                or norm_width <= 0:
+            raise KernelError("gemm_skinny: row_sumsq must be a contiguous float32 [rows, parts] tensor, with the norm's width")
+        _check(lib.lcu_gemm_skinny_bf16_scaled(_ptr(x), x.stride(0), _ptr(w), w.stride(0), _ptr(out), out.stride(0), m, n, k,
+                                               _EPILOGUES[epi], tiles, waves, _ptr(row_sumsq), row_sumsq.shape[1],
+                                               int(norm_width), ctypes.c_float(eps), _stream()), "gemm_skinny (scaled rows)")
+        return out
     _check(lib.lcu_gemm_skinny_bf16(_ptr(x), x.stride(0), _ptr(w), w.stride(0), _ptr(out), out.stride(0), m, n, k,
-                                    _EPILOGUES[epi], tiles or ((4 if m > 8 else 2) if swiglu else _skinny_tiles(width, m)),
-                                    waves or (8 if width <= 8192 else 4), _stream()),
+                                    _EPILOGUES[epi], tiles, waves, _stream()),
            "gemm_skinny")
     return out
+
+
+ADD_NORM_MAX_ROWS = 16
+
+
+def gemm_skinny_add_norm(x: torch.Tensor, w: torch.Tensor, residual: torch.Tensor, norm_weight: torch.Tensor,
+                         tiles: Optional[int] = None, waves: Optional[int] = None):
+    """The product that ends a branch, the residual sum and the next norm's weight in one
+    kernel: ``residual += x @ w.T`` (float32, in place); returns ``(h, sumsq)`` with
+    ``h = bfloat16(residual * norm_weight)``, not yet normalised, and ``sumsq [rows, parts]``,
+    the workgroups' shares of each row's sum of squares, for ``gemm_skinny(..., row_sumsq=)``.
+    At most 16 rows."""
+    _gpu(x, w, residual, norm_weight)
+    _rows(x, "skinny x"); _rows(w, "skinny w"); _rows(residual, "residual")
+    m, k = x.shape
+    n = w.shape[0]
+    if w.shape[1] != k or m > ADD_NORM_MAX_ROWS or not skinny_supported(x, w, torch.float32):
+        raise KernelError(f"gemm_skinny_add_norm: x {tuple(x.shape)} {x.dtype} with w {tuple(w.shape)} {w.dtype} is not supported")
+    if residual.dtype != torch.float32 or residual.shape != (m, n):
+        raise KernelError(f"gemm_skinny_add_norm: the residual must be float32 {(m, n)}")
+    if norm_weight.shape != (n,) or not norm_weight.is_contiguous():
+        raise KernelError(f"gemm_skinny_add_norm: the norm's weight must be a contiguous [{n}] tensor")
+    tiles = tiles or (1 if n <= 8192 else 2)
+    waves = waves or (8 if n <= 8192 else 4)
+    parts = (n + 16 * tiles - 1) // (16 * tiles)
+    h = torch.empty((m, n), dtype=torch.bfloat16, device=x.device)
+    sumsq = torch.empty((m, parts), dtype=torch.float32, device=x.device)
+    lib = build.load("gemm_skinny")
+    _check(lib.lcu_gemm_skinny_bf16_add_norm(_ptr(x), x.stride(0), _ptr(w), w.stride(0), _ptr(residual), residual.stride(0),
+                                             m, n, k, _ptr(norm_weight), _type(norm_weight, "norm weight"), _ptr(h),
+                                             h.stride(0), _ptr(sumsq), parts, tiles, waves, _stream()),
+           "gemm_skinny_add_norm")
+    return h, sumsq
 
 
 def skinny_f32_supported(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype) -> bool:

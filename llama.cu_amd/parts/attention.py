@@ -14,8 +14,8 @@ from typing import Dict, Optional
 import torch
 
 from ..kernels import ops
-from .base import BuildContext, PagedKV, Part, PartSpec, TensorSpec, make_part, register_part
-from .linear import linear
+from .base import BuildContext, PagedKV, Part, PartSpec, ScaledRows, TensorSpec, make_part, register_part
+from .linear import linear, linear_into_norm
 
 
 class Attention(Part):
@@ -60,7 +60,11 @@ class Attention(Part):
         self.page_size = build.page_size
         self.dtype = build.dtype
 
-    def forward(self, h: torch.Tensor, step, cache) -> torch.Tensor:
+    # forward(..., into=(residual, norm)) may end with the residual sum and that norm's weight
+    # in the output projection and return ScaledRows instead of the branch's output
+    ends_in_norm = True
+
+    def forward(self, h: torch.Tensor, step, cache, into=None):
         nh, nkv, dh = self.heads, self.kv_heads, self.head_dim
         qkv = linear(h, self.w_qkv, out_dtype=self.dtype)
         self.position.apply(qkv, step.positions, nh, 0 if self.shares_kv else nkv, dh)
@@ -76,6 +80,11 @@ class Attention(Part):
         out = torch.empty((h.shape[0], nh * dh), dtype=self.dtype, device=h.device)
         ops.paged_attention(qkv, out, cache.pages, step, cache.group, nh, nkv, dh, self.page_size, self.scale,
                             self.window)
+        if into is not None:
+            residual, norm = into
+            fused = linear_into_norm(out, self.w_o, residual, norm.weight)
+            if fused is not None:
+                return ScaledRows(fused[0], fused[1], norm.size, norm.eps)
         return linear(out, self.w_o, out_dtype=self.dtype)
 
 

@@ -99,6 +99,21 @@ class BuildContext:
     page_size: int
 
 
+@dataclass
+class ScaledRows:
+    """Rows on their way from a norm to a matrix product whose normalisation is still to be
+    applied: the norm's weight is in already, and row ``i`` of whatever is multiplied with
+    them is to be multiplied by ``rsqrt(sum(sumsq[i]) / width + eps)``.  A mixer that can end
+    with the residual sum and the next norm's weight in its last product hands these to a
+    feed-forward that can apply the factor in its first product's epilogue, and no norm
+    kernel runs between them.  A part that does not know of this never sees one: the block
+    offers it only to parts that say they take it."""
+    rows: torch.Tensor          # [n, width], the compute type
+    sumsq: torch.Tensor         # [n, parts] float32 shares of the rows' sums of squares
+    width: int
+    eps: float
+
+
 class Part:
     # Whether a step through this part may be captured into a graph and replayed: true only
     # if all it does is launch work on the current stream whose shape depends on the batch's

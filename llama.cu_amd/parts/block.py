@@ -13,7 +13,7 @@ from typing import Dict, Optional
 
 import torch
 
-from .base import BuildContext, Part, PartSpec, TensorSpec, make_part, prefixed, register_part
+from .base import BuildContext, Part, PartSpec, ScaledRows, TensorSpec, make_part, prefixed, register_part
 
 
 class PreNormBlock(Part):
@@ -24,6 +24,9 @@ class PreNormBlock(Part):
         self.norm2 = make_part("norm", norm2)
         self.ffn = make_part("ffn", ffn)
         self.graph_safe = all(p.graph_safe for p in (self.norm1, self.mixer, self.norm2, self.ffn))
+        # parts that say so may pass rows between them whose normalisation is still to be applied
+        self._fuse = (getattr(self.mixer, "ends_in_norm", False) and getattr(self.norm2, "deferrable", False)
+                      and callable(getattr(self.ffn, "takes_scaled_rows", None)))
 
     def _children(self):
         return [(self.specs[k].name, getattr(self, k)) for k in ("norm1", "mixer", "norm2", "ffn")]
@@ -45,7 +48,14 @@ class PreNormBlock(Part):
 
     def forward(self, x: torch.Tensor, pending: Optional[torch.Tensor], step, cache) -> torch.Tensor:
         h = self.norm1.forward(x, pending)
-        a = self.mixer.forward(h, step, cache)
+        if self._fuse and self.ffn.takes_scaled_rows(h):
+            # the mixer may end with the residual sum and the second norm's weight in its last
+            # product; then the feed-forward applies the norm's factor in its first one
+            a = self.mixer.forward(h, step, cache, into=(x, self.norm2))
+            if isinstance(a, ScaledRows):
+                return self.ffn.forward(a)
+        else:
+            a = self.mixer.forward(h, step, cache)
         h2 = self.norm2.forward(x, a)
         return self.ffn.forward(h2)
 

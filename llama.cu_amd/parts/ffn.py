@@ -12,7 +12,7 @@ from typing import Dict
 import torch
 
 from ..kernels import ops
-from .base import BuildContext, Part, TensorSpec, register_part
+from .base import BuildContext, Part, ScaledRows, TensorSpec, register_part
 from .linear import linear
 
 
@@ -36,7 +36,18 @@ class SwiGLU(Part):
         self.w_down = tensors["down_proj.weight"].contiguous()
         self.dtype = build.dtype
 
-    def forward(self, h: torch.Tensor) -> torch.Tensor:
+    def takes_scaled_rows(self, h: torch.Tensor) -> bool:
+        """Whether ``forward`` could be given ScaledRows in the place of rows like ``h``: the
+        factor then goes into the first product's epilogue."""
+        return (self.dtype == torch.bfloat16 and h.shape[0] <= ops.ADD_NORM_MAX_ROWS
+                and ops.skinny_supported(h, self.w_gate_up, self.dtype))
+
+    def forward(self, h) -> torch.Tensor:
+        if isinstance(h, ScaledRows):
+            if not ops.skinny_supported(h.rows, self.w_gate_up, self.dtype):
+                raise ops.KernelError("feed-forward: rows that wait for their normalisation need the kernel for few rows")
+            act = ops.gemm_skinny(h.rows, self.w_gate_up, swiglu=True, row_sumsq=h.sumsq, norm_width=h.width, eps=h.eps)
+            return linear(act, self.w_down, out_dtype=self.dtype)
         if self.dtype == torch.bfloat16 and h.shape[0] <= ops.SKINNY_ROWS and ops.skinny_supported(h, self.w_gate_up, self.dtype):
             # few rows: one pass over the weights, the activation in the product's epilogue
             act = ops.gemm_skinny(h, self.w_gate_up, swiglu=True)

@@ -40,3 +40,14 @@ def linear(x: torch.Tensor, weight: torch.Tensor, out_dtype: Optional[torch.dtyp
     if ops.skinny_f32_supported(x, weight, out_dtype):
         return ops.gemm_skinny_f32(x, weight, out=out, accumulate=accumulate)
     return ops.gemm_nt(x, weight, out=out, out_dtype=out_dtype, accumulate=accumulate)
+
+
+def linear_into_norm(a: torch.Tensor, weight: torch.Tensor, residual: torch.Tensor, norm_weight: torch.Tensor):
+    """``residual += a @ weight.T`` and the rows for the product after the next norm, in one
+    kernel: returns ``(rows, sumsq)`` for a ``ScaledRows``, or None if the kernel for it does
+    not take these operands (then nothing has been done)."""
+    if not (a.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and a.shape[0] <= ops.ADD_NORM_MAX_ROWS
+            and residual.dtype == torch.float32 and ops.skinny_supported(a, weight, torch.float32)
+            and norm_weight.dtype in (torch.bfloat16, torch.float32)):
+        return None
+    return ops.gemm_skinny_add_norm(a, weight, residual, norm_weight)

@@ -37,4 +37,10 @@ class RMSNorm(Part):
         return ops.rmsnorm(x, self.weight, self.eps, out, delta=delta, write_back=True)
 
 
+    # This norm is a factor per row times a weight per column, so its factor may be applied
+    # after a matrix product instead of before (see ScaledRows); whoever does that reads
+    # ``weight``, ``size`` and ``eps``.
+    deferrable = True
+
+
 register_part("norm", "rmsnorm", RMSNorm)

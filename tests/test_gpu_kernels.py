@@ -433,6 +433,53 @@ def test_gemm_skinny_refuses_what_it_cannot_take():
     assert not ops.skinny_supported(rnd(65, 64).to(torch.bfloat16).cuda(), rnd(16, 64).to(torch.bfloat16).cuda(), torch.bfloat16)
 
 
+@pytest.mark.parametrize("m,n,k,tiles,wdtype", [(1, 16, 8, 1, "bfloat16"), (8, 304, 136, 1, "float32"), (16, 4096, 1000, 1, "bfloat16"),
+                                                (5, 104, 64, 2, "bfloat16"), (13, 1000, 4096, 2, "float32")])
+def test_gemm_skinny_residual_sum_and_norm_weight_in_the_epilogue(m, n, k, tiles, wdtype):
+    """``residual += x w^T``; the new rows times the norm's weight as bfloat16, not yet normalised;
+    the workgroups' shares of the rows' sums of squares.  Then a second product applies the
+    norm's factor per row in its epilogue, plain and with SwiGLU: together they equal residual
+    sum, RMS norm and product done one after the other."""
+    from llama_cu_amd.kernels import ops
+    eps = 1e-5
+    x = rnd(m, k, seed=m + k).to(torch.bfloat16)
+    w = rnd(n, k, seed=n, scale=0.3).to(torch.bfloat16)
+    res = rnd(m, n, seed=3) * 3.0
+    nw = (1.0 + 0.2 * rnd(n, seed=4)).to(DT[wdtype])
+    res_g = res.clone().cuda()
+    h, sumsq = ops.gemm_skinny_add_norm(x.cuda(), w.cuda(), res_g, nw.cuda(), tiles=tiles)
+    new = res.double() + plain.linear(x, w)
+    close(res_g, new, "float32", "residual")
+    assert sumsq.shape == (m, (n + 16 * tiles - 1) // (16 * tiles))
+    close(sumsq.sum(dim=1), (new ** 2).sum(dim=1), "float32", "sums of squares")
+    close(h, new * nw.double()[None, :], "bfloat16", "rows with the norm's weight")
+    # the product that follows: n features in, n2 out
+    n2 = 72
+    w2 = rnd(2 * n2, n, seed=5, scale=0.2).to(torch.bfloat16)
+    normed = plain.rms_norm(new, nw, eps)
+    got = ops.gemm_skinny(h, w2.cuda(), row_sumsq=sumsq, norm_width=n, eps=eps)
+    close(got, plain.linear(normed, w2), "bfloat16", "scaled product")
+    got = ops.gemm_skinny(h, w2.cuda(), swiglu=True, row_sumsq=sumsq, norm_width=n, eps=eps)
+    gu = plain.linear(normed, w2)
+    close(got, plain.swiglu(gu[:, :n2], gu[:, n2:]), "bfloat16", "scaled product with SwiGLU")
+    # the same shares on every call: no atomics
+    res_g2 = res.clone().cuda()
+    h2, sumsq2 = ops.gemm_skinny_add_norm(x.cuda(), w.cuda(), res_g2, nw.cuda(), tiles=tiles)
+    assert torch.equal(sumsq, sumsq2) and torch.equal(h, h2) and torch.equal(res_g, res_g2)
+
+
+def test_gemm_skinny_add_norm_refuses_what_it_cannot_take():
+    from llama_cu_amd.kernels import ops
+    x = rnd(17, 64).to(torch.bfloat16).cuda()
+    w = rnd(32, 64).to(torch.bfloat16).cuda()
+    with pytest.raises(ops.KernelError):
+        ops.gemm_skinny_add_norm(x, w, torch.zeros(17, 32).cuda(), torch.ones(32).cuda())        # more than 16 rows
+    with pytest.raises(ops.KernelError):
+        ops.gemm_skinny_add_norm(x[:4], w, torch.zeros(4, 32, dtype=torch.bfloat16).cuda(), torch.ones(32).cuda())
+    with pytest.raises(ops.KernelError):
+        ops.gemm_skinny(x[:4], w, row_sumsq=torch.zeros(3, 2).cuda(), norm_width=64, eps=1e-5)    # rows do not match
+
+
 @pytest.mark.parametrize("m,n,k", [(1, 16, 4), (8, 301, 172), (17, 100, 64), (70, 4096, 352), (300, 1000, 4096)])
 def test_gemm_skinny_f32(m, n, k):
     from llama_cu_amd.kernels import ops
