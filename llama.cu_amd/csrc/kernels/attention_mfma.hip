@@ -237,7 +237,10 @@ __device__ __forceinline__ void load_q(const bf16_t *__restrict__ qrow, bool val
 }
 
 // ============================================================================ decode
-constexpr int DEC_WAVES = 4;
+#ifndef LCU_DEC_WAVES
+#define LCU_DEC_WAVES 4
+#endif
+constexpr int DEC_WAVES = LCU_DEC_WAVES;
 #ifndef LCU_DEC_MIN_WAVES
 #define LCU_DEC_MIN_WAVES 2      // two waves per SIMD: measured faster than one with more registers
 #endif

@@ -99,8 +99,8 @@ class ModelRunner:
         self.builder = BatchBuilder(self.cache, self.max_batch_tokens, self.max_seqs, max_pages, self.device)
         # captured decode steps, by batch size: (graph, its logits tensor)
         self.use_graphs = bool(use_graphs) and self.model.graph_safe
-        self._graphs: Dict[int, Any] = {}
-        self._seen: Dict[int, int] = {}
+        self._graphs: Dict[tuple, Any] = {}        # (batch size, key parts) -> (graph, its logits)
+        self._seen: Dict[tuple, int] = {}
 
     # ------------------------------------------------------------ construction helpers
     @classmethod
@@ -168,29 +168,32 @@ class ModelRunner:
         b = step.n_req
         if not (self.use_graphs and step.decode_only and step.n_logits == b and b <= self.GRAPH_MAX_BATCH):
             return self.model.forward(step, self.caches)
-        # the number of key parts of the decode attention must not change between replays
-        step.attn_splits = self._decode_splits(b)
-        entry = self._graphs.get(b)
+        # the number of key parts of the decode attention must not change between replays: a
+        # graph is made for a batch size and a number of parts (which follows the longest
+        # context rounded up to a power of two, so it changes rarely)
+        step.attn_splits = self._decode_splits(b, step.max_ctx_len)
+        key = (b, step.attn_splits)
+        entry = self._graphs.get(key)
         if entry is None:
-            self._seen[b] = self._seen.get(b, 0) + 1
-            if self._seen[b] <= self.GRAPH_AFTER:
+            self._seen[key] = self._seen.get(key, 0) + 1
+            if self._seen[key] <= self.GRAPH_AFTER:
                 return self.model.forward(step, self.caches)
             torch.cuda.synchronize(self.device)
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph):
                 logits = self.model.forward(step, self.caches)
-            entry = self._graphs[b] = (graph, logits)
+            entry = self._graphs[key] = (graph, logits)
         graph, logits = entry
         graph.replay()
         return logits
 
-    def _decode_splits(self, batch: int) -> int:
+    def _decode_splits(self, batch: int, max_ctx_len: int) -> int:
         from ..kernels.ops import decode_splits
         best = 1
         for need in self.model.cache_needs():
             if isinstance(need, PagedKV):
                 heads = getattr(self.model.layers[0].mixer, "heads", need.kv_heads)
-                best = max(best, decode_splits(batch, heads, need.kv_heads, self.max_model_len))
+                best = max(best, decode_splits(batch, heads, need.kv_heads, max_ctx_len))
         return best
 
     def step(self, req_ids: Sequence[int], tokens: Sequence[Sequence[int]],

@@ -381,10 +381,14 @@ def attention_prefill(q, out, cache, block_table, q_start, ctx_len, task_req, ta
 
 def decode_splits(n_req: int, n_heads: int, n_kv_heads: int, max_ctx_len: int) -> int:
     """Into how many parts the decode kernel cuts each request's keys: about one workgroup
-    for each of the 256 compute units, no part shorter than 256 keys (measured: more parts
-    cost more in the merge than they gain)."""
+    for each of the 256 compute units, no part shorter than 512 keys, at most 32 parts
+    (measured on the Llama-3-8B shape from 2k to 128k keys: more parts cost more in the merge
+    than they gain; a single request with 128k keys wants 32).  The length counts rounded up
+    to a power of two, so that a growing context changes the choice, and with it the
+    rounding of the result and the captured graph that fits, only rarely."""
     base = n_req * n_kv_heads * ((n_heads // n_kv_heads + 15) // 16)
-    return max(1, min(8, 256 // max(base, 1), (max_ctx_len + 255) // 256))
+    rounded = 1 << max(int(max_ctx_len) - 1, 0).bit_length()     # up to a power of two: the choice changes rarely
+    return max(1, min(32, 256 // max(base, 1), rounded // 512))
 
 
 def paged_attention(q: torch.Tensor, out: torch.Tensor, cache: torch.Tensor, step, group: int, n_heads: int,

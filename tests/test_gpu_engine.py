@@ -156,7 +156,7 @@ def test_captured_decode_steps_equal_eager_ones():
 
     eager, _ = decode(False)
     graphed, runner = decode(True)
-    assert 3 in runner._graphs                              # the batch size was captured and replayed
+    assert any(key[0] == 3 for key in runner._graphs)       # the batch size was captured and replayed
     for i, (a, b) in enumerate(zip(eager, graphed)):
         assert torch.equal(a, b), f"decode step {i} differs between eager and captured"
 

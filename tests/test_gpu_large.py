@@ -49,5 +49,5 @@ def test_whole_portions_and_decoding_at_full_layer_sizes(big, dtype):
         for i, n in enumerate(names):
             got[n][head[n] + k] = logits[i]
     if dtype == "bfloat16":
-        assert 2 in runner._graphs
+        assert any(key[0] == 2 for key in runner._graphs)
     common.assert_matches_plain(got, want, dtype, f"8B-sized layers/{dtype}")
