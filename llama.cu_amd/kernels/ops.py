@@ -442,6 +442,12 @@ def skinny_supported(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype) -
             and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
 
 
+def skinny_weight_ok(w: torch.Tensor) -> bool:
+    """Whether the weight-streaming kernel takes ``w`` as its weight (for any rows it takes)."""
+    return (w.dtype == torch.bfloat16 and w.dim() == 2 and w.is_cuda and w.shape[1] % 8 == 0 and w.stride(1) == 1
+            and w.stride(0) % 8 == 0 and w.data_ptr() % 16 == 0)
+
+
 def skinny_preferred(m: int, n: int, k: int, out_dtype: torch.dtype) -> bool:
     """Whether the weight-streaming kernel is the faster choice for a plain bfloat16 product
     of ``m`` rows with an ``[n, k]`` weight (measured against the library on the Llama-3-8B

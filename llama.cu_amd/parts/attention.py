@@ -64,9 +64,20 @@ class Attention(Part):
     # in the output projection and return ScaledRows instead of the branch's output
     ends_in_norm = True
 
-    def forward(self, h: torch.Tensor, step, cache, into=None):
+    def takes_scaled_rows(self, n_rows: int) -> bool:
+        """Whether ``forward`` could be given ScaledRows of ``n_rows`` rows in the place of
+        plain rows: only where the kernel for few rows is the faster one for the q, k, v
+        product anyway."""
+        return (self.dtype == torch.bfloat16 and n_rows <= ops.ADD_NORM_MAX_ROWS and ops.skinny_weight_ok(self.w_qkv)
+                and ops.skinny_preferred(n_rows, self.w_qkv.shape[0], self.w_qkv.shape[1], self.dtype))
+
+    def forward(self, h, step, cache, into=None):
         nh, nkv, dh = self.heads, self.kv_heads, self.head_dim
-        qkv = linear(h, self.w_qkv, out_dtype=self.dtype)
+        if isinstance(h, ScaledRows):
+            qkv = ops.gemm_skinny(h.rows, self.w_qkv, row_sumsq=h.sumsq, norm_width=h.width, eps=h.eps)
+            h = h.rows
+        else:
+            qkv = linear(h, self.w_qkv, out_dtype=self.dtype)
         self.position.apply(qkv, step.positions, nh, 0 if self.shares_kv else nkv, dh)
         rot = self.position.rotary_tables()
         cos, sin, rot_dim, pairing = rot if rot is not None else (None, None, 0, 0)

@@ -46,18 +46,32 @@ class PreNormBlock(Part):
     def cache_need(self):
         return self.mixer.cache_need()
 
-    def forward(self, x: torch.Tensor, pending: Optional[torch.Tensor], step, cache) -> torch.Tensor:
-        h = self.norm1.forward(x, pending)
-        if self._fuse and self.ffn.takes_scaled_rows(h):
+    ends_in_next_norm = True     # forward takes ``next_norm``
+
+    def takes_scaled_rows(self, n_rows: int) -> bool:
+        """Whether ``forward`` could be given, as ``pending``, ScaledRows of ``n_rows`` rows made
+        with this block's first norm in the place of the last branch's output."""
+        fn = getattr(self.mixer, "takes_scaled_rows", None)
+        return getattr(self.norm1, "deferrable", False) and callable(fn) and fn(n_rows)
+
+    def forward(self, x: torch.Tensor, pending, step, cache, next_norm=None):
+        """``pending``: the last branch's output, not yet added to ``x`` (or None, or ScaledRows
+        made with ``norm1`` by the block before, the sum then being in ``x`` already).
+        ``next_norm``: the norm that will follow this block, if whoever runs it takes
+        ScaledRows; then the feed-forward may end in it.  Returns the new ``pending``."""
+        h = pending if isinstance(pending, ScaledRows) else self.norm1.forward(x, pending)
+        n_rows = x.shape[0]
+        ffn_into = (x, next_norm) if next_norm is not None and getattr(self.ffn, "ends_in_norm", False) else None
+        if self._fuse and self.ffn.takes_scaled_rows(n_rows):
             # the mixer may end with the residual sum and the second norm's weight in its last
             # product; then the feed-forward applies the norm's factor in its first one
             a = self.mixer.forward(h, step, cache, into=(x, self.norm2))
             if isinstance(a, ScaledRows):
-                return self.ffn.forward(a)
+                return self.ffn.forward(a, into=ffn_into) if ffn_into else self.ffn.forward(a)
         else:
             a = self.mixer.forward(h, step, cache)
         h2 = self.norm2.forward(x, a)
-        return self.ffn.forward(h2)
+        return self.ffn.forward(h2, into=ffn_into) if ffn_into else self.ffn.forward(h2)
 
 
 register_part("block", "prenorm", PreNormBlock)

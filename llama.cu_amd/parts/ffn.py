@@ -13,7 +13,7 @@ import torch
 
 from ..kernels import ops
 from .base import BuildContext, Part, ScaledRows, TensorSpec, register_part
-from .linear import linear
+from .linear import linear, linear_into_norm
 
 
 class SwiGLU(Part):
@@ -36,24 +36,33 @@ class SwiGLU(Part):
         self.w_down = tensors["down_proj.weight"].contiguous()
         self.dtype = build.dtype
 
-    def takes_scaled_rows(self, h: torch.Tensor) -> bool:
-        """Whether ``forward`` could be given ScaledRows in the place of rows like ``h``: the
-        factor then goes into the first product's epilogue."""
-        return (self.dtype == torch.bfloat16 and h.shape[0] <= ops.ADD_NORM_MAX_ROWS
-                and ops.skinny_supported(h, self.w_gate_up, self.dtype))
+    def takes_scaled_rows(self, n_rows: int) -> bool:
+        """Whether ``forward`` could be given ScaledRows of ``n_rows`` rows in the place of
+        plain rows: the factor then goes into the first product's epilogue."""
+        return self.dtype == torch.bfloat16 and n_rows <= ops.ADD_NORM_MAX_ROWS and ops.skinny_weight_ok(self.w_gate_up)
 
-    def forward(self, h) -> torch.Tensor:
+    # forward(..., into=(residual, norm)) may end with the residual sum and that norm's weight
+    # in the down projection and return ScaledRows instead of the branch's output
+    ends_in_norm = True
+
+    def forward(self, h, into=None):
         if isinstance(h, ScaledRows):
             if not ops.skinny_supported(h.rows, self.w_gate_up, self.dtype):
                 raise ops.KernelError("feed-forward: rows that wait for their normalisation need the kernel for few rows")
             act = ops.gemm_skinny(h.rows, self.w_gate_up, swiglu=True, row_sumsq=h.sumsq, norm_width=h.width, eps=h.eps)
-            return linear(act, self.w_down, out_dtype=self.dtype)
-        if self.dtype == torch.bfloat16 and h.shape[0] <= ops.SKINNY_ROWS and ops.skinny_supported(h, self.w_gate_up, self.dtype):
+        elif self.dtype == torch.bfloat16 and h.shape[0] <= ops.SKINNY_ROWS and ops.skinny_supported(h, self.w_gate_up, self.dtype):
             # few rows: one pass over the weights, the activation in the product's epilogue
             act = ops.gemm_skinny(h, self.w_gate_up, swiglu=True)
         else:
             gu = linear(h, self.w_gate_up, out_dtype=self.dtype)
             act = ops.swiglu(gu)
+        if into is not None and act.dtype == torch.bfloat16 and ops.skinny_preferred(
+                act.shape[0], self.w_down.shape[0], self.w_down.shape[1], torch.bfloat16):
+            # only where the kernel for few rows is the faster one for this product anyway
+            residual, norm = into
+            fused = linear_into_norm(act, self.w_down, residual, norm.weight)
+            if fused is not None:
+                return ScaledRows(fused[0], fused[1], norm.size, norm.eps)
         return linear(act, self.w_down, out_dtype=self.dtype)
 
 

@@ -122,8 +122,15 @@ class DecoderModel:
         with ops.stream_scope():                  # the whole pass goes to one stream, asked for once
             x = self.embedding.forward(step.tokens)
             pending = None
-            for i, e in enumerate(self.spec.run_order):
-                pending = self.layers[e.layer].forward(x, pending, step, caches[i])
+            order = self.spec.run_order
+            for i, e in enumerate(order):
+                # a block may end in the next block's first norm, if that block takes such rows
+                follower = self.layers[order[i + 1].layer] if i + 1 < len(order) else None
+                takes = getattr(follower, "takes_scaled_rows", None)
+                if callable(takes) and getattr(self.layers[e.layer], "ends_in_next_norm", False) and takes(x.shape[0]):
+                    pending = self.layers[e.layer].forward(x, pending, step, caches[i], next_norm=follower.norm1)
+                else:
+                    pending = self.layers[e.layer].forward(x, pending, step, caches[i])
             if step.n_logits == 0:
                 return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=x.device)
             xs = ops.gather_rows(x, step.logit_rows)
