@@ -6,7 +6,7 @@
 // returns the first entry with c[i] >= p (llama.cu/src/op/random_sample/sample.cuh:71-87,
 // 186-207, with library sort, scan and reduce).  The same token comes out here without
 // sorting: the entry with c[i] >= p is found by a radix select over the bit patterns of
-// the logits, most significant byte first, on histograms of counts and of weights.
+// the logits, most significant digit first, on histograms of counts and of weights.
 // Weights are summed as 64-bit fixed-point integers (w * 2^45), so the sums do not
 // depend on the order of the additions and a draw is reproducible bit for bit.  Equal
 // logits are ordered by index, as a stable sort orders them.
@@ -27,6 +27,20 @@ __device__ __forceinline__ float key_value(uint32_t k) {
 __device__ __forceinline__ unsigned long long fixed_weight(float logit, float max_logit, float inv_t) {
     const float w = expf((logit - max_logit) * inv_t);
     return (unsigned long long)((double)w * FIXED_ONE);
+}
+
+// Every element of a row, for the threads of a block together: four neighbouring logits per
+// load where the row allows it and several loads in flight (a row is read by one workgroup,
+// so latency, not bandwidth, is what counts).  f(index, value); no order is promised.
+template <class F>
+__device__ __forceinline__ void scan_row(const float *__restrict__ row, int vocab, F f) {
+    const int vec_end = (((size_t)row % 16) == 0) ? (vocab / 4) * 4 : 0;
+#pragma unroll 4
+    for (int i = threadIdx.x * 4; i < vec_end; i += blockDim.x * 4) {
+        const float4 v = *(const float4 *)(row + i);
+        f(i, v.x); f(i + 1, v.y); f(i + 2, v.z); f(i + 3, v.w);
+    }
+    for (int i = vec_end + threadIdx.x; i < vocab; i += blockDim.x) f(i, row[i]);
 }
 
 // ---------------------------------------------------------------- arg-max
@@ -84,47 +98,110 @@ struct SelectState {
     unsigned long long mass_above;     // their summed weights
 };
 
+// The digits of the radix select, most significant first: 12, 12 and 8 bits.  The first digit
+// holds the sign, the exponent and three bits of the mantissa: with one byte (sign and seven
+// bits of the exponent) nearly all logits of a row fall into a handful of bins and their
+// atomic additions queue up behind each other.
+constexpr int SELECT_PASSES = 3;
+constexpr int SELECT_BINS = 4096;
+__device__ __forceinline__ int select_shift(int pass) { return pass == 0 ? 20 : (pass == 1 ? 8 : 0); }
+__device__ __forceinline__ int select_bits(int pass) { return pass == 2 ? 8 : 12; }
+
+struct SelectScratch {
+    unsigned int cnt[SELECT_BINS];
+    unsigned long long mass[SELECT_BINS];
+    unsigned int wave_cnt[SAMPLE_THREADS / WAVE];
+    unsigned long long wave_mass[SAMPLE_THREADS / WAVE];
+    int best, last_nonempty;
+    SelectState st;
+};
+
 // One radix select over the row.  by_mass == 0: the target-th largest entry (target >= 1).
 // by_mass == 1: the first entry, in descending order, whose inclusive prefix sum of weights
 // reaches target.  On return st.prefix is that entry's key and the two sums count what is
-// strictly larger.
+// strictly larger.  Every thread of the block must call it.
 __device__ void radix_select(const float *row, int vocab, float max_logit, float inv_t, int by_mass,
-                             unsigned long long target, SelectState &st, unsigned int *cnt,
-                             unsigned long long *mass, SelectState *shared_st) {
+                             unsigned long long target, SelectState &st, SelectScratch &sc) {
     st.prefix = 0; st.count_above = 0; st.mass_above = 0;
-    for (int pass = 0; pass < 4; ++pass) {
-        const int shift = 24 - 8 * pass;
-        for (int d = threadIdx.x; d < 256; d += blockDim.x) { cnt[d] = 0; mass[d] = 0; }
+    const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE, nwaves = blockDim.x / WAVE;
+    for (int pass = 0; pass < SELECT_PASSES; ++pass) {
+        const int shift = select_shift(pass), bits = select_bits(pass), nbins = 1 << bits;
+        for (int d = threadIdx.x; d < SELECT_BINS; d += blockDim.x) { sc.cnt[d] = 0; sc.mass[d] = 0; }
+        if (threadIdx.x == 0) { sc.best = SELECT_BINS; sc.last_nonempty = -1; }
         __syncthreads();
-        for (int i = threadIdx.x; i < vocab; i += blockDim.x) {
-            const float v = row[i];
+        const int above = shift + bits;                      // the bits that earlier passes have fixed
+        const uint32_t fixed = st.prefix;
+        scan_row(row, vocab, [&](int, float v) {
             const uint32_t k = order_key(v);
-            if (pass > 0 && (k >> (shift + 8)) != (st.prefix >> (shift + 8))) continue;
-            const int d = (k >> shift) & 255;
-            atomicAdd(&cnt[d], 1u);
-            atomicAdd(&mass[d], fixed_weight(v, max_logit, inv_t));
+            if (pass > 0 && (k >> above) != (fixed >> above)) return;
+            const int d = (k >> shift) & (nbins - 1);
+            atomicAdd(&sc.cnt[d], 1u);
+            atomicAdd(&sc.mass[d], fixed_weight(v, max_logit, inv_t));
+        });
+        __syncthreads();
+        // Walk the bins from the largest digit down, all threads together: thread t has the
+        // places 4t .. 4t+3 of that walk (place q is digit nbins-1-q); an exclusive scan over
+        // the threads gives what lies above its places.
+        const int per = SELECT_BINS / SAMPLE_THREADS;
+        unsigned int c_mine = 0;
+        unsigned long long m_mine = 0;
+#pragma unroll
+        for (int e = 0; e < per; ++e) {
+            const int q = threadIdx.x * per + e;
+            if (q < nbins) { c_mine += sc.cnt[nbins - 1 - q]; m_mine += sc.mass[nbins - 1 - q]; }
+        }
+        unsigned int c_scan = c_mine;
+        unsigned long long m_scan = m_mine;
+#pragma unroll
+        for (int off = 1; off < WAVE; off <<= 1) {
+            const unsigned int c_up = __shfl_up(c_scan, off, WAVE);
+            const unsigned long long m_up = __shfl_up(m_scan, off, WAVE);
+            if (lane >= off) { c_scan += c_up; m_scan += m_up; }
+        }
+        if (lane == WAVE - 1) { sc.wave_cnt[wave] = c_scan; sc.wave_mass[wave] = m_scan; }
+        __syncthreads();
+        unsigned long long c_before = st.count_above, m_before = st.mass_above, c_all = 0, m_all = 0;
+        for (int w = 0; w < nwaves; ++w) {
+            if (w < wave) { c_before += sc.wave_cnt[w]; m_before += sc.wave_mass[w]; }
+            c_all += sc.wave_cnt[w]; m_all += sc.wave_mass[w];
+        }
+        c_before += c_scan - c_mine;                         // exclusive within the wave
+        m_before += m_scan - m_mine;
+        bool found = false;
+        unsigned long long c_at = 0, m_at = 0;
+        int q_at = 0;
+#pragma unroll
+        for (int e = 0; e < per; ++e) {
+            const int q = threadIdx.x * per + e;
+            if (q >= nbins) break;
+            const unsigned int c = sc.cnt[nbins - 1 - q];
+            const unsigned long long m = sc.mass[nbins - 1 - q];
+            if (c) {
+                atomicMax(&sc.last_nonempty, q);
+                const unsigned long long have = by_mass ? m_before + m : c_before + c;
+                if (!found && have >= target) { found = true; c_at = c_before; m_at = m_before; q_at = q; }
+            }
+            c_before += c;
+            m_before += m;
+        }
+        if (found) atomicMin(&sc.best, q_at);
+        __syncthreads();
+        if (sc.best < SELECT_BINS) {
+            if (found && q_at == sc.best) {                   // exactly one thread: the owner of that place
+                sc.st.prefix = st.prefix | ((uint32_t)(nbins - 1 - q_at) << shift);
+                sc.st.count_above = c_at;
+                sc.st.mass_above = m_at;
+            }
+        } else if (threadIdx.x == 0) {
+            // the target lies beyond the row's total: take the last entry
+            const int q = sc.last_nonempty < 0 ? nbins - 1 : sc.last_nonempty;
+            const int d = nbins - 1 - q;
+            sc.st.prefix = st.prefix | ((uint32_t)d << shift);
+            sc.st.count_above = st.count_above + c_all - (sc.last_nonempty < 0 ? 0 : sc.cnt[d]);
+            sc.st.mass_above = st.mass_above + m_all - (sc.last_nonempty < 0 ? 0 : sc.mass[d]);
         }
         __syncthreads();
-        if (threadIdx.x == 0) {
-            SelectState s = st;
-            int chosen = -1, last_nonempty = -1;
-            for (int d = 255; d >= 0; --d) {
-                if (!cnt[d]) continue;
-                last_nonempty = d;
-                const unsigned long long have = by_mass ? s.mass_above + mass[d] : s.count_above + cnt[d];
-                if (have >= target) { chosen = d; break; }
-                s.count_above += cnt[d];
-                s.mass_above += mass[d];
-            }
-            if (chosen < 0) {          // the target lies beyond the row's total: take the last entry
-                chosen = last_nonempty < 0 ? 0 : last_nonempty;
-                if (last_nonempty >= 0) { s.count_above -= cnt[chosen]; s.mass_above -= mass[chosen]; }
-            }
-            s.prefix = st.prefix | ((uint32_t)chosen << shift);
-            *shared_st = s;
-        }
-        __syncthreads();
-        st = *shared_st;
+        st = sc.st;
         __syncthreads();
     }
 }
@@ -133,9 +210,7 @@ __global__ void __launch_bounds__(SAMPLE_THREADS)
 sample_kernel(const float *__restrict__ logits, int ld, int vocab, const float *__restrict__ temperature,
               const float *__restrict__ top_p, const int *__restrict__ top_k, const float *__restrict__ uniform,
               int *__restrict__ out) {
-    __shared__ unsigned int cnt[256];
-    __shared__ unsigned long long mass[256];
-    __shared__ SelectState shared_st;
+    __shared__ SelectScratch sc;
     __shared__ float red[SAMPLE_THREADS / WAVE];
     __shared__ unsigned long long red64[SAMPLE_THREADS / WAVE];
     __shared__ int seg_count[SAMPLE_THREADS];
@@ -149,7 +224,7 @@ sample_kernel(const float *__restrict__ logits, int ld, int vocab, const float *
 
     // the largest logit
     float mx = -INFINITY;
-    for (int i = threadIdx.x; i < vocab; i += blockDim.x) mx = fmaxf(mx, row[i]);
+    scan_row(row, vocab, [&](int, float v) { mx = fmaxf(mx, v); });
     mx = wave_max(mx);
     if (lane == 0) red[wave] = mx;
     __syncthreads();
@@ -159,7 +234,7 @@ sample_kernel(const float *__restrict__ logits, int ld, int vocab, const float *
 
     // the sum of all weights
     unsigned long long total = 0;
-    for (int i = threadIdx.x; i < vocab; i += blockDim.x) total += fixed_weight(row[i], mx, inv_t);
+    scan_row(row, vocab, [&](int, float v) { total += fixed_weight(v, mx, inv_t); });
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) total += __shfl_xor(total, off, WAVE);
     if (lane == 0) red64[wave] = total;
@@ -173,7 +248,7 @@ sample_kernel(const float *__restrict__ logits, int ld, int vocab, const float *
     unsigned long long limit_k = total;
     int k = top_k[r];
     if (k >= 1 && k < vocab) {
-        radix_select(row, vocab, mx, inv_t, 0, (unsigned long long)k, st, cnt, mass, &shared_st);
+        radix_select(row, vocab, mx, inv_t, 0, (unsigned long long)k, st, sc);
         const unsigned long long w_tie = fixed_weight(key_value(st.prefix), mx, inv_t);
         limit_k = st.mass_above + ((unsigned long long)k - st.count_above) * w_tie;
     }
@@ -183,7 +258,7 @@ sample_kernel(const float *__restrict__ logits, int ld, int vocab, const float *
     unsigned long long target = (unsigned long long)((double)uniform[r] * lim);
     if (target > total) target = total;
 
-    radix_select(row, vocab, mx, inv_t, 1, target, st, cnt, mass, &shared_st);
+    radix_select(row, vocab, mx, inv_t, 1, target, st, sc);
 
     // among equal logits: the m-th in index order, m = ceil((p - mass_above) / w)
     const uint32_t key = st.prefix;
@@ -191,27 +266,41 @@ sample_kernel(const float *__restrict__ logits, int ld, int vocab, const float *
     unsigned long long m = 1;
     if (w_tie > 0 && target > st.mass_above) m = (target - st.mass_above + w_tie - 1) / w_tie;
     if (m < 1) m = 1;
-    const int seg = (vocab + blockDim.x - 1) / blockDim.x;
-    const int lo = threadIdx.x * seg, hi = (lo + seg < vocab) ? lo + seg : vocab;
-    int mine = 0;
-    for (int i = lo; i < hi; ++i) mine += order_key(row[i]) == key;
-    seg_count[threadIdx.x] = mine;
-    if (threadIdx.x == 0) result = -1;
+    // Mostly one logit has that key: count them in a fast pass and take the one.
+    __shared__ int n_found, first_found;
+    if (threadIdx.x == 0) { n_found = 0; first_found = 0x7fffffff; result = -1; }
     __syncthreads();
-    if (threadIdx.x == 0) {
-        // exclusive prefix counts, serial: 1024 additions
-        int run = 0;
-        for (int t = 0; t < (int)blockDim.x; ++t) { const int c = seg_count[t]; seg_count[t] = run; run += c; }
-        red64[0] = (unsigned long long)run;
-    }
+    int seen_here = 0, first_here = 0x7fffffff;
+    scan_row(row, vocab, [&](int i, float v) {
+        if (order_key(v) == key) { ++seen_here; first_here = i < first_here ? i : first_here; }
+    });
+    if (seen_here) { atomicAdd(&n_found, seen_here); atomicMin(&first_found, first_here); }
     __syncthreads();
-    const unsigned long long n_ties = red64[0];
-    if (m > n_ties) m = n_ties;
-    const int before = seg_count[threadIdx.x];
-    if (mine > 0 && (unsigned long long)before < m && m <= (unsigned long long)(before + mine)) {
-        int seen = before;
-        for (int i = lo; i < hi; ++i)
-            if (order_key(row[i]) == key && (unsigned long long)(++seen) == m) { result = i; break; }
+    if (n_found <= 1) {
+        if (threadIdx.x == 0) result = n_found == 1 ? first_found : -1;
+    } else {
+        // several equal logits: the m-th in index order; every thread counts a stretch of the row
+        const int seg = (vocab + blockDim.x - 1) / blockDim.x;
+        const int lo = threadIdx.x * seg, hi = (lo + seg < vocab) ? lo + seg : vocab;
+        int mine = 0;
+        for (int i = lo; i < hi; ++i) mine += order_key(row[i]) == key;
+        seg_count[threadIdx.x] = mine;
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            // exclusive prefix counts, serial: 1024 additions
+            int run = 0;
+            for (int t = 0; t < (int)blockDim.x; ++t) { const int c = seg_count[t]; seg_count[t] = run; run += c; }
+            red64[0] = (unsigned long long)run;
+        }
+        __syncthreads();
+        const unsigned long long n_ties = red64[0];
+        if (m > n_ties) m = n_ties;
+        const int before = seg_count[threadIdx.x];
+        if (mine > 0 && (unsigned long long)before < m && m <= (unsigned long long)(before + mine)) {
+            int seen = before;
+            for (int i = lo; i < hi; ++i)
+                if (order_key(row[i]) == key && (unsigned long long)(++seen) == m) { result = i; break; }
+        }
     }
     __syncthreads();
     if (threadIdx.x == 0) out[r] = result < 0 ? 0 : result;
