@@ -65,3 +65,31 @@ def test_float32_does_not_depend_on_cutting(models):
         for name in reqs:
             for pos in results[0][name]:
                 assert np.array_equal(results[0][name][pos], other[name][pos]), (name, pos)
+
+
+@pytest.mark.parametrize("seed", [1, 2, 3, 4, 5, 6])
+def test_random_configurations_match_plain(seed):
+    """Configurations drawn at random from what config.json allows: head sizes in steps of 16
+    up to 256, any number of heads and groups, widths and vocabularies that are no power of
+    two, both pairings of the rotation, tied and untied output; replayed whole, with a decoded
+    tail, in portions and mixed, in 32-bit and in bfloat16."""
+    import random
+    rng = random.Random(seed)
+    nkv = rng.choice([1, 2, 3, 5])
+    cfg = dict(architectures=["LlamaForCausalLM"], num_hidden_layers=rng.choice([1, 2]),
+               hidden_size=rng.choice([40, 72, 88, 104, 136, 200, 264]), num_attention_heads=nkv * rng.choice([1, 2, 3, 4, 7, 8]),
+               num_key_value_heads=nkv, head_dim=rng.choice([16, 32, 48, 64, 80, 96, 112, 128, 144, 192, 256]),
+               intermediate_size=rng.choice([56, 100, 172, 232, 352]), vocab_size=rng.choice([257, 301, 384, 1000, 1537]),
+               max_position_embeddings=256, rope_theta=rng.choice([1e4, 5e5, 333.0]),
+               rms_norm_eps=rng.choice([1e-5, 1e-6, 1e-3]), tie_word_embeddings=rng.random() < 0.5,
+               rope_interleaved=rng.random() < 0.3)
+    lens = [rng.randrange(1, 150) for _ in range(4)]
+    for dtype, tdt, std in (("float32", torch.float32, 0.15), ("bfloat16", torch.bfloat16, common.BF16_STD)):
+        folder = common.make_folder(cfg, seed=seed, dtype=tdt, std=std)
+        reqs = common.random_requests(cfg["vocab_size"], lens, seed=seed)
+        want = common.plain_logits(folder, reqs)
+        for mode in ("whole", "tail", "portions", "mixed"):
+            steps, max_tokens = TRACES[mode](reqs)
+            outputs = common.run_trace_inprocess(folder, dtype, steps, max_tokens)
+            got = common.collect(steps, outputs, cfg["vocab_size"])
+            common.assert_matches_plain(got, want, dtype, f"{cfg}/{dtype}/{mode}")
