@@ -362,6 +362,21 @@ def test_attention_decode_kernel(nh, nkv, dh, page, window, splits):
     close(out, want, "bfloat16")
 
 
+@pytest.mark.parametrize("nh,nkv,dh,page", [(8, 2, 128, 16), (4, 1, 64, 32)])
+def test_attention_decode_kernel_long_context_in_many_parts(nh, nkv, dh, page):
+    """One request with thousands of keys: its keys are cut into 32 parts (the most), each
+    walked by another workgroup, and merged; a key far back dominates."""
+    from llama_cu_amd.kernels import ops
+    ctx_lens = [9001, 700]
+    q, cache, step, want = paged_case("bfloat16", nh, nkv, dh, page, [1, 1], ctx_lens, 0, seed=dh)
+    assert ops.decode_splits(1, nh, nkv, 9001) == 32
+    for splits in (None, 32):
+        step.attn_splits = splits
+        out = torch.empty(q.shape[0], nh * dh, dtype=torch.bfloat16, device="cuda")
+        ops.paged_attention(q.cuda(), out, cache.cuda(), step, 0, nh, nkv, dh, page, dh ** -0.5, 0)
+        close(out, want, "bfloat16")
+
+
 @pytest.mark.parametrize("nh,nkv,dh,page", [(8, 2, 64, 16), (32, 8, 128, 16), (3, 1, 128, 32), (7, 7, 64, 16), (4, 1, 32, 32), (6, 3, 96, 16)])
 def test_attention_prefill_kernel_long(nh, nkv, dh, page):
     """Whole prompts and portions with history on the matrix cores, long enough that a
