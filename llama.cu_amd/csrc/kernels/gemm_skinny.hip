@@ -15,6 +15,12 @@
 //     MT such tiles for up to 64 tokens.
 // The waves' partial sums are added in LDS in a fixed order.
 //
+// W may also be given packed (lcu_pack_weight / the wrapper's pack_weight): the 16 x 128 block
+// of a tile and a macro-step lies in 4 KB of its own, ordered [j][lane][8] as the lanes load it,
+// the blocks of a tile one after the other.  Then every load instruction of a wave reads 1 KB
+// in one piece and a workgroup streams one contiguous run of memory, which HBM serves
+// faster than pieces of 256 bytes out of 16 or 32 rows that lie kilobytes apart.
+//
 // Epilogues: store bfloat16; store float32 (logits); add into float32 (the residual
 // stream); SwiGLU, where the workgroup's two tiles are the gate rows n and the up rows
 // n + N/2 of one matrix and silu(gate) * up is stored.
@@ -60,14 +66,17 @@ struct Frag {
 // The lane's loads of macro-step s: k = 128 s + 32 grp + 8 j .. + 7 for j = 0..3.
 template <int NT, int MT>
 __device__ __forceinline__ void load_frag(Frag<NT, MT> &f, const bf16_t *const (&wrow)[NT], const bf16_t *const (&xrow)[MT],
-                                          const bool (&xvalid)[MT], int s, int grp, int K) {
+                                          const bool (&xvalid)[MT], int s, int grp, int K, int packed) {
     const int kb = 128 * s + 32 * grp;
     const u32x4 zero = u32x4{0u, 0u, 0u, 0u};
     if (128 * (s + 1) <= K) {
+        // packed: wrow is the lane's place in the tile's first block; blocks are 2048 elements,
+        // the four loads of a block 512 apart
+        const int w0 = packed ? 2048 * s : kb, wj = packed ? 512 : 8;
 #pragma unroll
         for (int t = 0; t < NT; ++t)
 #pragma unroll
-            for (int j = 0; j < 4; ++j) f.w[t][j] = *(const u32x4 *)(wrow[t] + kb + 8 * j);
+            for (int j = 0; j < 4; ++j) f.w[t][j] = *(const u32x4 *)(wrow[t] + w0 + wj * j);
 #pragma unroll
         for (int m = 0; m < MT; ++m)
 #pragma unroll
@@ -98,7 +107,7 @@ __device__ __forceinline__ void mul_frag(const Frag<NT, MT> &f, f32x4 (&acc)[NT]
 template <int NT, int MT, int EPI, int SK_WAVES>
 __global__ void __launch_bounds__(SK_WAVES *WAVE)
 gemm_skinny_kernel(const bf16_t *__restrict__ X, int ldx, const bf16_t *__restrict__ W, int ldw, void *__restrict__ Y,
-                   int ldy, int M, int N, int K, SkinnyExtra ex) {
+                   int ldy, int M, int N, int K, int w_packed, SkinnyExtra ex) {
     __shared__ float red[SK_WAVES][NT * MT * 4][WAVE];
     __shared__ float row_scale[16 * MT];
     const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
@@ -114,7 +123,8 @@ gemm_skinny_kernel(const bf16_t *__restrict__ X, int ldx, const bf16_t *__restri
         int row = EPI == EPI_SWIGLU ? n0 + 16 * (t % (NT / 2 > 0 ? NT / 2 : 1)) + l16 + half * n_out : n0 + 16 * t + l16;
         const int limit = EPI == EPI_SWIGLU ? (half + 1) * n_out : N;
         row = row < limit ? row : limit - 1;                          // a row beyond the end is read, not stored
-        wrow[t] = W + (size_t)row * ldw;
+        wrow[t] = w_packed ? W + ((size_t)(row / 16) * (K / 128)) * 2048 + (size_t)lane * 8   // (the tile of the row)
+                           : W + (size_t)row * ldw;
     }
     const bf16_t *xrow[MT];
     bool xvalid[MT];
@@ -167,7 +177,7 @@ gemm_skinny_kernel(const bf16_t *__restrict__ X, int ldx, const bf16_t *__restri
     int s = wave;
 #pragma unroll
     for (int i = 0; i < STAGES; ++i)
-        if (s + i * SK_WAVES < nsteps) load_frag<NT, MT>(f[i], wrow, xrow, xvalid, s + i * SK_WAVES, grp, K);
+        if (s + i * SK_WAVES < nsteps) load_frag<NT, MT>(f[i], wrow, xrow, xvalid, s + i * SK_WAVES, grp, K, w_packed);
     for (; s < nsteps; s += STAGES * SK_WAVES) {
 #pragma unroll
         for (int i = 0; i < STAGES; ++i) {
@@ -175,7 +185,7 @@ gemm_skinny_kernel(const bf16_t *__restrict__ X, int ldx, const bf16_t *__restri
             if (cur < nsteps) {
                 mul_frag<NT, MT>(f[i], acc);
                 if (cur + STAGES * SK_WAVES < nsteps)
-                    load_frag<NT, MT>(f[i], wrow, xrow, xvalid, cur + STAGES * SK_WAVES, grp, K);
+                    load_frag<NT, MT>(f[i], wrow, xrow, xvalid, cur + STAGES * SK_WAVES, grp, K, w_packed);
             }
         }
     }
@@ -268,10 +278,10 @@ gemm_skinny_kernel(const bf16_t *__restrict__ X, int ldx, const bf16_t *__restri
 
 template <int NT, int MT, int WAVES>
 static int launch_epi(const void *X, int ldx, const void *W, int ldw, void *Y, int ldy, int M, int N, int K, int epi,
-                      const SkinnyExtra &ex, hipStream_t stream) {
+                      int packed, const SkinnyExtra &ex, hipStream_t stream) {
     dim3 block(WAVES * WAVE);
     const dim3 grid((N + 16 * NT - 1) / (16 * NT));
-#define GO(E) gemm_skinny_kernel<NT, MT, E, WAVES><<<grid, block, 0, stream>>>((const bf16_t *)X, ldx, (const bf16_t *)W, ldw, Y, ldy, M, N, K, ex)
+#define GO(E) gemm_skinny_kernel<NT, MT, E, WAVES><<<grid, block, 0, stream>>>((const bf16_t *)X, ldx, (const bf16_t *)W, ldw, Y, ldy, M, N, K, packed, ex)
     switch (epi) {
     case EPI_BF16: GO(EPI_BF16); break;
     case EPI_F32: GO(EPI_F32); break;
@@ -288,10 +298,10 @@ static int launch_epi(const void *X, int ldx, const void *W, int ldw, void *Y, i
 
 template <int NT, int MT, int WAVES>
 static int launch_swiglu(const void *X, int ldx, const void *W, int ldw, void *Y, int ldy, int M, int N, int K,
-                         const SkinnyExtra &ex, hipStream_t stream) {
+                         int packed, const SkinnyExtra &ex, hipStream_t stream) {
     const int groups = (N / 2 + 8 * NT - 1) / (8 * NT);
     gemm_skinny_kernel<NT, MT, EPI_SWIGLU, WAVES><<<dim3(groups), dim3(WAVES * WAVE), 0, stream>>>(
-        (const bf16_t *)X, ldx, (const bf16_t *)W, ldw, Y, ldy, M, N, K, ex);
+        (const bf16_t *)X, ldx, (const bf16_t *)W, ldw, Y, ldy, M, N, K, packed, ex);
     LCU_LAUNCH_CHECK();
     return LCU_OK;
 }
@@ -302,16 +312,18 @@ static int launch_swiglu(const void *X, int ldx, const void *W, int ldw, void *Y
 // features per workgroup (1, 2 or 4; more tiles reuse X more, fewer give more workgroups);
 // waves: 4 or 8 waves share a workgroup's K.
 static int skinny_bf16(const void *X, int ldx, const void *W, int ldw, void *Y, int ldy, int M, int N, int K, int epilogue,
-                       int tiles, int waves, const SkinnyExtra &ex, hipStream_t stream) {
+                       int tiles, int waves, int packed, const SkinnyExtra &ex, hipStream_t stream) {
     if (M <= 0 || N <= 0) return LCU_OK;
+    // a packed weight is whole blocks of 16 rows x 128 k (and for SwiGLU each half is)
+    if (packed && (K % 128 || N % 16 || (epilogue == EPI_SWIGLU && N % 32))) return LCU_BAD_ARGUMENT;
     if (M > 64 || K <= 0 || K % 8 || ldx % 8 || ldw % 8 || ldx < K || ldw < K) return LCU_BAD_ARGUMENT;
     if (waves != 4 && waves != 8) return LCU_BAD_ARGUMENT;
     const int mt = (M + 15) / 16;
     if (epilogue == EPI_SWIGLU) {
         if (N % 2 || ldy < N / 2) return LCU_BAD_ARGUMENT;
         // tiles: gate and up tiles together (2: one of each, 4: two of each)
-#define SW(NT_, MT_) return waves == 8 ? launch_swiglu<NT_, MT_, 8>(X, ldx, W, ldw, Y, ldy, M, N, K, ex, stream) \
-                                       : launch_swiglu<NT_, MT_, 4>(X, ldx, W, ldw, Y, ldy, M, N, K, ex, stream)
+#define SW(NT_, MT_) return waves == 8 ? launch_swiglu<NT_, MT_, 8>(X, ldx, W, ldw, Y, ldy, M, N, K, packed, ex, stream) \
+                                       : launch_swiglu<NT_, MT_, 4>(X, ldx, W, ldw, Y, ldy, M, N, K, packed, ex, stream)
         if (tiles == 4 && mt <= 2) {
             if (mt == 1) SW(4, 1);
             SW(4, 2);
@@ -326,8 +338,8 @@ static int skinny_bf16(const void *X, int ldx, const void *W, int ldw, void *Y, 
     }
     if (ldy < N) return LCU_BAD_ARGUMENT;
     if (tiles == 4 && mt > 2) tiles = 2;      // 4 x 4 tiles of accumulators and operands do not fit the registers
-#define EP(NT_, MT_) return waves == 8 ? launch_epi<NT_, MT_, 8>(X, ldx, W, ldw, Y, ldy, M, N, K, epilogue, ex, stream) \
-                                       : launch_epi<NT_, MT_, 4>(X, ldx, W, ldw, Y, ldy, M, N, K, epilogue, ex, stream)
+#define EP(NT_, MT_) return waves == 8 ? launch_epi<NT_, MT_, 8>(X, ldx, W, ldw, Y, ldy, M, N, K, epilogue, packed, ex, stream) \
+                                       : launch_epi<NT_, MT_, 4>(X, ldx, W, ldw, Y, ldy, M, N, K, epilogue, packed, ex, stream)
 #define PICK(NT_)          \
     switch (mt) {          \
     case 1: EP(NT_, 1);    \
@@ -344,10 +356,10 @@ static int skinny_bf16(const void *X, int ldx, const void *W, int ldw, void *Y, 
 }
 
 LCU_API int lcu_gemm_skinny_bf16(const void *X, int ldx, const void *W, int ldw, void *Y, int ldy, int M, int N, int K,
-                                 int epilogue, int tiles, int waves, hipStream_t stream) {
+                                 int epilogue, int tiles, int waves, int w_packed, hipStream_t stream) {
     if (epilogue == EPI_ADD_NORM) return LCU_BAD_ARGUMENT;
     const SkinnyExtra none = {};
-    return skinny_bf16(X, ldx, W, ldw, Y, ldy, M, N, K, epilogue, tiles, waves, none, stream);
+    return skinny_bf16(X, ldx, W, ldw, Y, ldy, M, N, K, epilogue, tiles, waves, w_packed, none, stream);
 }
 
 // The product that ends a branch, the residual sum and the next norm's weight in one kernel:
@@ -356,24 +368,24 @@ LCU_API int lcu_gemm_skinny_bf16(const void *X, int ldx, const void *W, int ldw,
 // squares.  At most 16 rows, tiles 1 or 2.
 LCU_API int lcu_gemm_skinny_bf16_add_norm(const void *X, int ldx, const void *W, int ldw, float *res, int ldres, int M, int N,
                                           int K, const void *norm_w, int norm_w_type, void *h_out, int ldh, float *sumsq_out,
-                                          int sumsq_cols, int tiles, int waves, hipStream_t stream) {
+                                          int sumsq_cols, int tiles, int waves, int w_packed, hipStream_t stream) {
     if (M > 16 || (tiles != 1 && tiles != 2) || !res || !norm_w || !h_out || !sumsq_out || ldh < N || ldres < N ||
         (norm_w_type != LCU_F32 && norm_w_type != LCU_BF16) || sumsq_cols != (N + 16 * tiles - 1) / (16 * tiles))
         return LCU_BAD_ARGUMENT;
     SkinnyExtra ex = {};
     ex.norm_w = norm_w; ex.norm_w_type = norm_w_type; ex.h_out = (bf16_t *)h_out; ex.ldh = ldh; ex.sumsq_out = sumsq_out;
-    return skinny_bf16(X, ldx, W, ldw, res, ldres, M, N, K, EPI_ADD_NORM, tiles, waves, ex, stream);
+    return skinny_bf16(X, ldx, W, ldw, res, ldres, M, N, K, EPI_ADD_NORM, tiles, waves, w_packed, ex, stream);
 }
 
 // A product whose rows of X wait for their normalisation: row i of the product is multiplied by
 // rsqrt(sum(sumsq_in[i][0 .. n_in)) / norm_width + eps) before the epilogue (not EPI_ADD_NORM).
 LCU_API int lcu_gemm_skinny_bf16_scaled(const void *X, int ldx, const void *W, int ldw, void *Y, int ldy, int M, int N, int K,
-                                        int epilogue, int tiles, int waves, const float *sumsq_in, int n_in, int norm_width,
-                                        float eps, hipStream_t stream) {
+                                        int epilogue, int tiles, int waves, int w_packed, const float *sumsq_in, int n_in,
+                                        int norm_width, float eps, hipStream_t stream) {
     if (epilogue == EPI_ADD_NORM || !sumsq_in || n_in <= 0 || norm_width <= 0) return LCU_BAD_ARGUMENT;
     SkinnyExtra ex = {};
     ex.sumsq_in = sumsq_in; ex.n_in = n_in; ex.norm_width = norm_width; ex.eps = eps;
-    return skinny_bf16(X, ldx, W, ldw, Y, ldy, M, N, K, epilogue, tiles, waves, ex, stream);
+    return skinny_bf16(X, ldx, W, ldw, Y, ldy, M, N, K, epilogue, tiles, waves, w_packed, ex, stream);
 }
 
 

@@ -49,7 +49,7 @@ class ModelRunner:
     def __init__(self, spec: ModelSpec, tensors: Dict[str, torch.Tensor], dtype, device="cuda:0",
                  page_size: int = 16, max_tokens: Optional[int] = None, num_pages: Optional[int] = None,
                  max_seqs: int = 8, max_batch_tokens: int = 2048, max_model_len: Optional[int] = None,
-                 kv_fraction: float = 0.85, use_graphs: bool = True):
+                 kv_fraction: float = 0.85, use_graphs: bool = True, pack_weights: bool = True):
         self.device = require_gpu(device)
         self.dtype = DTYPES[dtype]
         self.spec = spec
@@ -60,7 +60,7 @@ class ModelRunner:
         self.max_seqs, self.max_batch_tokens = int(max_seqs), int(max_batch_tokens)
         torch.cuda.set_device(self.device)
         self.model = DecoderModel(spec)
-        build = BuildContext(self.dtype, self.device, spec.max_positions, self.page_size)
+        build = BuildContext(self.dtype, self.device, spec.max_positions, self.page_size, bool(pack_weights))
         self.model.load(tensors, build)
 
         # cache groups: one per distinct window among the layers that page keys and values

@@ -442,25 +442,48 @@ def skinny_supported(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype) -
             and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
 
 
+def packable(w: torch.Tensor) -> bool:
+    """Whether ``pack_weight`` takes ``w``: bfloat16 ``[n, k]`` of whole blocks of 16 rows x 128 k."""
+    return w.dtype == torch.bfloat16 and w.dim() == 2 and w.shape[0] % 16 == 0 and w.shape[1] % 128 == 0
+
+
+def pack_weight(w: torch.Tensor) -> torch.Tensor:
+    """``w [n, k]`` in the order in which the weight-streaming kernel loads it: the block of
+    16 rows and 128 k of a tile and a macro-step in 4 KB of its own, inside it
+    ``[load j][lane = 16 * group + row][8 k]`` (k = 32 * group + 8 * j + 0..7), the blocks of a
+    tile one after the other.  The result has the shape of ``w`` and is given to
+    ``gemm_skinny(..., packed=True)``."""
+    if not packable(w):
+        raise KernelError(f"pack_weight: need a bfloat16 [n, k] weight with n % 16 == 0 and k % 128 == 0, got {tuple(w.shape)} {w.dtype}")
+    n, k = w.shape
+    return w.view(n // 16, 16, k // 128, 4, 4, 8).permute(0, 2, 4, 3, 1, 5).contiguous().view(n, k)
+
+
 def skinny_weight_ok(w: torch.Tensor) -> bool:
     """Whether the weight-streaming kernel takes ``w`` as its weight (for any rows it takes)."""
     return (w.dtype == torch.bfloat16 and w.dim() == 2 and w.is_cuda and w.shape[1] % 8 == 0 and w.stride(1) == 1
             and w.stride(0) % 8 == 0 and w.data_ptr() % 16 == 0)
 
 
-def skinny_preferred(m: int, n: int, k: int, out_dtype: torch.dtype) -> bool:
+def skinny_preferred(m: int, n: int, k: int, out_dtype: torch.dtype, packed: bool = False) -> bool:
     """Whether the weight-streaming kernel is the faster choice for a plain bfloat16 product
     of ``m`` rows with an ``[n, k]`` weight (measured against the library on the Llama-3-8B
-    shapes): always for very few rows and for float32 output; for 5 to 16 rows only for small
-    weights (the library's split over K wins on the large ones)."""
+    shapes): always for very few rows and for float32 output; with a packed weight up to 8
+    rows; beyond that, up to 16 rows, only for small weights (the library's split over K wins
+    on the large ones)."""
     if m > SKINNY_ROWS:
         return False
-    return m <= 4 or out_dtype == torch.float32 or n * k <= (1 << 24)
+    return m <= (8 if packed else 4) or out_dtype == torch.float32 or n * k <= (1 << 24)
 
 
-def _skinny_tiles(n_features: int, m: int) -> int:
-    """Output tiles of 16 features per workgroup: as many as still leave about four
-    workgroups for each of the 256 compute units."""
+def _skinny_tiles(n_features: int, m: int, packed: bool = False) -> int:
+    """Output tiles of 16 features per workgroup (measured on the Llama-3-8B shapes).  Plain
+    weights: as many as still leave about four workgroups for each of the 256 compute units.
+    Packed weights: two from 6144 features on, four for the widest with more than 8 rows."""
+    if packed:
+        if n_features >= 65536 and m > 8:
+            return 4
+        return 2 if n_features >= 6144 else 1
     for tiles in (4, 2):
         if n_features // (16 * tiles) >= 1024 and (tiles < 4 or m <= 32):
             return tiles
@@ -470,13 +493,17 @@ def _skinny_tiles(n_features: int, m: int) -> int:
 def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = None,
                 out_dtype: Optional[torch.dtype] = None, accumulate: bool = False, swiglu: bool = False,
                 tiles: Optional[int] = None, waves: Optional[int] = None,
-                row_sumsq: Optional[torch.Tensor] = None, norm_width: int = 0, eps: float = 0.0) -> torch.Tensor:
+                row_sumsq: Optional[torch.Tensor] = None, norm_width: int = 0, eps: float = 0.0,
+                packed: bool = False) -> torch.Tensor:
     """``out (+)= x @ w.T`` for at most 64 rows of bfloat16 ``x`` by streaming ``w`` once.
     ``swiglu``: ``w`` holds gate rows, then up rows; ``out = silu(x @ gate.T) * (x @ up.T)``.
     ``row_sumsq [m, parts]``: the rows of ``x`` wait for their normalisation (see
     ``gemm_skinny_add_norm``); row ``i`` of the product is multiplied by
-    ``rsqrt(sum(row_sumsq[i]) / norm_width + eps)`` before the epilogue."""
+    ``rsqrt(sum(row_sumsq[i]) / norm_width + eps)`` before the epilogue.
+    ``packed``: ``w`` is the result of ``pack_weight``."""
     _gpu(x, w, out, row_sumsq)
+    if packed and not (packable(w) and w.is_contiguous()):
+        raise KernelError("gemm_skinny: a packed weight is a contiguous result of pack_weight")
     _rows(x, "skinny x"); _rows(w, "skinny w")
     m, k = x.shape
     n = w.shape[0]
@@ -498,7 +525,7 @@ def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = 
     _rows(out, "skinny out")
     if out.shape != (m, width):
         raise KernelError(f"gemm_skinny out: shape {tuple(out.shape)}, expected {(m, width)}")
-    tiles = tiles or ((4 if m > 8 else 2) if swiglu else _skinny_tiles(width, m))
+    tiles = tiles or ((4 if (m > 8 or packed) else 2) if swiglu else _skinny_tiles(width, m, packed))
     waves = waves or (8 if width <= 8192 else 4)
     lib = build.load("gemm_skinny")
     if row_sumsq is not None:
@@ -506,11 +533,11 @@ def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = 
                 or norm_width <= 0:
             raise KernelError("gemm_skinny: row_sumsq must be a contiguous float32 [rows, parts] tensor, with the norm's width")
         _check(lib.lcu_gemm_skinny_bf16_scaled(_ptr(x), x.stride(0), _ptr(w), w.stride(0), _ptr(out), out.stride(0), m, n, k,
-                                               _EPILOGUES[epi], tiles, waves, _ptr(row_sumsq), row_sumsq.shape[1],
+                                               _EPILOGUES[epi], tiles, waves, int(packed), _ptr(row_sumsq), row_sumsq.shape[1],
                                                int(norm_width), ctypes.c_float(eps), _stream()), "gemm_skinny (scaled rows)")
         return out
     _check(lib.lcu_gemm_skinny_bf16(_ptr(x), x.stride(0), _ptr(w), w.stride(0), _ptr(out), out.stride(0), m, n, k,
-                                    _EPILOGUES[epi], tiles, waves, _stream()),
+                                    _EPILOGUES[epi], tiles, waves, int(packed), _stream()),
            "gemm_skinny")
     return out
 
@@ -519,7 +546,7 @@ ADD_NORM_MAX_ROWS = 16
 
 
 def gemm_skinny_add_norm(x: torch.Tensor, w: torch.Tensor, residual: torch.Tensor, norm_weight: torch.Tensor,
-                         tiles: Optional[int] = None, waves: Optional[int] = None):
+                         tiles: Optional[int] = None, waves: Optional[int] = None, packed: bool = False):
     """The product that ends a branch, the residual sum and the next norm's weight in one
     kernel: ``residual += x @ w.T`` (float32, in place); returns ``(h, sumsq)`` with
     ``h = bfloat16(residual * norm_weight)``, not yet normalised, and ``sumsq [rows, parts]``,
@@ -527,6 +554,8 @@ def gemm_skinny_add_norm(x: torch.Tensor, w: torch.Tensor, residual: torch.Tenso
     At most 16 rows."""
     _gpu(x, w, residual, norm_weight)
     _rows(x, "skinny x"); _rows(w, "skinny w"); _rows(residual, "residual")
+    if packed and not (packable(w) and w.is_contiguous()):
+        raise KernelError("gemm_skinny_add_norm: a packed weight is a contiguous result of pack_weight")
     m, k = x.shape
     n = w.shape[0]
     if w.shape[1] != k or m > ADD_NORM_MAX_ROWS or not skinny_supported(x, w, torch.float32):
@@ -543,7 +572,7 @@ def gemm_skinny_add_norm(x: torch.Tensor, w: torch.Tensor, residual: torch.Tenso
     lib = build.load("gemm_skinny")
     _check(lib.lcu_gemm_skinny_bf16_add_norm(_ptr(x), x.stride(0), _ptr(w), w.stride(0), _ptr(residual), residual.stride(0),
                                              m, n, k, _ptr(norm_weight), _type(norm_weight, "norm weight"), _ptr(h),
-                                             h.stride(0), _ptr(sumsq), parts, tiles, waves, _stream()),
+                                             h.stride(0), _ptr(sumsq), parts, tiles, waves, int(packed), _stream()),
            "gemm_skinny_add_norm")
     return h, sumsq
 

@@ -15,7 +15,7 @@ import torch
 
 from ..kernels import ops
 from .base import BuildContext, PagedKV, Part, PartSpec, ScaledRows, TensorSpec, make_part, register_part
-from .linear import linear, linear_into_norm
+from .linear import Weight, linear, linear_into_norm, linear_scaled, skinny_takes
 
 
 class Attention(Part):
@@ -49,13 +49,13 @@ class Attention(Part):
 
     def load(self, tensors, build: BuildContext) -> None:
         if self.shares_kv:
-            self.w_qkv = tensors["q_proj.weight"].contiguous()
+            self.w_qkv = Weight(tensors["q_proj.weight"], build)
         else:
             parts = [tensors["q_proj.weight"], tensors["k_proj.weight"], tensors["v_proj.weight"]]
             if len({p.dtype for p in parts}) != 1:
                 parts = [p.float() for p in parts]
-            self.w_qkv = torch.cat(parts, dim=0).contiguous()
-        self.w_o = tensors["o_proj.weight"].contiguous()
+            self.w_qkv = Weight(torch.cat(parts, dim=0), build)
+        self.w_o = Weight(tensors["o_proj.weight"], build)
         self.position.load({}, build)
         self.page_size = build.page_size
         self.dtype = build.dtype
@@ -68,13 +68,12 @@ class Attention(Part):
         """Whether ``forward`` could be given ScaledRows of ``n_rows`` rows in the place of
         plain rows: only where the kernel for few rows is the faster one for the q, k, v
         product anyway."""
-        return (self.dtype == torch.bfloat16 and n_rows <= ops.ADD_NORM_MAX_ROWS and ops.skinny_weight_ok(self.w_qkv)
-                and ops.skinny_preferred(n_rows, self.w_qkv.shape[0], self.w_qkv.shape[1], self.dtype))
+        return self.dtype == torch.bfloat16 and n_rows <= ops.ADD_NORM_MAX_ROWS and skinny_takes(n_rows, self.w_qkv, preferred=True)
 
     def forward(self, h, step, cache, into=None):
         nh, nkv, dh = self.heads, self.kv_heads, self.head_dim
         if isinstance(h, ScaledRows):
-            qkv = ops.gemm_skinny(h.rows, self.w_qkv, row_sumsq=h.sumsq, norm_width=h.width, eps=h.eps)
+            qkv = linear_scaled(h, self.w_qkv)
             h = h.rows
         else:
             qkv = linear(h, self.w_qkv, out_dtype=self.dtype)

@@ -97,6 +97,7 @@ class BuildContext:
     device: torch.device
     max_positions: int
     page_size: int
+    pack_weights: bool = True        # keep a second copy of bfloat16 matrices in the order the decode kernel streams them
 
 
 @dataclass

@@ -13,7 +13,7 @@ import torch
 
 from ..kernels import ops
 from .base import BuildContext, Part, ScaledRows, TensorSpec, register_part
-from .linear import linear, linear_into_norm
+from .linear import Weight, linear, linear_into_norm, linear_swiglu, skinny_takes
 
 
 class SwiGLU(Part):
@@ -32,14 +32,14 @@ class SwiGLU(Part):
         g, u = tensors["gate_proj.weight"], tensors["up_proj.weight"]
         if g.dtype != u.dtype:
             g, u = g.float(), u.float()
-        self.w_gate_up = torch.cat([g, u], dim=0).contiguous()
-        self.w_down = tensors["down_proj.weight"].contiguous()
+        self.w_gate_up = Weight(torch.cat([g, u], dim=0), build)
+        self.w_down = Weight(tensors["down_proj.weight"], build)
         self.dtype = build.dtype
 
     def takes_scaled_rows(self, n_rows: int) -> bool:
         """Whether ``forward`` could be given ScaledRows of ``n_rows`` rows in the place of
         plain rows: the factor then goes into the first product's epilogue."""
-        return self.dtype == torch.bfloat16 and n_rows <= ops.ADD_NORM_MAX_ROWS and ops.skinny_weight_ok(self.w_gate_up)
+        return self.dtype == torch.bfloat16 and n_rows <= ops.ADD_NORM_MAX_ROWS and skinny_takes(n_rows, self.w_gate_up)
 
     # forward(..., into=(residual, norm)) may end with the residual sum and that norm's weight
     # in the down projection and return ScaledRows instead of the branch's output
@@ -47,17 +47,16 @@ class SwiGLU(Part):
 
     def forward(self, h, into=None):
         if isinstance(h, ScaledRows):
-            if not ops.skinny_supported(h.rows, self.w_gate_up, self.dtype):
+            if not ops.skinny_supported(h.rows, self.w_gate_up.plain, self.dtype):
                 raise ops.KernelError("feed-forward: rows that wait for their normalisation need the kernel for few rows")
-            act = ops.gemm_skinny(h.rows, self.w_gate_up, swiglu=True, row_sumsq=h.sumsq, norm_width=h.width, eps=h.eps)
-        elif self.dtype == torch.bfloat16 and h.shape[0] <= ops.SKINNY_ROWS and ops.skinny_supported(h, self.w_gate_up, self.dtype):
+            act = linear_swiglu(h.rows, self.w_gate_up, row_sumsq=h.sumsq, norm_width=h.width, eps=h.eps)
+        elif self.dtype == torch.bfloat16 and h.shape[0] <= ops.SKINNY_ROWS and ops.skinny_supported(h, self.w_gate_up.plain, self.dtype):
             # few rows: one pass over the weights, the activation in the product's epilogue
-            act = ops.gemm_skinny(h, self.w_gate_up, swiglu=True)
+            act = linear_swiglu(h, self.w_gate_up)
         else:
             gu = linear(h, self.w_gate_up, out_dtype=self.dtype)
             act = ops.swiglu(gu)
-        if into is not None and act.dtype == torch.bfloat16 and ops.skinny_preferred(
-                act.shape[0], self.w_down.shape[0], self.w_down.shape[1], torch.bfloat16):
+        if into is not None and act.dtype == torch.bfloat16 and skinny_takes(act.shape[0], self.w_down, preferred=True):
             # only where the kernel for few rows is the faster one for this product anyway
             residual, norm = into
             fused = linear_into_norm(act, self.w_down, residual, norm.weight)

@@ -16,7 +16,7 @@ import torch
 
 from ..kernels import ops
 from .base import BuildContext, ModelSpec, Part, PartSpec, TensorSpec, make_part, prefixed, register_part
-from .linear import linear
+from .linear import Weight, linear
 
 
 class TokenEmbedding(Part):
@@ -54,7 +54,7 @@ class OutputHead(Part):
 
     def load(self, tensors, build: BuildContext, table: Optional[torch.Tensor] = None) -> None:
         own = tensors.get("weight")
-        self.weight = table if (self.tied or own is None) else own.contiguous()
+        self.weight = Weight(table if (self.tied or own is None) else own, build)
 
     def forward(self, y: torch.Tensor) -> torch.Tensor:
         return linear(y, self.weight, out_dtype=torch.float32)

@@ -483,6 +483,39 @@ def test_gemm_skinny_residual_sum_and_norm_weight_in_the_epilogue(m, n, k, tiles
     assert torch.equal(sumsq, sumsq2) and torch.equal(h, h2) and torch.equal(res_g, res_g2)
 
 
+@pytest.mark.parametrize("m,n,k", [(1, 16, 128), (8, 304, 256), (16, 4096, 1024), (13, 96, 384)])
+def test_gemm_skinny_with_a_packed_weight_equals_the_plain_one_bit_for_bit(m, n, k):
+    """``pack_weight`` only changes where the kernel finds its operands, not what it adds in
+    which order: every epilogue gives the same bits as with the plain weight.  The packed
+    copy is checked against its definition too."""
+    from llama_cu_amd.kernels import ops
+    x = rnd(m, k, seed=m).to(torch.bfloat16).cuda()
+    w = rnd(n, k, seed=n, scale=0.3).to(torch.bfloat16)
+    p = ops.pack_weight(w.cuda())
+    assert p.shape == w.shape
+    # [tile of 16 rows][block of 128 k][load j][lane = 16 * group + row][8 k], k = 32 * group + 8 * j + e
+    flat = p.cpu().view(n // 16, k // 128, 4, 4, 16, 8)
+    for (t, b, j, g, r, e) in [(0, 0, 0, 0, 0, 0), (n // 16 - 1, k // 128 - 1, 3, 2, 15, 7), (0, k // 128 - 1, 1, 3, 4, 2)]:
+        assert flat[t, b, j, g, r, e] == w[16 * t + r, 128 * b + 32 * g + 8 * j + e]
+    wg = w.cuda()
+    for tiles in (1, 2, 4):
+        assert torch.equal(ops.gemm_skinny(x, wg, tiles=tiles), ops.gemm_skinny(x, p, tiles=tiles, packed=True))
+    assert torch.equal(ops.gemm_skinny(x, wg, out_dtype=torch.float32), ops.gemm_skinny(x, p, out_dtype=torch.float32, packed=True))
+    if n % 32 == 0:
+        assert torch.equal(ops.gemm_skinny(x, wg, swiglu=True), ops.gemm_skinny(x, p, swiglu=True, packed=True))
+    res = rnd(m, n, seed=3).cuda()
+    nw = (1.0 + 0.2 * rnd(n, seed=4)).to(torch.bfloat16).cuda()
+    r1, r2 = res.clone(), res.clone()
+    h1, s1 = ops.gemm_skinny_add_norm(x, wg, r1, nw)
+    h2, s2 = ops.gemm_skinny_add_norm(x, p, r2, nw, packed=True)
+    assert torch.equal(r1, r2) and torch.equal(h1, h2) and torch.equal(s1, s2)
+    close(ops.gemm_skinny(x, p, packed=True), plain.linear(x.cpu(), w), "bfloat16")
+    with pytest.raises(ops.KernelError):
+        ops.pack_weight(rnd(24, 128).to(torch.bfloat16).cuda())            # no whole tiles of 16 rows
+    with pytest.raises(ops.KernelError):
+        ops.gemm_skinny(x, wg[:, :k - 8], packed=True)
+
+
 def test_gemm_skinny_add_norm_refuses_what_it_cannot_take():
     from llama_cu_amd.kernels import ops
     x = rnd(17, 64).to(torch.bfloat16).cuda()
