@@ -25,12 +25,13 @@
 // stream); SwiGLU, where the workgroup's two tiles are the gate rows n and the up rows
 // n + N/2 of one matrix and silu(gate) * up is stored.
 #include "common.h"
+#include "kv_layout.h"
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 
-enum { EPI_BF16 = 0, EPI_F32 = 1, EPI_ADD_F32 = 2, EPI_SWIGLU = 3, EPI_ADD_NORM = 4 };
+enum { EPI_BF16 = 0, EPI_F32 = 1, EPI_ADD_F32 = 2, EPI_SWIGLU = 3, EPI_ADD_NORM = 4, EPI_QKV_ROPE = 5 };
 
 // What two epilogues need beside Y, so that no kernel stands between a projection that ends
 // a branch and the product that follows the next norm:
@@ -40,6 +41,11 @@ enum { EPI_BF16 = 0, EPI_F32 = 1, EPI_ADD_F32 = 2, EPI_SWIGLU = 3, EPI_ADD_NORM 
 //   row scale (any other epilogue, sumsq_in not null): the rows of X are such rows; a row of
 //     the product is multiplied by rsqrt(sum of its shares / norm_width + eps) before the
 //     epilogue (the normalisation is a factor per row, so it commutes with the product).
+//   EPI_QKV_ROPE: W holds the q, k and v projections (rows q heads, k heads, v heads, head_dim
+//     each).  A workgroup's two tiles are 16 dims of a head and the 16 dims head_dim/2 further,
+//     the pairs of the rotation (half-split pairing over the whole head): the epilogue rotates q
+//     and k by the token's position, writes q to q_out and k and v straight into the token's
+//     place in the paged cache.  No rotation kernel runs after this product.
 // The shares are added in a fixed order: no atomics, results do not depend on timing.
 struct SkinnyExtra {
     const void *norm_w;        // [N] norm weight of EPI_ADD_NORM
@@ -51,6 +57,15 @@ struct SkinnyExtra {
     int n_in;
     int norm_width;
     float eps;
+    // EPI_QKV_ROPE
+    const int *positions;      // [M]
+    const int *slots;          // [M] page * page_size + place, or -1: store nothing
+    const float *cos_t, *sin_t;  // [max_pos, head_dim / 2]
+    int max_pos;
+    bf16_t *cache;             // this layer's pages
+    bf16_t *q_out;             // [M, heads * head_dim] rows ldq apart
+    int ldq;
+    int heads, kv_heads, head_dim, page;
 };
 
 __device__ __forceinline__ f32x4 mfma16(u32x4 a, u32x4 b, f32x4 c) {
@@ -116,11 +131,15 @@ gemm_skinny_kernel(const bf16_t *__restrict__ X, int ldx, const bf16_t *__restri
     const int n_out = EPI == EPI_SWIGLU ? N / 2 : N;                 // width of Y
     // SwiGLU: the first NT/2 tiles are gate rows, the other NT/2 the up rows N/2 further
     const int n0 = blockIdx.x * 16 * (EPI == EPI_SWIGLU ? NT / 2 : NT);
+    // q/k/v with rotation: workgroup b has, of head b / (head_dim/32), the dims 16 c .. and head_dim/2 + 16 c ..
+    const int rope_head = EPI == EPI_QKV_ROPE ? blockIdx.x / (ex.head_dim / 32) : 0;
+    const int rope_c = EPI == EPI_QKV_ROPE ? blockIdx.x % (ex.head_dim / 32) : 0;
     const bf16_t *wrow[NT];
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
         const int half = t / (NT / 2 > 0 ? NT / 2 : 1);              // 0: gate tiles, 1: up tiles (SwiGLU)
         int row = EPI == EPI_SWIGLU ? n0 + 16 * (t % (NT / 2 > 0 ? NT / 2 : 1)) + l16 + half * n_out : n0 + 16 * t + l16;
+        if (EPI == EPI_QKV_ROPE) row = rope_head * ex.head_dim + t * (ex.head_dim / 2) + 16 * rope_c + l16;
         const int limit = EPI == EPI_SWIGLU ? (half + 1) * n_out : N;
         row = row < limit ? row : limit - 1;                          // a row beyond the end is read, not stored
         wrow[t] = w_packed ? W + ((size_t)(row / 16) * (K / 128)) * 2048 + (size_t)lane * 8   // (the tile of the row)
@@ -221,6 +240,49 @@ gemm_skinny_kernel(const bf16_t *__restrict__ X, int ldx, const bf16_t *__restri
                 for (int r = 0; r < 4; ++r) acc[t][m][r] *= rs;
         }
     }
+    if (EPI == EPI_QKV_ROPE) {
+        // the lane holds dims i = 16 c + 4 grp + r (tile 0) and i + head_dim/2 (tile 1) of token l16
+        const int tok = l16, dh = ex.head_dim, half_dim = dh / 2;
+        if (tok >= M) return;
+        const int pos = ex.positions[tok];
+        const bool in_table = pos >= 0 && pos < ex.max_pos;
+        const int slot = ex.slots ? ex.slots[tok] : -1;
+        const bool is_q = rope_head < ex.heads, is_k = !is_q && rope_head < ex.heads + ex.kv_heads;
+        bf16_t *pg = nullptr;
+        int place = 0;
+        if (!is_q && slot >= 0) {
+            pg = ex.cache + (size_t)(slot / ex.page) * kv_page_elems(ex.kv_heads, dh, ex.page);
+            place = slot % ex.page;
+        }
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int i = 16 * rope_c + 4 * grp + r;
+            float a = acc[0][0][r], b = acc[NT - 1][0][r];
+            if (is_q || is_k) {
+                float c = __uint_as_float(0x7fc00000u), sn = c;         // a position outside the table gives NaN
+                if (in_table) { c = ex.cos_t[(size_t)pos * half_dim + i]; sn = ex.sin_t[(size_t)pos * half_dim + i]; }
+                const float ra = a * c - b * sn, rb = a * sn + b * c;
+                a = ra; b = rb;
+            }
+            const bf16_t va = from_f32<bf16_t>(a), vb = from_f32<bf16_t>(b);
+            if (is_q) {
+                bf16_t *qo = ex.q_out + (size_t)tok * ex.ldq + (size_t)rope_head * dh;
+                qo[i] = va;
+                qo[i + half_dim] = vb;
+            } else if (pg) {
+                if (is_k) {
+                    const int kvh = rope_head - ex.heads;
+                    pg[kv_key_offset(kvh, place, i, dh, ex.page)] = va;
+                    pg[kv_key_offset(kvh, place, i + half_dim, dh, ex.page)] = vb;
+                } else {
+                    const int kvh = rope_head - ex.heads - ex.kv_heads;
+                    pg[kv_value_offset(ex.kv_heads, kvh, place, i, dh, ex.page)] = va;
+                    pg[kv_value_offset(ex.kv_heads, kvh, place, i + half_dim, dh, ex.page)] = vb;
+                }
+            }
+        }
+        return;
+    }
     if (EPI == EPI_ADD_NORM) {
 #pragma unroll
         for (int m = 0; m < MT; ++m) {
@@ -288,6 +350,14 @@ static int launch_epi(const void *X, int ldx, const void *W, int ldw, void *Y, i
     case EPI_ADD_F32: GO(EPI_ADD_F32); break;
     case EPI_ADD_NORM:
         if constexpr (MT == 1 && NT <= 2) { GO(EPI_ADD_NORM); break; }      // made for decoding: at most 16 rows
+        return LCU_UNSUPPORTED;
+    case EPI_QKV_ROPE:
+        if constexpr (MT == 1 && NT == 2) {
+            const dim3 rgrid((ex.heads + 2 * ex.kv_heads) * (ex.head_dim / 32));
+            gemm_skinny_kernel<NT, MT, EPI_QKV_ROPE, WAVES><<<rgrid, block, 0, stream>>>(
+                (const bf16_t *)X, ldx, (const bf16_t *)W, ldw, Y, ldy, M, N, K, packed, ex);
+            break;
+        }
         return LCU_UNSUPPORTED;
     default: return LCU_BAD_ARGUMENT;
     }
@@ -386,6 +456,33 @@ LCU_API int lcu_gemm_skinny_bf16_scaled(const void *X, int ldx, const void *W, i
     SkinnyExtra ex = {};
     ex.sumsq_in = sumsq_in; ex.n_in = n_in; ex.norm_width = norm_width; ex.eps = eps;
     return skinny_bf16(X, ldx, W, ldw, Y, ldy, M, N, K, epilogue, tiles, waves, w_packed, ex, stream);
+}
+
+
+// The q, k and v projections with the rotation and the cache write in the epilogue.  W: [(heads +
+// 2 kv_heads) * head_dim, K] (q heads, then k heads, then v heads).  q_out: [M, heads * head_dim]
+// rows ldq apart takes the rotated queries; the rotated keys and the values go to cache (this
+// layer's pages, laid out as kv_layout.h says) at slots[m] (page * page_size + place; -1: nothing
+// is stored).  cos_t, sin_t: [max_pos, head_dim / 2] float32; pairs are (i, i + head_dim / 2).
+// At most 16 rows; head_dim a multiple of 32.  sumsq_in (may be null): the rows of X wait for
+// their normalisation, as in lcu_gemm_skinny_bf16_scaled.
+LCU_API int lcu_gemm_skinny_bf16_qkv_rope(const void *X, int ldx, const void *W, int ldw, int M, int K, void *q_out, int ldq,
+                                          const int *positions, const int *slots, const float *cos_t, const float *sin_t,
+                                          int max_pos, void *cache, int heads, int kv_heads, int head_dim, int page,
+                                          int waves, int w_packed, const float *sumsq_in, int n_in, int norm_width, float eps,
+                                          hipStream_t stream) {
+    if (M <= 0) return LCU_OK;
+    if (M > 16 || heads <= 0 || kv_heads <= 0 || head_dim <= 0 || head_dim % 32 || page <= 0 || page % 8 || !q_out ||
+        !positions || !cos_t || !sin_t || max_pos <= 0 || !cache || ldq < heads * head_dim ||
+        (sumsq_in && (n_in <= 0 || norm_width <= 0)))
+        return LCU_BAD_ARGUMENT;
+    SkinnyExtra ex = {};
+    ex.sumsq_in = sumsq_in; ex.n_in = n_in; ex.norm_width = norm_width; ex.eps = eps;
+    ex.positions = positions; ex.slots = slots; ex.cos_t = cos_t; ex.sin_t = sin_t; ex.max_pos = max_pos;
+    ex.cache = (bf16_t *)cache; ex.q_out = (bf16_t *)q_out; ex.ldq = ldq;
+    ex.heads = heads; ex.kv_heads = kv_heads; ex.head_dim = head_dim; ex.page = page;
+    const int N = (heads + 2 * kv_heads) * head_dim;
+    return skinny_bf16(X, ldx, W, ldw, q_out, N, M, N, K, EPI_QKV_ROPE, 2, waves, w_packed, ex, stream);
 }
 
 

@@ -577,6 +577,57 @@ def gemm_skinny_add_norm(x: torch.Tensor, w: torch.Tensor, residual: torch.Tenso
     return h, sumsq
 
 
+QKV_ROPE_MAX_ROWS = 16
+
+
+def qkv_rope_supported(x: torch.Tensor, w: torch.Tensor, heads: int, kv_heads: int, head_dim: int) -> bool:
+    """Whether ``gemm_skinny_qkv_rope`` takes these operands: at most 16 rows, bfloat16, whole
+    heads whose halves are multiples of 16."""
+    return (x.dim() == 2 and x.shape[0] <= QKV_ROPE_MAX_ROWS and head_dim % 32 == 0
+            and w.shape[0] == (heads + 2 * kv_heads) * head_dim and skinny_supported(x, w, torch.bfloat16))
+
+
+def gemm_skinny_qkv_rope(x: torch.Tensor, w: torch.Tensor, positions: torch.Tensor, slots: torch.Tensor,
+                         cos: torch.Tensor, sin: torch.Tensor, cache: torch.Tensor, heads: int, kv_heads: int,
+                         head_dim: int, page_size: int, row_sumsq: Optional[torch.Tensor] = None, norm_width: int = 0,
+                         eps: float = 0.0, packed: bool = False, waves: Optional[int] = None) -> torch.Tensor:
+    """The q, k, v product of an attention layer with the rotation and the cache write in its
+    epilogue: ``w`` holds the rows of q, k and v (whole heads, in this order); returns the rotated
+    queries ``[rows, heads * head_dim]``; the rotated keys and the values of row ``i`` are written
+    into ``cache`` at ``slots[i]`` (negative: not stored).  Pairs are ``(i, i + head_dim / 2)`` and
+    the rotation covers the whole head.  ``row_sumsq``: as in ``gemm_skinny``."""
+    _gpu(x, w, positions, slots, cos, sin, cache, row_sumsq)
+    if packed and not (packable(w) and w.is_contiguous()):
+        raise KernelError("gemm_skinny_qkv_rope: a packed weight is a contiguous result of pack_weight")
+    _rows(x, "skinny x"); _rows(w, "skinny w")
+    m, k = x.shape
+    if w.shape[1] != k or not qkv_rope_supported(x, w, heads, kv_heads, head_dim):
+        raise KernelError(f"gemm_skinny_qkv_rope: x {tuple(x.shape)} {x.dtype} with w {tuple(w.shape)} {w.dtype}, {heads} + 2 * "
+                          f"{kv_heads} heads of {head_dim} is not supported")
+    _i32(positions, "positions", m); _i32(slots, "cache slots", m)
+    if cos.shape != sin.shape or cos.dtype != torch.float32 or sin.dtype != torch.float32 or cos.dim() != 2 \
+            or cos.shape[1] * 2 != head_dim or not cos.is_contiguous() or not sin.is_contiguous():
+        raise KernelError("rotation tables must be two contiguous float32 tensors [max_pos, head_dim/2]")
+    _contig(cache, "cache")
+    if cache.dtype != torch.bfloat16 or cache.dim() != 3 or cache.shape[1] != 2 \
+            or cache.shape[2] != kv_heads * head_dim * page_size:
+        raise KernelError(f"cache: {cache.dtype} {tuple(cache.shape)}, expected bfloat16 [pages, 2, {kv_heads * head_dim * page_size}]")
+    n_in = 0
+    if row_sumsq is not None:
+        if row_sumsq.dtype != torch.float32 or row_sumsq.dim() != 2 or row_sumsq.shape[0] != m or not row_sumsq.is_contiguous() \
+                or norm_width <= 0:
+            raise KernelError("gemm_skinny_qkv_rope: row_sumsq must be a contiguous float32 [rows, parts] tensor, with the norm's width")
+        n_in = row_sumsq.shape[1]
+    q = torch.empty((m, heads * head_dim), dtype=torch.bfloat16, device=x.device)
+    waves = waves or 8
+    lib = build.load("gemm_skinny")
+    _check(lib.lcu_gemm_skinny_bf16_qkv_rope(_ptr(x), x.stride(0), _ptr(w), w.stride(0), m, k, _ptr(q), q.stride(0),
+                                             _ptr(positions), _ptr(slots), _ptr(cos), _ptr(sin), cos.shape[0], _ptr(cache),
+                                             heads, kv_heads, head_dim, page_size, waves, int(packed), _ptr(row_sumsq), n_in,
+                                             int(norm_width), ctypes.c_float(eps), _stream()), "gemm_skinny_qkv_rope")
+    return q
+
+
 def skinny_f32_supported(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype) -> bool:
     """Whether the float32 weight-streaming kernel takes this product: all float32, K a
     multiple of 4 (16-byte loads)."""

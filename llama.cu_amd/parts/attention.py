@@ -15,7 +15,8 @@ import torch
 
 from ..kernels import ops
 from .base import BuildContext, PagedKV, Part, PartSpec, ScaledRows, TensorSpec, make_part, register_part
-from .linear import Weight, linear, linear_into_norm, linear_scaled, skinny_takes
+from .linear import Weight, linear, linear_into_norm, linear_qkv_rope, linear_scaled, skinny_takes
+from .position import NoPosition
 
 
 class Attention(Part):
@@ -57,6 +58,8 @@ class Attention(Part):
             self.w_qkv = Weight(torch.cat(parts, dim=0), build)
         self.w_o = Weight(tensors["o_proj.weight"], build)
         self.position.load({}, build)
+        # a position encoding that is its rotation tables alone (apply() does nothing of its own)
+        self._rotation_only = getattr(type(self.position), "apply", None) is NoPosition.apply
         self.page_size = build.page_size
         self.dtype = build.dtype
 
@@ -72,22 +75,29 @@ class Attention(Part):
 
     def forward(self, h, step, cache, into=None):
         nh, nkv, dh = self.heads, self.kv_heads, self.head_dim
-        if isinstance(h, ScaledRows):
-            qkv = linear_scaled(h, self.w_qkv)
-            h = h.rows
-        else:
-            qkv = linear(h, self.w_qkv, out_dtype=self.dtype)
-        self.position.apply(qkv, step.positions, nh, 0 if self.shares_kv else nkv, dh)
-        rot = self.position.rotary_tables()
-        cos, sin, rot_dim, pairing = rot if rot is not None else (None, None, 0, 0)
-        store = cache.writes and not self.shares_kv
         if self.shares_kv == cache.writes:
             raise ops.KernelError("attention: a layer that shares another's keys and values must be given that "
                                   "layer's cache in the run order (and only such a layer)")
-        ops.rope_kv_store(qkv, step.positions, nh, nkv, dh, cos, sin, rot_dim, pairing,
-                          cache.pages if store else None, step.slots(cache.group) if store else None,
-                          self.page_size)
-        out = torch.empty((h.shape[0], nh * dh), dtype=self.dtype, device=h.device)
+        rot = self.position.rotary_tables()
+        cos, sin, rot_dim, pairing = rot if rot is not None else (None, None, 0, 0)
+        store = cache.writes and not self.shares_kv
+        n_rows = (h.rows if isinstance(h, ScaledRows) else h).shape[0]
+        qkv = None
+        if store and self._rotation_only and rot is not None and pairing == 0 and rot_dim == dh \
+                and self.dtype == torch.bfloat16 and skinny_takes(n_rows, self.w_qkv, preferred=True):
+            # few rows: the product rotates q and k and writes k and v into the pages itself
+            qkv = linear_qkv_rope(h, self.w_qkv, step.positions, step.slots(cache.group), cos, sin, cache.pages,
+                                  nh, nkv, dh, self.page_size)
+        if qkv is None:
+            if isinstance(h, ScaledRows):
+                qkv = linear_scaled(h, self.w_qkv)
+            else:
+                qkv = linear(h, self.w_qkv, out_dtype=self.dtype)
+            self.position.apply(qkv, step.positions, nh, 0 if self.shares_kv else nkv, dh)
+            ops.rope_kv_store(qkv, step.positions, nh, nkv, dh, cos, sin, rot_dim, pairing,
+                              cache.pages if store else None, step.slots(cache.group) if store else None,
+                              self.page_size)
+        out = torch.empty((n_rows, nh * dh), dtype=self.dtype, device=qkv.device)
         ops.paged_attention(qkv, out, cache.pages, step, cache.group, nh, nkv, dh, self.page_size, self.scale,
                             self.window)
         if into is not None:

@@ -19,6 +19,7 @@ from typing import Optional, Union
 import torch
 
 from ..kernels import ops
+from .base import ScaledRows
 
 
 class Weight:
@@ -113,3 +114,22 @@ def linear_into_norm(a: torch.Tensor, weight: Union[torch.Tensor, Weight], resid
     if packed is not None:
         return ops.gemm_skinny_add_norm(a, packed, residual, norm_weight, packed=True)
     return ops.gemm_skinny_add_norm(a, weight, residual, norm_weight)
+
+
+def linear_qkv_rope(h, weight: Union[torch.Tensor, Weight], positions, slots, cos, sin, cache_pages, heads: int,
+                    kv_heads: int, head_dim: int, page_size: int):
+    """The q, k, v product with the rotation of q and k and the write of k and v into the cache in
+    its epilogue (``h``: bfloat16 rows or ScaledRows): returns the rotated queries, or None if the
+    kernel for it does not take these operands (then nothing has been done)."""
+    weight, packed = _split(weight)
+    rows = h.rows if isinstance(h, ScaledRows) else h
+    if not (rows.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and cache_pages.dtype == torch.bfloat16
+            and ops.qkv_rope_supported(rows, weight, heads, kv_heads, head_dim)):
+        return None
+    kw = dict(row_sumsq=h.sumsq, norm_width=h.width, eps=h.eps) if isinstance(h, ScaledRows) else {}
+    if packed is not None:
+        return ops.gemm_skinny_qkv_rope(rows, packed, positions, slots, cos, sin, cache_pages, heads, kv_heads, head_dim,
+                                        page_size, packed=True, **kw)
+    return ops.gemm_skinny_qkv_rope(rows, weight, positions, slots, cos, sin, cache_pages, heads, kv_heads, head_dim,
+                                    page_size, **kw)
+

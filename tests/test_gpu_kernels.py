@@ -516,6 +516,62 @@ def test_gemm_skinny_with_a_packed_weight_equals_the_plain_one_bit_for_bit(m, n,
         ops.gemm_skinny(x, wg[:, :k - 8], packed=True)
 
 
+@pytest.mark.parametrize("m,k,nh,nkv,dh,page,packed,scaled", [(1, 64, 4, 2, 32, 8, False, False), (8, 256, 6, 2, 64, 16, True, True),
+                                                              (16, 136, 3, 1, 96, 24, False, True), (5, 512, 8, 8, 128, 32, True, False),
+                                                              (13, 128, 5, 5, 160, 16, True, False)])
+def test_gemm_skinny_q_k_v_with_rotation_and_cache_write(m, k, nh, nkv, dh, page, packed, scaled):
+    """The product of few rows with the q, k and v weights whose epilogue rotates q and k and
+    writes k and v into the pages: against product, rotation and cache layout done one after
+    the other; a token that stores nothing; nothing else in the cache is touched."""
+    from llama_cu_amd.kernels import ops
+    from llama_cu_amd.parts.position import Rotary
+    max_pos, pages, theta, eps = 300, 7, 10000.0, 1e-5
+    n = (nh + 2 * nkv) * dh
+    cos, sin = Rotary(dh, theta, max_pos).host_tables()
+    sin_p, cos_p = plain.rope_tables(max_pos, dh, theta)
+    x = rnd(m, k, seed=m + k).to(torch.bfloat16)
+    w = rnd(n, k, seed=n, scale=0.3).to(torch.bfloat16)
+    pos = random.Random(1).sample(range(max_pos), m)
+    slots = random.Random(2).sample(range(pages * page), m)
+    if m > 2:
+        slots[2] = -1
+    cache = torch.full((pages, 2, nkv * dh * page), 7.0, dtype=torch.bfloat16).cuda()
+    kw, rows = {}, x.double()
+    if scaled:
+        sumsq = rnd(m, 5, seed=9).abs() * 40.0
+        kw = dict(row_sumsq=sumsq.cuda(), norm_width=k, eps=eps)
+        rows = rows * torch.rsqrt(sumsq.double().sum(dim=1) / k + eps)[:, None]
+    wg = ops.pack_weight(w.cuda()) if packed else w.cuda()
+    q_got = ops.gemm_skinny_qkv_rope(x.cuda(), wg, torch.tensor(pos, dtype=torch.int32).cuda(),
+                                     torch.tensor(slots, dtype=torch.int32).cuda(), torch.from_numpy(cos).cuda(),
+                                     torch.from_numpy(sin).cuda(), cache, nh, nkv, dh, page, packed=packed, **kw)
+    qkv = plain.linear(rows, w)
+    q = qkv[:, :nh * dh].view(m, nh, dh)
+    kk = qkv[:, nh * dh:(nh + nkv) * dh].view(m, nkv, dh)
+    v = qkv[:, (nh + nkv) * dh:].view(m, nkv, dh)
+    close(q_got.reshape(m, nh, dh), plain.rope(q, pos, sin_p, cos_p, "half"), "bfloat16", "q")
+    k_want = plain.rope(kk, pos, sin_p, cos_p, "half")
+    flat = cache.cpu().view(pages, -1)
+    expect = torch.full_like(flat, 7.0).double()
+    written = torch.zeros_like(flat, dtype=torch.bool)
+    for t in range(m):
+        if slots[t] < 0:
+            continue
+        pg, tok = slots[t] // page, slots[t] % page
+        for h in range(nkv):
+            for c in range(dh):
+                expect[pg, key_offset(h, tok, c, dh, page)] = k_want[t, h, c]
+                expect[pg, value_offset(nkv, h, tok, c, dh, page)] = v[t, h, c]
+                written[pg, key_offset(h, tok, c, dh, page)] = written[pg, value_offset(nkv, h, tok, c, dh, page)] = True
+    close(flat, expect, "bfloat16", "cache")
+    assert bool((flat[~written] == 7.0).all())                              # nothing else was touched
+    with pytest.raises(ops.KernelError):                                    # halves of a head that are no multiple of 16
+        ops.gemm_skinny_qkv_rope(x.cuda(), rnd(4 * 48, k).to(torch.bfloat16).cuda(), torch.zeros(m, dtype=torch.int32).cuda(),
+                                 torch.zeros(m, dtype=torch.int32).cuda(), torch.zeros(max_pos, 24).cuda(),
+                                 torch.zeros(max_pos, 24).cuda(), torch.zeros(2, 2, 48 * page, dtype=torch.bfloat16).cuda(),
+                                 2, 1, 48, page)
+
+
 def test_gemm_skinny_add_norm_refuses_what_it_cannot_take():
     from llama_cu_amd.kernels import ops
     x = rnd(17, 64).to(torch.bfloat16).cuda()
