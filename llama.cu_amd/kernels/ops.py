@@ -468,12 +468,13 @@ def skinny_weight_ok(w: torch.Tensor) -> bool:
 def skinny_preferred(m: int, n: int, k: int, out_dtype: torch.dtype, packed: bool = False) -> bool:
     """Whether the weight-streaming kernel is the faster choice for a plain bfloat16 product
     of ``m`` rows with an ``[n, k]`` weight (measured against the library on the Llama-3-8B
-    shapes): always for very few rows and for float32 output; with a packed weight up to 8
-    rows; beyond that, up to 16 rows, only for small weights (the library's split over K wins
-    on the large ones)."""
+    shapes): always for very few rows and for float32 output; with a packed weight up to 16
+    rows (there it equals the library on the large weights, and its epilogues save the kernels
+    around the product); without one, beyond 4 rows, only for small weights (the library's
+    split over K wins on the large ones)."""
     if m > SKINNY_ROWS:
         return False
-    return m <= (8 if packed else 4) or out_dtype == torch.float32 or n * k <= (1 << 24)
+    return m <= (SKINNY_ROWS if packed else 4) or out_dtype == torch.float32 or n * k <= (1 << 24)
 
 
 def _skinny_tiles(n_features: int, m: int, packed: bool = False) -> int:
