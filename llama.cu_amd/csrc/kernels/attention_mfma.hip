@@ -336,22 +336,48 @@ attention_decode_kernel(const bf16_t *__restrict__ q, int q_stride, bf16_t *__re
 // device-wide fence per workgroup, which writes back and invalidates the whole L2: measured
 // several times slower than this second launch.)
 template <int DH>
-__global__ void attention_merge_kernel(bf16_t *__restrict__ out, int out_stride, const float *__restrict__ part_o,
-                                       const float *__restrict__ part_ml, const int *__restrict__ q_start,
-                                       const int *__restrict__ req_list, int nh, int n_splits) {
-    const int ri = blockIdx.x, head = blockIdx.y;
+__global__ void __launch_bounds__(DH / 4)
+attention_merge_kernel(bf16_t *__restrict__ out, int out_stride, const float *__restrict__ part_o,
+                       const float *__restrict__ part_ml, const int *__restrict__ q_start,
+                       const int *__restrict__ req_list, int nh, int n_splits) {
+    // a thread has four dims of one (token, head); the loads of up to eight parts are issued
+    // together, so the kernel takes one trip to memory and not one per part
+    constexpr int GROUP = 8;
+    const int ri = blockIdx.x, head = blockIdx.y, d0 = 4 * threadIdx.x;
     const int token = q_start[req_list ? req_list[ri] : ri];
     const size_t base = ((size_t)ri * nh + head) * n_splits;
-    float M = -INFINITY;
-    for (int s = 0; s < n_splits; ++s) M = fmaxf(M, part_ml[(base + s) * 2]);
-    float L = 0.f;
-    for (int s = 0; s < n_splits; ++s) L += part_ml[(base + s) * 2 + 1] * exp2f(part_ml[(base + s) * 2] - M);
-    const float inv = 1.0f / L;
-    for (int d = threadIdx.x; d < DH; d += blockDim.x) {
-        float val = 0.f;
-        for (int s = 0; s < n_splits; ++s) val += part_o[(base + s) * DH + d] * exp2f(part_ml[(base + s) * 2] - M);
-        out[(size_t)token * out_stride + (size_t)head * DH + d] = from_f32<bf16_t>(val * inv);
+    float M = -INFINITY, L = 0.f;
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    for (int s0 = 0; s0 < n_splits; s0 += GROUP) {
+        float m[GROUP], l[GROUP];
+        f32x4 o[GROUP];
+#pragma unroll
+        for (int i = 0; i < GROUP; ++i) {
+            const int s = s0 + i < n_splits ? s0 + i : n_splits - 1;        // past the end: the last part again, weight 0
+            m[i] = part_ml[(base + s) * 2];
+            l[i] = part_ml[(base + s) * 2 + 1];
+            o[i] = *(const f32x4 *)(part_o + (base + s) * DH + d0);
+        }
+        float Mn = M;
+#pragma unroll
+        for (int i = 0; i < GROUP; ++i) Mn = fmaxf(Mn, m[i]);
+        const float M_safe = Mn == -INFINITY ? 0.f : Mn;
+        const float keep = exp2f(M - M_safe);                                // 0 at the first group
+        L *= keep;
+        acc *= keep;
+#pragma unroll
+        for (int i = 0; i < GROUP; ++i) {
+            const float f = s0 + i < n_splits ? exp2f(m[i] - M_safe) : 0.f;
+            L += l[i] * f;
+            acc += o[i] * f;
+        }
+        M = Mn;
     }
+    const float inv = 1.0f / L;
+    u32x2 w;
+    w.x = pack_bf16(acc[0] * inv, acc[1] * inv);
+    w.y = pack_bf16(acc[2] * inv, acc[3] * inv);
+    *(u32x2 *)(out + (size_t)token * out_stride + (size_t)head * DH + d0) = w;
 }
 
 template <int DH>
@@ -368,7 +394,7 @@ static int launch_decode(const void *q, int q_stride, void *out, int out_stride,
         ctx_len, req_list, nh, nkvh, page, scale_log2, window, n_splits, part_o, part_ml);
     LCU_LAUNCH_CHECK();
     if (n_splits > 1) {
-        attention_merge_kernel<DH><<<dim3(n_req, nh), dim3(WAVE), 0, stream>>>((bf16_t *)out, out_stride, part_o, part_ml,
+        attention_merge_kernel<DH><<<dim3(n_req, nh), dim3(DH / 4), 0, stream>>>((bf16_t *)out, out_stride, part_o, part_ml,
                                                                                 q_start, req_list, nh, n_splits);
         LCU_LAUNCH_CHECK();
     }
