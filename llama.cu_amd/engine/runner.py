@@ -49,7 +49,7 @@ class ModelRunner:
     def __init__(self, spec: ModelSpec, tensors: Dict[str, torch.Tensor], dtype, device="cuda:0",
                  page_size: int = 16, max_tokens: Optional[int] = None, num_pages: Optional[int] = None,
                  max_seqs: int = 8, max_batch_tokens: int = 2048, max_model_len: Optional[int] = None,
-                 kv_fraction: float = 0.85, use_graphs: bool = True, pack_weights: bool = True):
+                 kv_fraction: float = 0.85, use_graphs: bool = True, pack_weights: Optional[bool] = None):
         self.device = require_gpu(device)
         self.dtype = DTYPES[dtype]
         self.spec = spec
@@ -60,7 +60,14 @@ class ModelRunner:
         self.max_seqs, self.max_batch_tokens = int(max_seqs), int(max_batch_tokens)
         torch.cuda.set_device(self.device)
         self.model = DecoderModel(spec)
-        build = BuildContext(self.dtype, self.device, spec.max_positions, self.page_size, bool(pack_weights))
+        if pack_weights is None:
+            # the second, packed copy of the matrices is worth its memory only while most of the
+            # card stays free for the cache: an 8B model takes it, a 70B model on one card does not
+            matrices = sum(t.numel() * t.element_size() for t in tensors.values() if t.dim() == 2)
+            free, total = torch.cuda.mem_get_info(self.device)
+            pack_weights = self.dtype == torch.bfloat16 and free - matrices >= 0.3 * total
+        self.pack_weights = bool(pack_weights)
+        build = BuildContext(self.dtype, self.device, spec.max_positions, self.page_size, self.pack_weights)
         self.model.load(tensors, build)
 
         # cache groups: one per distinct window among the layers that page keys and values

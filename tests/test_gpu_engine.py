@@ -161,6 +161,29 @@ def test_captured_decode_steps_equal_eager_ones():
         assert torch.equal(a, b), f"decode step {i} differs between eager and captured"
 
 
+def test_the_packed_copy_of_the_weights_changes_no_logit():
+    """With and without the second copy of the matrices in the decode kernels' order the
+    model gives the same bits, prompt and decoding; the copy is made by default where the
+    memory allows."""
+    from llama_cu_amd.engine.runner import ModelRunner
+    folder = common.make_folder(common.TINY_B, seed=33, dtype=torch.bfloat16, std=common.BF16_STD)
+    reqs = list(common.random_requests(384, [9, 40], seed=9).values())
+
+    def run(pack):
+        runner = ModelRunner.from_folder(folder, dtype="bfloat16", max_tokens=512, max_seqs=2, pack_weights=pack)
+        outs = [runner.step([0, 1], reqs).float().cpu()]
+        for i in range(4):
+            outs.append(runner.step([0, 1], [[3 + i], [200 - i]]).float().cpu())
+        return outs, runner
+
+    plain_outs, r0 = run(False)
+    packed_outs, r1 = run(None)
+    assert not r0.pack_weights and r1.pack_weights
+    assert r1.model.layers[0].mixer.w_qkv.packed is not None and r0.model.layers[0].mixer.w_qkv.packed is None
+    for a, b in zip(plain_outs, packed_outs):
+        assert torch.equal(a, b)
+
+
 def _run(engine, prompts, params=None, max_steps=20, ignore_eos=False, keep=False):
     """Tokens and finish reasons per request, through ``step()`` until idle."""
     from llama_cu_amd.sampling import GREEDY
