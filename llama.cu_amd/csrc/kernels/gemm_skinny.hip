@@ -241,43 +241,47 @@ gemm_skinny_kernel(const bf16_t *__restrict__ X, int ldx, const bf16_t *__restri
         }
     }
     if (EPI == EPI_QKV_ROPE) {
-        // the lane holds dims i = 16 c + 4 grp + r (tile 0) and i + head_dim/2 (tile 1) of token l16
-        const int tok = l16, dh = ex.head_dim, half_dim = dh / 2;
-        if (tok >= M) return;
-        const int pos = ex.positions[tok];
-        const bool in_table = pos >= 0 && pos < ex.max_pos;
-        const int slot = ex.slots ? ex.slots[tok] : -1;
+        // the lane holds dims i = 16 c + 4 grp + r (tile 0) and i + head_dim/2 (tile 1) of token 16 m + l16
+        const int dh = ex.head_dim, half_dim = dh / 2;
         const bool is_q = rope_head < ex.heads, is_k = !is_q && rope_head < ex.heads + ex.kv_heads;
-        bf16_t *pg = nullptr;
-        int place = 0;
-        if (!is_q && slot >= 0) {
-            pg = ex.cache + (size_t)(slot / ex.page) * kv_page_elems(ex.kv_heads, dh, ex.page);
-            place = slot % ex.page;
-        }
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const int i = 16 * rope_c + 4 * grp + r;
-            float a = acc[0][0][r], b = acc[NT - 1][0][r];
-            if (is_q || is_k) {
-                float c = __uint_as_float(0x7fc00000u), sn = c;         // a position outside the table gives NaN
-                if (in_table) { c = ex.cos_t[(size_t)pos * half_dim + i]; sn = ex.sin_t[(size_t)pos * half_dim + i]; }
-                const float ra = a * c - b * sn, rb = a * sn + b * c;
-                a = ra; b = rb;
+        for (int m = 0; m < MT; ++m) {
+            const int tok = 16 * m + l16;
+            if (tok >= M) continue;
+            const int pos = ex.positions[tok];
+            const bool in_table = pos >= 0 && pos < ex.max_pos;
+            const int slot = ex.slots ? ex.slots[tok] : -1;
+            bf16_t *pg = nullptr;
+            int place = 0;
+            if (!is_q && slot >= 0) {
+                pg = ex.cache + (size_t)(slot / ex.page) * kv_page_elems(ex.kv_heads, dh, ex.page);
+                place = slot % ex.page;
             }
-            const bf16_t va = from_f32<bf16_t>(a), vb = from_f32<bf16_t>(b);
-            if (is_q) {
-                bf16_t *qo = ex.q_out + (size_t)tok * ex.ldq + (size_t)rope_head * dh;
-                qo[i] = va;
-                qo[i + half_dim] = vb;
-            } else if (pg) {
-                if (is_k) {
-                    const int kvh = rope_head - ex.heads;
-                    pg[kv_key_offset(kvh, place, i, dh, ex.page)] = va;
-                    pg[kv_key_offset(kvh, place, i + half_dim, dh, ex.page)] = vb;
-                } else {
-                    const int kvh = rope_head - ex.heads - ex.kv_heads;
-                    pg[kv_value_offset(ex.kv_heads, kvh, place, i, dh, ex.page)] = va;
-                    pg[kv_value_offset(ex.kv_heads, kvh, place, i + half_dim, dh, ex.page)] = vb;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int i = 16 * rope_c + 4 * grp + r;
+                float a = acc[0][m][r], b = acc[NT - 1][m][r];
+                if (is_q || is_k) {
+                    float c = __uint_as_float(0x7fc00000u), sn = c;         // a position outside the table gives NaN
+                    if (in_table) { c = ex.cos_t[(size_t)pos * half_dim + i]; sn = ex.sin_t[(size_t)pos * half_dim + i]; }
+                    const float ra = a * c - b * sn, rb = a * sn + b * c;
+                    a = ra; b = rb;
+                }
+                const bf16_t va = from_f32<bf16_t>(a), vb = from_f32<bf16_t>(b);
+                if (is_q) {
+                    bf16_t *qo = ex.q_out + (size_t)tok * ex.ldq + (size_t)rope_head * dh;
+                    qo[i] = va;
+                    qo[i + half_dim] = vb;
+                } else if (pg) {
+                    if (is_k) {
+                        const int kvh = rope_head - ex.heads;
+                        pg[kv_key_offset(kvh, place, i, dh, ex.page)] = va;
+                        pg[kv_key_offset(kvh, place, i + half_dim, dh, ex.page)] = vb;
+                    } else {
+                        const int kvh = rope_head - ex.heads - ex.kv_heads;
+                        pg[kv_value_offset(ex.kv_heads, kvh, place, i, dh, ex.page)] = va;
+                        pg[kv_value_offset(ex.kv_heads, kvh, place, i + half_dim, dh, ex.page)] = vb;
+                    }
                 }
             }
         }
@@ -349,10 +353,10 @@ static int launch_epi(const void *X, int ldx, const void *W, int ldw, void *Y, i
     case EPI_F32: GO(EPI_F32); break;
     case EPI_ADD_F32: GO(EPI_ADD_F32); break;
     case EPI_ADD_NORM:
-        if constexpr (MT == 1 && NT <= 2) { GO(EPI_ADD_NORM); break; }      // made for decoding: at most 16 rows
+        if constexpr (MT <= 2 && NT <= 2) { GO(EPI_ADD_NORM); break; }      // made for decoding: at most 32 rows
         return LCU_UNSUPPORTED;
     case EPI_QKV_ROPE:
-        if constexpr (MT == 1 && NT == 2) {
+        if constexpr (MT <= 2 && NT == 2) {
             const dim3 rgrid((ex.heads + 2 * ex.kv_heads) * (ex.head_dim / 32));
             gemm_skinny_kernel<NT, MT, EPI_QKV_ROPE, WAVES><<<rgrid, block, 0, stream>>>(
                 (const bf16_t *)X, ldx, (const bf16_t *)W, ldw, Y, ldy, M, N, K, packed, ex);
@@ -435,11 +439,11 @@ LCU_API int lcu_gemm_skinny_bf16(const void *X, int ldx, const void *W, int ldw,
 // The product that ends a branch, the residual sum and the next norm's weight in one kernel:
 // res[M, N] (float32, rows ldres apart) += X W^T; h_out[M, N] = bfloat16(res * norm_w), not yet
 // normalised; sumsq_out[M][ceil(N / (16 tiles))] = each workgroup's share of the rows' sums of
-// squares.  At most 16 rows, tiles 1 or 2.
+// squares.  At most 32 rows, tiles 1 or 2.
 LCU_API int lcu_gemm_skinny_bf16_add_norm(const void *X, int ldx, const void *W, int ldw, float *res, int ldres, int M, int N,
                                           int K, const void *norm_w, int norm_w_type, void *h_out, int ldh, float *sumsq_out,
                                           int sumsq_cols, int tiles, int waves, int w_packed, hipStream_t stream) {
-    if (M > 16 || (tiles != 1 && tiles != 2) || !res || !norm_w || !h_out || !sumsq_out || ldh < N || ldres < N ||
+    if (M > 32 || (tiles != 1 && tiles != 2) || !res || !norm_w || !h_out || !sumsq_out || ldh < N || ldres < N ||
         (norm_w_type != LCU_F32 && norm_w_type != LCU_BF16) || sumsq_cols != (N + 16 * tiles - 1) / (16 * tiles))
         return LCU_BAD_ARGUMENT;
     SkinnyExtra ex = {};
@@ -464,7 +468,7 @@ LCU_API int lcu_gemm_skinny_bf16_scaled(const void *X, int ldx, const void *W, i
 // rows ldq apart takes the rotated queries; the rotated keys and the values go to cache (this
 // layer's pages, laid out as kv_layout.h says) at slots[m] (page * page_size + place; -1: nothing
 // is stored).  cos_t, sin_t: [max_pos, head_dim / 2] float32; pairs are (i, i + head_dim / 2).
-// At most 16 rows; head_dim a multiple of 32.  sumsq_in (may be null): the rows of X wait for
+// At most 32 rows; head_dim a multiple of 32.  sumsq_in (may be null): the rows of X wait for
 // their normalisation, as in lcu_gemm_skinny_bf16_scaled.
 LCU_API int lcu_gemm_skinny_bf16_qkv_rope(const void *X, int ldx, const void *W, int ldw, int M, int K, void *q_out, int ldq,
                                           const int *positions, const int *slots, const float *cos_t, const float *sin_t,
@@ -472,7 +476,7 @@ LCU_API int lcu_gemm_skinny_bf16_qkv_rope(const void *X, int ldx, const void *W,
                                           int waves, int w_packed, const float *sumsq_in, int n_in, int norm_width, float eps,
                                           hipStream_t stream) {
     if (M <= 0) return LCU_OK;
-    if (M > 16 || heads <= 0 || kv_heads <= 0 || head_dim <= 0 || head_dim % 32 || page <= 0 || page % 8 || !q_out ||
+    if (M > 32 || heads <= 0 || kv_heads <= 0 || head_dim <= 0 || head_dim % 32 || page <= 0 || page % 8 || !q_out ||
         !positions || !cos_t || !sin_t || max_pos <= 0 || !cache || ldq < heads * head_dim ||
         (sumsq_in && (n_in <= 0 || norm_width <= 0)))
         return LCU_BAD_ARGUMENT;

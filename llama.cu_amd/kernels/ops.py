@@ -429,7 +429,14 @@ def paged_attention(q: torch.Tensor, out: torch.Tensor, cache: torch.Tensor, ste
 
 
 SKINNY_MAX_ROWS = 64      # what the kernel takes
-SKINNY_ROWS = 16          # up to here it beats the library's product (measured on the Llama-3-8B shapes)
+SKINNY_ROWS = 16          # up to here it beats the library's product (measured on the Llama-3-8B shapes) ...
+SKINNY_ROWS_PACKED = 24   # ... and up to here when it reads a packed weight and its epilogues save the kernels around it
+                          # (whole decode steps of the Llama-3-8B shape: +9 % at 17 rows, +4 % at 24, -2 % at 32)
+
+
+def skinny_max_rows(packed: bool) -> int:
+    """The most rows for which the weight-streaming kernel is ever chosen over the library."""
+    return SKINNY_ROWS_PACKED if packed else SKINNY_ROWS
 _EPILOGUES = {"bf16": 0, "f32": 1, "add_f32": 2, "swiglu": 3}
 
 
@@ -468,13 +475,13 @@ def skinny_weight_ok(w: torch.Tensor) -> bool:
 def skinny_preferred(m: int, n: int, k: int, out_dtype: torch.dtype, packed: bool = False) -> bool:
     """Whether the weight-streaming kernel is the faster choice for a plain bfloat16 product
     of ``m`` rows with an ``[n, k]`` weight (measured against the library on the Llama-3-8B
-    shapes): always for very few rows and for float32 output; with a packed weight up to 16
-    rows (there it equals the library on the large weights, and its epilogues save the kernels
-    around the product); without one, beyond 4 rows, only for small weights (the library's
-    split over K wins on the large ones)."""
-    if m > SKINNY_ROWS:
+    shapes): always for very few rows and for float32 output; with a packed weight up to 24
+    rows (there it is within a tenth of the library on the large weights, and its epilogues save
+    the kernels around the product); without one, beyond 4 and up to 16 rows, only for small
+    weights (the library's split over K wins on the large ones)."""
+    if m > skinny_max_rows(packed):
         return False
-    return m <= (SKINNY_ROWS if packed else 4) or out_dtype == torch.float32 or n * k <= (1 << 24)
+    return m <= (SKINNY_ROWS_PACKED if packed else 4) or out_dtype == torch.float32 or n * k <= (1 << 24)
 
 
 def _skinny_tiles(n_features: int, m: int, packed: bool = False) -> int:
@@ -543,7 +550,7 @@ def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = 
     return out
 
 
-ADD_NORM_MAX_ROWS = 16
+ADD_NORM_MAX_ROWS = 32
 
 
 def gemm_skinny_add_norm(x: torch.Tensor, w: torch.Tensor, residual: torch.Tensor, norm_weight: torch.Tensor,
@@ -552,7 +559,7 @@ def gemm_skinny_add_norm(x: torch.Tensor, w: torch.Tensor, residual: torch.Tenso
     kernel: ``residual += x @ w.T`` (float32, in place); returns ``(h, sumsq)`` with
     ``h = bfloat16(residual * norm_weight)``, not yet normalised, and ``sumsq [rows, parts]``,
     the workgroups' shares of each row's sum of squares, for ``gemm_skinny(..., row_sumsq=)``.
-    At most 16 rows."""
+    At most 32 rows."""
     _gpu(x, w, residual, norm_weight)
     _rows(x, "skinny x"); _rows(w, "skinny w"); _rows(residual, "residual")
     if packed and not (packable(w) and w.is_contiguous()):
@@ -578,11 +585,11 @@ def gemm_skinny_add_norm(x: torch.Tensor, w: torch.Tensor, residual: torch.Tenso
     return h, sumsq
 
 
-QKV_ROPE_MAX_ROWS = 16
+QKV_ROPE_MAX_ROWS = 32
 
 
 def qkv_rope_supported(x: torch.Tensor, w: torch.Tensor, heads: int, kv_heads: int, head_dim: int) -> bool:
-    """Whether ``gemm_skinny_qkv_rope`` takes these operands: at most 16 rows, bfloat16, whole
+    """Whether ``gemm_skinny_qkv_rope`` takes these operands: at most 32 rows, bfloat16, whole
     heads whose halves are multiples of 16."""
     return (x.dim() == 2 and x.shape[0] <= QKV_ROPE_MAX_ROWS and head_dim % 32 == 0
             and w.shape[0] == (heads + 2 * kv_heads) * head_dim and skinny_supported(x, w, torch.bfloat16))

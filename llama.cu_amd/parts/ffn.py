@@ -13,7 +13,7 @@ import torch
 
 from ..kernels import ops
 from .base import BuildContext, Part, ScaledRows, TensorSpec, register_part
-from .linear import Weight, linear, linear_into_norm, linear_swiglu, skinny_takes
+from .linear import Weight, linear, linear_into_norm, linear_swiglu, skinny_row_limit, skinny_takes
 
 
 class SwiGLU(Part):
@@ -39,7 +39,8 @@ class SwiGLU(Part):
     def takes_scaled_rows(self, n_rows: int) -> bool:
         """Whether ``forward`` could be given ScaledRows of ``n_rows`` rows in the place of
         plain rows: the factor then goes into the first product's epilogue."""
-        return self.dtype == torch.bfloat16 and n_rows <= ops.ADD_NORM_MAX_ROWS and skinny_takes(n_rows, self.w_gate_up)
+        return (self.dtype == torch.bfloat16 and n_rows <= min(ops.ADD_NORM_MAX_ROWS, skinny_row_limit(self.w_gate_up))
+                and skinny_takes(n_rows, self.w_gate_up))
 
     # forward(..., into=(residual, norm)) may end with the residual sum and that norm's weight
     # in the down projection and return ScaledRows instead of the branch's output
@@ -50,7 +51,8 @@ class SwiGLU(Part):
             if not ops.skinny_supported(h.rows, self.w_gate_up.plain, self.dtype):
                 raise ops.KernelError("feed-forward: rows that wait for their normalisation need the kernel for few rows")
             act = linear_swiglu(h.rows, self.w_gate_up, row_sumsq=h.sumsq, norm_width=h.width, eps=h.eps)
-        elif self.dtype == torch.bfloat16 and h.shape[0] <= ops.SKINNY_ROWS and ops.skinny_supported(h, self.w_gate_up.plain, self.dtype):
+        elif (self.dtype == torch.bfloat16 and h.shape[0] <= skinny_row_limit(self.w_gate_up)
+              and ops.skinny_supported(h, self.w_gate_up.plain, self.dtype)):
             # few rows: one pass over the weights, the activation in the product's epilogue
             act = linear_swiglu(h, self.w_gate_up)
         else:

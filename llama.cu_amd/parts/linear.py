@@ -67,7 +67,7 @@ def linear(x: torch.Tensor, weight: Union[torch.Tensor, Weight], out_dtype: Opti
         if out is None:
             return torch.matmul(x, weight.t())
         return torch.matmul(x, weight.t(), out=out)
-    if all_bf16 and out_dtype == torch.float32 and not accumulate and out is None and x.shape[0] > ops.SKINNY_ROWS:
+    if all_bf16 and out_dtype == torch.float32 and not accumulate and out is None and x.shape[0] > ops.skinny_max_rows(packed is not None):
         return torch.mm(x, weight.t(), out_dtype=torch.float32)      # 32-bit accumulation, stored unrounded (logits)
     if ops.skinny_f32_supported(x, weight, out_dtype):
         return ops.gemm_skinny_f32(x, weight, out=out, accumulate=accumulate)
@@ -91,6 +91,11 @@ def linear_scaled(rows, weight: Union[torch.Tensor, Weight]):
     if packed is not None:
         return ops.gemm_skinny(rows.rows, packed, packed=True, **kw)
     return ops.gemm_skinny(rows.rows, weight, **kw)
+
+
+def skinny_row_limit(weight: Union[torch.Tensor, Weight]) -> int:
+    """Up to how many rows the weight-streaming kernel may be chosen for this weight."""
+    return ops.skinny_max_rows(_split(weight)[1] is not None)
 
 
 def skinny_takes(n_rows: int, weight: Union[torch.Tensor, Weight], preferred: bool = False) -> bool:

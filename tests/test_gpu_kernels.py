@@ -449,7 +449,8 @@ def test_gemm_skinny_refuses_what_it_cannot_take():
 
 
 @pytest.mark.parametrize("m,n,k,tiles,wdtype", [(1, 16, 8, 1, "bfloat16"), (8, 304, 136, 1, "float32"), (16, 4096, 1000, 1, "bfloat16"),
-                                                (5, 104, 64, 2, "bfloat16"), (13, 1000, 4096, 2, "float32")])
+                                                (5, 104, 64, 2, "bfloat16"), (13, 1000, 4096, 2, "float32"),
+                                                (17, 304, 256, 1, "bfloat16"), (32, 1000, 512, 2, "float32"), (27, 96, 136, 2, "bfloat16")])
 def test_gemm_skinny_residual_sum_and_norm_weight_in_the_epilogue(m, n, k, tiles, wdtype):
     """``residual += x w^T``; the new rows times the norm's weight as bfloat16, not yet normalised;
     the workgroups' shares of the rows' sums of squares.  Then a second product applies the
@@ -483,7 +484,7 @@ def test_gemm_skinny_residual_sum_and_norm_weight_in_the_epilogue(m, n, k, tiles
     assert torch.equal(sumsq, sumsq2) and torch.equal(h, h2) and torch.equal(res_g, res_g2)
 
 
-@pytest.mark.parametrize("m,n,k", [(1, 16, 128), (8, 304, 256), (16, 4096, 1024), (13, 96, 384)])
+@pytest.mark.parametrize("m,n,k", [(1, 16, 128), (8, 304, 256), (16, 4096, 1024), (13, 96, 384), (30, 608, 256)])
 def test_gemm_skinny_with_a_packed_weight_equals_the_plain_one_bit_for_bit(m, n, k):
     """``pack_weight`` only changes where the kernel finds its operands, not what it adds in
     which order: every epilogue gives the same bits as with the plain weight.  The packed
@@ -518,7 +519,8 @@ def test_gemm_skinny_with_a_packed_weight_equals_the_plain_one_bit_for_bit(m, n,
 
 @pytest.mark.parametrize("m,k,nh,nkv,dh,page,packed,scaled", [(1, 64, 4, 2, 32, 8, False, False), (8, 256, 6, 2, 64, 16, True, True),
                                                               (16, 136, 3, 1, 96, 24, False, True), (5, 512, 8, 8, 128, 32, True, False),
-                                                              (13, 128, 5, 5, 160, 16, True, False)])
+                                                              (13, 128, 5, 5, 160, 16, True, False), (17, 256, 4, 2, 64, 16, True, True),
+                                                              (32, 136, 3, 3, 32, 8, False, False), (29, 128, 8, 2, 128, 16, True, True)])
 def test_gemm_skinny_q_k_v_with_rotation_and_cache_write(m, k, nh, nkv, dh, page, packed, scaled):
     """The product of few rows with the q, k and v weights whose epilogue rotates q and k and
     writes k and v into the pages: against product, rotation and cache layout done one after
@@ -574,10 +576,10 @@ def test_gemm_skinny_q_k_v_with_rotation_and_cache_write(m, k, nh, nkv, dh, page
 
 def test_gemm_skinny_add_norm_refuses_what_it_cannot_take():
     from llama_cu_amd.kernels import ops
-    x = rnd(17, 64).to(torch.bfloat16).cuda()
+    x = rnd(33, 64).to(torch.bfloat16).cuda()
     w = rnd(32, 64).to(torch.bfloat16).cuda()
     with pytest.raises(ops.KernelError):
-        ops.gemm_skinny_add_norm(x, w, torch.zeros(17, 32).cuda(), torch.ones(32).cuda())        # more than 16 rows
+        ops.gemm_skinny_add_norm(x, w, torch.zeros(33, 32).cuda(), torch.ones(32).cuda())        # more than 32 rows
     with pytest.raises(ops.KernelError):
         ops.gemm_skinny_add_norm(x[:4], w, torch.zeros(4, 32, dtype=torch.bfloat16).cuda(), torch.ones(32).cuda())
     with pytest.raises(ops.KernelError):
