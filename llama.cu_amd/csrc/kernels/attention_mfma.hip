@@ -526,29 +526,37 @@ constexpr int PRE_RING = 3;               // buffers of 64 keys in LDS: one is r
 // A page holds less than 4 GiB (the host checks).
 template <int DH>
 __device__ __forceinline__ void stage_issue(u32x4 *__restrict__ buf, const bf16_t *__restrict__ cache,
-                                            const int *__restrict__ bt, int max_pages, int page, size_t page_elems,
-                                            int nkvh, int kvh, int k0) {
-    const uint32_t v_off = (uint32_t)(nkvh + kvh) * DH * page;
-    const int wave = threadIdx.x / WAVE;
+                                            const int *__restrict__ bt, int max_pages, int page, uint32_t tile_magic,
+                                            size_t page_elems, int nkvh, int kvh, int k0, int wave_id) {
+    // Everything but the lane's offset is made in scalar registers from the wave's number: a wave's
+    // 64 chunks lie in one region of one step (regions are multiples of 64 chunks), and a tile of 16
+    // keys lies in one page.  Tile T is in page T / (page / 16): with tile_magic =
+    // floor(2^32 / (page / 16)) + 1 the quotient is the high word of T * tile_magic (exact while
+    // T * page / 16 < 2^32; 0 stands for pages of 16 keys, where the page is the tile).
+    constexpr uint32_t E = sizeof(bf16_t);
+    const int tiles_per_page = page / 16;
+    int tid = threadIdx.x;
+    asm volatile("" : "+v"(tid));                  // made anew in every step, not kept in registers across the loop
+    const int lane = tid & (WAVE - 1);
+    const uint32_t k_lane = ((uint32_t)(lane >> 4) * page + (lane & 15)) * 8 * E;       // keys [dim/8][token][8]
+    const uint32_t v_lane = ((uint32_t)(lane >> 1) * page + (lane & 1) * 8) * E;        // values [dim][token]
 #pragma unroll
     for (int i = 0; i < DH / 32; ++i) {
-        const int c2 = threadIdx.x + 512 * i;
-        const int sub = c2 / (8 * DH), c = c2 % (8 * DH);
-        const int region = c / (2 * DH), w = c % (2 * DH), t = region & 1;
-        const int j = k0 + 32 * sub + 16 * t;
-        int pi = j / page;
+        const int cw = wave_id * WAVE + 512 * i;                  // the wave's first chunk
+        const int sub = cw / (8 * DH), c = cw % (8 * DH);
+        const int region = c / (2 * DH), w0 = c % (2 * DH), t = region & 1;
+        const uint32_t tile = (uint32_t)(k0 >> 4) + 2 * sub + t;
+        int pi = tile_magic ? (int)__umulhi(tile, tile_magic) : (int)tile;
+        const uint32_t tok0 = (tile - (uint32_t)pi * tiles_per_page) * 16;
         pi = pi < max_pages ? pi : max_pages - 1;
-        const int page_id = bt[__builtin_amdgcn_readfirstlane(pi)];
-        const int tok0 = j % page;
-        // within the page, in elements: keys [dim/8][token][8], values [dim][token]
-        const uint32_t lane_off = region < 2 ? ((uint32_t)(kvh * (DH / 8) + w / 16) * page + (w % 16)) * 8
-                                             : v_off + (uint32_t)(w / 2) * page + (w % 2) * 8;
-        const uint32_t tok_off = __builtin_amdgcn_readfirstlane(region < 2 ? tok0 * 8 : tok0);
+        const int page_id = bt[pi];
+        const uint32_t s_off = region < 2 ? ((uint32_t)(kvh * (DH / 8) + w0 / 16) * page + tok0) * 8 * E
+                                          : ((uint32_t)((nkvh + kvh) * DH + w0 / 2) * page + tok0) * E;
         // a buffer load whose buffer is the page: all of the address but the lane's offset is scalar
         const __amdgpu_buffer_rsrc_t pg = __builtin_amdgcn_make_buffer_rsrc(
-            const_cast<bf16_t *>(cache + (size_t)page_id * page_elems), 0, (uint32_t)(page_elems * sizeof(bf16_t)), 0x00020000);
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(pg, (__attribute__((address_space(3))) void *)(buf + 512 * i + WAVE * wave), 16,
-                                                 lane_off * (uint32_t)sizeof(bf16_t), tok_off * (uint32_t)sizeof(bf16_t), 0, 0);
+            const_cast<bf16_t *>(cache + (size_t)page_id * page_elems), 0, (uint32_t)(page_elems * E), 0x00020000);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(pg, (__attribute__((address_space(3))) void *)(buf + 512 * i + WAVE * wave_id), 16,
+                                                 region < 2 ? k_lane : v_lane, s_off, 0, 0);
     }
 }
 
@@ -566,11 +574,12 @@ __device__ __forceinline__ void wait_loads() {
 template <int DH, int QB>
 __device__ __forceinline__ void ring_step(const u32x4 *__restrict__ src, u32x4 *__restrict__ dst,
                                           const bf16_t *__restrict__ cache, const int *__restrict__ bt, int max_pages, int page,
-                                          size_t page_elems, int nkvh, int kvh, int k0_copy, int blk, int blk_end,
+                                          uint32_t tile_magic, size_t page_elems, int nkvh, int kvh, int k0_copy, int wave_id,
+                                          int blk, int blk_end,
                                           bool wave_has, int p_max, int p_min, int lo_min, int lo_max,
                                           const int (&tok_row)[QB], int pos_of_tok, int window, const u32x4 (&qv)[QB][DH / 32],
                                           AttnState<DH, QB> &st, float scale_log2) {
-    stage_issue<DH>(dst, cache, bt, max_pages, page, page_elems, nkvh, kvh, k0_copy);
+    stage_issue<DH>(dst, cache, bt, max_pages, page, tile_magic, page_elems, nkvh, kvh, k0_copy, wave_id);
     const int k0 = blk * 32;
     // the lane's coordinates are made anew in every step: kept across the loop they would
     // be spilled, and a reload from scratch waits for all the copies in flight
@@ -609,7 +618,7 @@ attention_prefill_kernel(const bf16_t *__restrict__ q, int q_stride, bf16_t *__r
                          const bf16_t *__restrict__ cache, const int *__restrict__ block_table, int max_pages,
                          const int *__restrict__ q_start, const int *__restrict__ ctx_len,
                          const int *__restrict__ task_req, const int *__restrict__ task_tok0, int n_tasks,
-                         int tasks_per_wg, int nh, int nkvh, int page, float scale_log2, int window) {
+                         int tasks_per_wg, int nh, int nkvh, int page, uint32_t tile_magic, float scale_log2, int window) {
     extern __shared__ u32x4 lds_ring[];            // [PRE_RING][16 * DH]; at the end the halves' states
     // the wave's number as a scalar: what follows from it (its rows' limits) then lives in scalar registers
     const int wave_id = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
@@ -668,13 +677,15 @@ attention_prefill_kernel(const bf16_t *__restrict__ q, int q_stride, bf16_t *__r
     const int n_dsteps = (blk_end - blk0 + 1) / 2;
 #pragma unroll
     for (int d = 0; d < PRE_RING - 1; ++d)
-        stage_issue<DH>(lds_ring + d * 16 * DH, cache, bt, max_pages, page, page_elems, nkvh, kvh, (blk0 + 2 * d) * 32);
+        stage_issue<DH>(lds_ring + d * 16 * DH, cache, bt, max_pages, page, tile_magic, page_elems, nkvh, kvh, (blk0 + 2 * d) * 32,
+                        wave_id);
     int slot = 0, fill = PRE_RING - 1;
     for (int d = 0; d < n_dsteps; ++d) {
         wait_loads<(PRE_RING - 2) * (DH / 32)>();
         lds_barrier();
         ring_step<DH, QB>(lds_ring + slot * 16 * DH + half * 8 * DH, lds_ring + fill * 16 * DH, cache, bt, max_pages, page,
-                          page_elems, nkvh, kvh, (blk0 + 2 * (d + PRE_RING - 1)) * 32, blk0 + 2 * d + half, blk_end, wave_has,
+                          tile_magic, page_elems, nkvh, kvh, (blk0 + 2 * (d + PRE_RING - 1)) * 32, wave_id, blk0 + 2 * d + half,
+                          blk_end, wave_has,
                           p_max, p_min, lo_min, lo_max, tok_row, pos_of_tok, window, qv, st, scale_log2);
         slot = slot + 1 == PRE_RING ? 0 : slot + 1;
         fill = fill + 1 == PRE_RING ? 0 : fill + 1;
@@ -746,7 +757,8 @@ static int launch_prefill(const void *q, int q_stride, void *out, int out_stride
     }
     attention_prefill_kernel<DH, QB><<<grid, block, lds_bytes, stream>>>(
         (const bf16_t *)q, q_stride, (bf16_t *)out, out_stride, (const bf16_t *)cache, block_table, max_pages, q_start,
-        ctx_len, task_req, task_tok0, n_tasks, tasks_per_wg, nh, nkvh, page, scale * 1.4426950408889634f, window);
+        ctx_len, task_req, task_tok0, n_tasks, tasks_per_wg, nh, nkvh, page,
+        page == 16 ? 0u : (uint32_t)(0x100000000ull / (unsigned)(page / 16)) + 1u, scale * 1.4426950408889634f, window);
     LCU_LAUNCH_CHECK();
     return LCU_OK;
 }
