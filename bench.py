@@ -55,12 +55,18 @@ def prefill_flops(c, t):
     return matmul + attention
 
 
-def run_decode(engine, cfg, batch, steps, warmup, rng, sync):
+def rounds_of(prompt_len):
+    """Rounds that a prompt's prefill takes (portions of PREFILL_TOKENS): earlier requests decode meanwhile."""
+    return (prompt_len + PREFILL_TOKENS - 1) // PREFILL_TOKENS
+
+
+def run_decode(engine, cfg, batch, steps, warmup, rng, sync, prompt_len=PROMPT_LEN):
     """Prefill ``batch`` prompts, then time ``steps`` decode steps.  Returns (seconds,
     tokens decoded in them, mean context length during the timed steps)."""
     from llama_cu_amd.sampling import GREEDY
-    ids = [engine.add_request([rng.randrange(cfg.vocab_size) for _ in range(PROMPT_LEN)], GREEDY,
-                              max_steps=steps + warmup + 2 * batch + 8, ignore_eos=True) for _ in range(batch)]
+    ids = [engine.add_request([rng.randrange(cfg.vocab_size) for _ in range(prompt_len)], GREEDY,
+                              max_steps=steps + warmup + 2 * batch * rounds_of(prompt_len) + 8, ignore_eos=True)
+           for _ in range(batch)]
     # prefill rounds: until every request has produced its first token
     while any(engine.sched.info(i).generated == 0 for i in ids):
         engine.step()
@@ -137,6 +143,9 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the shape has (named in config)")
+    ap.add_argument("--prompt-len", type=int, default=PROMPT_LEN,
+                    help="tokens of each request's prompt (other context lengths than the default run's; the context "
+                         "limit grows with it)")
     ap.add_argument("--dtype", choices=["bfloat16", "float32"], default="bfloat16")
     ap.add_argument("--no-points", action="store_true", help="skip decoding at batch 1 and 64 and the prefill")
     ap.add_argument("--only-prefill", action="store_true", help="time the 2048-token prefill alone (for profiles)")
@@ -158,6 +167,10 @@ def main() -> int:
     full_layers = shape["num_hidden_layers"]
     if args.layers:
         shape["num_hidden_layers"] = args.layers
+    grow = args.steps + args.warmup + 2 * max(args.batch, 64) * rounds_of(args.prompt_len) + 64
+    need_ctx = args.prompt_len + grow + 64
+    while shape["max_position_embeddings"] < need_ctx:
+        shape["max_position_embeddings"] *= 2
     cfg = LlamaConfig.from_dict(shape)
     dt_name = "bf16" if args.dtype == "bfloat16" else "f32"
     elem = 2 if args.dtype == "bfloat16" else 4
@@ -166,7 +179,7 @@ def main() -> int:
     page = 16
     biggest = max(args.batch, 1 if (args.no_points or args.only_prefill) else 64)
     # a request decodes while later ones still prefill: room for that too
-    per_req = PROMPT_LEN + args.steps + args.warmup + 2 * biggest + 64
+    per_req = max(args.prompt_len, PROMPT_LEN) + grow
     engine = Engine.from_config(cfg, seed=0, dtype=args.dtype, page_size=page,
                                 max_tokens=biggest * ((per_req + page - 1) // page * page) + PREFILL_TOKENS + page,
                                 max_seqs=biggest + 2, max_batch_tokens=max(PREFILL_TOKENS, biggest), prefill_chunk=PREFILL_TOKENS)
@@ -176,16 +189,16 @@ def main() -> int:
         print(json.dumps({"prefill": {"value": round(PREFILL_TOKENS / pt, 1), "tokens": PREFILL_TOKENS, "ms": round(pt * 1e3, 3),
                                       "frac": round(prefill_flops(cfg, PREFILL_TOKENS) / pt / MATRIX_PEAK[dt_name], 4)}}))
         return 0
-    seconds, produced, mean_ctx = run_decode(engine, cfg, args.batch, args.steps, args.warmup, rng, sync)
+    seconds, produced, mean_ctx = run_decode(engine, cfg, args.batch, args.steps, args.warmup, rng, sync, args.prompt_len)
     ms_per_step = seconds / args.steps * 1e3
     value = produced / seconds
     step_bytes = weight_bytes(cfg, elem) + args.batch * mean_ctx * kv_bytes_per_token(cfg, elem)
     achieved = step_bytes / (seconds / args.steps)
     line = {
-        "metric": "decode tok/s (Llama-3-8B shape, prompts of 2048 tokens)", "value": round(value, 2), "unit": "tok/s",
+        "metric": f"decode tok/s (Llama-3-8B shape, prompts of {args.prompt_len} tokens)", "value": round(value, 2), "unit": "tok/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": dt_name, "data": "synthetic",
-        "config": {"model": "Llama-3-8B shape, random weights", "global_batch": args.batch, "seq_len": PROMPT_LEN,
+        "config": {"model": "Llama-3-8B shape, random weights", "global_batch": args.batch, "seq_len": args.prompt_len,
                    "parallelism": "none (1 GPU)", "context": cfg.max_position_embeddings,
                    "layers": cfg.num_hidden_layers, "layers_of_shape": full_layers, "hidden_size": cfg.hidden_size,
                    "heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads, "head_dim": cfg.head_dim,
