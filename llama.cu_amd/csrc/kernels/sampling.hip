@@ -44,24 +44,34 @@ __device__ __forceinline__ void scan_row(const float *__restrict__ row, int voca
 }
 
 // ---------------------------------------------------------------- arg-max
-// The largest logit of each row; among equals the lowest index.  NaN never wins.
+// The largest logit of each row; among equals the lowest index.  NaN never wins.  A row is cut
+// into gridDim.y parts, one workgroup each (a single workgroup reads a long row at the speed of
+// one compute unit); with more than one part the parts' winners go to part_val / part_idx
+// [rows][parts] and argmax_merge_kernel picks among them.
 __global__ void __launch_bounds__(SAMPLE_THREADS)
-argmax_kernel(const float *__restrict__ logits, int ld, int vocab, int *__restrict__ out) {
+argmax_kernel(const float *__restrict__ logits, int ld, int vocab, int *__restrict__ out, float *__restrict__ part_val,
+              int *__restrict__ part_idx) {
     const float *row = logits + (size_t)blockIdx.x * ld;
+    const int parts = gridDim.y, part = blockIdx.y;
+    // the part's share of the row, in units of four logits
+    const int quads = (vocab + 3) / 4;
+    const int lo = (int)((long long)quads * part / parts) * 4;
+    int hi = (int)((long long)quads * (part + 1) / parts) * 4;
+    hi = hi < vocab ? hi : vocab;
     float best = -INFINITY;
     int bi = 0x7fffffff;
-    // four neighbouring logits per load where the row allows it (many loads in flight: a
-    // row is read by one workgroup, so latency, not bandwidth, is what counts)
-    const int vec_end = (((size_t)row % 16) == 0) ? (vocab / 4) * 4 : 0;
+    // four neighbouring logits per load where the row allows it (many loads in flight: latency,
+    // not bandwidth, is what counts)
+    const int vec_end = (((size_t)row % 16) == 0) ? lo + ((hi - lo) / 4) * 4 : lo;
 #pragma unroll 4
-    for (int i = threadIdx.x * 4; i < vec_end; i += blockDim.x * 4) {
+    for (int i = lo + threadIdx.x * 4; i < vec_end; i += blockDim.x * 4) {
         const float4 v = *(const float4 *)(row + i);
         const float e[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
         for (int k = 0; k < 4; ++k)
             if (e[k] > best || (e[k] == best && i + k < bi)) { best = e[k]; bi = i + k; }
     }
-    for (int i = vec_end + threadIdx.x; i < vocab; i += blockDim.x) {
+    for (int i = vec_end + threadIdx.x; i < hi; i += blockDim.x) {
         const float v = row[i];
         if (v > best || (v == best && i < bi)) { best = v; bi = i; }
     }
@@ -79,15 +89,45 @@ argmax_kernel(const float *__restrict__ logits, int ld, int vocab, int *__restri
     if (threadIdx.x == 0) {
         for (int w = 1; w < (int)(blockDim.x / WAVE); ++w)
             if (sv[w] > best || (sv[w] == best && si[w] < bi)) { best = sv[w]; bi = si[w]; }
-        out[blockIdx.x] = bi == 0x7fffffff ? 0 : bi;
+        if (parts == 1) {
+            out[blockIdx.x] = bi == 0x7fffffff ? 0 : bi;
+        } else {
+            part_val[(size_t)blockIdx.x * parts + part] = best;
+            part_idx[(size_t)blockIdx.x * parts + part] = bi;
+        }
     }
 }
 
-LCU_API int lcu_argmax(const float *logits, int ld, int rows, int vocab, int *out, hipStream_t stream) {
+__global__ void argmax_merge_kernel(const float *__restrict__ part_val, const int *__restrict__ part_idx, int parts,
+                                    int *__restrict__ out) {
+    float best = -INFINITY;
+    int bi = 0x7fffffff;
+    for (int p = threadIdx.x; p < parts; p += WAVE) {
+        const float v = part_val[(size_t)blockIdx.x * parts + p];
+        const int i = part_idx[(size_t)blockIdx.x * parts + p];
+        if (v > best || (v == best && i < bi)) { best = v; bi = i; }
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        const float ov = __shfl_xor(best, off, WAVE);
+        const int oi = __shfl_xor(bi, off, WAVE);
+        if (ov > best || (ov == best && oi < bi)) { best = ov; bi = oi; }
+    }
+    if (threadIdx.x == 0) out[blockIdx.x] = bi == 0x7fffffff ? 0 : bi;
+}
+
+// parts: into how many workgroups a row is cut (1: one kernel, no scratch); part_val, part_idx:
+// [rows * parts] when parts > 1.
+LCU_API int lcu_argmax(const float *logits, int ld, int rows, int vocab, int *out, int parts, float *part_val, int *part_idx,
+                       hipStream_t stream) {
     if (rows <= 0) return LCU_OK;
-    if (vocab <= 0 || ld < vocab) return LCU_BAD_ARGUMENT;
-    argmax_kernel<<<dim3(rows), dim3(SAMPLE_THREADS), 0, stream>>>(logits, ld, vocab, out);
+    if (vocab <= 0 || ld < vocab || parts < 1 || parts > 1024 || (parts > 1 && (!part_val || !part_idx))) return LCU_BAD_ARGUMENT;
+    argmax_kernel<<<dim3(rows, parts), dim3(SAMPLE_THREADS), 0, stream>>>(logits, ld, vocab, out, part_val, part_idx);
     LCU_LAUNCH_CHECK();
+    if (parts > 1) {
+        argmax_merge_kernel<<<dim3(rows), dim3(WAVE), 0, stream>>>(part_val, part_idx, parts, out);
+        LCU_LAUNCH_CHECK();
+    }
     return LCU_OK;
 }
 

@@ -44,6 +44,7 @@ class StepContext:
     ctx_lens: List[int] = field(default_factory=list)
     req_ids: List[int] = field(default_factory=list)
     state_slots: List[int] = field(default_factory=list)    # ``state_slot`` on the host
+    logits_all: bool = False                    # the logits of every token are wanted, in order (logit_rows is 0, 1, ...)
     attn_splits: Optional[int] = None           # fixed number of key parts for the decode kernel (captured graphs)
     scratch: dict = field(default_factory=dict)  # what kernels' wrappers derive from the batch once per step
     # tokens that the step before sampled and the host does not know yet: tokens[feed_dst[i]] is
@@ -157,7 +158,7 @@ class BatchBuilder:
             n=n, n_req=n_req, tokens=self._d("tokens", n), positions=self._d("positions", n),
             req_of_token=self._d("req_of_token", n), q_start=self._d("q_start", n_req + 1),
             ctx_len=self._d("ctx_len", n_req), state_slot=self._d("state_slot", n_req),
-            logit_rows=self._d("logit_rows", len(rows)), n_logits=len(rows),
+            logit_rows=self._d("logit_rows", len(rows)), n_logits=len(rows), logits_all=rows == list(range(n)),
             block_tables=[self._d(f"block_table{g}", n_req * mp).view(n_req, mp) for g, mp in enumerate(self.max_pages)],
             slot_maps=[self._d(f"slots{g}", n) for g in range(len(self.max_pages))],
             q_lens=n_new, ctx_lens=ctx_lens, req_ids=list(req_ids),

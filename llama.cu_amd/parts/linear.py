@@ -84,10 +84,10 @@ def linear_swiglu(h, weight: Union[torch.Tensor, Weight], row_sumsq=None, norm_w
     return ops.gemm_skinny(h, weight, swiglu=True, **kw)
 
 
-def linear_scaled(rows, weight: Union[torch.Tensor, Weight]):
+def linear_scaled(rows, weight: Union[torch.Tensor, Weight], out_dtype: Optional[torch.dtype] = None):
     """``rows.rows @ weight.T`` with the rows' normalisation applied in the epilogue (``rows``: ScaledRows)."""
     weight, packed = _split(weight)
-    kw = dict(row_sumsq=rows.sumsq, norm_width=rows.width, eps=rows.eps)
+    kw = dict(row_sumsq=rows.sumsq, norm_width=rows.width, eps=rows.eps, out_dtype=out_dtype)
     if packed is not None:
         return ops.gemm_skinny(rows.rows, packed, packed=True, **kw)
     return ops.gemm_skinny(rows.rows, weight, **kw)

@@ -15,8 +15,8 @@ from typing import Dict, List, Optional
 import torch
 
 from ..kernels import ops
-from .base import BuildContext, ModelSpec, Part, PartSpec, TensorSpec, make_part, prefixed, register_part
-from .linear import Weight, linear
+from .base import BuildContext, ModelSpec, Part, PartSpec, ScaledRows, TensorSpec, make_part, prefixed, register_part
+from .linear import Weight, linear, linear_scaled, skinny_takes
 
 
 class TokenEmbedding(Part):
@@ -55,8 +55,16 @@ class OutputHead(Part):
     def load(self, tensors, build: BuildContext, table: Optional[torch.Tensor] = None) -> None:
         own = tensors.get("weight")
         self.weight = Weight(table if (self.tied or own is None) else own, build)
+        self.dtype = build.dtype
 
-    def forward(self, y: torch.Tensor) -> torch.Tensor:
+    def takes_scaled_rows(self, n_rows: int) -> bool:
+        """Whether ``forward`` could be given ScaledRows of ``n_rows`` rows made with the final norm."""
+        return (self.dtype == torch.bfloat16 and n_rows <= ops.ADD_NORM_MAX_ROWS
+                and skinny_takes(n_rows, self.weight, preferred=True))
+
+    def forward(self, y) -> torch.Tensor:
+        if isinstance(y, ScaledRows):
+            return linear_scaled(y, self.weight, out_dtype=torch.float32)
         return linear(y, self.weight, out_dtype=torch.float32)
 
 
@@ -124,16 +132,28 @@ class DecoderModel:
             pending = None
             order = self.spec.run_order
             for i, e in enumerate(order):
-                # a block may end in the next block's first norm, if that block takes such rows
-                follower = self.layers[order[i + 1].layer] if i + 1 < len(order) else None
+                # a block may end in the norm that follows it, if what comes then takes such rows: the
+                # next block with its first norm, or, when every token's logits are wanted, the output
+                # matrix with the final norm
+                if i + 1 < len(order):
+                    follower = self.layers[order[i + 1].layer]
+                    norm = getattr(follower, "norm1", None)
+                else:
+                    follower = self.head if step.logits_all and getattr(self.final_norm, "deferrable", False) else None
+                    norm = self.final_norm
                 takes = getattr(follower, "takes_scaled_rows", None)
                 if callable(takes) and getattr(self.layers[e.layer], "ends_in_next_norm", False) and takes(x.shape[0]):
-                    pending = self.layers[e.layer].forward(x, pending, step, caches[i], next_norm=follower.norm1)
+                    pending = self.layers[e.layer].forward(x, pending, step, caches[i], next_norm=norm)
                 else:
                     pending = self.layers[e.layer].forward(x, pending, step, caches[i])
             if step.n_logits == 0:
                 return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=x.device)
-            xs = ops.gather_rows(x, step.logit_rows)
-            ps = ops.gather_rows(pending, step.logit_rows) if pending is not None else None
+            if isinstance(pending, ScaledRows):          # the last block ended in the final norm
+                return self.head.forward(pending)
+            if step.logits_all:
+                xs, ps = x, pending
+            else:
+                xs = ops.gather_rows(x, step.logit_rows)
+                ps = ops.gather_rows(pending, step.logit_rows) if pending is not None else None
             y = self.final_norm.forward(xs, ps)
             return self.head.forward(y)

@@ -39,10 +39,15 @@ def argmax(logits: torch.Tensor) -> torch.Tensor:
     _gpu(logits)
     if logits.dim() != 2 or logits.dtype != torch.float32 or logits.stride(1) != 1:
         raise KernelError("argmax: logits must be float32 [rows, vocab] with contiguous rows")
-    out = torch.empty(logits.shape[0], dtype=torch.int32, device=logits.device)
+    rows, vocab = logits.shape
+    out = torch.empty(rows, dtype=torch.int32, device=logits.device)
+    # a long row is read by several workgroups, whose winners a second kernel compares
+    parts = max(1, min(16, vocab // 8192))
+    part_val = torch.empty(rows * parts, dtype=torch.float32, device=logits.device) if parts > 1 else None
+    part_idx = torch.empty(rows * parts, dtype=torch.int32, device=logits.device) if parts > 1 else None
     lib = build.load("sampling")
-    _check(lib.lcu_argmax(_ptr(logits), logits.stride(0), logits.shape[0], logits.shape[1], _ptr(out), _stream()),
-           "argmax")
+    _check(lib.lcu_argmax(_ptr(logits), logits.stride(0), rows, vocab, _ptr(out), parts, _ptr(part_val), _ptr(part_idx),
+                          _stream()), "argmax")
     return out
 
 
