@@ -253,7 +253,7 @@ __device__ __forceinline__ void attn_compute_lds(const u32x4 *__restrict__ buf, 
     for (int t = 0; t < 2; ++t) {
         const u32x2 *vb = (const u32x2 *)(buf + 4 * DH + t * 2 * DH);
 #pragma unroll
-        for (int dt = 0; dt < DH / 16; ++dt) v[dt][t] = vb[(16 * dt + l16) * 4 + grp];
+        for (int dt = 0; dt < DH / 16; ++dt) v[dt][t] = vb[(32 * dt + 16 * (grp >> 1) + l16) * 2 + (grp & 1)];
     }
     u32x4 pb[QB];
     attn_softmax<DH, QB, MASK>(s, k0, st, p_row, lo_row, scale_log2, grp, pb);
@@ -509,11 +509,14 @@ constexpr int PRE_WAVES = PRE_QWAVES * PRE_HALVES;
 constexpr int PRE_QB = LCU_PRE_QB;
 constexpr int PRE_RING = 3;               // buffers of 64 keys in LDS: one is read, two are on their way
 
-// The keys and values of two steps of 32, copied into LDS as they lie in their pages: per step
-// and tile of 16 keys first the keys [dim/8][token][8], then (after both key tiles) the values
-// [dim][token].  In units of 16 bytes a step holds 8*DH chunks: [K tile 0 | K tile 1 | V tile 0
-// | V tile 1], 2*DH chunks each; a buffer holds two steps.  A thread of the workgroup copies
-// chunks tid, tid + 512, ...
+// The keys and values of two steps of 32, copied into LDS in chunks of 16 bytes: per step and
+// tile of 16 keys first the keys as they lie in their page, [dim/8][token][8], then (after both
+// key tiles) the values, whose page holds [dim][token]: a chunk is 8 tokens of one dim, and of
+// every 16 dims first come the 16 chunks of tokens 0..7, then those of tokens 8..15 (the lanes that
+// read one half of 16 dims then read neighbouring bytes; with the page's own order four of them
+// fell into one bank, and the bank conflicts took a quarter of the kernel's time).  A step holds
+// 8*DH chunks: [K tile 0 | K tile 1 | V tile 0 | V tile 1], 2*DH chunks each; a buffer holds two
+// steps.  A thread of the workgroup copies chunks tid, tid + 512, ...
 //
 // The copy goes from memory straight into LDS (global_load_lds_dwordx4: no registers hold the
 // data on its way, lane l of a wave writes the 16 bytes l of the wave's 1 KB), so the loads of
@@ -539,7 +542,9 @@ __device__ __forceinline__ void stage_issue(u32x4 *__restrict__ buf, const bf16_
     asm volatile("" : "+v"(tid));                  // made anew in every step, not kept in registers across the loop
     const int lane = tid & (WAVE - 1);
     const uint32_t k_lane = ((uint32_t)(lane >> 4) * page + (lane & 15)) * 8 * E;       // keys [dim/8][token][8]
-    const uint32_t v_lane = ((uint32_t)(lane >> 1) * page + (lane & 1) * 8) * E;        // values [dim][token]
+    // values [dim][token]: of 16 dims first the chunks with tokens 0..7, then those with tokens 8..15
+    // (so that the 32 lanes that read one half of 16 dims read 256 bytes in a row: no two in one bank)
+    const uint32_t v_lane = ((uint32_t)(16 * (lane >> 5) + (lane & 15)) * page + ((lane >> 4) & 1) * 8) * E;
 #pragma unroll
     for (int i = 0; i < DH / 32; ++i) {
         const int cw = wave_id * WAVE + 512 * i;                  // the wave's first chunk
