@@ -153,7 +153,9 @@ constexpr float RESCALE_SLACK = 6.0f;
 
 // The softmax of the step, online: new maxima and sums, the output rescaled, the weights as
 // bfloat16 operands.
-template <int DH, int QB, bool MASK>
+// PERM: the lane's eight scores are the keys k0 + 8 grp .. + 7 in a row (the prefill kernel reads
+// its key tiles from LDS in that order); else four keys of each tile, k0 + 16 t + 4 grp .. + 3.
+template <int DH, int QB, bool MASK, bool PERM = false>
 __device__ __forceinline__ void attn_softmax(const f32x4 (&s)[QB][2], int k0, AttnState<DH, QB> &st, const int (&p_row)[QB],
                                              const int (&lo_row)[QB], float scale_log2, int grp, u32x4 (&pb)[QB]) {
 #pragma unroll
@@ -164,7 +166,7 @@ __device__ __forceinline__ void attn_softmax(const f32x4 (&s)[QB][2], int k0, At
         if (MASK) {
 #pragma unroll
             for (int r = 0; r < 8; ++r) {
-                const int j = k0 + 16 * (r / 4) + 4 * grp + (r % 4);
+                const int j = PERM ? k0 + 8 * grp + r : k0 + 16 * (r / 4) + 4 * grp + (r % 4);
                 if (j > p_row[b] || j < lo_row[b]) v[r] = -INFINITY;
             }
         }
@@ -220,6 +222,29 @@ __device__ __forceinline__ void attn_mix(const u32x2 (&v)[DH / 16][2], const u32
     }
 }
 
+// The same with the lane's values being the keys k0 + 8 grp .. + 7 of dim 16 dt + lane % 16, as one
+// 16-byte chunk of the page holds them.
+template <int DH, int QB, bool MASK>
+__device__ __forceinline__ void attn_mix_perm(const u32x4 (&v)[DH / 16], const u32x4 (&pb)[QB], int k0, int p_max, int lo_min,
+                                              int grp, AttnState<DH, QB> &st) {
+    uint32_t keep[4] = {0xffffffffu, 0xffffffffu, 0xffffffffu, 0xffffffffu};
+    if (MASK) {
+        // values of keys that no row sees are taken as zero: their memory may hold anything
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const int j = k0 + 8 * grp + e;
+            if (j > p_max || j < lo_min) keep[e / 2] &= (e & 1) ? 0x0000ffffu : 0xffff0000u;   // clears element e of its dword
+        }
+    }
+#pragma unroll
+    for (int dt = 0; dt < DH / 16; ++dt) {
+        u32x4 a = v[dt];
+        if (MASK) { a.x &= keep[0]; a.y &= keep[1]; a.z &= keep[2]; a.w &= keep[3]; }
+#pragma unroll
+        for (int b = 0; b < QB; ++b) st.o[b][dt] = mfma16(a, pb[b], st.o[b][dt]);
+    }
+}
+
 template <int DH, int QB, bool MASK>
 __device__ __forceinline__ void attn_compute(const KVFrag<DH> &f, int k0, const u32x4 (&q)[QB][DH / 32],
                                              AttnState<DH, QB> &st, const int (&p_row)[QB], const int (&lo_row)[QB],
@@ -238,26 +263,29 @@ template <int DH, int QB, bool MASK>
 __device__ __forceinline__ void attn_compute_lds(const u32x4 *__restrict__ buf, int k0, const u32x4 (&q)[QB][DH / 32],
                                                  AttnState<DH, QB> &st, const int (&p_row)[QB], const int (&lo_row)[QB],
                                                  int p_max, int lo_min, float scale_log2, int l16, int grp) {
+    // Row i of the matrix instruction's key tile t is key 8 (i / 4) + 4 t + i % 4 of the step, so that a
+    // lane's eight scores (rows 4 grp .. + 3 of both tiles) are eight keys in a row, and with them its
+    // values one chunk of 16 bytes: one read, the operand as it arrives.  In LDS key tile i / 8 holds
+    // that key at place i % 8 + 8 t of its row (stage_issue orders the tokens so): the lanes of a read
+    // take neighbouring bytes.
     f32x4 s[QB][2];
     {
         u32x4 k[2][DH / 32];
+        const u32x4 *kb0 = buf + (l16 >> 3) * 2 * DH + grp * 16 + (l16 & 7);
 #pragma unroll
         for (int t = 0; t < 2; ++t)
 #pragma unroll
-            for (int kb = 0; kb < DH / 32; ++kb) k[t][kb] = buf[t * 2 * DH + (4 * kb + grp) * 16 + l16];
+            for (int kb = 0; kb < DH / 32; ++kb) k[t][kb] = kb0[4 * kb * 16 + 8 * t];
         attn_scores<DH, QB>(k, q, s);
     }
     __builtin_amdgcn_sched_barrier(0);             // the values' reads stay below the scores
-    u32x2 v[DH / 16][2];
+    u32x4 v[DH / 16];
+    const u32x4 *vb = buf + 4 * DH + (grp >> 1) * 2 * DH + (grp & 1) * 16 + l16;
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
-        const u32x2 *vb = (const u32x2 *)(buf + 4 * DH + t * 2 * DH);
-#pragma unroll
-        for (int dt = 0; dt < DH / 16; ++dt) v[dt][t] = vb[(32 * dt + 16 * (grp >> 1) + l16) * 2 + (grp & 1)];
-    }
+    for (int dt = 0; dt < DH / 16; ++dt) v[dt] = vb[32 * dt];
     u32x4 pb[QB];
-    attn_softmax<DH, QB, MASK>(s, k0, st, p_row, lo_row, scale_log2, grp, pb);
-    attn_mix<DH, QB, MASK>(v, pb, k0, p_max, lo_min, grp, st);
+    attn_softmax<DH, QB, MASK, true>(s, k0, st, p_row, lo_row, scale_log2, grp, pb);
+    attn_mix_perm<DH, QB, MASK>(v, pb, k0, p_max, lo_min, grp, st);
 }
 
 // Masks only where a row needs them (the choice is the same for the whole wave).
@@ -541,7 +569,10 @@ __device__ __forceinline__ void stage_issue(u32x4 *__restrict__ buf, const bf16_
     int tid = threadIdx.x;
     asm volatile("" : "+v"(tid));                  // made anew in every step, not kept in registers across the loop
     const int lane = tid & (WAVE - 1);
-    const uint32_t k_lane = ((uint32_t)(lane >> 4) * page + (lane & 15)) * 8 * E;       // keys [dim/8][token][8]
+    // keys [dim/8][token][8]; place p of a row of 16 takes token p with bits 2 and 3 swapped (0-3, 8-11,
+    // 4-7, 12-15: the order in which attn_compute_lds reads them)
+    const uint32_t k_tok = (lane & 3) | ((lane & 4) << 1) | ((lane & 8) >> 1);
+    const uint32_t k_lane = ((uint32_t)(lane >> 4) * page + k_tok) * 8 * E;
     // values [dim][token]: of 16 dims first the chunks with tokens 0..7, then those with tokens 8..15
     // (so that the 32 lanes that read one half of 16 dims read 256 bytes in a row: no two in one bank)
     const uint32_t v_lane = ((uint32_t)(16 * (lane >> 5) + (lane & 15)) * page + ((lane >> 4) & 1) * 8) * E;
