@@ -151,6 +151,17 @@ __device__ __forceinline__ void attn_scores(const u32x4 (&k)[2][DH / 32], const 
 
 constexpr float RESCALE_SLACK = 6.0f;
 
+// The largest of the values that the lanes l, l + 16, l + 32 and l + 48 hold, in all four of them.
+// The rows of 16 lanes are swapped in the vector unit (v_permlane16_swap, v_permlane32_swap): a
+// shuffle through LDS takes an order of magnitude longer, and the softmax waits for this value.
+__device__ __forceinline__ float max_over_groups(float x) {
+    const unsigned u = __float_as_uint(x);
+    const auto a = __builtin_amdgcn_permlane16_swap(u, u, false, false);     // (rows 0 0 2 2, rows 1 1 3 3)
+    const unsigned v = __float_as_uint(fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1])));
+    const auto b = __builtin_amdgcn_permlane32_swap(v, v, false, false);     // (lower half twice, upper half twice)
+    return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+
 // The softmax of the step, online: new maxima and sums, the output rescaled, the weights as
 // bfloat16 operands.
 // PERM: the lane's eight scores are the keys k0 + 8 grp .. + 7 in a row (the prefill kernel reads
@@ -173,8 +184,7 @@ __device__ __forceinline__ void attn_softmax(const f32x4 (&s)[QB][2], int k0, At
         float mx = v[0];
 #pragma unroll
         for (int r = 1; r < 8; ++r) mx = fmaxf(mx, v[r]);
-        mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
-        mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
+        mx = max_over_groups(mx);
         // The reference point of the exponentials need not be the exact maximum: it moves only
         // when the maximum has grown by more than 2^RESCALE_SLACK, so the weights stay below
         // that and the output is rarely rescaled (the result is the same up to rounding).
