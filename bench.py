@@ -47,11 +47,13 @@ def kv_bytes_per_token(c, elem):
     return c.num_hidden_layers * 2 * c.num_key_value_heads * c.head_dim * elem
 
 
-def prefill_flops(c, t):
+def prefill_flops(c, t, history=0):
+    """Of a step that feeds ``t`` tokens of a prompt after ``history`` tokens that the cache holds."""
     d, dh, nh, nkv, di = c.hidden_size, c.head_dim, c.num_attention_heads, c.num_key_value_heads, c.intermediate_size
     per_token = 2 * ((nh + 2 * nkv) * dh * d + d * nh * dh + 2 * di * d + d * di)
     matmul = c.num_hidden_layers * per_token * t + 2 * c.vocab_size * d      # the output matrix for the last row only
-    attention = c.num_hidden_layers * 2 * 2 * nh * dh * t * (t + 1) / 2      # causal: QK^T and PV over t(t+1)/2 pairs
+    pairs = t * history + t * (t + 1) / 2                                    # causal: every key before, half of the step's own
+    attention = c.num_hidden_layers * 2 * 2 * nh * dh * pairs                # QK^T and PV
     return matmul + attention
 
 
@@ -88,12 +90,15 @@ def run_decode(engine, cfg, batch, steps, warmup, rng, sync, prompt_len=PROMPT_L
     return dt, produced, (ctx0 + ctx1) / 2.0
 
 
-def run_prefill(engine, cfg, rng, sync, repeats=3):
-    """Best time of one step that feeds a whole prompt of PREFILL_TOKENS tokens."""
+def run_prefill(engine, cfg, rng, sync, repeats=3, history=0):
+    """Best time of one step that feeds PREFILL_TOKENS tokens of a prompt: a whole prompt, or,
+    with ``history``, the portion after that many tokens (fed before, untimed)."""
     best = None
     for k in range(repeats + 1):
         toks = [rng.randrange(cfg.vocab_size) for _ in range(PREFILL_TOKENS)]
         rid = 10_000 + k
+        for at in range(0, history, PREFILL_TOKENS):
+            engine.runner.step([rid], [[rng.randrange(cfg.vocab_size) for _ in range(min(PREFILL_TOKENS, history - at))]], want=[[]])
         sync()
         t0 = time.perf_counter()
         engine.runner.step([rid], [toks])
@@ -149,6 +154,8 @@ def main() -> int:
     ap.add_argument("--dtype", choices=["bfloat16", "float32"], default="bfloat16")
     ap.add_argument("--no-points", action="store_true", help="skip decoding at batch 1 and 64 and the prefill")
     ap.add_argument("--only-prefill", action="store_true", help="time the 2048-token prefill alone (for profiles)")
+    ap.add_argument("--prefill-history", type=int, default=0,
+                    help="with --only-prefill: time the 2048 tokens that follow this many tokens of the same prompt")
     ap.add_argument("--kernel-summary", metavar="DB", help="print the per-step kernel table of a rocprofv3 database and exit")
     ap.add_argument("--summary-steps", type=int, default=8)
     args = ap.parse_args()
@@ -168,7 +175,7 @@ def main() -> int:
     if args.layers:
         shape["num_hidden_layers"] = args.layers
     grow = args.steps + args.warmup + 2 * max(args.batch, 64) * rounds_of(args.prompt_len) + 64
-    need_ctx = args.prompt_len + grow + 64
+    need_ctx = max(args.prompt_len + grow + 64, args.prefill_history + PREFILL_TOKENS)
     while shape["max_position_embeddings"] < need_ctx:
         shape["max_position_embeddings"] *= 2
     cfg = LlamaConfig.from_dict(shape)
@@ -181,13 +188,14 @@ def main() -> int:
     # a request decodes while later ones still prefill: room for that too
     per_req = max(args.prompt_len, PROMPT_LEN) + grow
     engine = Engine.from_config(cfg, seed=0, dtype=args.dtype, page_size=page,
-                                max_tokens=biggest * ((per_req + page - 1) // page * page) + PREFILL_TOKENS + page,
+                                max_tokens=biggest * ((per_req + page - 1) // page * page) + args.prefill_history + PREFILL_TOKENS + page,
                                 max_seqs=biggest + 2, max_batch_tokens=max(PREFILL_TOKENS, biggest), prefill_chunk=PREFILL_TOKENS)
 
     if args.only_prefill:
-        pt = run_prefill(engine, cfg, rng, sync, repeats=args.steps)
+        pt = run_prefill(engine, cfg, rng, sync, repeats=args.steps, history=args.prefill_history)
+        flops = prefill_flops(cfg, PREFILL_TOKENS, args.prefill_history)
         print(json.dumps({"prefill": {"value": round(PREFILL_TOKENS / pt, 1), "tokens": PREFILL_TOKENS, "ms": round(pt * 1e3, 3),
-                                      "frac": round(prefill_flops(cfg, PREFILL_TOKENS) / pt / MATRIX_PEAK[dt_name], 4)}}))
+                                      "frac": round(flops / pt / MATRIX_PEAK[dt_name], 4), "history": args.prefill_history}}))
         return 0
     seconds, produced, mean_ctx = run_decode(engine, cfg, args.batch, args.steps, args.warmup, rng, sync, args.prompt_len)
     ms_per_step = seconds / args.steps * 1e3
