@@ -9,9 +9,12 @@
 //                                          8-byte loads in the cache's value layout),
 //                                          B = P^T: exactly the lane's own S^T values
 // In S^T a lane owns one query row (lane % 16) and 8 of each 32 keys, so the softmax's
-// maximum and sum run over a lane's registers and two cross-lane steps.  Scores, the
-// running maximum and sum and the output are 32-bit; P is rounded to bfloat16 for the
-// second product.
+// maximum and sum run over a lane's registers and two cross-lane steps.  Which 8 keys is the
+// kernel's choice, by the order in which it feeds the keys' rows to the first product: the decode
+// kernel, which loads from the pages, takes 4 keys of each tile of 16 (keys of a tile are
+// neighbours in memory); the prefill kernel, which reads from its copy in LDS, takes 8 keys in a
+// row (its values are then one 16-byte read).  Scores, the running maximum and sum and the
+// output are 32-bit; P is rounded to bfloat16 for the second product.
 //
 // A "row" is one (token, head) pair; 16 rows that share a request and a key/value head
 // form a block: the heads of a group for one token, for several tokens if the group is
@@ -21,7 +24,7 @@
 //                   key/value head and one of `n_splits` equal parts of its keys; the
 //                   waves take 32-key steps in turn and merge through LDS; parts are
 //                   merged by a second kernel.
-//   prefill kernel  any number of tokens per request (also one).  A workgroup of 4 waves
+//   prefill kernel  any number of tokens per request (also one).  A workgroup of 8 waves
 //                   takes consecutive tokens of one request; the keys and values of a step
 //                   are copied to LDS once and shared by the waves.
 #include "common.h"
