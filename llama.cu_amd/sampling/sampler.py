@@ -67,8 +67,13 @@ def sample_rows(logits: torch.Tensor, temperature: Sequence[float], top_p: Seque
     kk = torch.tensor([min(int(k), vocab) for k in top_k], dtype=torch.int32).to(dev)
     out = torch.empty(rows, dtype=torch.int32, device=dev)
     lib = build.load("sampling")
+    # a long row is cut into parts, one workgroup each: about one workgroup per compute unit in all
+    parts = max(1, min(16, 256 // rows, vocab // 4096))
+    lib.lcu_sample_scratch_bytes.restype = ctypes.c_size_t
+    scratch = torch.zeros(int(lib.lcu_sample_scratch_bytes(rows, parts)), dtype=torch.uint8, device=dev)
+    any_top_k = any(int(k) < vocab for k in top_k)
     _check(lib.lcu_sample(_ptr(logits), logits.stride(0), rows, vocab, _ptr(fl[0]), _ptr(fl[1]), _ptr(kk), _ptr(fl[2]),
-                          _ptr(out), _stream()), "sample")
+                          _ptr(out), int(any_top_k), parts, _ptr(scratch), _stream()), "sample")
     return out
 
 
@@ -76,8 +81,11 @@ class Sampler:
     def sample_device(self, logits: torch.Tensor, params: Sequence[SamplingParams],
                       keys: Sequence[Tuple[int, int]]) -> torch.Tensor:
         """A token for every row, left on the device (int32)."""
-        out = argmax(logits)
         random_rows = [i for i, p in enumerate(params) if not p.is_argmax]
+        if random_rows and len(random_rows) == logits.shape[0]:
+            return sample_rows(logits, [p.temperature for p in params], [p.top_p for p in params], [p.top_k for p in params],
+                               [uniform(p.seed, k[0], k[1]) for p, k in zip(params, keys)])
+        out = argmax(logits)
         if random_rows:
             idx = torch.tensor(random_rows, dtype=torch.long).to(logits.device)
             sub = logits if len(random_rows) == logits.shape[0] else logits[idx]
