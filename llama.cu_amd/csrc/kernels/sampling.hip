@@ -17,8 +17,9 @@ constexpr double FIXED_ONE = 35184372088832.0;   // 2^45: the sum of 2^19 weight
 constexpr int MAX_VOCAB = 1 << 19;
 
 __device__ __forceinline__ uint32_t order_key(float x) {
-    // ascending float order -> ascending unsigned order
-    const uint32_t u = __float_as_uint(x);
+    // ascending float order -> ascending unsigned order; -0 counts as +0 (equal values are ordered
+    // by index, as a stable sort by value orders them)
+    const uint32_t u = x == 0.0f ? 0u : __float_as_uint(x);
     return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
 }
 __device__ __forceinline__ float key_value(uint32_t k) {

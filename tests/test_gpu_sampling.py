@@ -43,6 +43,25 @@ def test_sample_kernel_matches_plain_sampler(vocab, temperature, top_p, top_k):
             _assert_draw_within_rounding(l[r], temperature, top_p, top_k, u[r], got[r])
 
 
+@pytest.mark.parametrize("rows", [3, 40])
+def test_equal_logits_across_the_parts_of_a_long_row(rows):
+    """A long row is cut into parts, one workgroup each.  With few distinct values thousands of
+    logits are equal, spread over all parts: the draw is the m-th of them in index order, as a
+    stable sort has them; with and without a cut at top_k that falls among equals."""
+    from llama_cu_amd.sampling import sample_rows
+    vocab = 70001
+    g = torch.Generator().manual_seed(rows)
+    l = (torch.randn(rows, vocab, generator=g) * 2.0).round() * 0.5        # steps of a half: a few dozen values
+    rng = np.random.default_rng(rows)
+    u = [0.0, 0.999999] + [float(x) for x in rng.random(rows - 2)]
+    for top_p, top_k in ((1.0, 10 ** 9), (0.9, 5000), (1.0, 37)):
+        got = sample_rows(l.cuda(), [0.7] * rows, [top_p] * rows, [top_k] * rows, u).tolist()
+        for r in range(rows):
+            want = plain.sample(l[r], 0.7, top_p, top_k, u[r])
+            if got[r] != want:
+                _assert_draw_within_rounding(l[r], 0.7, top_p, top_k, u[r], got[r])
+
+
 def _assert_draw_within_rounding(logits, temperature, top_p, top_k, u, token, tol=2e-6):
     """``token`` is the right answer for a number within ``tol`` of ``u``: in the sorted
     order of llama.cu/src/op/random_sample/sample.cuh:186-207 its span of the cumulative
