@@ -117,6 +117,25 @@ def chat(args) -> int:
             rid = None
 
 
+def random_model(args) -> int:
+    """Write a model folder with random weights from a configuration and a seed (the reference
+    has no such mode; without files to download this is how a model of a given shape is had)."""
+    import json
+
+    import torch
+
+    from . import models  # noqa: F401  (registers the architectures)
+    from .config import architecture_of
+    from .weights import write_random_model
+    with open(args.config) as f:
+        data = json.load(f)
+    config = architecture_of(data, args.config).config_from_dict(data)
+    dtype = {"bfloat16": torch.bfloat16, "float32": torch.float32}[args.dtype]
+    folder = write_random_model(args.folder, config, args.seed, dtype=dtype, std=args.std)
+    print(f"[info] wrote {folder}/config.json and model.safetensors (seed {args.seed}, {args.dtype})", file=sys.stderr)
+    return 0
+
+
 def main(argv: Optional[List[str]] = None) -> int:
     ap = argparse.ArgumentParser(prog="llama.cu_amd")
     sub = ap.add_subparsers(dest="command", required=True)
@@ -128,5 +147,12 @@ def main(argv: Optional[List[str]] = None) -> int:
     c = sub.add_parser("chat", help="chat in console")
     _base(c)
     c.set_defaults(func=chat)
+    r = sub.add_parser("random-model", help="write a model folder with random weights")
+    r.add_argument("config", metavar="CONFIG", help="a config.json of a registered architecture")
+    r.add_argument("folder", metavar="FOLDER", help="where config.json and model.safetensors are written")
+    r.add_argument("--seed", type=int, default=0)
+    r.add_argument("--dtype", choices=["bfloat16", "float32"], default="bfloat16", help="type of the stored matrices")
+    r.add_argument("--std", type=float, default=0.02, help="standard deviation of the matrices' entries")
+    r.set_defaults(func=random_model)
     args = ap.parse_args(argv)
     return args.func(args)

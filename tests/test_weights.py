@@ -154,3 +154,21 @@ def test_random_weights_of_an_untied_model_hold_an_output_matrix(tmp_path):
     t = load_weights(open_safetensors(d), expected(common.TINY_A), torch.float32, torch.device("cpu"))
     assert t["lm_head.weight"].shape == (256, 64)
     assert not torch.equal(t["lm_head.weight"], t["model.embed_tokens.weight"])
+
+
+def test_random_model_command_writes_a_folder_that_loads(tmp_path):
+    """``llama.cu_amd random-model CONFIG FOLDER --seed N``: the folder holds config.json and every
+    tensor that the model expects, and the same seed gives the same bytes."""
+    import json
+    import llama_cu_amd.cli as cli
+    cfg_path = tmp_path / "cfg.json"
+    cfg_path.write_text(json.dumps(common.TINY_A))
+    assert cli.main(["random-model", str(cfg_path), str(tmp_path / "m1"), "--seed", "4", "--dtype", "float32"]) == 0
+    assert cli.main(["random-model", str(cfg_path), str(tmp_path / "m2"), "--seed", "4", "--dtype", "float32"]) == 0
+    a = (tmp_path / "m1" / "model.safetensors").read_bytes()
+    assert a == (tmp_path / "m2" / "model.safetensors").read_bytes()
+    assert json.loads((tmp_path / "m1" / "config.json").read_text())["hidden_size"] == common.TINY_A["hidden_size"]
+    files = open_safetensors(str(tmp_path / "m1"))
+    names = {n for f in files for n in f.names()}
+    assert "model.embed_tokens.weight" in names and "model.layers.1.mlp.down_proj.weight" in names
+
