@@ -30,18 +30,28 @@ __device__ __forceinline__ unsigned long long fixed_weight(float logit, float ma
     return (unsigned long long)((double)w * FIXED_ONE);
 }
 
-// Every element of a row, for the threads of a block together: four neighbouring logits per
-// load where the row allows it and several loads in flight (a row is read by one workgroup,
-// so latency, not bandwidth, is what counts).  f(index, value); no order is promised.
+// A row is cut into `parts` stretches, one workgroup each; their borders are multiples of four
+// logits.
+__device__ __forceinline__ void part_range(int vocab, int part, int parts, int &lo, int &hi) {
+    const int quads = (vocab + 3) / 4;
+    lo = (int)((long long)quads * part / parts) * 4;
+    hi = (int)((long long)quads * (part + 1) / parts) * 4;
+    hi = hi < vocab ? hi : vocab;
+}
+
+// Every element of the stretch [lo, hi) of a row (lo a multiple of 4), for the threads of a block
+// together: four neighbouring logits per load where the row allows it and several loads in flight
+// (a stretch is read by one workgroup, so latency, not bandwidth, is what counts).  f(index,
+// value); no order is promised.
 template <class F>
-__device__ __forceinline__ void scan_row(const float *__restrict__ row, int vocab, F f) {
-    const int vec_end = (((size_t)row % 16) == 0) ? (vocab / 4) * 4 : 0;
+__device__ __forceinline__ void scan_part(const float *__restrict__ row, int lo, int hi, F f) {
+    const int vec_end = (((size_t)row % 16) == 0) ? lo + ((hi - lo) / 4) * 4 : lo;
 #pragma unroll 4
-    for (int i = threadIdx.x * 4; i < vec_end; i += blockDim.x * 4) {
+    for (int i = lo + threadIdx.x * 4; i < vec_end; i += blockDim.x * 4) {
         const float4 v = *(const float4 *)(row + i);
         f(i, v.x); f(i + 1, v.y); f(i + 2, v.z); f(i + 3, v.w);
     }
-    for (int i = vec_end + threadIdx.x; i < vocab; i += blockDim.x) f(i, row[i]);
+    for (int i = vec_end + threadIdx.x; i < hi; i += blockDim.x) f(i, row[i]);
 }
 
 // ---------------------------------------------------------------- arg-max
@@ -54,28 +64,13 @@ argmax_kernel(const float *__restrict__ logits, int ld, int vocab, int *__restri
               int *__restrict__ part_idx) {
     const float *row = logits + (size_t)blockIdx.x * ld;
     const int parts = gridDim.y, part = blockIdx.y;
-    // the part's share of the row, in units of four logits
-    const int quads = (vocab + 3) / 4;
-    const int lo = (int)((long long)quads * part / parts) * 4;
-    int hi = (int)((long long)quads * (part + 1) / parts) * 4;
-    hi = hi < vocab ? hi : vocab;
+    int lo, hi;
+    part_range(vocab, part, parts, lo, hi);
     float best = -INFINITY;
     int bi = 0x7fffffff;
-    // four neighbouring logits per load where the row allows it (many loads in flight: latency,
-    // not bandwidth, is what counts)
-    const int vec_end = (((size_t)row % 16) == 0) ? lo + ((hi - lo) / 4) * 4 : lo;
-#pragma unroll 4
-    for (int i = lo + threadIdx.x * 4; i < vec_end; i += blockDim.x * 4) {
-        const float4 v = *(const float4 *)(row + i);
-        const float e[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-        for (int k = 0; k < 4; ++k)
-            if (e[k] > best || (e[k] == best && i + k < bi)) { best = e[k]; bi = i + k; }
-    }
-    for (int i = vec_end + threadIdx.x; i < hi; i += blockDim.x) {
-        const float v = row[i];
+    scan_part(row, lo, hi, [&](int i, float v) {
         if (v > best || (v == best && i < bi)) { best = v; bi = i; }
-    }
+    });
     __shared__ float sv[SAMPLE_THREADS / WAVE];
     __shared__ int si[SAMPLE_THREADS / WAVE];
 #pragma unroll
@@ -251,25 +246,6 @@ struct RowState {
     SelectState st;                    // the select that is under way, or its result
 };
 
-__device__ __forceinline__ void part_range(int vocab, int part, int parts, int &lo, int &hi) {
-    const int quads = (vocab + 3) / 4;                 // the parts' borders are multiples of four logits
-    lo = (int)((long long)quads * part / parts) * 4;
-    hi = (int)((long long)quads * (part + 1) / parts) * 4;
-    hi = hi < vocab ? hi : vocab;
-}
-
-// Every element of the stretch [lo, hi) of a row (lo a multiple of 4), as scan_row does for a row.
-template <class F>
-__device__ __forceinline__ void scan_part(const float *__restrict__ row, int lo, int hi, F f) {
-    const int vec_end = (((size_t)row % 16) == 0) ? lo + ((hi - lo) / 4) * 4 : lo;
-#pragma unroll 4
-    for (int i = lo + threadIdx.x * 4; i < vec_end; i += blockDim.x * 4) {
-        const float4 v = *(const float4 *)(row + i);
-        f(i, v.x); f(i + 1, v.y); f(i + 2, v.z); f(i + 3, v.w);
-    }
-    for (int i = vec_end + threadIdx.x; i < hi; i += blockDim.x) f(i, row[i]);
-}
-
 __device__ __forceinline__ bool row_cuts_at_k(int k, int vocab) { return k >= 1 && k < vocab; }
 
 __global__ void __launch_bounds__(SAMPLE_THREADS)
@@ -402,7 +378,7 @@ sample_pick_kernel(const float *__restrict__ logits, int ld, int vocab, const fl
                    const RowState *__restrict__ state, const int *__restrict__ part_count,
                    const int *__restrict__ part_first, int parts, int *__restrict__ out) {
     __shared__ int seg_count[SAMPLE_THREADS];
-    __shared__ int result, seg_total;
+    __shared__ int result;
     const int r = blockIdx.x;
     const float *row = logits + (size_t)r * ld;
     const RowState &rs = state[r];
@@ -443,7 +419,6 @@ sample_pick_kernel(const float *__restrict__ logits, int ld, int vocab, const fl
         // exclusive prefix counts, serial: 1024 additions
         int run = 0;
         for (int t = 0; t < (int)blockDim.x; ++t) { const int c = seg_count[t]; seg_count[t] = run; run += c; }
-        seg_total = run;
     }
     __syncthreads();
     const unsigned long long before = before_part + (unsigned long long)seg_count[threadIdx.x];
