@@ -431,12 +431,16 @@ def paged_attention(q: torch.Tensor, out: torch.Tensor, cache: torch.Tensor, ste
 SKINNY_MAX_ROWS = 64      # what the kernel takes
 SKINNY_ROWS = 16          # up to here it beats the library's product (measured on the Llama-3-8B shapes) ...
 SKINNY_ROWS_PACKED = 24   # ... and up to here when it reads a packed weight and its epilogues save the kernels around it
-                          # (whole decode steps of the Llama-3-8B shape: +9 % at 17 rows, +4 % at 24, -2 % at 32)
+                          # (whole decode steps of the Llama-3-8B shape: +9 % at 17 rows, +4 % at 24)
+SKINNY_ROWS_SHORT_K = 32  # ... and up to here for packed weights with K <= 8192 (q/k/v, output, gate/up: +4.5 % at 28
+                          # rows, +2 % at 32; with the down projection as well the step at 32 rows was 2 % slower)
 
 
 def skinny_max_rows(packed: bool) -> int:
     """The most rows for which the weight-streaming kernel is ever chosen over the library."""
-    return SKINNY_ROWS_PACKED if packed else SKINNY_ROWS
+    return SKINNY_ROWS_SHORT_K if packed else SKINNY_ROWS
+
+
 _EPILOGUES = {"bf16": 0, "f32": 1, "add_f32": 2, "swiglu": 3}
 
 
@@ -476,11 +480,13 @@ def skinny_preferred(m: int, n: int, k: int, out_dtype: torch.dtype, packed: boo
     """Whether the weight-streaming kernel is the faster choice for a plain bfloat16 product
     of ``m`` rows with an ``[n, k]`` weight (measured against the library on the Llama-3-8B
     shapes): always for very few rows and for float32 output; with a packed weight up to 24
-    rows (there it is within a tenth of the library on the large weights, and its epilogues save
+    rows, and up to 32 where K is at most 8192 (there it is within a tenth of the library on the large weights, and its epilogues save
     the kernels around the product); without one, beyond 4 and up to 16 rows, only for small
     weights (the library's split over K wins on the large ones)."""
     if m > skinny_max_rows(packed):
         return False
+    if packed and m > SKINNY_ROWS_PACKED:
+        return k <= 8192                  # up to 32 rows, but not the products with a long K (the down projection)
     return m <= (SKINNY_ROWS_PACKED if packed else 4) or out_dtype == torch.float32 or n * k <= (1 << 24)
 
 
