@@ -17,6 +17,19 @@ __global__ void embedding_gather_kernel(TO *__restrict__ out, const TT *__restri
         return;
     }
     const TT *t = table + (size_t)id * d;
+    if (d % 8 == 0 && ((size_t)t % (8 * sizeof(TT))) == 0 && ((size_t)o % (8 * sizeof(TO))) == 0) {
+        // eight neighbouring elements per load (a row is read once, from memory: few, wide loads)
+        struct alignas(8 * sizeof(TT)) In8 { TT v[8]; };
+        struct alignas(8 * sizeof(TO)) Out8 { TO v[8]; };
+        for (int c = threadIdx.x * 8; c < d; c += blockDim.x * 8) {
+            const In8 in = *(const In8 *)(t + c);
+            Out8 res;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) res.v[e] = from_f32<TO>(to_f32(in.v[e]));
+            *(Out8 *)(o + c) = res;
+        }
+        return;
+    }
     for (int c = threadIdx.x; c < d; c += blockDim.x) o[c] = from_f32<TO>(to_f32(t[c]));
 }
 
