@@ -77,12 +77,14 @@ LCU_API int lcu_gather_rows(void *out, const void *x, int type, const int *rows,
 
 // ---------------------------------------------------------------- RMS norm (+ residual sum)
 // One block per row.  If `delta` is given: x += delta first (in 32-bit, written back
-// when x is 32-bit: x is then the residual stream).  Then
+// when x is 32-bit: x is then the residual stream); delta may be `planes` planes [n, d],
+// `plane_stride` elements apart (a product's partial sums over slices of K), which are added
+// one after the other in the order of the planes.  Then
 //   y = x * rsqrt(sum(x^2)/d + eps) * w        (32-bit, one rounding at the store)
 // The order of the sum depends on d and the block size only, not on the batch.
 template <class TX, class TD, class TW, class TO>
 __global__ void rmsnorm_kernel(TX *__restrict__ x, const TD *__restrict__ delta, const TW *__restrict__ w,
-                               TO *__restrict__ out, int d, float eps, int write_back) {
+                               TO *__restrict__ out, int d, float eps, int write_back, int planes, size_t plane_stride) {
     __shared__ float scratch[16];
     TX *xr = x + (size_t)blockIdx.x * d;
     const TD *dr = delta ? delta + (size_t)blockIdx.x * d : nullptr;
@@ -90,7 +92,7 @@ __global__ void rmsnorm_kernel(TX *__restrict__ x, const TD *__restrict__ delta,
     for (int c = threadIdx.x; c < d; c += blockDim.x) {
         float v = to_f32(xr[c]);
         if (dr) {
-            v += to_f32(dr[c]);
+            for (int p = 0; p < planes; ++p) v += to_f32(dr[p * plane_stride + c]);
             if (write_back) xr[c] = from_f32<TX>(v);
         }
         acc += v * v;
@@ -100,7 +102,8 @@ __global__ void rmsnorm_kernel(TX *__restrict__ x, const TD *__restrict__ delta,
     TO *o = out + (size_t)blockIdx.x * d;
     for (int c = threadIdx.x; c < d; c += blockDim.x) {
         float v = to_f32(xr[c]);
-        if (dr && !write_back) v += to_f32(dr[c]);
+        if (dr && !write_back)
+            for (int p = 0; p < planes; ++p) v += to_f32(dr[p * plane_stride + c]);
         o[c] = from_f32<TO>(rms * v * to_f32(w[c]));
     }
 }
@@ -115,7 +118,7 @@ template <class T> struct alignas(4 * sizeof(T)) Vec4 { T v[4]; };
 template <class TX, class TD, class TW, class TO>
 __global__ void __launch_bounds__(NORM_THREADS)
 rmsnorm_fast_kernel(TX *__restrict__ x, const TD *__restrict__ delta, const TW *__restrict__ w, TO *__restrict__ out,
-                    int d, float eps, int write_back) {
+                    int d, float eps, int write_back, int planes, size_t plane_stride) {
     __shared__ float scratch[16];
     TX *xr = x + (size_t)blockIdx.x * d;
     const TD *dr = delta ? delta + (size_t)blockIdx.x * d : nullptr;
@@ -129,10 +132,14 @@ rmsnorm_fast_kernel(TX *__restrict__ x, const TD *__restrict__ delta, const TW *
 #pragma unroll
             for (int e = 0; e < 4; ++e) v[i][e] = to_f32(xv.v[e]);
             if (dr) {
-                const Vec4<TD> dv = *(const Vec4<TD> *)(dr + c);
+                for (int p = 0; p < planes; ++p) {
+                    const Vec4<TD> dv = *(const Vec4<TD> *)(dr + p * plane_stride + c);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) v[i][e] += to_f32(dv.v[e]);
+                }
                 Vec4<TX> back;
 #pragma unroll
-                for (int e = 0; e < 4; ++e) { v[i][e] += to_f32(dv.v[e]); back.v[e] = from_f32<TX>(v[i][e]); }
+                for (int e = 0; e < 4; ++e) back.v[e] = from_f32<TX>(v[i][e]);
                 if (write_back) *(Vec4<TX> *)(xr + c) = back;
             }
 #pragma unroll
@@ -157,22 +164,22 @@ rmsnorm_fast_kernel(TX *__restrict__ x, const TD *__restrict__ delta, const TW *
 
 template <class TX, class TD, class TO>
 static int rmsnorm_w(void *x, const void *delta, const void *w, int w_type, void *out, int n, int d, float eps,
-                     int write_back, hipStream_t stream) {
+                     int write_back, hipStream_t stream, int planes = 1, size_t plane_stride = 0) {
     dim3 grid(n), block(d >= 2048 ? 512 : 256);
     if (d % 4 == 0 && d <= NORM_THREADS * NORM_ITEMS * 4) {
         if (w_type == LCU_F32)
-            rmsnorm_fast_kernel<TX, TD, float, TO><<<grid, dim3(NORM_THREADS), 0, stream>>>((TX *)x, (const TD *)delta, (const float *)w, (TO *)out, d, eps, write_back);
+            rmsnorm_fast_kernel<TX, TD, float, TO><<<grid, dim3(NORM_THREADS), 0, stream>>>((TX *)x, (const TD *)delta, (const float *)w, (TO *)out, d, eps, write_back, planes, plane_stride);
         else if (w_type == LCU_BF16)
-            rmsnorm_fast_kernel<TX, TD, bf16_t, TO><<<grid, dim3(NORM_THREADS), 0, stream>>>((TX *)x, (const TD *)delta, (const bf16_t *)w, (TO *)out, d, eps, write_back);
+            rmsnorm_fast_kernel<TX, TD, bf16_t, TO><<<grid, dim3(NORM_THREADS), 0, stream>>>((TX *)x, (const TD *)delta, (const bf16_t *)w, (TO *)out, d, eps, write_back, planes, plane_stride);
         else
             return LCU_BAD_ARGUMENT;
         LCU_LAUNCH_CHECK();
         return LCU_OK;
     }
     if (w_type == LCU_F32)
-        rmsnorm_kernel<TX, TD, float, TO><<<grid, block, 0, stream>>>((TX *)x, (const TD *)delta, (const float *)w, (TO *)out, d, eps, write_back);
+        rmsnorm_kernel<TX, TD, float, TO><<<grid, block, 0, stream>>>((TX *)x, (const TD *)delta, (const float *)w, (TO *)out, d, eps, write_back, planes, plane_stride);
     else if (w_type == LCU_BF16)
-        rmsnorm_kernel<TX, TD, bf16_t, TO><<<grid, block, 0, stream>>>((TX *)x, (const TD *)delta, (const bf16_t *)w, (TO *)out, d, eps, write_back);
+        rmsnorm_kernel<TX, TD, bf16_t, TO><<<grid, block, 0, stream>>>((TX *)x, (const TD *)delta, (const bf16_t *)w, (TO *)out, d, eps, write_back, planes, plane_stride);
     else
         return LCU_BAD_ARGUMENT;
     LCU_LAUNCH_CHECK();
@@ -188,6 +195,18 @@ LCU_API int lcu_rmsnorm(void *x, int x_type, const void *delta, const void *w, i
     if (x_type == LCU_F32 && act_type == LCU_F32) return rmsnorm_w<float, float, float>(x, delta, w, w_type, out, n, d, eps, write_back, stream);
     if (x_type == LCU_F32 && act_type == LCU_BF16) return rmsnorm_w<float, bf16_t, bf16_t>(x, delta, w, w_type, out, n, d, eps, write_back, stream);
     if (x_type == LCU_BF16 && act_type == LCU_BF16) return rmsnorm_w<bf16_t, bf16_t, bf16_t>(x, delta, w, w_type, out, n, d, eps, write_back, stream);
+    return LCU_BAD_ARGUMENT;
+}
+
+// The same with the branch's output as `planes` float32 planes [n, d], one after the other:
+// x (float32) += plane 0 + plane 1 + ... (in this order), then the norm.  d a multiple of 4.
+LCU_API int lcu_rmsnorm_planes(float *x, const float *planes_ptr, int planes, const void *w, int w_type, void *out,
+                               int act_type, int n, int d, float eps, int write_back, hipStream_t stream) {
+    if (n <= 0) return LCU_OK;
+    if (d <= 0 || d % 4 || planes <= 0 || !planes_ptr) return LCU_BAD_ARGUMENT;
+    const size_t stride = (size_t)n * d;
+    if (act_type == LCU_F32) return rmsnorm_w<float, float, float>(x, planes_ptr, w, w_type, out, n, d, eps, write_back, stream, planes, stride);
+    if (act_type == LCU_BF16) return rmsnorm_w<float, float, bf16_t>(x, planes_ptr, w, w_type, out, n, d, eps, write_back, stream, planes, stride);
     return LCU_BAD_ARGUMENT;
 }
 

@@ -1,0 +1,240 @@
+// Y[M, N] = X[M, K] * W[N, K]^T for 33 to 64 rows (decoding many requests), bfloat16 operands,
+// 32-bit accumulation on the matrix cores.  W is streamed once from HBM; what sets this kernel
+// apart from the one for few rows is where X comes from.  With 64 rows a wave that loads its own
+// piece of X moves twice as many bytes of X as of W and has no registers left to keep loads of W
+// in flight.  Here
+//
+//   * a workgroup is four consumer waves and one producer wave.  The four consumers work on the
+//     same k at the same time, each on its own tile of 16 output features (for SwiGLU a gate
+//     tile and the up tile that belongs to it), so one piece of X serves all of them;
+//   * the producer wave does nothing but copy X, macro-step (128 k) by macro-step, from memory
+//     (it comes from the L2 cache) into a ring of three buffers in LDS, two macro-steps ahead.
+//     Its waits for its loads do not touch the consumers' loads: a wave's loads come back in
+//     order, so a consumer that waited for X would wait for every load of W issued before it;
+//   * a consumer keeps the loads of W of several macro-steps in flight (16 registers a tile and step),
+//     reads X as matrix operands from LDS (rows 272 bytes apart: the 16 lanes of a read fall
+//     into different banks) and multiplies: v_mfma_f32_16x16x32_bf16, A = W tile, B = X^T;
+//   * a product with few output features is cut over K into slices (grid.y), so that the whole
+//     chip streams W: each slice writes its partial sums as float32 to its own plane of the
+//     output, [slice][M][N], and the kernel that follows (residual sum and norm) adds the planes
+//     in a fixed order.  Nothing is added atomically: results do not depend on timing.
+//
+// W is plain rows or packed as gemm_skinny.hip describes it (16 x 128 blocks of 4 KB).
+#include "common.h"
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+
+enum { MID_EPI_BF16 = 0, MID_EPI_PARTIAL_F32 = 1, MID_EPI_SWIGLU = 2 };
+
+#ifndef LCU_MID_STAGES
+#define LCU_MID_STAGES 8
+#endif
+constexpr int MID_STAGE_TILES = LCU_MID_STAGES;    // tiles of W in flight per wave: stages times tiles of a wave
+#ifndef LCU_MID_CONSUMERS
+#define LCU_MID_CONSUMERS 4
+#endif
+constexpr int MID_CONSUMERS = LCU_MID_CONSUMERS;
+constexpr int MID_XROW = 272;                 // bytes between the rows of X in LDS (256 + 16)
+constexpr int MID_XBUFS = 3;
+
+__device__ __forceinline__ f32x4 mid_mfma(u32x4 a, u32x4 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+}
+
+template <int NT, int MT, int EPI>
+__global__ void __launch_bounds__((MID_CONSUMERS + 1) * WAVE)
+gemm_mid_kernel(const bf16_t *__restrict__ X, int ldx, const bf16_t *__restrict__ W, int ldw, void *__restrict__ Y, int ldy,
+                int M, int N, int K, int w_packed, int steps_per_slice) {
+    __shared__ __attribute__((aligned(16))) char xs[MID_XBUFS][16 * MT * MID_XROW];
+    const int lane = threadIdx.x & (WAVE - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
+    const int l16 = lane & 15, grp = lane >> 4;
+    const int steps_total = K / 128;
+    const int s_begin = blockIdx.y * steps_per_slice;
+    const int s_end = min(steps_total, s_begin + steps_per_slice);
+    const int nst = s_end - s_begin;                 // the same for every wave of the workgroup (at least 1)
+
+    if (wave == MID_CONSUMERS) {
+        // ---------------------------------------------------------------- producer of X
+        // chunk c = 64 i + lane of a macro-step: row c / 16, 16 bytes at k = 8 (c % 16).  The loads go
+        // through a buffer resource that ends with the slice's last k of row M - 1 and stand under
+        // no branch (a branch around a load makes the compiler wait for every load in flight): a
+        // row from M on has an offset beyond the end and reads zeros, a macro-step beyond the
+        // slice reads what lies there or zeros and is not used.
+        const __amdgpu_buffer_rsrc_t xb = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<bf16_t *>(X + (size_t)128 * s_begin), 0, (uint32_t)(((size_t)(M - 1) * ldx + 128 * nst) * 2), 0x00020000);
+        uint32_t src[MT * 4];
+        int dst[MT * 4];
+#pragma unroll
+        for (int i = 0; i < MT * 4; ++i) {
+            const int c = 64 * i + lane, tok = c >> 4, kc = c & 15;
+            src[i] = tok < M ? (uint32_t)(tok * ldx + 8 * kc) * 2 : 0x80000000u;
+            dst[i] = tok * MID_XROW + 16 * kc;
+        }
+        u32x4 xr[2][MT * 4];
+#define MID_LOAD_X(b, step)                                                                                         \
+    _Pragma("unroll") for (int i = 0; i < MT * 4; ++i) xr[b][i] =                                                  \
+        __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(xb, src[i], (uint32_t)(step) * 256u, 0))
+        // macro-steps 0 and 1 go straight into their buffers
+        MID_LOAD_X(0, 0);
+        MID_LOAD_X(1, 1);
+#pragma unroll
+        for (int b = 0; b < 2; ++b)
+#pragma unroll
+            for (int i = 0; i < MT * 4; ++i) *(u32x4 *)(xs[b] + dst[i]) = xr[b][i];
+        MID_LOAD_X(0, 2);
+        MID_LOAD_X(1, 3);
+        lds_barrier();
+        // in iteration s: macro-step s + 2 goes into buffer (s + 2) % 3, the loads of s + 4 start
+        int buf = 2;
+        for (int s = 0; s < nst; s += 2) {
+#pragma unroll
+            for (int b = 0; b < 2; ++b) {
+                const int cur = s + b;
+                if (cur < nst) {
+#pragma unroll
+                    for (int i = 0; i < MT * 4; ++i) *(u32x4 *)(xs[buf] + dst[i]) = xr[b][i];
+                    MID_LOAD_X(b, cur + 4);
+                    buf = buf == MID_XBUFS - 1 ? 0 : buf + 1;
+                    lds_barrier();
+                }
+            }
+        }
+#undef MID_LOAD_X
+        return;
+    }
+
+    // -------------------------------------------------------------------- consumers of W
+    // tile t of the wave: rows of W.  SwiGLU: tile 0 a gate tile, tile 1 the up tile N/2 further.
+    const int tile0 = blockIdx.x * MID_CONSUMERS + wave;
+    const int n_tiles = (EPI == MID_EPI_SWIGLU ? N / 2 : N) / 16;
+    const bool live = tile0 < n_tiles;               // a wave beyond the last tile reads the last one and stores nothing
+    // W comes through buffer resources, one per tile, that end with the slice: the loads of the
+    // ring stand under no branch, and a macro-step beyond the slice reads zeros (packed) or
+    // what lies further in the rows (plain; past the matrix's last row zeros) and is not used.
+    __amdgpu_buffer_rsrc_t wb[NT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+        const int tile = (live ? tile0 : n_tiles - 1) + t * n_tiles;
+        wb[t] = w_packed ? __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t *>(W + ((size_t)tile * steps_total + s_begin) * 2048), 0,
+                                                             (uint32_t)nst * 4096u, 0x00020000)
+                         : __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t *>(W + (size_t)16 * tile * ldw + (size_t)128 * s_begin), 0,
+                                                             (uint32_t)(((size_t)15 * ldw + 128 * nst) * 2), 0x00020000);
+    }
+    const uint32_t w_lane = w_packed ? (uint32_t)lane * 16u : (uint32_t)(l16 * ldw + 32 * grp) * 2u;
+    const uint32_t w_step = w_packed ? 4096u : 256u, w_j = w_packed ? 1024u : 16u;
+    f32x4 acc[NT][MT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int m = 0; m < MT; ++m) acc[t][m] = f32x4{0.f, 0.f, 0.f, 0.f};
+    constexpr int MID_STAGES = MID_STAGE_TILES / NT;
+    u32x4 w[MID_STAGES][NT][4];
+#define MID_LOAD_W(i, step)                                                                                     \
+    _Pragma("unroll") for (int t = 0; t < NT; ++t) _Pragma("unroll") for (int j = 0; j < 4; ++j) w[i][t][j] =  \
+        __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(wb[t], w_lane + w_j * j, (uint32_t)(step) * w_step, 0))
+#pragma unroll
+    for (int i = 0; i < MID_STAGES; ++i) MID_LOAD_W(i, i);
+    const int x_off = l16 * MID_XROW + 64 * grp;     // the lane's operand of row tile 0, instruction 0
+    lds_barrier();                                   // macro-steps 0 and 1 of X are in LDS
+    int buf = 0;
+    for (int s = 0; s < nst; s += MID_STAGES) {
+#pragma unroll
+        for (int i = 0; i < MID_STAGES; ++i) {
+            const int cur = s + i;
+            if (cur < nst) {
+                u32x4 xf[MT][4];
+#pragma unroll
+                for (int m = 0; m < MT; ++m)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) xf[m][j] = *(const u32x4 *)(xs[buf] + x_off + 16 * m * MID_XROW + 16 * j);
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+#pragma unroll
+                    for (int t = 0; t < NT; ++t)
+#pragma unroll
+                        for (int m = 0; m < MT; ++m) acc[t][m] = mid_mfma(w[i][t][j], xf[m][j], acc[t][m]);
+                MID_LOAD_W(i, cur + MID_STAGES);
+                buf = buf == MID_XBUFS - 1 ? 0 : buf + 1;
+                lds_barrier();
+            }
+        }
+    }
+#undef MID_LOAD_W
+    if (!live) return;
+    // ---- epilogue: the lane holds, per tile, features 4 grp + r of token 16 m + l16
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+        const int tok = 16 * m + l16;
+        if (tok >= M) continue;
+        const int n = 16 * tile0 + 4 * grp;
+        if (EPI == MID_EPI_SWIGLU) {
+            float o[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const float gate = acc[0][m][r], up = acc[NT - 1][m][r];
+                o[r] = gate * (1.0f / (1.0f + expf(-gate))) * up;
+            }
+            uint2 pk = {pack2_bf16(o[0], o[1]), pack2_bf16(o[2], o[3])};
+            *(uint2 *)((bf16_t *)Y + (size_t)tok * ldy + n) = pk;
+        } else if (EPI == MID_EPI_BF16) {
+            uint2 pk = {pack2_bf16(acc[0][m][0], acc[0][m][1]), pack2_bf16(acc[0][m][2], acc[0][m][3])};
+            *(uint2 *)((bf16_t *)Y + (size_t)tok * ldy + n) = pk;
+        } else {
+            float *plane = (float *)Y + (size_t)blockIdx.y * M * ldy;
+            *(f32x4 *)(plane + (size_t)tok * ldy + n) = acc[0][m];
+        }
+    }
+}
+
+template <int NT, int EPI>
+static int mid_launch(const void *X, int ldx, const void *W, int ldw, void *Y, int ldy, int M, int N, int K, int packed,
+                      int slices, hipStream_t stream) {
+    const int n_tiles = (EPI == MID_EPI_SWIGLU ? N / 2 : N) / 16;
+    const int steps = K / 128, per = (steps + slices - 1) / slices;
+    const dim3 grid((n_tiles + MID_CONSUMERS - 1) / MID_CONSUMERS, (steps + per - 1) / per);
+    const dim3 block((MID_CONSUMERS + 1) * WAVE);
+    if (M <= 32)
+        gemm_mid_kernel<NT, 2, EPI><<<grid, block, 0, stream>>>((const bf16_t *)X, ldx, (const bf16_t *)W, ldw, Y, ldy, M, N, K, packed, per);
+    else if (M <= 48)
+        gemm_mid_kernel<NT, 3, EPI><<<grid, block, 0, stream>>>((const bf16_t *)X, ldx, (const bf16_t *)W, ldw, Y, ldy, M, N, K, packed, per);
+    else
+        gemm_mid_kernel<NT, 4, EPI><<<grid, block, 0, stream>>>((const bf16_t *)X, ldx, (const bf16_t *)W, ldw, Y, ldy, M, N, K, packed, per);
+    LCU_LAUNCH_CHECK();
+    return LCU_OK;
+}
+
+// X: [M, K] bfloat16 rows ldx apart, M <= 64; W: [N, K] bfloat16, rows ldw apart or packed; K a
+// multiple of 128, N of 16 (SwiGLU: of 32; W holds N/2 gate rows, then N/2 up rows).
+// epilogue MID_EPI_BF16: Y [M, N] bfloat16 rows ldy apart (slices must be 1);
+//          MID_EPI_SWIGLU: Y [M, N/2] bfloat16 = silu(gate) * up (slices must be 1);
+//          MID_EPI_PARTIAL_F32: Y [slices_used][M][ldy] float32, plane s the sum over slice s of K;
+//          the planes that exist are ceil(steps / ceil(steps / slices)) with steps = K / 128
+//          (lcu_gemm_mid_planes gives the number).
+LCU_API int lcu_gemm_mid_planes(int K, int slices) {
+    if (K <= 0 || K % 128 || slices <= 0) return LCU_BAD_ARGUMENT;
+    const int steps = K / 128, per = (steps + slices - 1) / slices;
+    return (steps + per - 1) / per;
+}
+
+LCU_API int lcu_gemm_mid_bf16(const void *X, int ldx, const void *W, int ldw, void *Y, int ldy, int M, int N, int K,
+                              int epilogue, int slices, int w_packed, hipStream_t stream) {
+    if (M <= 0 || N <= 0) return LCU_OK;
+    if (M > 64 || K <= 0 || K % 128 || N % 16 || ldx % 8 || ldx < K || slices <= 0 || slices > 64) return LCU_BAD_ARGUMENT;
+    if (!w_packed && (ldw % 8 || ldw < K)) return LCU_BAD_ARGUMENT;
+    if ((uintptr_t)X % 16 || (uintptr_t)W % 16 || (uintptr_t)Y % 16) return LCU_BAD_ARGUMENT;
+    switch (epilogue) {
+    case MID_EPI_BF16:
+        if (slices != 1 || ldy < N || ldy % 4) return LCU_BAD_ARGUMENT;
+        return mid_launch<1, MID_EPI_BF16>(X, ldx, W, ldw, Y, ldy, M, N, K, w_packed, 1, stream);
+    case MID_EPI_PARTIAL_F32:
+        if (ldy < N || ldy % 4) return LCU_BAD_ARGUMENT;
+        return mid_launch<1, MID_EPI_PARTIAL_F32>(X, ldx, W, ldw, Y, ldy, M, N, K, w_packed, slices, stream);
+    case MID_EPI_SWIGLU:
+        if (slices != 1 || N % 32 || ldy < N / 2 || ldy % 4) return LCU_BAD_ARGUMENT;
+        return mid_launch<2, MID_EPI_SWIGLU>(X, ldx, W, ldw, Y, ldy, M, N, K, w_packed, 1, stream);
+    default: return LCU_BAD_ARGUMENT;
+    }
+}

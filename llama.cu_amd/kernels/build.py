@@ -33,7 +33,7 @@ HOST_FLAGS = ["-O2", "-std=c++17", "-shared", "-fPIC", "-Wall"]
 HIP_FLAGS += os.environ.get("LCU_HIP_FLAGS", "").split()
 
 KERNEL_LIBRARIES = ["elementwise", "rope_kv", "attention_generic", "attention_mfma", "gemm_generic", "gemm_skinny",
-                    "sampling"]
+                    "gemm_mid", "sampling"]
 HOST_LIBRARY = "host"
 
 _loaded: Dict[str, ctypes.CDLL] = {}

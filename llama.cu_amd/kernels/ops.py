@@ -137,7 +137,9 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor
             delta: Optional[torch.Tensor] = None, write_back: bool = True) -> torch.Tensor:
     """``y = x' * rsqrt(mean(x'^2) + eps) * weight`` with ``x' = x + delta`` (``x`` if there is
     no ``delta``), all in 32-bit.  With ``write_back`` the sum ``x'`` replaces ``x`` (the
-    residual stream takes in the branch's output)."""
+    residual stream takes in the branch's output).  ``delta`` may also be float32 planes
+    ``[planes, n, d]`` (a product's partial sums, ``gemm_mid(..., slices=)``) beside a float32
+    ``x``: they are added one after the other, in the order of the planes."""
     _gpu(x, weight, out, delta)
     _rows(x, "norm input"); _contig(x, "norm input"); _contig(out, "norm out"); _contig(weight, "norm weight")
     n, d = x.shape
@@ -145,11 +147,20 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor
         raise KernelError(f"norm out: shape {tuple(out.shape)}, expected {(n, d)}")
     if weight.shape != (d,):
         raise KernelError(f"norm weight: shape {tuple(weight.shape)}, expected {(d,)}")
+    xt, at = _type(x, "norm input"), _type(out, "norm out")
+    if delta is not None and delta.dim() == 3:
+        _contig(delta, "norm delta")
+        if delta.shape[1:] != (n, d) or delta.dtype != torch.float32 or x.dtype != torch.float32 or d % 4:
+            raise KernelError("norm delta: planes must be float32 [planes, n, d] beside a float32 input, d a multiple of 4")
+        lib = build.load("elementwise")
+        _check(lib.lcu_rmsnorm_planes(_ptr(x), _ptr(delta), delta.shape[0], _ptr(weight), _type(weight, "norm weight"),
+                                      _ptr(out), at, n, d, ctypes.c_float(eps), int(bool(write_back)), _stream()),
+               "rmsnorm (planes)")
+        return out
     if delta is not None:
         _contig(delta, "norm delta")
         if delta.shape != (n, d) or delta.dtype != out.dtype:
             raise KernelError("norm delta: must have the output's shape and type")
-    xt, at = _type(x, "norm input"), _type(out, "norm out")
     if (xt, at) not in ((F32, F32), (F32, BF16), (BF16, BF16)):
         raise KernelError(f"norm: input {x.dtype} with output {out.dtype} is not supported")
     lib = build.load("elementwise")
@@ -553,6 +564,63 @@ def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = 
     _check(lib.lcu_gemm_skinny_bf16(_ptr(x), x.stride(0), _ptr(w), w.stride(0), _ptr(out), out.stride(0), m, n, k,
                                     _EPILOGUES[epi], tiles, waves, int(packed), _stream()),
            "gemm_skinny")
+    return out
+
+
+MID_MAX_ROWS = 64
+
+
+def mid_supported(x: torch.Tensor, w: torch.Tensor) -> bool:
+    """Whether ``gemm_mid`` takes these operands: up to 64 bfloat16 rows with K a multiple of 128
+    and a bfloat16 weight of a multiple of 16 rows."""
+    return (x.is_cuda and w.is_cuda and x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and x.dim() == 2
+            and w.dim() == 2 and 0 < x.shape[0] <= MID_MAX_ROWS and x.shape[1] == w.shape[1] and w.shape[1] % 128 == 0
+            and w.shape[0] % 16 == 0 and x.stride(1) == 1 and w.stride(1) == 1 and x.stride(0) % 8 == 0
+            and w.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
+
+
+def mid_planes(k: int, slices: int) -> int:
+    """The number of planes ``gemm_mid(..., slices=)`` writes for a weight with ``k`` columns."""
+    steps = k // 128
+    per = -(-steps // slices)
+    return -(-steps // per)
+
+
+def gemm_mid(x: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = None, swiglu: bool = False,
+             slices: Optional[int] = None, packed: bool = False) -> torch.Tensor:
+    """``x @ w.T`` for 33 to 64 rows of bfloat16 ``x`` (it takes fewer too), streaming ``w`` once while
+    the waves of a workgroup share ``x`` through LDS.  ``slices=None``: ``out [m, n]`` bfloat16
+    (``swiglu``: ``w`` holds gate rows, then up rows, ``out [m, n/2] = silu(gate) * up``).
+    ``slices=s``: K is cut into (at most) ``s`` slices and ``out [planes, m, n]`` float32 holds
+    each slice's sum; whoever reads it adds the planes (``rmsnorm(..., delta=planes)`` does).
+    ``packed``: ``w`` is the result of ``pack_weight``."""
+    _gpu(x, w, out)
+    _rows(x, "mid x"); _rows(w, "mid w")
+    if packed and not (packable(w) and w.is_contiguous()):
+        raise KernelError("gemm_mid: a packed weight is a contiguous result of pack_weight")
+    if not mid_supported(x, w):
+        raise KernelError(f"gemm_mid: x {tuple(x.shape)} {x.dtype} with w {tuple(w.shape)} {w.dtype} is not supported "
+                          f"(at most {MID_MAX_ROWS} bfloat16 rows, K a multiple of 128, a multiple of 16 features)")
+    m, k = x.shape
+    n = w.shape[0]
+    if swiglu:
+        if n % 32 or slices is not None:
+            raise KernelError("gemm_mid: the SwiGLU epilogue needs a multiple of 32 rows of w and no slices")
+        epi, shape, dtype = 2, (m, n // 2), torch.bfloat16
+    elif slices is None:
+        epi, shape, dtype = 0, (m, n), torch.bfloat16
+    else:
+        if not 1 <= slices <= 64:
+            raise KernelError("gemm_mid: 1 to 64 slices")
+        epi, shape, dtype = 1, (mid_planes(k, slices), m, n), torch.float32
+    if out is None:
+        out = torch.empty(shape, dtype=dtype, device=x.device)
+    if out.shape != shape or out.dtype != dtype or out.stride(-1) != 1 or out.data_ptr() % 16 or out.stride(-2) % 4 \
+            or (out.dim() == 3 and out.stride(0) != m * out.stride(1)):
+        raise KernelError(f"gemm_mid out: need {dtype} {shape} with rows a multiple of 4 elements apart and planes one after the other")
+    lib = build.load("gemm_mid")
+    _check(lib.lcu_gemm_mid_bf16(_ptr(x), x.stride(0), _ptr(w), w.stride(0), _ptr(out), out.stride(-2), m, n, k, epi,
+                                 slices or 1, int(packed), _stream()), "gemm_mid")
     return out
 
 

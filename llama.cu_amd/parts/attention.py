@@ -15,7 +15,8 @@ import torch
 
 from ..kernels import ops
 from .base import BuildContext, PagedKV, Part, PartSpec, ScaledRows, TensorSpec, make_part, register_part
-from .linear import Weight, linear, linear_into_norm, linear_qkv_rope, linear_scaled, skinny_takes
+from .linear import (Weight, linear, linear_into_norm, linear_planes, linear_qkv_rope, linear_scaled, mid_takes,
+                     skinny_takes)
 from .position import NoPosition
 
 
@@ -66,6 +67,8 @@ class Attention(Part):
     # forward(..., into=(residual, norm)) may end with the residual sum and that norm's weight
     # in the output projection and return ScaledRows instead of the branch's output
     ends_in_norm = True
+    # forward(..., planes_ok=True) may return the branch's output as float32 planes of partial sums
+    ends_in_planes = True
 
     def takes_scaled_rows(self, n_rows: int) -> bool:
         """Whether ``forward`` could be given ScaledRows of ``n_rows`` rows in the place of
@@ -73,7 +76,7 @@ class Attention(Part):
         product anyway."""
         return self.dtype == torch.bfloat16 and n_rows <= ops.ADD_NORM_MAX_ROWS and skinny_takes(n_rows, self.w_qkv, preferred=True)
 
-    def forward(self, h, step, cache, into=None):
+    def forward(self, h, step, cache, into=None, planes_ok=False):
         nh, nkv, dh = self.heads, self.kv_heads, self.head_dim
         if self.shares_kv == cache.writes:
             raise ops.KernelError("attention: a layer that shares another's keys and values must be given that "
@@ -105,6 +108,8 @@ class Attention(Part):
             fused = linear_into_norm(out, self.w_o, residual, norm.weight)
             if fused is not None:
                 return ScaledRows(fused[0], fused[1], norm.size, norm.eps)
+        if planes_ok and self.dtype == torch.bfloat16 and mid_takes(n_rows, self.w_o):
+            return linear_planes(out, self.w_o)
         return linear(out, self.w_o, out_dtype=self.dtype)
 
 

@@ -47,6 +47,12 @@ class PreNormBlock(Part):
         return self.mixer.cache_need()
 
     ends_in_next_norm = True     # forward takes ``next_norm``
+    ends_in_planes = True        # forward takes ``planes_ok``
+
+    @property
+    def takes_planes(self) -> bool:
+        """Whether ``pending`` may be float32 planes of partial sums: the first norm adds them."""
+        return bool(getattr(self.norm1, "takes_planes", False))
 
     def takes_scaled_rows(self, n_rows: int) -> bool:
         """Whether ``forward`` could be given, as ``pending``, ScaledRows of ``n_rows`` rows made
@@ -54,24 +60,32 @@ class PreNormBlock(Part):
         fn = getattr(self.mixer, "takes_scaled_rows", None)
         return getattr(self.norm1, "deferrable", False) and callable(fn) and fn(n_rows)
 
-    def forward(self, x: torch.Tensor, pending, step, cache, next_norm=None):
+    def forward(self, x: torch.Tensor, pending, step, cache, next_norm=None, planes_ok=False):
         """``pending``: the last branch's output, not yet added to ``x`` (or None, or ScaledRows
         made with ``norm1`` by the block before, the sum then being in ``x`` already).
         ``next_norm``: the norm that will follow this block, if whoever runs it takes
-        ScaledRows; then the feed-forward may end in it.  Returns the new ``pending``."""
+        ScaledRows; then the feed-forward may end in it.  ``planes_ok``: whoever takes the new
+        ``pending`` adds float32 planes of partial sums as well as plain rows.  Returns the new
+        ``pending``."""
         h = pending if isinstance(pending, ScaledRows) else self.norm1.forward(x, pending)
         n_rows = x.shape[0]
         ffn_into = (x, next_norm) if next_norm is not None and getattr(self.ffn, "ends_in_norm", False) else None
+        ffn_kw = {"into": ffn_into} if ffn_into else {}
+        if planes_ok and getattr(self.ffn, "ends_in_planes", False):
+            ffn_kw["planes_ok"] = True
+        mixer_kw = {}
+        if getattr(self.norm2, "takes_planes", False) and getattr(self.mixer, "ends_in_planes", False):
+            mixer_kw["planes_ok"] = True
         if self._fuse and self.ffn.takes_scaled_rows(n_rows):
             # the mixer may end with the residual sum and the second norm's weight in its last
             # product; then the feed-forward applies the norm's factor in its first one
-            a = self.mixer.forward(h, step, cache, into=(x, self.norm2))
+            a = self.mixer.forward(h, step, cache, into=(x, self.norm2), **mixer_kw)
             if isinstance(a, ScaledRows):
-                return self.ffn.forward(a, into=ffn_into) if ffn_into else self.ffn.forward(a)
+                return self.ffn.forward(a, **ffn_kw)
         else:
-            a = self.mixer.forward(h, step, cache)
+            a = self.mixer.forward(h, step, cache, **mixer_kw)
         h2 = self.norm2.forward(x, a)
-        return self.ffn.forward(h2, into=ffn_into) if ffn_into else self.ffn.forward(h2)
+        return self.ffn.forward(h2, **ffn_kw)
 
 
 register_part("block", "prenorm", PreNormBlock)

@@ -13,7 +13,8 @@ import torch
 
 from ..kernels import ops
 from .base import BuildContext, Part, ScaledRows, TensorSpec, register_part
-from .linear import Weight, linear, linear_into_norm, linear_swiglu, skinny_row_limit, skinny_takes
+from .linear import (Weight, linear, linear_into_norm, linear_planes, linear_swiglu, linear_swiglu_mid, mid_swiglu_takes,
+                     mid_takes, skinny_row_limit, skinny_takes)
 
 
 class SwiGLU(Part):
@@ -45,8 +46,10 @@ class SwiGLU(Part):
     # forward(..., into=(residual, norm)) may end with the residual sum and that norm's weight
     # in the down projection and return ScaledRows instead of the branch's output
     ends_in_norm = True
+    # forward(..., planes_ok=True) may return the branch's output as float32 planes of partial sums
+    ends_in_planes = True
 
-    def forward(self, h, into=None):
+    def forward(self, h, into=None, planes_ok=False):
         if isinstance(h, ScaledRows):
             if not ops.skinny_supported(h.rows, self.w_gate_up.plain, self.dtype):
                 raise ops.KernelError("feed-forward: rows that wait for their normalisation need the kernel for few rows")
@@ -55,6 +58,9 @@ class SwiGLU(Part):
               and ops.skinny_supported(h, self.w_gate_up.plain, self.dtype)):
             # few rows: one pass over the weights, the activation in the product's epilogue
             act = linear_swiglu(h, self.w_gate_up)
+        elif self.dtype == torch.bfloat16 and mid_swiglu_takes(h.shape[0], self.w_gate_up) and ops.mid_supported(h, self.w_gate_up.plain):
+            # 33 to 64 rows: the rows shared through LDS, the activation in the product's epilogue
+            act = linear_swiglu_mid(h, self.w_gate_up)
         else:
             gu = linear(h, self.w_gate_up, out_dtype=self.dtype)
             act = ops.swiglu(gu)
@@ -64,6 +70,8 @@ class SwiGLU(Part):
             fused = linear_into_norm(act, self.w_down, residual, norm.weight)
             if fused is not None:
                 return ScaledRows(fused[0], fused[1], norm.size, norm.eps)
+        if planes_ok and act.dtype == torch.bfloat16 and mid_takes(act.shape[0], self.w_down):
+            return linear_planes(act, self.w_down)
         return linear(act, self.w_down, out_dtype=self.dtype)
 
 

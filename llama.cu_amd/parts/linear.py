@@ -93,6 +93,49 @@ def linear_scaled(rows, weight: Union[torch.Tensor, Weight], out_dtype: Optional
     return ops.gemm_skinny(rows.rows, weight, **kw)
 
 
+def _mid_slices(n_features: int, k: int) -> int:
+    """Into how many slices of K the kernel for 33 to 64 rows cuts a product, so that about one
+    workgroup (64 features and a slice) stands on each of the 256 compute units; a slice keeps at
+    least four macro-steps of 128."""
+    groups = -(-n_features // 64)
+    return max(1, min(round(256 / groups), 8, k // 512))
+
+
+def mid_takes(n_rows: int, weight: Union[torch.Tensor, Weight]) -> bool:
+    """Whether the kernel for 33 to 64 rows is the faster choice for this many bfloat16 rows and
+    this weight (measured against the library on the Llama-3-8B shapes: the products with few
+    output features, which are cut over K, 10 to 30 % faster with a packed weight, the down
+    projection with a plain one too)."""
+    w, packed = _split(weight)
+    if not (32 < n_rows <= ops.MID_MAX_ROWS and w.dtype == torch.bfloat16 and w.is_cuda and w.dim() == 2
+            and w.shape[1] % 128 == 0 and w.shape[0] % 16 == 0):
+        return False
+    return _mid_slices(w.shape[0], w.shape[1]) >= 3 and (packed is not None or w.shape[1] >= 8192)
+
+
+def linear_planes(a: torch.Tensor, weight: Union[torch.Tensor, Weight]) -> torch.Tensor:
+    """``a @ weight.T`` as float32 planes ``[planes, rows, out]`` of partial sums over slices of K
+    (``mid_takes`` says when); the norm that follows adds them to the residual stream."""
+    w, packed = _split(weight)
+    slices = _mid_slices(w.shape[0], w.shape[1])
+    if packed is not None:
+        return ops.gemm_mid(a, packed, slices=slices, packed=True)
+    return ops.gemm_mid(a, w, slices=slices)
+
+
+def mid_swiglu_takes(n_rows: int, weight: Union[torch.Tensor, Weight]) -> bool:
+    """Whether the gate/up product of this many rows goes to the kernel for 33 to 64 rows with
+    SwiGLU in its epilogue (with a packed weight it is faster than the library's product and the
+    activation kernel after it)."""
+    w, packed = _split(weight)
+    return (32 < n_rows <= ops.MID_MAX_ROWS and packed is not None and w.shape[0] % 32 == 0 and w.shape[1] % 128 == 0
+            and w.shape[0] >= 8192)
+
+
+def linear_swiglu_mid(h: torch.Tensor, weight: Union[torch.Tensor, Weight]) -> torch.Tensor:
+    return ops.gemm_mid(h, _split(weight)[1], swiglu=True, packed=True)
+
+
 def skinny_row_limit(weight: Union[torch.Tensor, Weight]) -> int:
     """Up to how many rows the weight-streaming kernel may be chosen for this weight."""
     return ops.skinny_max_rows(_split(weight)[1] is not None)

@@ -31,8 +31,9 @@ class RMSNorm(Part):
         self.dtype = build.dtype
 
     def forward(self, x: torch.Tensor, delta: Optional[torch.Tensor] = None) -> torch.Tensor:
-        """``x`` (float32 residual stream) takes in ``delta`` if there is one; returns the
-        normalised rows in the compute type."""
+        """``x`` (float32 residual stream) takes in ``delta`` if there is one (rows in the compute
+        type, or float32 planes ``[planes, n, d]`` of partial sums); returns the normalised rows
+        in the compute type."""
         out = torch.empty(x.shape, dtype=self.dtype, device=x.device)
         return ops.rmsnorm(x, self.weight, self.eps, out, delta=delta, write_back=True)
 
@@ -41,6 +42,10 @@ class RMSNorm(Part):
     # after a matrix product instead of before (see ScaledRows); whoever does that reads
     # ``weight``, ``size`` and ``eps``.
     deferrable = True
+
+    # ``delta`` may be planes of partial sums: a product cut over K leaves its slices' sums for
+    # this kernel to add.  A branch hands them only to a norm that says so.
+    takes_planes = True
 
 
 register_part("norm", "rmsnorm", RMSNorm)

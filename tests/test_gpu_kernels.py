@@ -448,6 +448,90 @@ def test_gemm_skinny_refuses_what_it_cannot_take():
     assert not ops.skinny_supported(rnd(65, 64).to(torch.bfloat16).cuda(), rnd(16, 64).to(torch.bfloat16).cuda(), torch.bfloat16)
 
 
+# ------------------------------------------------------------------ product for 33 to 64 rows
+@pytest.mark.parametrize("m", [5, 33, 47, 48, 64])
+@pytest.mark.parametrize("n,k", [(16, 128), (208, 384), (1008, 1024), (64, 2176)])
+@pytest.mark.parametrize("packed", [False, True])
+def test_gemm_mid(m, n, k, packed):
+    from llama_cu_amd.kernels import ops
+    x = rnd(m, k, seed=m + k).to(torch.bfloat16)
+    w = rnd(n, k, seed=n).to(torch.bfloat16)
+    want = plain.linear(x, w)
+    wg = ops.pack_weight(w.cuda()) if packed else w.cuda()
+    # the rows of x lie in a larger buffer whose other rows are poison: nothing beyond row m may count
+    buf = torch.full((m + 3, k + 8), float("nan"), dtype=torch.bfloat16, device="cuda")
+    buf[:m, :k] = x.cuda()
+    xg = buf[:m, :k]
+    close(ops.gemm_mid(xg, wg, packed=packed), want, "bfloat16", "bf16 out")
+    for slices in (1, 2, 3, 5, 64):
+        planes = ops.gemm_mid(xg, wg, slices=slices, packed=packed)
+        assert planes.shape == (ops.mid_planes(k, slices), m, n) and planes.dtype == torch.float32
+        assert planes.shape[0] <= min(slices, k // 128)
+        close(planes.double().sum(0), want, "float32", f"{slices} slices")
+    # a slice's plane is that slice's sum alone
+    if k >= 256:
+        planes = ops.gemm_mid(xg, wg, slices=2, packed=packed)
+        half = 128 * (-(-(k // 128) // 2))
+        close(planes[0], plain.linear(x[:, :half], w[:, :half]), "float32", "first slice")
+
+
+@pytest.mark.parametrize("m,di,k", [(33, 16, 128), (40, 176, 256), (64, 1008, 640)])
+@pytest.mark.parametrize("packed", [False, True])
+def test_gemm_mid_swiglu(m, di, k, packed):
+    from llama_cu_amd.kernels import ops
+    x = rnd(m, k, seed=m).to(torch.bfloat16)
+    w = rnd(2 * di, k, seed=di, scale=0.3).to(torch.bfloat16)
+    gu = plain.linear(x, w)
+    wg = ops.pack_weight(w.cuda()) if packed else w.cuda()
+    close(ops.gemm_mid(x.cuda(), wg, swiglu=True, packed=packed), plain.swiglu(gu[:, :di], gu[:, di:]), "bfloat16")
+
+
+def test_gemm_mid_result_does_not_depend_on_the_batch_and_equals_the_sum_of_the_products():
+    from llama_cu_amd.kernels import ops
+    x = rnd(50, 512, seed=1).to(torch.bfloat16).cuda()
+    w = rnd(304, 512, seed=2).to(torch.bfloat16).cuda()
+    whole = ops.gemm_mid(x, w, slices=2)
+    one = ops.gemm_mid(x[23:24], w, slices=2)
+    assert torch.equal(whole[:, 23:24], one)
+    again = ops.gemm_mid(x, w, slices=2)
+    assert torch.equal(whole, again)
+
+
+def test_gemm_mid_refuses_what_it_cannot_take():
+    from llama_cu_amd.kernels import ops
+    w = rnd(16, 128).to(torch.bfloat16).cuda()
+    assert not ops.mid_supported(rnd(65, 128).to(torch.bfloat16).cuda(), w)                 # too many rows
+    assert not ops.mid_supported(rnd(40, 136).to(torch.bfloat16).cuda(), rnd(16, 136).to(torch.bfloat16).cuda())   # K no multiple of 128
+    assert not ops.mid_supported(rnd(40, 128).to(torch.bfloat16).cuda(), rnd(24, 128).to(torch.bfloat16).cuda())   # features no multiple of 16
+    assert not ops.mid_supported(rnd(40, 128).cuda(), w)                                      # float32 rows
+    with pytest.raises(ops.KernelError):
+        ops.gemm_mid(rnd(65, 128).to(torch.bfloat16).cuda(), w)
+    with pytest.raises(ops.KernelError):
+        ops.gemm_mid(rnd(40, 128).to(torch.bfloat16).cuda(), w, swiglu=True)                  # 16 rows are no gate and up tiles
+    with pytest.raises(ops.KernelError):
+        ops.gemm_mid(rnd(40, 128).to(torch.bfloat16).cuda(), w, slices=65)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("n,d,planes", [(1, 16, 1), (5, 172, 3), (40, 4096, 4), (2, 8200, 2)])
+def test_rmsnorm_adds_planes_of_partial_sums(dtype, n, d, planes):
+    from llama_cu_amd.kernels import ops
+    x = rnd(n, d, seed=1, scale=0.05)
+    parts = rnd(planes, n, d, seed=2, scale=0.05)
+    w = (1 + rnd(d, seed=3, scale=0.1)).to(DT[dtype])
+    xg = x.cuda()
+    out = torch.empty(n, d, dtype=DT[dtype], device="cuda")
+    ops.rmsnorm(xg, w.cuda(), 1e-5, out, delta=parts.cuda())
+    xs = x.double() + parts.double().sum(0)
+    close(xg, xs, "float32", "residual sum")
+    close(out, plain.rms_norm(xs, w, 1e-5), dtype, "norm")
+    # the planes are added one after the other: the same bits as adding them one by one
+    xg2 = x.cuda()
+    for p in range(planes):
+        ops.residual_add(xg2, parts[p].cuda())
+    assert torch.equal(xg, xg2)
+
+
 @pytest.mark.parametrize("m,n,k,tiles,wdtype", [(1, 16, 8, 1, "bfloat16"), (8, 304, 136, 1, "float32"), (16, 4096, 1000, 1, "bfloat16"),
                                                 (5, 104, 64, 2, "bfloat16"), (13, 1000, 4096, 2, "float32"),
                                                 (17, 304, 256, 1, "bfloat16"), (32, 1000, 512, 2, "float32"), (27, 96, 136, 2, "bfloat16")])

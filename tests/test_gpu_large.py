@@ -51,3 +51,40 @@ def test_whole_portions_and_decoding_at_full_layer_sizes(big, dtype):
     if dtype == "bfloat16":
         assert any(key[0] == 2 for key in runner._graphs)
     common.assert_matches_plain(got, want, dtype, f"8B-sized layers/{dtype}")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_steps_of_33_to_64_rows_at_full_layer_sizes(big, dtype, monkeypatch):
+    """Steps of 40 and 39 rows: in bfloat16 the output and down projections leave planes of partial
+    sums to the norm that follows, and gate/up ends in SwiGLU, in the kernel for 33 to 64 rows."""
+    from llama_cu_amd.engine.runner import ModelRunner
+    from llama_cu_amd.kernels import ops
+    calls = {"planes": 0, "swiglu": 0}
+    real = ops.gemm_mid
+
+    def counted(*a, **kw):
+        calls["swiglu" if kw.get("swiglu") else "planes"] += 1
+        return real(*a, **kw)
+    monkeypatch.setattr(ops, "gemm_mid", counted)
+    folder, reqs, want = big[dtype]
+    runner = ModelRunner.from_folder(folder, dtype=dtype, max_tokens=512, max_seqs=4)
+    r0, r1 = reqs["r0"], reqs["r1"]
+    got = {"r0": {}, "r1": {}}
+    logits = runner.step([0], [r0[:40]], [list(range(40))]).cpu().numpy()                    # 40 rows
+    for p in range(40):
+        got["r0"][p] = logits[p]
+    logits = runner.step([0, 1], [r0[40:58], r1[:21]], [list(range(18)), list(range(21))]).cpu().numpy()   # 39 rows
+    for p in range(18):
+        got["r0"][40 + p] = logits[p]
+    for p in range(21):
+        got["r1"][p] = logits[18 + p]
+    logits = runner.step([1, 0], [r1[21:], r0[58:]], [list(range(12)), list(range(12))]).cpu().numpy()     # 24 rows
+    for p in range(12):
+        got["r1"][21 + p] = logits[p]
+        got["r0"][58 + p] = logits[12 + p]
+    layers = SHAPE["num_hidden_layers"]
+    if dtype == "bfloat16":
+        assert calls["planes"] == 2 * 2 * layers and calls["swiglu"] == 2 * layers, calls
+    else:
+        assert calls == {"planes": 0, "swiglu": 0}
+    common.assert_matches_plain(got, want, dtype, f"8B-sized layers, 33 to 64 rows/{dtype}")
