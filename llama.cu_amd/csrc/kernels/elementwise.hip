@@ -110,13 +110,16 @@ __global__ void rmsnorm_kernel(TX *__restrict__ x, const TD *__restrict__ delta,
 
 // The same for rows of up to 8192 elements whose width is a multiple of 4: one read of
 // the row (four elements per thread and load), the row kept in registers between the sum
-// and the scaling.  The order of the sum depends on d only.
-constexpr int NORM_THREADS = 256, NORM_ITEMS = 8;
+// and the scaling.  The block has a thread for every four elements where 1024 threads
+// suffice and never fewer than 256 (few rows leave most of the chip idle: what counts is
+// how many loads a row has in flight); the planes are loaded four at a time.  The order of
+// the sum depends on d and the block's size, which depends on d only.
+constexpr int NORM_MIN_THREADS = 256, NORM_MAX_THREADS = 1024, NORM_ITEMS = 8;
 
 template <class T> struct alignas(4 * sizeof(T)) Vec4 { T v[4]; };
 
 template <class TX, class TD, class TW, class TO>
-__global__ void __launch_bounds__(NORM_THREADS)
+__global__ void __launch_bounds__(NORM_MAX_THREADS)
 rmsnorm_fast_kernel(TX *__restrict__ x, const TD *__restrict__ delta, const TW *__restrict__ w, TO *__restrict__ out,
                     int d, float eps, int write_back, int planes, size_t plane_stride) {
     __shared__ float scratch[16];
@@ -126,16 +129,22 @@ rmsnorm_fast_kernel(TX *__restrict__ x, const TD *__restrict__ delta, const TW *
     float acc = 0.f;
 #pragma unroll
     for (int i = 0; i < NORM_ITEMS; ++i) {
-        const int c = (i * NORM_THREADS + threadIdx.x) * 4;
+        const int c = (i * blockDim.x + threadIdx.x) * 4;
         if (c < d) {
             const Vec4<TX> xv = *(const Vec4<TX> *)(xr + c);
 #pragma unroll
             for (int e = 0; e < 4; ++e) v[i][e] = to_f32(xv.v[e]);
             if (dr) {
-                for (int p = 0; p < planes; ++p) {
-                    const Vec4<TD> dv = *(const Vec4<TD> *)(dr + p * plane_stride + c);
+                for (int p0 = 0; p0 < planes; p0 += 4) {
+                    Vec4<TD> dv[4];
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) v[i][e] += to_f32(dv.v[e]);
+                    for (int q = 0; q < 4; ++q) dv[q] = *(const Vec4<TD> *)(dr + (p0 + q < planes ? p0 + q : p0) * plane_stride + c);
+#pragma unroll
+                    for (int q = 0; q < 4; ++q)
+                        if (p0 + q < planes) {
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) v[i][e] += to_f32(dv[q].v[e]);
+                        }
                 }
                 Vec4<TX> back;
 #pragma unroll
@@ -151,7 +160,7 @@ rmsnorm_fast_kernel(TX *__restrict__ x, const TD *__restrict__ delta, const TW *
     TO *o = out + (size_t)blockIdx.x * d;
 #pragma unroll
     for (int i = 0; i < NORM_ITEMS; ++i) {
-        const int c = (i * NORM_THREADS + threadIdx.x) * 4;
+        const int c = (i * blockDim.x + threadIdx.x) * 4;
         if (c < d) {
             const Vec4<TW> wv = *(const Vec4<TW> *)(w + c);
             Vec4<TO> ov;
@@ -166,11 +175,12 @@ template <class TX, class TD, class TO>
 static int rmsnorm_w(void *x, const void *delta, const void *w, int w_type, void *out, int n, int d, float eps,
                      int write_back, hipStream_t stream, int planes = 1, size_t plane_stride = 0) {
     dim3 grid(n), block(d >= 2048 ? 512 : 256);
-    if (d % 4 == 0 && d <= NORM_THREADS * NORM_ITEMS * 4) {
+    if (d % 4 == 0 && d <= NORM_MIN_THREADS * NORM_ITEMS * 4) {
+        const int fast_threads = min(NORM_MAX_THREADS, max(NORM_MIN_THREADS, (d / 4 + WAVE - 1) / WAVE * WAVE));
         if (w_type == LCU_F32)
-            rmsnorm_fast_kernel<TX, TD, float, TO><<<grid, dim3(NORM_THREADS), 0, stream>>>((TX *)x, (const TD *)delta, (const float *)w, (TO *)out, d, eps, write_back, planes, plane_stride);
+            rmsnorm_fast_kernel<TX, TD, float, TO><<<grid, dim3(fast_threads), 0, stream>>>((TX *)x, (const TD *)delta, (const float *)w, (TO *)out, d, eps, write_back, planes, plane_stride);
         else if (w_type == LCU_BF16)
-            rmsnorm_fast_kernel<TX, TD, bf16_t, TO><<<grid, dim3(NORM_THREADS), 0, stream>>>((TX *)x, (const TD *)delta, (const bf16_t *)w, (TO *)out, d, eps, write_back, planes, plane_stride);
+            rmsnorm_fast_kernel<TX, TD, bf16_t, TO><<<grid, dim3(fast_threads), 0, stream>>>((TX *)x, (const TD *)delta, (const bf16_t *)w, (TO *)out, d, eps, write_back, planes, plane_stride);
         else
             return LCU_BAD_ARGUMENT;
         LCU_LAUNCH_CHECK();

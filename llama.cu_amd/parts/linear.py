@@ -105,9 +105,11 @@ def mid_takes(n_rows: int, weight: Union[torch.Tensor, Weight]) -> bool:
     """Whether the kernel for 33 to 64 rows is the faster choice for this many bfloat16 rows and
     this weight (measured against the library on the Llama-3-8B shapes: the products with few
     output features, which are cut over K, 10 to 30 % faster with a packed weight, the down
-    projection with a plain one too)."""
+    projection with a plain one too).  Where the weight-streaming kernel is not chosen for a
+    long K (the down projection from 25 rows on) it takes those rows too: 24 against 32 us."""
     w, packed = _split(weight)
-    if not (32 < n_rows <= ops.MID_MAX_ROWS and w.dtype == torch.bfloat16 and w.is_cuda and w.dim() == 2
+    fewest = ops.SKINNY_ROWS_PACKED if (packed is not None and w.dim() == 2 and w.shape[1] > 8192) else ops.SKINNY_ROWS_SHORT_K
+    if not (fewest < n_rows <= ops.MID_MAX_ROWS and w.dtype == torch.bfloat16 and w.is_cuda and w.dim() == 2
             and w.shape[1] % 128 == 0 and w.shape[0] % 16 == 0):
         return False
     return _mid_slices(w.shape[0], w.shape[1]) >= 3 and (packed is not None or w.shape[1] >= 8192)
