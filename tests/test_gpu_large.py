@@ -88,3 +88,34 @@ def test_steps_of_33_to_64_rows_at_full_layer_sizes(big, dtype, monkeypatch):
     else:
         assert calls == {"planes": 0, "swiglu": 0}
     common.assert_matches_plain(got, want, dtype, f"8B-sized layers, 33 to 64 rows/{dtype}")
+
+
+def test_captured_steps_of_36_requests_equal_eager_ones(big):
+    """36 requests decode together: the steps replayed from a captured graph (the kernel for 33 to
+    64 rows and its planes of partial sums inside it) give the bits of eager steps on every replay,
+    with eager work between the replays."""
+    from llama_cu_amd.engine.runner import ModelRunner
+    folder = big["bfloat16"][0]
+    rng = np.random.default_rng(5)
+    prompts = [[int(t) for t in rng.integers(SHAPE["vocab_size"], size=3 + i % 5)] for i in range(36)]
+    feeds = [[[int(t)] for t in rng.integers(SHAPE["vocab_size"], size=36)] for _ in range(6)]
+
+    def decode(use_graphs):
+        runner = ModelRunner.from_folder(folder, dtype="bfloat16", max_tokens=36 * 32 + 64, max_seqs=40, use_graphs=use_graphs)
+        ids = list(range(36))
+        runner.step(ids, prompts)
+        outs = []
+        for i, toks in enumerate(feeds):
+            outs.append(runner.step(ids, toks).float().cpu())
+            if i == 3:
+                runner.step([36], [[1, 2, 3, 4, 5]])
+                runner.end(36)
+            torch.cuda.synchronize()
+        return outs, runner
+
+    eager, _ = decode(False)
+    graphed, runner = decode(True)
+    assert any(key[0] == 36 for key in runner._graphs)
+    for i, (a, b) in enumerate(zip(eager, graphed)):
+        assert torch.isfinite(a).all()
+        assert torch.equal(a, b), f"decode step {i} differs between eager and captured"
