@@ -31,6 +31,16 @@ MATRIX_PEAK = {"bf16": 2.5e15, "f32": 157.3e12}
 SHAPE = dict(architectures=["LlamaForCausalLM"], num_hidden_layers=32, hidden_size=4096, num_attention_heads=32,
              num_key_value_heads=8, head_dim=128, intermediate_size=14336, vocab_size=128256,
              max_position_embeddings=8192, rope_theta=500000.0, rms_norm_eps=1e-5, tie_word_embeddings=False)
+# other shapes to measure the same step at (--shape): the 7B shape has a key/value head per head, a
+# smaller feed-forward and vocabulary; the 70B shape is twice as wide (give it --layers: 80 layers
+# of it take 141 GB)
+SHAPES = {
+    "llama3-8b": ("Llama-3-8B", SHAPE),
+    "llama2-7b": ("Llama-2-7B", dict(SHAPE, num_key_value_heads=32, intermediate_size=11008, vocab_size=32000,
+                                     max_position_embeddings=4096, rope_theta=10000.0)),
+    "llama3-70b": ("Llama-3-70B", dict(SHAPE, num_hidden_layers=80, hidden_size=8192, num_attention_heads=64,
+                                       intermediate_size=28672)),
+}
 PROMPT_LEN = 2048
 PREFILL_TOKENS = 2048
 
@@ -147,6 +157,7 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=128)
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--shape", choices=sorted(SHAPES), default="llama3-8b", help="the layer sizes (default: the Llama-3-8B shape)")
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the shape has (named in config)")
     ap.add_argument("--prompt-len", type=int, default=PROMPT_LEN,
                     help="tokens of each request's prompt (other context lengths than the default run's; the context "
@@ -170,7 +181,8 @@ def main() -> int:
     from llama_cu_amd.config import LlamaConfig
     from llama_cu_amd.engine.engine import Engine
 
-    shape = dict(SHAPE)
+    shape_name, shape = SHAPES[args.shape]
+    shape = dict(shape)
     full_layers = shape["num_hidden_layers"]
     if args.layers:
         shape["num_hidden_layers"] = args.layers
@@ -203,10 +215,10 @@ def main() -> int:
     step_bytes = weight_bytes(cfg, elem) + args.batch * mean_ctx * kv_bytes_per_token(cfg, elem)
     achieved = step_bytes / (seconds / args.steps)
     line = {
-        "metric": f"decode tok/s (Llama-3-8B shape, prompts of {args.prompt_len} tokens)", "value": round(value, 2), "unit": "tok/s",
+        "metric": f"decode tok/s ({shape_name} shape, prompts of {args.prompt_len} tokens)", "value": round(value, 2), "unit": "tok/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": dt_name, "data": "synthetic",
-        "config": {"model": "Llama-3-8B shape, random weights", "global_batch": args.batch, "seq_len": args.prompt_len,
+        "config": {"model": f"{shape_name} shape, random weights", "global_batch": args.batch, "seq_len": args.prompt_len,
                    "parallelism": "none (1 GPU)", "context": cfg.max_position_embeddings,
                    "layers": cfg.num_hidden_layers, "layers_of_shape": full_layers, "hidden_size": cfg.hidden_size,
                    "heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads, "head_dim": cfg.head_dim,

@@ -109,80 +109,97 @@ __global__ void rmsnorm_kernel(TX *__restrict__ x, const TD *__restrict__ delta,
 }
 
 // The same for rows of up to 8192 elements whose width is a multiple of 4: one read of
-// the row (four elements per thread and load), the row kept in registers between the sum
-// and the scaling.  The block has a thread for every four elements where 1024 threads
-// suffice and never fewer than 256 (few rows leave most of the chip idle: what counts is
-// how many loads a row has in flight); the planes are loaded four at a time.  The order of
-// the sum depends on d and the block's size, which depends on d only.
-constexpr int NORM_MIN_THREADS = 256, NORM_MAX_THREADS = 1024, NORM_ITEMS = 8;
+// the row (four elements per load), the row kept in registers between the sum and the
+// scaling.  The row is dealt to 1024 virtual threads, two loads each; a block has 1024
+// threads (few rows leave most of the chip idle: what counts then is how many loads a row has
+// in flight) or 256 that play four virtual threads each (many rows: fewer, longer-lived waves
+// stream faster).  The sums are added as the 1024 threads would add them, wave by wave, so
+// the result does not depend on the block's size, only on d.  The planes are loaded four at
+// a time.
+constexpr int NORM_VTHREADS = 1024, NORM_ITEMS = 2;
 
 template <class T> struct alignas(4 * sizeof(T)) Vec4 { T v[4]; };
 
-template <class TX, class TD, class TW, class TO>
-__global__ void __launch_bounds__(NORM_MAX_THREADS)
+template <int THREADS, class TX, class TD, class TW, class TO>
+__global__ void __launch_bounds__(THREADS)
 rmsnorm_fast_kernel(TX *__restrict__ x, const TD *__restrict__ delta, const TW *__restrict__ w, TO *__restrict__ out,
                     int d, float eps, int write_back, int planes, size_t plane_stride) {
-    __shared__ float scratch[16];
+    constexpr int PLAY = NORM_VTHREADS / THREADS;           // virtual threads per thread
+    __shared__ float scratch[NORM_VTHREADS / WAVE];
     TX *xr = x + (size_t)blockIdx.x * d;
     const TD *dr = delta ? delta + (size_t)blockIdx.x * d : nullptr;
-    float v[NORM_ITEMS][4];
-    float acc = 0.f;
+    float v[PLAY][NORM_ITEMS][4];
 #pragma unroll
-    for (int i = 0; i < NORM_ITEMS; ++i) {
-        const int c = (i * blockDim.x + threadIdx.x) * 4;
-        if (c < d) {
-            const Vec4<TX> xv = *(const Vec4<TX> *)(xr + c);
+    for (int j = 0; j < PLAY; ++j) {
+        float acc = 0.f;
 #pragma unroll
-            for (int e = 0; e < 4; ++e) v[i][e] = to_f32(xv.v[e]);
-            if (dr) {
-                for (int p0 = 0; p0 < planes; p0 += 4) {
-                    Vec4<TD> dv[4];
+        for (int i = 0; i < NORM_ITEMS; ++i) {
+            const int c = (i * NORM_VTHREADS + j * THREADS + threadIdx.x) * 4;
+            if (c < d) {
+                const Vec4<TX> xv = *(const Vec4<TX> *)(xr + c);
 #pragma unroll
-                    for (int q = 0; q < 4; ++q) dv[q] = *(const Vec4<TD> *)(dr + (p0 + q < planes ? p0 + q : p0) * plane_stride + c);
+                for (int e = 0; e < 4; ++e) v[j][i][e] = to_f32(xv.v[e]);
+                if (dr) {
+                    for (int p0 = 0; p0 < planes; p0 += 4) {
+                        Vec4<TD> dv[4];
 #pragma unroll
-                    for (int q = 0; q < 4; ++q)
-                        if (p0 + q < planes) {
+                        for (int q = 0; q < 4; ++q) dv[q] = *(const Vec4<TD> *)(dr + (p0 + q < planes ? p0 + q : p0) * plane_stride + c);
 #pragma unroll
-                            for (int e = 0; e < 4; ++e) v[i][e] += to_f32(dv[q].v[e]);
-                        }
+                        for (int q = 0; q < 4; ++q)
+                            if (p0 + q < planes) {
+#pragma unroll
+                                for (int e = 0; e < 4; ++e) v[j][i][e] += to_f32(dv[q].v[e]);
+                            }
+                    }
+                    Vec4<TX> back;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) back.v[e] = from_f32<TX>(v[j][i][e]);
+                    if (write_back) *(Vec4<TX> *)(xr + c) = back;
                 }
-                Vec4<TX> back;
 #pragma unroll
-                for (int e = 0; e < 4; ++e) back.v[e] = from_f32<TX>(v[i][e]);
-                if (write_back) *(Vec4<TX> *)(xr + c) = back;
+                for (int e = 0; e < 4; ++e) acc += v[j][i][e] * v[j][i][e];
             }
-#pragma unroll
-            for (int e = 0; e < 4; ++e) acc += v[i][e] * v[i][e];
         }
+        // the wave of the 1024 threads that these virtual threads are
+        acc = wave_sum(acc);
+        if ((threadIdx.x & (WAVE - 1)) == 0) scratch[j * (THREADS / WAVE) + threadIdx.x / WAVE] = acc;
     }
-    const float total = block_sum(acc, scratch);
+    __syncthreads();
+    float total = 0.f;
+#pragma unroll
+    for (int k = 0; k < NORM_VTHREADS / WAVE; ++k) total += scratch[k];
     const float rms = rsqrtf(total / (float)d + eps);
     TO *o = out + (size_t)blockIdx.x * d;
 #pragma unroll
-    for (int i = 0; i < NORM_ITEMS; ++i) {
-        const int c = (i * blockDim.x + threadIdx.x) * 4;
-        if (c < d) {
-            const Vec4<TW> wv = *(const Vec4<TW> *)(w + c);
-            Vec4<TO> ov;
+    for (int j = 0; j < PLAY; ++j)
 #pragma unroll
-            for (int e = 0; e < 4; ++e) ov.v[e] = from_f32<TO>(rms * v[i][e] * to_f32(wv.v[e]));
-            *(Vec4<TO> *)(o + c) = ov;
+        for (int i = 0; i < NORM_ITEMS; ++i) {
+            const int c = (i * NORM_VTHREADS + j * THREADS + threadIdx.x) * 4;
+            if (c < d) {
+                const Vec4<TW> wv = *(const Vec4<TW> *)(w + c);
+                Vec4<TO> ov;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) ov.v[e] = from_f32<TO>(rms * v[j][i][e] * to_f32(wv.v[e]));
+                *(Vec4<TO> *)(o + c) = ov;
+            }
         }
-    }
 }
 
 template <class TX, class TD, class TO>
 static int rmsnorm_w(void *x, const void *delta, const void *w, int w_type, void *out, int n, int d, float eps,
                      int write_back, hipStream_t stream, int planes = 1, size_t plane_stride = 0) {
     dim3 grid(n), block(d >= 2048 ? 512 : 256);
-    if (d % 4 == 0 && d <= NORM_MIN_THREADS * NORM_ITEMS * 4) {
-        const int fast_threads = min(NORM_MAX_THREADS, max(NORM_MIN_THREADS, (d / 4 + WAVE - 1) / WAVE * WAVE));
-        if (w_type == LCU_F32)
-            rmsnorm_fast_kernel<TX, TD, float, TO><<<grid, dim3(fast_threads), 0, stream>>>((TX *)x, (const TD *)delta, (const float *)w, (TO *)out, d, eps, write_back, planes, plane_stride);
-        else if (w_type == LCU_BF16)
-            rmsnorm_fast_kernel<TX, TD, bf16_t, TO><<<grid, dim3(fast_threads), 0, stream>>>((TX *)x, (const TD *)delta, (const bf16_t *)w, (TO *)out, d, eps, write_back, planes, plane_stride);
-        else
+    if (d % 4 == 0 && d <= NORM_VTHREADS * NORM_ITEMS * 4) {
+#define FAST(T_, TW_) rmsnorm_fast_kernel<T_, TX, TD, TW_, TO><<<grid, dim3(T_), 0, stream>>>((TX *)x, (const TD *)delta, (const TW_ *)w, (TO *)out, d, eps, write_back, planes, plane_stride)
+        const bool few = n <= 128;
+        if (w_type == LCU_F32) {
+            if (few) FAST(1024, float); else FAST(256, float);
+        } else if (w_type == LCU_BF16) {
+            if (few) FAST(1024, bf16_t); else FAST(256, bf16_t);
+        } else {
             return LCU_BAD_ARGUMENT;
+        }
+#undef FAST
         LCU_LAUNCH_CHECK();
         return LCU_OK;
     }

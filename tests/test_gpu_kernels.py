@@ -513,6 +513,20 @@ def test_gemm_mid_refuses_what_it_cannot_take():
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("d", [172, 4096, 8192])
+def test_rmsnorm_of_a_row_does_not_depend_on_the_number_of_rows(dtype, d):
+    """Many rows go to smaller blocks than few rows; the sum is added in the same order."""
+    from llama_cu_amd.kernels import ops
+    x = rnd(300, d, seed=4)
+    delta = rnd(300, d, seed=5).to(DT[dtype])
+    w = (1 + rnd(d, seed=6, scale=0.1)).to(DT[dtype]).cuda()
+    xa, xb = x.cuda(), x[7:9].cuda()
+    many = ops.rmsnorm(xa, w, 1e-5, torch.empty(300, d, dtype=DT[dtype], device="cuda"), delta=delta.cuda())
+    few = ops.rmsnorm(xb, w, 1e-5, torch.empty(2, d, dtype=DT[dtype], device="cuda"), delta=delta[7:9].cuda())
+    assert torch.equal(many[7:9], few) and torch.equal(xa[7:9], xb)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("n,d,planes", [(1, 16, 1), (5, 172, 3), (40, 4096, 4), (2, 8200, 2)])
 def test_rmsnorm_adds_planes_of_partial_sums(dtype, n, d, planes):
     from llama_cu_amd.kernels import ops
