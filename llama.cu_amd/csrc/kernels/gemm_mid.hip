@@ -43,10 +43,10 @@ __device__ __forceinline__ f32x4 mid_mfma(u32x4 a, u32x4 b, f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
 }
 
-template <int NT, int MT, int EPI>
+template <int NT, int MT, int EPI, bool PACKED>
 __global__ void __launch_bounds__((MID_CONSUMERS + 1) * WAVE)
 gemm_mid_kernel(const bf16_t *__restrict__ X, int ldx, const bf16_t *__restrict__ W, int ldw, void *__restrict__ Y, int ldy,
-                int M, int N, int K, int w_packed, int steps_per_slice) {
+                int M, int N, int K, int steps_per_slice) {
     __shared__ __attribute__((aligned(16))) char xs[MID_XBUFS][16 * MT * MID_XROW];
     const int lane = threadIdx.x & (WAVE - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
@@ -62,7 +62,8 @@ gemm_mid_kernel(const bf16_t *__restrict__ X, int ldx, const bf16_t *__restrict_
         // through a buffer resource that ends with the slice's last k of row M - 1 and stand under
         // no branch (a branch around a load makes the compiler wait for every load in flight): a
         // row from M on has an offset beyond the end and reads zeros, a macro-step beyond the
-        // slice reads what lies there or zeros and is not used.
+        // slice reads what lies there or zeros and is not used.  The whole offset is the lane's
+        // (the hardware checks the lane's offset against the end, not the scalar one).
         const __amdgpu_buffer_rsrc_t xb = __builtin_amdgcn_make_buffer_rsrc(
             const_cast<bf16_t *>(X + (size_t)128 * s_begin), 0, (uint32_t)(((size_t)(M - 1) * ldx + 128 * nst) * 2), 0x00020000);
         uint32_t src[MT * 4];
@@ -76,7 +77,7 @@ gemm_mid_kernel(const bf16_t *__restrict__ X, int ldx, const bf16_t *__restrict_
         u32x4 xr[2][MT * 4];
 #define MID_LOAD_X(b, step)                                                                                         \
     _Pragma("unroll") for (int i = 0; i < MT * 4; ++i) xr[b][i] =                                                  \
-        __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(xb, src[i], (uint32_t)(step) * 256u, 0))
+        __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(xb, src[i] + (uint32_t)(step) * 256u, 0, 0))
         // macro-steps 0 and 1 go straight into their buffers
         MID_LOAD_X(0, 0);
         MID_LOAD_X(1, 1);
@@ -118,13 +119,14 @@ gemm_mid_kernel(const bf16_t *__restrict__ X, int ldx, const bf16_t *__restrict_
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
         const int tile = (live ? tile0 : n_tiles - 1) + t * n_tiles;
-        wb[t] = w_packed ? __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t *>(W + ((size_t)tile * steps_total + s_begin) * 2048), 0,
+        wb[t] = PACKED ? __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t *>(W + ((size_t)tile * steps_total + s_begin) * 2048), 0,
                                                              (uint32_t)nst * 4096u, 0x00020000)
                          : __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t *>(W + (size_t)16 * tile * ldw + (size_t)128 * s_begin), 0,
                                                              (uint32_t)(((size_t)15 * ldw + 128 * nst) * 2), 0x00020000);
     }
-    const uint32_t w_lane = w_packed ? (uint32_t)lane * 16u : (uint32_t)(l16 * ldw + 32 * grp) * 2u;
-    const uint32_t w_step = w_packed ? 4096u : 256u, w_j = w_packed ? 1024u : 16u;
+    // the step and the load within it are constants of the instruction, the lane adds its place once a step
+    const uint32_t w_lane = PACKED ? (uint32_t)lane * 16u : (uint32_t)(l16 * ldw + 32 * grp) * 2u;
+    constexpr uint32_t w_step = PACKED ? 4096u : 256u, w_j = PACKED ? 1024u : 16u;
     f32x4 acc[NT][MT];
 #pragma unroll
     for (int t = 0; t < NT; ++t)
@@ -134,7 +136,7 @@ gemm_mid_kernel(const bf16_t *__restrict__ X, int ldx, const bf16_t *__restrict_
     u32x4 w[MID_STAGES][NT][4];
 #define MID_LOAD_W(i, step)                                                                                     \
     _Pragma("unroll") for (int t = 0; t < NT; ++t) _Pragma("unroll") for (int j = 0; j < 4; ++j) w[i][t][j] =  \
-        __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(wb[t], w_lane + w_j * j, (uint32_t)(step) * w_step, 0))
+        __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(wb[t], w_lane + (uint32_t)(step) * w_step + w_j * j, 0, 0))
 #pragma unroll
     for (int i = 0; i < MID_STAGES; ++i) MID_LOAD_W(i, i);
     const int x_off = l16 * MID_XROW + 64 * grp;     // the lane's operand of row tile 0, instruction 0
@@ -196,12 +198,15 @@ static int mid_launch(const void *X, int ldx, const void *W, int ldw, void *Y, i
     const int steps = K / 128, per = (steps + slices - 1) / slices;
     const dim3 grid((n_tiles + MID_CONSUMERS - 1) / MID_CONSUMERS, (steps + per - 1) / per);
     const dim3 block((MID_CONSUMERS + 1) * WAVE);
-    if (M <= 32)
-        gemm_mid_kernel<NT, 2, EPI><<<grid, block, 0, stream>>>((const bf16_t *)X, ldx, (const bf16_t *)W, ldw, Y, ldy, M, N, K, packed, per);
-    else if (M <= 48)
-        gemm_mid_kernel<NT, 3, EPI><<<grid, block, 0, stream>>>((const bf16_t *)X, ldx, (const bf16_t *)W, ldw, Y, ldy, M, N, K, packed, per);
-    else
-        gemm_mid_kernel<NT, 4, EPI><<<grid, block, 0, stream>>>((const bf16_t *)X, ldx, (const bf16_t *)W, ldw, Y, ldy, M, N, K, packed, per);
+#define GO(MT_, P_) gemm_mid_kernel<NT, MT_, EPI, P_><<<grid, block, 0, stream>>>((const bf16_t *)X, ldx, (const bf16_t *)W, ldw, Y, ldy, M, N, K, per)
+    if (M <= 32) {
+        if (packed) GO(2, true); else GO(2, false);
+    } else if (M <= 48) {
+        if (packed) GO(3, true); else GO(3, false);
+    } else {
+        if (packed) GO(4, true); else GO(4, false);
+    }
+#undef GO
     LCU_LAUNCH_CHECK();
     return LCU_OK;
 }
