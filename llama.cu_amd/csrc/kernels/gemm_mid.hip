@@ -1,4 +1,4 @@
-// Y[M, N] = X[M, K] * W[N, K]^T for 33 to 64 rows (decoding many requests), bfloat16 operands,
+// Y[M, N] = X[M, K] * W[N, K]^T for 17 to 64 rows (decoding many requests), bfloat16 operands,
 // 32-bit accumulation on the matrix cores.  W is streamed once from HBM; what sets this kernel
 // apart from the one for few rows is where X comes from.  With 64 rows a wave that loads its own
 // piece of X moves twice as many bytes of X as of W and has no registers left to keep loads of W
@@ -20,6 +20,11 @@
 //     in a fixed order.  Nothing is added atomically: results do not depend on timing.
 //
 // W is plain rows or packed as gemm_skinny.hip describes it (16 x 128 blocks of 4 KB).
+//
+// The rows of X may wait for their normalisation (sumsq_in not null: a factor per row,
+// rsqrt(sum of the row's shares / norm_width + eps), which commutes with the product): consumer
+// wave w loads the shares of rows 16 w .. 16 w + 15 before its first loads of W, so they are back
+// first, adds them in a fixed order and leaves the factors in LDS for the epilogue.
 #include "common.h"
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
@@ -46,8 +51,10 @@ __device__ __forceinline__ f32x4 mid_mfma(u32x4 a, u32x4 b, f32x4 c) {
 template <int NT, int MT, int EPI, bool PACKED>
 __global__ void __launch_bounds__((MID_CONSUMERS + 1) * WAVE)
 gemm_mid_kernel(const bf16_t *__restrict__ X, int ldx, const bf16_t *__restrict__ W, int ldw, void *__restrict__ Y, int ldy,
-                int M, int N, int K, int steps_per_slice) {
+                int M, int N, int K, int steps_per_slice, const float *__restrict__ sumsq_in, int n_in, int norm_width,
+                float eps) {
     __shared__ __attribute__((aligned(16))) char xs[MID_XBUFS][16 * MT * MID_XROW];
+    __shared__ float row_scale[16 * MT];
     const int lane = threadIdx.x & (WAVE - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
     const int l16 = lane & 15, grp = lane >> 4;
@@ -132,6 +139,28 @@ gemm_mid_kernel(const bf16_t *__restrict__ X, int ldx, const bf16_t *__restrict_
     for (int t = 0; t < NT; ++t)
 #pragma unroll
         for (int m = 0; m < MT; ++m) acc[t][m] = f32x4{0.f, 0.f, 0.f, 0.f};
+    // the rows' factors: lane group g adds the g-th quarter of a row's shares (sixteen 16-byte loads
+    // at a time), the quarters are added in the order of the shuffles
+    float scale_ss = 0.f;
+    const bool scales = sumsq_in != nullptr && wave < MT;
+    if (scales) {
+        const int tok = 16 * wave + l16;
+        const float *p = sumsq_in + (size_t)(tok < M ? tok : 0) * n_in;
+        if ((n_in & 15) == 0) {
+            const int q4 = n_in / 16;                         // float4s in a quarter
+            const f32x4 *p4 = (const f32x4 *)p + grp * q4;
+            for (int i = 0; i < q4; i += 16) {
+                f32x4 v[16];
+#pragma unroll
+                for (int e = 0; e < 16; ++e) v[e] = p4[i + e < q4 ? i + e : q4 - 1];
+#pragma unroll
+                for (int e = 0; e < 16; ++e)
+                    if (i + e < q4) scale_ss += (v[e][0] + v[e][1]) + (v[e][2] + v[e][3]);
+            }
+        } else {
+            for (int i = grp; i < n_in; i += 4) scale_ss += p[i];
+        }
+    }
     constexpr int MID_STAGES = MID_STAGE_TILES / NT;
     u32x4 w[MID_STAGES][NT][4];
 #define MID_LOAD_W(i, step)                                                                                     \
@@ -139,6 +168,11 @@ gemm_mid_kernel(const bf16_t *__restrict__ X, int ldx, const bf16_t *__restrict_
         __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(wb[t], w_lane + (uint32_t)(step) * w_step + w_j * j, 0, 0))
 #pragma unroll
     for (int i = 0; i < MID_STAGES; ++i) MID_LOAD_W(i, i);
+    if (scales) {
+        scale_ss += __shfl_xor(scale_ss, 16, WAVE);
+        scale_ss += __shfl_xor(scale_ss, 32, WAVE);
+        if (grp == 0) row_scale[16 * wave + l16] = rsqrtf(scale_ss / (float)norm_width + eps);
+    }
     const int x_off = l16 * MID_XROW + 64 * grp;     // the lane's operand of row tile 0, instruction 0
     lds_barrier();                                   // macro-steps 0 and 1 of X are in LDS
     int buf = 0;
@@ -167,6 +201,16 @@ gemm_mid_kernel(const bf16_t *__restrict__ X, int ldx, const bf16_t *__restrict_
 #undef MID_LOAD_W
     if (!live) return;
     // ---- epilogue: the lane holds, per tile, features 4 grp + r of token 16 m + l16
+    if (sumsq_in != nullptr) {                       // (the factors were written before the loop's barriers)
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+            const float rs = row_scale[16 * m + l16];
+#pragma unroll
+            for (int t = 0; t < NT; ++t)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) acc[t][m][r] *= rs;
+        }
+    }
 #pragma unroll
     for (int m = 0; m < MT; ++m) {
         const int tok = 16 * m + l16;
@@ -191,14 +235,20 @@ gemm_mid_kernel(const bf16_t *__restrict__ X, int ldx, const bf16_t *__restrict_
     }
 }
 
+struct MidScale {
+    const float *sumsq_in;
+    int n_in, norm_width;
+    float eps;
+};
+
 template <int NT, int EPI>
 static int mid_launch(const void *X, int ldx, const void *W, int ldw, void *Y, int ldy, int M, int N, int K, int packed,
-                      int slices, hipStream_t stream) {
+                      int slices, const MidScale &sc, hipStream_t stream) {
     const int n_tiles = (EPI == MID_EPI_SWIGLU ? N / 2 : N) / 16;
     const int steps = K / 128, per = (steps + slices - 1) / slices;
     const dim3 grid((n_tiles + MID_CONSUMERS - 1) / MID_CONSUMERS, (steps + per - 1) / per);
     const dim3 block((MID_CONSUMERS + 1) * WAVE);
-#define GO(MT_, P_) gemm_mid_kernel<NT, MT_, EPI, P_><<<grid, block, 0, stream>>>((const bf16_t *)X, ldx, (const bf16_t *)W, ldw, Y, ldy, M, N, K, per)
+#define GO(MT_, P_) gemm_mid_kernel<NT, MT_, EPI, P_><<<grid, block, 0, stream>>>((const bf16_t *)X, ldx, (const bf16_t *)W, ldw, Y, ldy, M, N, K, per, sc.sumsq_in, sc.n_in, sc.norm_width, sc.eps)
     if (M <= 32) {
         if (packed) GO(2, true); else GO(2, false);
     } else if (M <= 48) {
@@ -224,22 +274,38 @@ LCU_API int lcu_gemm_mid_planes(int K, int slices) {
     return (steps + per - 1) / per;
 }
 
-LCU_API int lcu_gemm_mid_bf16(const void *X, int ldx, const void *W, int ldw, void *Y, int ldy, int M, int N, int K,
-                              int epilogue, int slices, int w_packed, hipStream_t stream) {
+static int mid_bf16(const void *X, int ldx, const void *W, int ldw, void *Y, int ldy, int M, int N, int K, int epilogue,
+                    int slices, int w_packed, const MidScale &sc, hipStream_t stream) {
     if (M <= 0 || N <= 0) return LCU_OK;
     if (M > 64 || K <= 0 || K % 128 || N % 16 || ldx % 8 || ldx < K || slices <= 0 || slices > 64) return LCU_BAD_ARGUMENT;
     if (!w_packed && (ldw % 8 || ldw < K)) return LCU_BAD_ARGUMENT;
-    if ((uintptr_t)X % 16 || (uintptr_t)W % 16 || (uintptr_t)Y % 16) return LCU_BAD_ARGUMENT;
+    if ((uintptr_t)X % 16 || (uintptr_t)W % 16 || (uintptr_t)Y % 16 || (uintptr_t)sc.sumsq_in % 16) return LCU_BAD_ARGUMENT;
     switch (epilogue) {
     case MID_EPI_BF16:
         if (slices != 1 || ldy < N || ldy % 4) return LCU_BAD_ARGUMENT;
-        return mid_launch<1, MID_EPI_BF16>(X, ldx, W, ldw, Y, ldy, M, N, K, w_packed, 1, stream);
+        return mid_launch<1, MID_EPI_BF16>(X, ldx, W, ldw, Y, ldy, M, N, K, w_packed, 1, sc, stream);
     case MID_EPI_PARTIAL_F32:
         if (ldy < N || ldy % 4) return LCU_BAD_ARGUMENT;
-        return mid_launch<1, MID_EPI_PARTIAL_F32>(X, ldx, W, ldw, Y, ldy, M, N, K, w_packed, slices, stream);
+        return mid_launch<1, MID_EPI_PARTIAL_F32>(X, ldx, W, ldw, Y, ldy, M, N, K, w_packed, slices, sc, stream);
     case MID_EPI_SWIGLU:
         if (slices != 1 || N % 32 || ldy < N / 2 || ldy % 4) return LCU_BAD_ARGUMENT;
-        return mid_launch<2, MID_EPI_SWIGLU>(X, ldx, W, ldw, Y, ldy, M, N, K, w_packed, 1, stream);
+        return mid_launch<2, MID_EPI_SWIGLU>(X, ldx, W, ldw, Y, ldy, M, N, K, w_packed, 1, sc, stream);
     default: return LCU_BAD_ARGUMENT;
     }
+}
+
+LCU_API int lcu_gemm_mid_bf16(const void *X, int ldx, const void *W, int ldw, void *Y, int ldy, int M, int N, int K,
+                              int epilogue, int slices, int w_packed, hipStream_t stream) {
+    const MidScale none = {nullptr, 0, 0, 0.f};
+    return mid_bf16(X, ldx, W, ldw, Y, ldy, M, N, K, epilogue, slices, w_packed, none, stream);
+}
+
+// The same with rows of X that wait for their normalisation: row i of the product is multiplied by
+// rsqrt(sum(sumsq_in[i][0 .. n_in)) / norm_width + eps) before the epilogue.  sumsq_in: [M][n_in] float32.
+LCU_API int lcu_gemm_mid_bf16_scaled(const void *X, int ldx, const void *W, int ldw, void *Y, int ldy, int M, int N, int K,
+                                     int epilogue, int slices, int w_packed, const float *sumsq_in, int n_in,
+                                     int norm_width, float eps, hipStream_t stream) {
+    if (!sumsq_in || n_in <= 0 || norm_width <= 0) return LCU_BAD_ARGUMENT;
+    const MidScale sc = {sumsq_in, n_in, norm_width, eps};
+    return mid_bf16(X, ldx, W, ldw, Y, ldy, M, N, K, epilogue, slices, w_packed, sc, stream);
 }

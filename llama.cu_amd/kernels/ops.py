@@ -587,14 +587,16 @@ def mid_planes(k: int, slices: int) -> int:
 
 
 def gemm_mid(x: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = None, swiglu: bool = False,
-             slices: Optional[int] = None, packed: bool = False) -> torch.Tensor:
+             slices: Optional[int] = None, packed: bool = False, row_sumsq: Optional[torch.Tensor] = None,
+             norm_width: int = 0, eps: float = 0.0) -> torch.Tensor:
     """``x @ w.T`` for 33 to 64 rows of bfloat16 ``x`` (it takes fewer too), streaming ``w`` once while
     the waves of a workgroup share ``x`` through LDS.  ``slices=None``: ``out [m, n]`` bfloat16
     (``swiglu``: ``w`` holds gate rows, then up rows, ``out [m, n/2] = silu(gate) * up``).
     ``slices=s``: K is cut into (at most) ``s`` slices and ``out [planes, m, n]`` float32 holds
     each slice's sum; whoever reads it adds the planes (``rmsnorm(..., delta=planes)`` does).
-    ``packed``: ``w`` is the result of ``pack_weight``."""
-    _gpu(x, w, out)
+    ``packed``: ``w`` is the result of ``pack_weight``.  ``row_sumsq [m, parts]``: the rows of ``x``
+    wait for their normalisation, as in ``gemm_skinny``."""
+    _gpu(x, w, out, row_sumsq)
     _rows(x, "mid x"); _rows(w, "mid w")
     if packed and not (packable(w) and w.is_contiguous()):
         raise KernelError("gemm_mid: a packed weight is a contiguous result of pack_weight")
@@ -619,6 +621,14 @@ def gemm_mid(x: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = Non
             or (out.dim() == 3 and out.stride(0) != m * out.stride(1)):
         raise KernelError(f"gemm_mid out: need {dtype} {shape} with rows a multiple of 4 elements apart and planes one after the other")
     lib = build.load("gemm_mid")
+    if row_sumsq is not None:
+        if row_sumsq.dtype != torch.float32 or row_sumsq.dim() != 2 or row_sumsq.shape[0] != m or not row_sumsq.is_contiguous() \
+                or norm_width <= 0 or row_sumsq.data_ptr() % 16:
+            raise KernelError("gemm_mid: row_sumsq must be a contiguous float32 [rows, parts] tensor, with the norm's width")
+        _check(lib.lcu_gemm_mid_bf16_scaled(_ptr(x), x.stride(0), _ptr(w), w.stride(0), _ptr(out), out.stride(-2), m, n, k, epi,
+                                            slices or 1, int(packed), _ptr(row_sumsq), row_sumsq.shape[1], int(norm_width),
+                                            ctypes.c_float(eps), _stream()), "gemm_mid (scaled rows)")
+        return out
     _check(lib.lcu_gemm_mid_bf16(_ptr(x), x.stride(0), _ptr(w), w.stride(0), _ptr(out), out.stride(-2), m, n, k, epi,
                                  slices or 1, int(packed), _stream()), "gemm_mid")
     return out

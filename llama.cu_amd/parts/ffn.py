@@ -50,17 +50,19 @@ class SwiGLU(Part):
     ends_in_planes = True
 
     def forward(self, h, into=None, planes_ok=False):
-        if isinstance(h, ScaledRows):
+        if isinstance(h, ScaledRows) and mid_swiglu_takes(h.rows.shape[0], self.w_gate_up) and ops.mid_supported(h.rows, self.w_gate_up.plain):
+            act = linear_swiglu_mid(h, self.w_gate_up)
+        elif isinstance(h, ScaledRows):
             if not ops.skinny_supported(h.rows, self.w_gate_up.plain, self.dtype):
                 raise ops.KernelError("feed-forward: rows that wait for their normalisation need the kernel for few rows")
             act = linear_swiglu(h.rows, self.w_gate_up, row_sumsq=h.sumsq, norm_width=h.width, eps=h.eps)
+        elif self.dtype == torch.bfloat16 and mid_swiglu_takes(h.shape[0], self.w_gate_up) and ops.mid_supported(h, self.w_gate_up.plain):
+            # 17 to 64 rows: the rows shared through LDS, the activation in the product's epilogue
+            act = linear_swiglu_mid(h, self.w_gate_up)
         elif (self.dtype == torch.bfloat16 and h.shape[0] <= skinny_row_limit(self.w_gate_up)
               and ops.skinny_supported(h, self.w_gate_up.plain, self.dtype)):
             # few rows: one pass over the weights, the activation in the product's epilogue
             act = linear_swiglu(h, self.w_gate_up)
-        elif self.dtype == torch.bfloat16 and mid_swiglu_takes(h.shape[0], self.w_gate_up) and ops.mid_supported(h, self.w_gate_up.plain):
-            # 33 to 64 rows: the rows shared through LDS, the activation in the product's epilogue
-            act = linear_swiglu_mid(h, self.w_gate_up)
         else:
             gu = linear(h, self.w_gate_up, out_dtype=self.dtype)
             act = ops.swiglu(gu)

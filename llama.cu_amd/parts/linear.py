@@ -126,15 +126,19 @@ def linear_planes(a: torch.Tensor, weight: Union[torch.Tensor, Weight]) -> torch
 
 
 def mid_swiglu_takes(n_rows: int, weight: Union[torch.Tensor, Weight]) -> bool:
-    """Whether the gate/up product of this many rows goes to the kernel for 33 to 64 rows with
+    """Whether the gate/up product of this many rows goes to the kernel that shares the rows through LDS, with
     SwiGLU in its epilogue (with a packed weight it is faster than the library's product and the
-    activation kernel after it)."""
+    activation kernel after it, and from 17 rows on than the weight-streaming kernel: 46 against
+    52 to 55 us on the Llama-3-8B shape)."""
     w, packed = _split(weight)
-    return (32 < n_rows <= ops.MID_MAX_ROWS and packed is not None and w.shape[0] % 32 == 0 and w.shape[1] % 128 == 0
+    return (16 < n_rows <= ops.MID_MAX_ROWS and packed is not None and w.shape[0] % 32 == 0 and w.shape[1] % 128 == 0
             and w.shape[0] >= 8192)
 
 
-def linear_swiglu_mid(h: torch.Tensor, weight: Union[torch.Tensor, Weight]) -> torch.Tensor:
+def linear_swiglu_mid(h, weight: Union[torch.Tensor, Weight]) -> torch.Tensor:
+    """``h``: bfloat16 rows or ScaledRows (the factor then goes into the epilogue)."""
+    if isinstance(h, ScaledRows):
+        return ops.gemm_mid(h.rows, _split(weight)[1], swiglu=True, packed=True, row_sumsq=h.sumsq, norm_width=h.width, eps=h.eps)
     return ops.gemm_mid(h, _split(weight)[1], swiglu=True, packed=True)
 
 

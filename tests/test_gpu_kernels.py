@@ -486,6 +486,28 @@ def test_gemm_mid_swiglu(m, di, k, packed):
     close(ops.gemm_mid(x.cuda(), wg, swiglu=True, packed=packed), plain.swiglu(gu[:, :di], gu[:, di:]), "bfloat16")
 
 
+@pytest.mark.parametrize("m,di,k,parts", [(17, 16, 128, 1), (32, 176, 256, 256), (40, 1008, 640, 48), (64, 64, 128, 100)])
+def test_gemm_mid_rows_that_wait_for_their_normalisation(m, di, k, parts):
+    """The rows' factor, rsqrt(sum of the row's shares / width + eps), goes into the epilogue: of
+    SwiGLU, of the plain product and of every plane of partial sums."""
+    from llama_cu_amd.kernels import ops
+    x = rnd(m, k, seed=m).to(torch.bfloat16)
+    w = rnd(2 * di, k, seed=di, scale=0.3).to(torch.bfloat16)
+    # shares in a buffer with poison behind them: only a row's own shares may count
+    shares = torch.full((m + 1, parts), float("nan"))
+    shares[:m] = rnd(m, parts, seed=3).abs() * k / parts
+    sg = shares.cuda()[:m]
+    eps, width = 1e-3, k
+    factor = torch.rsqrt(shares[:m].double().sum(1, keepdim=True) / width + eps)
+    gu = plain.linear(x, w) * factor
+    for packed in (False, True):
+        wg = ops.pack_weight(w.cuda()) if packed else w.cuda()
+        kw = dict(packed=packed, row_sumsq=sg, norm_width=width, eps=eps)
+        close(ops.gemm_mid(x.cuda(), wg, swiglu=True, **kw), plain.swiglu(gu[:, :di], gu[:, di:]), "bfloat16", "SwiGLU")
+        close(ops.gemm_mid(x.cuda(), wg, **kw), gu, "bfloat16", "plain product")
+        close(ops.gemm_mid(x.cuda(), wg, slices=2, **kw).double().sum(0), gu, "float32", "planes")
+
+
 def test_gemm_mid_result_does_not_depend_on_the_batch_and_equals_the_sum_of_the_products():
     from llama_cu_amd.kernels import ops
     x = rnd(50, 512, seed=1).to(torch.bfloat16).cuda()
