@@ -1,10 +1,11 @@
-// Y[M, N] = X[M, K] * W[N, K]^T for 17 to 64 rows (decoding many requests), bfloat16 operands,
+// Y[M, N] = X[M, K] * W[N, K]^T for 17 to 128 rows (decoding many requests), bfloat16 operands,
 // 32-bit accumulation on the matrix cores.  W is streamed once from HBM; what sets this kernel
 // apart from the one for few rows is where X comes from.  With 64 rows a wave that loads its own
 // piece of X moves twice as many bytes of X as of W and has no registers left to keep loads of W
 // in flight.  Here
 //
-//   * a workgroup is four consumer waves and one producer wave.  The four consumers work on the
+//   * a workgroup is four consumer waves and one producer wave (two from 65 rows on, 64 rows
+//     each).  The four consumers work on the
 //     same k at the same time, each on its own tile of 16 output features (for SwiGLU a gate
 //     tile and the up tile that belongs to it), so one piece of X serves all of them;
 //   * the producer wave does nothing but copy X, macro-step (128 k) by macro-step, from memory
@@ -48,13 +49,70 @@ __device__ __forceinline__ f32x4 mid_mfma(u32x4 a, u32x4 b, f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
 }
 
+constexpr int mid_producers(int MT) { return MT > 4 ? 2 : 1; }
+constexpr int mid_lds_bytes(int MT) { return MID_XBUFS * 16 * MT * MID_XROW + 16 * MT * (int)sizeof(float); }
+
+// Producer wave P copies the rows 64 P .. of X, macro-step by macro-step, into the ring in LDS.
+// chunk c = 64 i + lane of a macro-step: row 64 P + c / 16, 16 bytes at k = 8 (c % 16).  The loads
+// go through a buffer resource that ends with the slice's last k of row M - 1 and stand under no
+// branch (a branch around a load makes the compiler wait for every load in flight): a row from M
+// on has an offset beyond the end and reads zeros, a macro-step beyond the slice reads what lies
+// there or zeros and is not used.  The whole offset is the lane's (the hardware checks the
+// lane's offset against the end, not the scalar one).
+template <int MT, int P>
+__device__ __forceinline__ void mid_produce(char *xs, const bf16_t *__restrict__ X, int ldx, int M, int s_begin, int nst, int lane) {
+    constexpr int LOADS = (P == 0 ? (MT < 4 ? MT : 4) : MT - 4) * 4;      // four rows a load
+    constexpr int BUF = 16 * MT * MID_XROW;
+    const __amdgpu_buffer_rsrc_t xb = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<bf16_t *>(X + (size_t)128 * s_begin), 0, (uint32_t)(((size_t)(M - 1) * ldx + 128 * nst) * 2), 0x00020000);
+    uint32_t src[LOADS];
+    int dst[LOADS];
+#pragma unroll
+    for (int i = 0; i < LOADS; ++i) {
+        const int c = 64 * i + lane, tok = 64 * P + (c >> 4), kc = c & 15;
+        src[i] = tok < M ? (uint32_t)(tok * ldx + 8 * kc) * 2 : 0x80000000u;
+        dst[i] = tok * MID_XROW + 16 * kc;
+    }
+    u32x4 xr[2][LOADS];
+#define MID_LOAD_X(b, step)                                                                                         \
+    _Pragma("unroll") for (int i = 0; i < LOADS; ++i) xr[b][i] =                                                   \
+        __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(xb, src[i] + (uint32_t)(step) * 256u, 0, 0))
+    // macro-steps 0 and 1 go straight into their buffers
+    MID_LOAD_X(0, 0);
+    MID_LOAD_X(1, 1);
+#pragma unroll
+    for (int b = 0; b < 2; ++b)
+#pragma unroll
+        for (int i = 0; i < LOADS; ++i) *(u32x4 *)(xs + b * BUF + dst[i]) = xr[b][i];
+    MID_LOAD_X(0, 2);
+    MID_LOAD_X(1, 3);
+    lds_barrier();
+    // in iteration s: macro-step s + 2 goes into buffer (s + 2) % 3, the loads of s + 4 start
+    int buf = 2;
+    for (int s = 0; s < nst; s += 2) {
+#pragma unroll
+        for (int b = 0; b < 2; ++b) {
+            const int cur = s + b;
+            if (cur < nst) {
+#pragma unroll
+                for (int i = 0; i < LOADS; ++i) *(u32x4 *)(xs + buf * BUF + dst[i]) = xr[b][i];
+                MID_LOAD_X(b, cur + 4);
+                buf = buf == MID_XBUFS - 1 ? 0 : buf + 1;
+                lds_barrier();
+            }
+        }
+    }
+#undef MID_LOAD_X
+}
+
 template <int NT, int MT, int EPI, bool PACKED>
-__global__ void __launch_bounds__((MID_CONSUMERS + 1) * WAVE)
+__global__ void __launch_bounds__((MID_CONSUMERS + mid_producers(MT)) * WAVE)
 gemm_mid_kernel(const bf16_t *__restrict__ X, int ldx, const bf16_t *__restrict__ W, int ldw, void *__restrict__ Y, int ldy,
                 int M, int N, int K, int steps_per_slice, const float *__restrict__ sumsq_in, int n_in, int norm_width,
                 float eps) {
-    __shared__ __attribute__((aligned(16))) char xs[MID_XBUFS][16 * MT * MID_XROW];
-    __shared__ float row_scale[16 * MT];
+    extern __shared__ __attribute__((aligned(16))) char xs[];      // the ring of X, then the rows' factors
+    constexpr int BUF = 16 * MT * MID_XROW;
+    float *row_scale = (float *)(xs + MID_XBUFS * BUF);
     const int lane = threadIdx.x & (WAVE - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
     const int l16 = lane & 15, grp = lane >> 4;
@@ -64,54 +122,14 @@ gemm_mid_kernel(const bf16_t *__restrict__ X, int ldx, const bf16_t *__restrict_
     const int nst = s_end - s_begin;                 // the same for every wave of the workgroup (at least 1)
 
     if (wave == MID_CONSUMERS) {
-        // ---------------------------------------------------------------- producer of X
-        // chunk c = 64 i + lane of a macro-step: row c / 16, 16 bytes at k = 8 (c % 16).  The loads go
-        // through a buffer resource that ends with the slice's last k of row M - 1 and stand under
-        // no branch (a branch around a load makes the compiler wait for every load in flight): a
-        // row from M on has an offset beyond the end and reads zeros, a macro-step beyond the
-        // slice reads what lies there or zeros and is not used.  The whole offset is the lane's
-        // (the hardware checks the lane's offset against the end, not the scalar one).
-        const __amdgpu_buffer_rsrc_t xb = __builtin_amdgcn_make_buffer_rsrc(
-            const_cast<bf16_t *>(X + (size_t)128 * s_begin), 0, (uint32_t)(((size_t)(M - 1) * ldx + 128 * nst) * 2), 0x00020000);
-        uint32_t src[MT * 4];
-        int dst[MT * 4];
-#pragma unroll
-        for (int i = 0; i < MT * 4; ++i) {
-            const int c = 64 * i + lane, tok = c >> 4, kc = c & 15;
-            src[i] = tok < M ? (uint32_t)(tok * ldx + 8 * kc) * 2 : 0x80000000u;
-            dst[i] = tok * MID_XROW + 16 * kc;
-        }
-        u32x4 xr[2][MT * 4];
-#define MID_LOAD_X(b, step)                                                                                         \
-    _Pragma("unroll") for (int i = 0; i < MT * 4; ++i) xr[b][i] =                                                  \
-        __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(xb, src[i] + (uint32_t)(step) * 256u, 0, 0))
-        // macro-steps 0 and 1 go straight into their buffers
-        MID_LOAD_X(0, 0);
-        MID_LOAD_X(1, 1);
-#pragma unroll
-        for (int b = 0; b < 2; ++b)
-#pragma unroll
-            for (int i = 0; i < MT * 4; ++i) *(u32x4 *)(xs[b] + dst[i]) = xr[b][i];
-        MID_LOAD_X(0, 2);
-        MID_LOAD_X(1, 3);
-        lds_barrier();
-        // in iteration s: macro-step s + 2 goes into buffer (s + 2) % 3, the loads of s + 4 start
-        int buf = 2;
-        for (int s = 0; s < nst; s += 2) {
-#pragma unroll
-            for (int b = 0; b < 2; ++b) {
-                const int cur = s + b;
-                if (cur < nst) {
-#pragma unroll
-                    for (int i = 0; i < MT * 4; ++i) *(u32x4 *)(xs[buf] + dst[i]) = xr[b][i];
-                    MID_LOAD_X(b, cur + 4);
-                    buf = buf == MID_XBUFS - 1 ? 0 : buf + 1;
-                    lds_barrier();
-                }
-            }
-        }
-#undef MID_LOAD_X
+        mid_produce<MT, 0>(xs, X, ldx, M, s_begin, nst, lane);
         return;
+    }
+    if constexpr (MT > 4) {
+        if (wave == MID_CONSUMERS + 1) {
+            mid_produce<MT, 1>(xs, X, ldx, M, s_begin, nst, lane);
+            return;
+        }
     }
 
     // -------------------------------------------------------------------- consumers of W
@@ -161,7 +179,7 @@ gemm_mid_kernel(const bf16_t *__restrict__ X, int ldx, const bf16_t *__restrict_
             for (int i = grp; i < n_in; i += 4) scale_ss += p[i];
         }
     }
-    constexpr int MID_STAGES = MID_STAGE_TILES / NT;
+    constexpr int MID_STAGES = (MT > 4 && NT > 1 ? MID_STAGE_TILES * 3 / 4 : MID_STAGE_TILES) / NT;
     u32x4 w[MID_STAGES][NT][4];
 #define MID_LOAD_W(i, step)                                                                                     \
     _Pragma("unroll") for (int t = 0; t < NT; ++t) _Pragma("unroll") for (int j = 0; j < 4; ++j) w[i][t][j] =  \
@@ -181,17 +199,16 @@ gemm_mid_kernel(const bf16_t *__restrict__ X, int ldx, const bf16_t *__restrict_
         for (int i = 0; i < MID_STAGES; ++i) {
             const int cur = s + i;
             if (cur < nst) {
-                u32x4 xf[MT][4];
 #pragma unroll
-                for (int m = 0; m < MT; ++m)
+                for (int j = 0; j < 4; ++j) {
+                    u32x4 xf[MT];
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) xf[m][j] = *(const u32x4 *)(xs[buf] + x_off + 16 * m * MID_XROW + 16 * j);
-#pragma unroll
-                for (int j = 0; j < 4; ++j)
+                    for (int m = 0; m < MT; ++m) xf[m] = *(const u32x4 *)(xs + buf * BUF + x_off + 16 * m * MID_XROW + 16 * j);
 #pragma unroll
                     for (int t = 0; t < NT; ++t)
 #pragma unroll
-                        for (int m = 0; m < MT; ++m) acc[t][m] = mid_mfma(w[i][t][j], xf[m][j], acc[t][m]);
+                        for (int m = 0; m < MT; ++m) acc[t][m] = mid_mfma(w[i][t][j], xf[m], acc[t][m]);
+                }
                 MID_LOAD_W(i, cur + MID_STAGES);
                 buf = buf == MID_XBUFS - 1 ? 0 : buf + 1;
                 lds_barrier();
@@ -247,21 +264,39 @@ static int mid_launch(const void *X, int ldx, const void *W, int ldw, void *Y, i
     const int n_tiles = (EPI == MID_EPI_SWIGLU ? N / 2 : N) / 16;
     const int steps = K / 128, per = (steps + slices - 1) / slices;
     const dim3 grid((n_tiles + MID_CONSUMERS - 1) / MID_CONSUMERS, (steps + per - 1) / per);
-    const dim3 block((MID_CONSUMERS + 1) * WAVE);
-#define GO(MT_, P_) gemm_mid_kernel<NT, MT_, EPI, P_><<<grid, block, 0, stream>>>((const bf16_t *)X, ldx, (const bf16_t *)W, ldw, Y, ldy, M, N, K, per, sc.sumsq_in, sc.n_in, sc.norm_width, sc.eps)
-    if (M <= 32) {
-        if (packed) GO(2, true); else GO(2, false);
-    } else if (M <= 48) {
-        if (packed) GO(3, true); else GO(3, false);
-    } else {
-        if (packed) GO(4, true); else GO(4, false);
-    }
+    // the ring of 65 to 128 rows takes more LDS than a kernel has without asking
+#define GO(MT_, P_)                                                                                                         \
+    do {                                                                                                                    \
+        auto kernel = gemm_mid_kernel<NT, MT_, EPI, P_>;                                                                    \
+        if (mid_lds_bytes(MT_) > 64 * 1024) {                                                                               \
+            static bool asked = false;                                                                                      \
+            if (!asked) {                                                                                                   \
+                hipError_t e = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,      \
+                                                   mid_lds_bytes(MT_));                                                     \
+                if (e != hipSuccess) return (int)e;                                                                         \
+                asked = true;                                                                                               \
+            }                                                                                                               \
+        }                                                                                                                   \
+        kernel<<<grid, dim3((MID_CONSUMERS + mid_producers(MT_)) * WAVE), mid_lds_bytes(MT_), stream>>>(                    \
+            (const bf16_t *)X, ldx, (const bf16_t *)W, ldw, Y, ldy, M, N, K, per, sc.sumsq_in, sc.n_in, sc.norm_width, sc.eps); \
+    } while (0)
+#define GO_MT(MT_)                 \
+    do {                           \
+        if (packed) GO(MT_, true); \
+        else GO(MT_, false);       \
+    } while (0)
+    if (M <= 32) GO_MT(2);
+    else if (M <= 48) GO_MT(3);
+    else if (M <= 64) GO_MT(4);
+    else if (M <= 96) GO_MT(6);
+    else GO_MT(8);
+#undef GO_MT
 #undef GO
     LCU_LAUNCH_CHECK();
     return LCU_OK;
 }
 
-// X: [M, K] bfloat16 rows ldx apart, M <= 64; W: [N, K] bfloat16, rows ldw apart or packed; K a
+// X: [M, K] bfloat16 rows ldx apart, M <= 128 (rows that wait for their normalisation: M <= 64); W: [N, K] bfloat16, rows ldw apart or packed; K a
 // multiple of 128, N of 16 (SwiGLU: of 32; W holds N/2 gate rows, then N/2 up rows).
 // epilogue MID_EPI_BF16: Y [M, N] bfloat16 rows ldy apart (slices must be 1);
 //          MID_EPI_SWIGLU: Y [M, N/2] bfloat16 = silu(gate) * up (slices must be 1);
@@ -277,7 +312,7 @@ LCU_API int lcu_gemm_mid_planes(int K, int slices) {
 static int mid_bf16(const void *X, int ldx, const void *W, int ldw, void *Y, int ldy, int M, int N, int K, int epilogue,
                     int slices, int w_packed, const MidScale &sc, hipStream_t stream) {
     if (M <= 0 || N <= 0) return LCU_OK;
-    if (M > 64 || K <= 0 || K % 128 || N % 16 || ldx % 8 || ldx < K || slices <= 0 || slices > 64) return LCU_BAD_ARGUMENT;
+    if (M > 128 || (sc.sumsq_in && M > 64) || K <= 0 || K % 128 || N % 16 || ldx % 8 || ldx < K || slices <= 0 || slices > 64) return LCU_BAD_ARGUMENT;
     if (!w_packed && (ldw % 8 || ldw < K)) return LCU_BAD_ARGUMENT;
     if ((uintptr_t)X % 16 || (uintptr_t)W % 16 || (uintptr_t)Y % 16 || (uintptr_t)sc.sumsq_in % 16) return LCU_BAD_ARGUMENT;
     switch (epilogue) {

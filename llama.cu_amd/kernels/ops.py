@@ -567,11 +567,12 @@ def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = 
     return out
 
 
-MID_MAX_ROWS = 64
+MID_MAX_ROWS = 128
+MID_MAX_SCALED_ROWS = 64
 
 
 def mid_supported(x: torch.Tensor, w: torch.Tensor) -> bool:
-    """Whether ``gemm_mid`` takes these operands: up to 64 bfloat16 rows with K a multiple of 128
+    """Whether ``gemm_mid`` takes these operands: up to 128 bfloat16 rows with K a multiple of 128
     and a bfloat16 weight of a multiple of 16 rows."""
     return (x.is_cuda and w.is_cuda and x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and x.dim() == 2
             and w.dim() == 2 and 0 < x.shape[0] <= MID_MAX_ROWS and x.shape[1] == w.shape[1] and w.shape[1] % 128 == 0
@@ -589,7 +590,7 @@ def mid_planes(k: int, slices: int) -> int:
 def gemm_mid(x: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = None, swiglu: bool = False,
              slices: Optional[int] = None, packed: bool = False, row_sumsq: Optional[torch.Tensor] = None,
              norm_width: int = 0, eps: float = 0.0) -> torch.Tensor:
-    """``x @ w.T`` for 33 to 64 rows of bfloat16 ``x`` (it takes fewer too), streaming ``w`` once while
+    """``x @ w.T`` for 17 to 128 rows of bfloat16 ``x`` (it takes fewer too), streaming ``w`` once while
     the waves of a workgroup share ``x`` through LDS.  ``slices=None``: ``out [m, n]`` bfloat16
     (``swiglu``: ``w`` holds gate rows, then up rows, ``out [m, n/2] = silu(gate) * up``).
     ``slices=s``: K is cut into (at most) ``s`` slices and ``out [planes, m, n]`` float32 holds
@@ -623,8 +624,9 @@ def gemm_mid(x: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = Non
     lib = build.load("gemm_mid")
     if row_sumsq is not None:
         if row_sumsq.dtype != torch.float32 or row_sumsq.dim() != 2 or row_sumsq.shape[0] != m or not row_sumsq.is_contiguous() \
-                or norm_width <= 0 or row_sumsq.data_ptr() % 16:
-            raise KernelError("gemm_mid: row_sumsq must be a contiguous float32 [rows, parts] tensor, with the norm's width")
+                or norm_width <= 0 or row_sumsq.data_ptr() % 16 or m > MID_MAX_SCALED_ROWS:
+            raise KernelError(f"gemm_mid: row_sumsq must be a contiguous float32 [rows, parts] tensor, with the norm's width, "
+                              f"for at most {MID_MAX_SCALED_ROWS} rows")
         _check(lib.lcu_gemm_mid_bf16_scaled(_ptr(x), x.stride(0), _ptr(w), w.stride(0), _ptr(out), out.stride(-2), m, n, k, epi,
                                             slices or 1, int(packed), _ptr(row_sumsq), row_sumsq.shape[1], int(norm_width),
                                             ctypes.c_float(eps), _stream()), "gemm_mid (scaled rows)")

@@ -94,7 +94,7 @@ def linear_scaled(rows, weight: Union[torch.Tensor, Weight], out_dtype: Optional
 
 
 def _mid_slices(n_features: int, k: int) -> int:
-    """Into how many slices of K the kernel for 33 to 64 rows cuts a product, so that about one
+    """Into how many slices of K the kernel for 17 to 128 rows cuts a product, so that about one
     workgroup (64 features and a slice) stands on each of the 256 compute units; a slice keeps at
     least four macro-steps of 128."""
     groups = -(-n_features // 64)
@@ -102,10 +102,10 @@ def _mid_slices(n_features: int, k: int) -> int:
 
 
 def mid_takes(n_rows: int, weight: Union[torch.Tensor, Weight]) -> bool:
-    """Whether the kernel for 33 to 64 rows is the faster choice for this many bfloat16 rows and
+    """Whether the kernel for 17 to 128 rows is the faster choice for this many bfloat16 rows and
     this weight (measured against the library on the Llama-3-8B shapes: the products with few
-    output features, which are cut over K, 10 to 30 % faster with a packed weight, the down
-    projection with a plain one too).  Where the weight-streaming kernel is not chosen for a
+    output features, which are cut over K, 10 to 30 % faster with a packed weight at 64 rows and
+    more beyond, the down projection with a plain one too).  Where the weight-streaming kernel is not chosen for a
     long K (the down projection from 25 rows on) it takes those rows too: 24 against 32 us."""
     w, packed = _split(weight)
     fewest = ops.SKINNY_ROWS_PACKED if (packed is not None and w.dim() == 2 and w.shape[1] > 8192) else ops.SKINNY_ROWS_SHORT_K
