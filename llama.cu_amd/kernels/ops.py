@@ -391,15 +391,26 @@ def attention_prefill(q, out, cache, block_table, q_start, ctx_len, task_req, ta
 
 
 def decode_splits(n_req: int, n_heads: int, n_kv_heads: int, max_ctx_len: int) -> int:
-    """Into how many parts the decode kernel cuts each request's keys: about one workgroup
-    for each of the 256 compute units, no part shorter than 512 keys, at most 32 parts
+    """Into how many parts the decode kernel cuts each request's keys.  Few requests: about one
+    workgroup for each of the 256 compute units, no part shorter than 512 keys, at most 32 parts
     (measured on the Llama-3-8B shape from 2k to 128k keys: more parts cost more in the merge
-    than they gain; a single request with 128k keys wants 32).  The length counts rounded up
-    to a power of two, so that a growing context changes the choice, and with it the
-    rounding of the result and the captured graph that fits, only rarely."""
-    base = n_req * n_kv_heads * ((n_heads // n_kv_heads + 15) // 16)
+    than they gain; a single request with 128k keys wants 32).  Between half the chip's worth of
+    workgroups and all of it (17 to 31 requests of 8 key/value heads), where one part leaves
+    compute units idle and two parts are a wave and a bit: one part up to 4k keys (whole decode
+    steps with 2k keys gained nothing from more), beyond that up to 4 parts of at least 2048
+    keys, the fewest with which the workgroups fill whole waves of 256 about as well as any (20
+    requests are 160 workgroups: over 8k keys 161 us in one part, 118 in three, the whole step
+    8.7 against 7.9 ms).  From 256 workgroups on one part: the chip is full, and more parts
+    gained nothing (48 requests over 8k keys: 13.1 ms a step in one part, 13.2 in two).  The
+    length counts rounded up to a power of two, so that a growing context changes the choice, and
+    with it the rounding of the result and the captured graph that fits, only rarely."""
+    base = max(1, n_req * n_kv_heads * ((n_heads // n_kv_heads + 15) // 16))
     rounded = 1 << max(int(max_ctx_len) - 1, 0).bit_length()     # up to a power of two: the choice changes rarely
-    return max(1, min(32, 256 // max(base, 1), rounded // 512))
+    if base <= 128:
+        return max(1, min(32, 256 // base, rounded // 512))
+    most = min(4, rounded // 2048) if (rounded >= 8192 and base < 256) else 1
+    fill = [(base * s / 256) / -(-base * s // 256) for s in range(1, most + 1)]
+    return 1 + next(i for i, f in enumerate(fill) if f >= max(fill) - 0.07)
 
 
 def paged_attention(q: torch.Tensor, out: torch.Tensor, cache: torch.Tensor, step, group: int, n_heads: int,

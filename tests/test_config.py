@@ -128,3 +128,16 @@ def test_the_model_s_layout_holds_the_configuration_s_values_and_nothing_else():
         assert blk["ffn"].params == {"hidden_size": cfg.hidden_size, "intermediate_size": cfg.intermediate_size}
         assert spec.head.params["tied"] == cfg.tie_word_embeddings
         assert spec.final_norm.params["eps"] == cfg.rms_norm_eps
+
+
+def test_decode_attention_split_rule():
+    """Into how many parts the decode attention cuts a request's keys: few requests fill the chip's
+    256 compute units, many requests of long contexts fill whole waves of workgroups."""
+    import llama_cu_amd  # noqa: F401
+    from llama_cu_amd.kernels.ops import decode_splits
+    assert decode_splits(1, 32, 8, 2100) == 8 and decode_splits(8, 32, 8, 2100) == 4 and decode_splits(16, 32, 8, 2100) == 2
+    assert decode_splits(1, 32, 8, 100) == 1 and decode_splits(1, 32, 8, 200000) == 32
+    for b in (20, 24, 40, 48, 64, 128):
+        assert decode_splits(b, 32, 8, 2100) == 1            # up to 4k keys: one part
+    assert decode_splits(20, 32, 8, 8192) == 3 and decode_splits(48, 32, 8, 8192) == 1 and decode_splits(64, 32, 8, 8192) == 1
+    assert decode_splits(20, 32, 8, 4097) == 3 and decode_splits(20, 32, 8, 4096) == 1
