@@ -66,14 +66,16 @@ class SwiGLU(Part):
         else:
             gu = linear(h, self.w_gate_up, out_dtype=self.dtype)
             act = ops.swiglu(gu)
+        if planes_ok and act.dtype == torch.bfloat16 and mid_takes(act.shape[0], self.w_down):
+            # from 17 rows on the product cut over K and the norm kernel that adds its planes are faster
+            # than the weight-streaming product with that norm in its epilogue (30 against 35 us)
+            return linear_planes(act, self.w_down)
         if into is not None and act.dtype == torch.bfloat16 and skinny_takes(act.shape[0], self.w_down, preferred=True):
             # only where the kernel for few rows is the faster one for this product anyway
             residual, norm = into
             fused = linear_into_norm(act, self.w_down, residual, norm.weight)
             if fused is not None:
                 return ScaledRows(fused[0], fused[1], norm.size, norm.eps)
-        if planes_ok and act.dtype == torch.bfloat16 and mid_takes(act.shape[0], self.w_down):
-            return linear_planes(act, self.w_down)
         return linear(act, self.w_down, out_dtype=self.dtype)
 
 
