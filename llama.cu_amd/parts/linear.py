@@ -112,7 +112,9 @@ def mid_takes(n_rows: int, weight: Union[torch.Tensor, Weight]) -> bool:
     if not (fewest < n_rows <= ops.MID_MAX_ROWS and w.dtype == torch.bfloat16 and w.is_cuda and w.dim() == 2
             and w.shape[1] % 128 == 0 and w.shape[0] % 16 == 0):
         return False
-    return _mid_slices(w.shape[0], w.shape[1]) >= 3 and (packed is not None or w.shape[1] >= 8192)
+    # products that are not cut over K stay with the library; a plain weight only with a long K (measured: the
+    # output projections of the 8B and 70B shapes with plain weights are no faster than the library's)
+    return _mid_slices(w.shape[0], w.shape[1]) >= 2 and (packed is not None or w.shape[1] > 8192)
 
 
 def linear_planes(a: torch.Tensor, weight: Union[torch.Tensor, Weight]) -> torch.Tensor:
