@@ -105,8 +105,9 @@ def mid_takes(n_rows: int, weight: Union[torch.Tensor, Weight]) -> bool:
     """Whether the kernel for 17 to 128 rows is the faster choice for this many bfloat16 rows and
     this weight (measured against the library on the Llama-3-8B shapes: the products with few
     output features, which are cut over K, 10 to 30 % faster with a packed weight at 64 rows and
-    more beyond, the down projection with a plain one too).  A packed weight with a long K (the down projection) it takes
-    from 17 rows on: 24 us and 5 for the norm kernel against 33 to 40 of the weight-streaming kernel."""
+    more beyond, the down projection with a plain one too).  A packed weight with a long K (the
+    down projection) it takes from 17 rows on: 24 us and 5 for the norm kernel against 33 to 40 of
+    the weight-streaming kernel."""
     w, packed = _split(weight)
     fewest = ops.SKINNY_ROWS if (packed is not None and w.dim() == 2 and w.shape[1] > 8192) else ops.SKINNY_ROWS_SHORT_K
     if not (fewest < n_rows <= ops.MID_MAX_ROWS and w.dtype == torch.bfloat16 and w.is_cuda and w.dim() == 2
