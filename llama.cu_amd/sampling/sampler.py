@@ -34,6 +34,13 @@ def uniform(seed: int, request: int, index: int) -> float:
     return (h >> 40) / float(1 << 24)
 
 
+def _to_device(values, dtype: torch.dtype, device) -> torch.Tensor:
+    """Host values to the device without waiting for the GPU: through pinned memory, as a copy on the
+    current stream.  (A copy from pageable memory makes the host wait until the stream has reached it,
+    and an engine that runs ahead would stand still for a whole step.)"""
+    return torch.tensor(values, dtype=dtype, pin_memory=True).to(device, non_blocking=True)
+
+
 def argmax(logits: torch.Tensor) -> torch.Tensor:
     """The index of the largest logit of each row (the lowest among equals), int32."""
     _gpu(logits)
@@ -63,8 +70,8 @@ def sample_rows(logits: torch.Tensor, temperature: Sequence[float], top_p: Seque
     if any(not t > 0 for t in temperature) or any(not 0 <= x < 1 for x in u):
         raise KernelError("sample: temperatures must be > 0 and uniform numbers in [0, 1)")
     dev = logits.device
-    fl = torch.tensor([list(temperature), list(top_p), list(u)], dtype=torch.float32).to(dev)
-    kk = torch.tensor([min(int(k), vocab) for k in top_k], dtype=torch.int32).to(dev)
+    fl = _to_device([list(temperature), list(top_p), list(u)], torch.float32, dev)
+    kk = _to_device([min(int(k), vocab) for k in top_k], torch.int32, dev)
     out = torch.empty(rows, dtype=torch.int32, device=dev)
     lib = build.load("sampling")
     # a long row is cut into parts, one workgroup each: about one workgroup per compute unit in all
@@ -87,7 +94,7 @@ class Sampler:
                                [uniform(p.seed, k[0], k[1]) for p, k in zip(params, keys)])
         out = argmax(logits)
         if random_rows:
-            idx = torch.tensor(random_rows, dtype=torch.long).to(logits.device)
+            idx = _to_device(random_rows, torch.long, logits.device)
             sub = logits if len(random_rows) == logits.shape[0] else logits[idx]
             drawn = sample_rows(sub, [params[i].temperature for i in random_rows], [params[i].top_p for i in random_rows],
                                 [params[i].top_k for i in random_rows],
