@@ -86,6 +86,13 @@ def _stream() -> ctypes.c_void_p:
     return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
 
 
+def to_device(values, dtype: torch.dtype, device) -> torch.Tensor:
+    """Host values to the device without waiting for the GPU: through pinned memory, as a copy on the
+    current stream.  (A copy from pageable memory makes the host wait until the stream has reached it:
+    an engine that runs ahead of the GPU would stand still for a whole step.)"""
+    return torch.tensor(values, dtype=dtype, pin_memory=True).to(device, non_blocking=True)
+
+
 def _ptr(t: Optional[torch.Tensor]) -> ctypes.c_void_p:
     return ctypes.c_void_p(0 if t is None else t.data_ptr())
 
@@ -374,7 +381,7 @@ def prefill_tasks(q_lens, ctx_lens, tokens_per_task: int, device, pair: Optional
         tasks, per_wg = paired, 2
     if not tasks:
         return None, None, 0, 1
-    both = torch.tensor([[t[1] for t in tasks], [t[2] for t in tasks]], dtype=torch.int32).to(device)
+    both = to_device([[t[1] for t in tasks], [t[2] for t in tasks]], torch.int32, device)
     return both[0], both[1], len(tasks), per_wg
 
 
@@ -437,7 +444,7 @@ def paged_attention(q: torch.Tensor, out: torch.Tensor, cache: torch.Tensor, ste
         singles = [r for r, n in enumerate(step.q_lens) if n == 1]
         use_decode = len(singles) >= 1
         tasks = prefill_tasks(step.q_lens, step.ctx_lens, tpt, q.device, skip_single=use_decode)
-        req_list = torch.tensor(singles, dtype=torch.int32).to(q.device) if use_decode else None
+        req_list = to_device(singles, torch.int32, q.device) if use_decode else None
         max_ctx = max([step.ctx_lens[r] for r in singles], default=0)
         step.scratch[key] = (tasks, req_list, len(singles) if use_decode else 0, max_ctx)
     (task_req, task_tok0, n_tasks, per_wg), req_list, n_single, max_ctx = step.scratch[key]

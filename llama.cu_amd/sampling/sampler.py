@@ -12,7 +12,7 @@ from typing import List, Sequence, Tuple
 import torch
 
 from ..kernels import build
-from ..kernels.ops import KernelError, _check, _gpu, _ptr, _stream
+from ..kernels.ops import KernelError, _check, _gpu, _ptr, _stream, to_device as _to_device
 from .params import SamplingParams
 
 _MASK = (1 << 64) - 1
@@ -32,13 +32,6 @@ def uniform(seed: int, request: int, index: int) -> float:
     h = _splitmix64(h ^ (request & _MASK))
     h = _splitmix64(h ^ (index & _MASK))
     return (h >> 40) / float(1 << 24)
-
-
-def _to_device(values, dtype: torch.dtype, device) -> torch.Tensor:
-    """Host values to the device without waiting for the GPU: through pinned memory, as a copy on the
-    current stream.  (A copy from pageable memory makes the host wait until the stream has reached it,
-    and an engine that runs ahead would stand still for a whole step.)"""
-    return torch.tensor(values, dtype=dtype, pin_memory=True).to(device, non_blocking=True)
 
 
 def argmax(logits: torch.Tensor) -> torch.Tensor:
