@@ -163,6 +163,7 @@ def main() -> int:
                     help="tokens of each request's prompt (other context lengths than the default run's; the context "
                          "limit grows with it)")
     ap.add_argument("--dtype", choices=["bfloat16", "float32"], default="bfloat16")
+    ap.add_argument("--page-size", type=int, default=16, help="tokens in a page of the cache (a multiple of 16)")
     ap.add_argument("--no-points", action="store_true", help="skip decoding at batch 1 and 64 and the prefill")
     ap.add_argument("--only-prefill", action="store_true", help="time the 2048-token prefill alone (for profiles)")
     ap.add_argument("--prefill-history", type=int, default=0,
@@ -195,7 +196,7 @@ def main() -> int:
     elem = 2 if args.dtype == "bfloat16" else 4
     rng = random.Random(0)
     sync = torch.cuda.synchronize
-    page = 16
+    page = args.page_size
     biggest = max(args.batch, 1 if (args.no_points or args.only_prefill) else 64)
     # a request decodes while later ones still prefill: room for that too
     per_req = max(args.prompt_len, PROMPT_LEN) + grow
