@@ -1,4 +1,4 @@
-// Y[M, N] = X[M, K] * W[N, K]^T for few rows (decoding: M <= 64), bfloat16 operands,
+// Y[M, N] = X[M, K] * W[N, K]^T for few rows (decoding: M <= 32), bfloat16 operands,
 // 32-bit accumulation on the matrix cores.  The work is streaming W once from HBM, so
 // the kernel is laid out around W's loads:
 //
@@ -12,7 +12,7 @@
 //     of a row back to back;
 //   * a wave keeps the loads of several macro-steps in flight while it multiplies one;
 //   * v_mfma_f32_16x16x32_bf16 with A = W tile, B = X^T: the 16 columns are 16 tokens,
-//     MT such tiles for up to 64 tokens.
+//     MT such tiles for up to 32 tokens (more rows go to gemm_mid.hip, which shares them through LDS).
 // The waves' partial sums are added in LDS in a fixed order.
 //
 // W may also be given packed (lcu_pack_weight / the wrapper's pack_weight): the 16 x 128 block
@@ -382,7 +382,7 @@ static int launch_swiglu(const void *X, int ldx, const void *W, int ldw, void *Y
 
 // X: [M, K] bfloat16 rows ldx apart; W: [N, K] bfloat16 rows ldw apart; Y: [M, N] rows ldy
 // apart (for the SwiGLU epilogue [M, N/2]: W holds N/2 gate rows, then N/2 up rows).
-// M <= 64; K, ldx and ldw multiples of 8 (16-byte loads); tiles: output tiles of 16
+// M <= 32; K, ldx and ldw multiples of 8 (16-byte loads); tiles: output tiles of 16
 // features per workgroup (1, 2 or 4; more tiles reuse X more, fewer give more workgroups);
 // waves: 4 or 8 waves share a workgroup's K.
 static int skinny_bf16(const void *X, int ldx, const void *W, int ldw, void *Y, int ldy, int M, int N, int K, int epilogue,
@@ -390,7 +390,7 @@ static int skinny_bf16(const void *X, int ldx, const void *W, int ldw, void *Y, 
     if (M <= 0 || N <= 0) return LCU_OK;
     // a packed weight is whole blocks of 16 rows x 128 k (and for SwiGLU each half is)
     if (packed && (K % 128 || N % 16 || (epilogue == EPI_SWIGLU && N % 32))) return LCU_BAD_ARGUMENT;
-    if (M > 64 || K <= 0 || K % 8 || ldx % 8 || ldw % 8 || ldx < K || ldw < K) return LCU_BAD_ARGUMENT;
+    if (M > 32 || K <= 0 || K % 8 || ldx % 8 || ldw % 8 || ldx < K || ldw < K) return LCU_BAD_ARGUMENT;
     if (waves != 4 && waves != 8) return LCU_BAD_ARGUMENT;
     const int mt = (M + 15) / 16;
     if (epilogue == EPI_SWIGLU) {
@@ -402,25 +402,16 @@ static int skinny_bf16(const void *X, int ldx, const void *W, int ldw, void *Y, 
             if (mt == 1) SW(4, 1);
             SW(4, 2);
         }
-        switch (mt) {
-        case 1: SW(2, 1);
-        case 2: SW(2, 2);
-        case 3: SW(2, 3);
-        default: SW(2, 4);
-        }
+        if (mt == 1) SW(2, 1);
+        SW(2, 2);
 #undef SW
     }
     if (ldy < N) return LCU_BAD_ARGUMENT;
-    if (tiles == 4 && mt > 2) tiles = 2;      // 4 x 4 tiles of accumulators and operands do not fit the registers
 #define EP(NT_, MT_) return waves == 8 ? launch_epi<NT_, MT_, 8>(X, ldx, W, ldw, Y, ldy, M, N, K, epilogue, packed, ex, stream) \
                                        : launch_epi<NT_, MT_, 4>(X, ldx, W, ldw, Y, ldy, M, N, K, epilogue, packed, ex, stream)
 #define PICK(NT_)          \
-    switch (mt) {          \
-    case 1: EP(NT_, 1);    \
-    case 2: EP(NT_, 2);    \
-    case 3: EP(NT_, 3);    \
-    default: EP(NT_, 4);   \
-    }
+    if (mt == 1) EP(NT_, 1); \
+    EP(NT_, 2);
     if (tiles == 1) { PICK(1) }
     if (tiles == 2) { PICK(2) }
     if (tiles == 4) { PICK(4) }

@@ -457,7 +457,7 @@ def paged_attention(q: torch.Tensor, out: torch.Tensor, cache: torch.Tensor, ste
     return out
 
 
-SKINNY_MAX_ROWS = 64      # what the kernel takes
+SKINNY_MAX_ROWS = 32      # what the kernel takes
 SKINNY_ROWS = 16          # up to here it beats the library's product (measured on the Llama-3-8B shapes) ...
 SKINNY_ROWS_PACKED = 24   # ... and up to here when it reads a packed weight and its epilogues save the kernels around it
                           # (whole decode steps of the Llama-3-8B shape: +9 % at 17 rows, +4 % at 24)
@@ -475,7 +475,7 @@ _EPILOGUES = {"bf16": 0, "f32": 1, "add_f32": 2, "swiglu": 3}
 
 def skinny_supported(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype) -> bool:
     """Whether the weight-streaming kernel for few rows takes this product: bfloat16
-    operands, at most 64 rows, K a multiple of 8 (16-byte loads)."""
+    operands, at most 32 rows, K a multiple of 8 (16-byte loads)."""
     return (x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and x.dim() == 2 and w.dim() == 2
             and 0 < x.shape[0] <= SKINNY_MAX_ROWS and x.shape[1] % 8 == 0 and x.stride(1) == 1 and w.stride(1) == 1
             and x.stride(0) % 8 == 0 and w.stride(0) % 8 == 0 and out_dtype in (torch.bfloat16, torch.float32)
@@ -538,7 +538,7 @@ def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = 
                 tiles: Optional[int] = None, waves: Optional[int] = None,
                 row_sumsq: Optional[torch.Tensor] = None, norm_width: int = 0, eps: float = 0.0,
                 packed: bool = False) -> torch.Tensor:
-    """``out (+)= x @ w.T`` for at most 64 rows of bfloat16 ``x`` by streaming ``w`` once.
+    """``out (+)= x @ w.T`` for at most 32 rows of bfloat16 ``x`` by streaming ``w`` once.
     ``swiglu``: ``w`` holds gate rows, then up rows; ``out = silu(x @ gate.T) * (x @ up.T)``.
     ``row_sumsq [m, parts]``: the rows of ``x`` wait for their normalisation (see
     ``gemm_skinny_add_norm``); row ``i`` of the product is multiplied by

@@ -404,7 +404,7 @@ def test_attention_float32_result_does_not_depend_on_the_batch():
 
 
 # ------------------------------------------------------------------ weight-streaming product for few rows
-@pytest.mark.parametrize("m", [1, 8, 16, 17, 40, 64])
+@pytest.mark.parametrize("m", [1, 8, 16, 17, 25, 32])
 @pytest.mark.parametrize("n,k", [(16, 8), (100, 64), (301, 136), (1000, 4096), (4096, 1000)])
 @pytest.mark.parametrize("tiles", [1, 2, 4])
 def test_gemm_skinny(m, n, k, tiles):
@@ -420,7 +420,7 @@ def test_gemm_skinny(m, n, k, tiles):
     close(cg, c.double() + want, "float32", "accumulate")
 
 
-@pytest.mark.parametrize("m,di,k", [(1, 8, 16), (8, 172, 64), (33, 1000, 128), (64, 14336, 256)])
+@pytest.mark.parametrize("m,di,k", [(1, 8, 16), (8, 172, 64), (23, 1000, 128), (32, 14336, 256)])
 def test_gemm_skinny_swiglu(m, di, k):
     from llama_cu_amd.kernels import ops
     x = rnd(m, k, seed=m).to(torch.bfloat16)
@@ -431,7 +431,7 @@ def test_gemm_skinny_swiglu(m, di, k):
 
 def test_gemm_skinny_result_does_not_depend_on_the_batch():
     from llama_cu_amd.kernels import ops
-    x = rnd(40, 512, seed=1).to(torch.bfloat16).cuda()
+    x = rnd(30, 512, seed=1).to(torch.bfloat16).cuda()
     w = rnd(300, 512, seed=2).to(torch.bfloat16).cuda()
     whole = ops.gemm_skinny(x, w, out_dtype=torch.float32)
     one = ops.gemm_skinny(x[23:24], w, out_dtype=torch.float32)
@@ -445,7 +445,7 @@ def test_gemm_skinny_refuses_what_it_cannot_take():
     assert not ops.skinny_supported(x, w, torch.bfloat16)
     with pytest.raises(ops.KernelError):
         ops.gemm_skinny(x, w)
-    assert not ops.skinny_supported(rnd(65, 64).to(torch.bfloat16).cuda(), rnd(16, 64).to(torch.bfloat16).cuda(), torch.bfloat16)
+    assert not ops.skinny_supported(rnd(33, 64).to(torch.bfloat16).cuda(), rnd(16, 64).to(torch.bfloat16).cuda(), torch.bfloat16)
 
 
 # ------------------------------------------------------------------ product for 33 to 64 rows
