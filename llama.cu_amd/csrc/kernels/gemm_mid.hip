@@ -20,7 +20,9 @@
 //     output, [slice][M][N], and the kernel that follows (residual sum and norm) adds the planes
 //     in a fixed order.  Nothing is added atomically: results do not depend on timing.
 //
-// W is plain rows or packed as gemm_skinny.hip describes it (16 x 128 blocks of 4 KB).
+// W is plain rows or packed as gemm_skinny.hip describes it (16 x 128 blocks of 4 KB).  (The reference
+// gives every product to its vendor library, llama.cu/src/op/linear.rs:91-118; at these row counts the
+// library streams the weights at half of what HBM gives.)
 //
 // The rows of X may wait for their normalisation (sumsq_in not null: a factor per row,
 // rsqrt(sum of the row's shares / norm_width + eps), which commutes with the product): consumer
