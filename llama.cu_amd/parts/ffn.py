@@ -13,8 +13,8 @@ import torch
 
 from ..kernels import ops
 from .base import BuildContext, Part, ScaledRows, TensorSpec, register_part
-from .linear import (Weight, linear, linear_into_norm, linear_planes, linear_swiglu, linear_swiglu_mid, mid_swiglu_takes,
-                     mid_takes, skinny_row_limit, skinny_takes)
+from .linear import (Weight, library_friendly_rows, linear, linear_into_norm, linear_planes, linear_swiglu,
+                     linear_swiglu_mid, mid_swiglu_takes, mid_takes, skinny_row_limit, skinny_takes)
 
 
 class SwiGLU(Part):
@@ -33,7 +33,17 @@ class SwiGLU(Part):
         g, u = tensors["gate_proj.weight"], tensors["up_proj.weight"]
         if g.dtype != u.dtype:
             g, u = g.float(), u.float()
-        self.w_gate_up = Weight(torch.cat([g, u], dim=0), build)
+        both = torch.cat([g, u], dim=0)
+        rows = self.intermediate_size
+        if build.dtype == torch.bfloat16 and both.dtype == torch.bfloat16 and both.is_cuda:
+            rows = library_friendly_rows(self.intermediate_size, self.hidden_size, both.device)
+        if rows != self.intermediate_size:
+            # the plain copy, which the library multiplies, gets rows of zeros behind each half; the
+            # copy that the decode kernels stream does not
+            zeros = torch.zeros((rows - self.intermediate_size, self.hidden_size), dtype=both.dtype, device=both.device)
+            self.w_gate_up = Weight(torch.cat([g, zeros, u, zeros], dim=0), build, packed_from=both)
+        else:
+            self.w_gate_up = Weight(both, build)
         self.w_down = Weight(tensors["down_proj.weight"], build)
         self.dtype = build.dtype
 
@@ -66,6 +76,8 @@ class SwiGLU(Part):
         else:
             gu = linear(h, self.w_gate_up, out_dtype=self.dtype)
             act = ops.swiglu(gu)
+        if act.shape[1] != self.intermediate_size:
+            act = act[:, :self.intermediate_size]      # without what the rows of zeros gave
         if planes_ok and act.dtype == torch.bfloat16 and mid_takes(act.shape[0], self.w_down):
             # from 17 rows on the product cut over K and the norm kernel that adds its planes are faster
             # than the weight-streaming product with that norm in its epilogue (30 against 35 us)

@@ -55,6 +55,28 @@ def test_feed_forward_part(dtype):
         close(part.forward(h.cuda()), plain.feed_forward(w, "L.", h), dtype)
 
 
+@pytest.mark.parametrize("pack", [True, False])
+def test_feed_forward_with_rows_of_zeros_for_the_library(monkeypatch, pack):
+    """Where the library's product is faster with more output features, each half of the plain
+    gate/up matrix gets rows of zeros; the copy that the decode kernels stream does not, and what
+    the zeros give is left out before the down projection: few rows, 17 to 128 and many rows give
+    what the plain formula gives."""
+    import llama_cu_amd.parts.ffn as ffn
+    from llama_cu_amd.parts import BuildContext, PartSpec, make_part
+    monkeypatch.setattr(ffn, "library_friendly_rows", lambda di, d, device: di + 96)
+    part = make_part("ffn", PartSpec("swiglu", {"hidden_size": 128, "intermediate_size": 8288}))
+    t = random_part_tensors(part, 2, "bfloat16", std=0.05)
+    part.load(dict(t), BuildContext(torch.bfloat16, torch.device("cuda:0"), 512, 16, pack))
+    assert part.w_gate_up.plain.shape == (2 * (8288 + 96), 128)
+    assert (part.w_gate_up.packed is not None) == pack and (not pack or part.w_gate_up.packed.shape == (2 * 8288, 128))
+    w = {"L.mlp." + k: v.cpu() for k, v in t.items()}
+    for n in (3, 20, 70, 200):
+        h = rnd(n, 128, seed=n).to(torch.bfloat16)
+        got = part.forward(h.cuda())
+        assert got.shape == (n, 128)
+        close(got, plain.feed_forward(w, "L.", h), "bfloat16", f"{n} rows")
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("interleaved", [False, True])
 def test_attention_mixer_part_whole_prompt_then_decode(dtype, interleaved):
