@@ -111,6 +111,9 @@ def library_friendly_rows(di: int, d: int, device) -> int:
         return di                                   # small matrices: nothing to gain, and timings of a few us say nothing
     key = (di, d, str(device))
     if key not in _friendly_rows:
+        free, _ = torch.cuda.mem_get_info(device)
+        if free < 4 * (2 * (di + 4096) * d * 2):
+            return di                               # no room to try (and none to spare for rows of zeros)
         x = torch.randn(2048, d, device=device, dtype=torch.bfloat16)
         times = {}
         for rows in sorted({di} | {-(-di // m) * m for m in (1024, 2048, 4096)}):
