@@ -29,7 +29,12 @@ TINY_C = dict(architectures=["LlamaForCausalLM"], num_hidden_layers=1, hidden_si
               num_key_value_heads=2, head_dim=48, intermediate_size=100, vocab_size=301,
               max_position_embeddings=200, rope_theta=777.0, rms_norm_eps=1e-3, tie_word_embeddings=False,
               rope_interleaved=True)
-TINY = {"A": TINY_A, "B": TINY_B, "C": TINY_C}
+# sizes that the kernel for 17 to 128 rows takes (K a multiple of 128, a feed-forward wide enough to be cut over
+# K): whole steps and mixed steps of 33 to 128 rows leave planes of partial sums to the next norm
+TINY_D = dict(architectures=["LlamaForCausalLM"], num_hidden_layers=2, hidden_size=256, num_attention_heads=4,
+              num_key_value_heads=2, head_dim=64, intermediate_size=1024, vocab_size=500,
+              max_position_embeddings=256, rope_theta=10000.0, rms_norm_eps=1e-5, tie_word_embeddings=False)
+TINY = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D}
 
 
 def make_folder(cfg_dict: dict, seed: int, dtype: torch.dtype, std: float = 0.15, folder: Optional[str] = None) -> str:
