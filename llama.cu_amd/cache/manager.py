@@ -32,7 +32,8 @@ class CacheGroup:
 
 _STATUS = {1: "not enough free pages", 2: "no free state slot", -1: "unknown request", -2: "request exists already",
            -3: "bad argument", -4: "a window has already given back pages below that length",
-           -5: "the manager's tables are corrupt"}
+           -5: "the manager's tables are corrupt",
+           -6: "the model keeps per-request state that cannot be cut back"}
 
 _configured = False
 
@@ -53,13 +54,17 @@ def _ints(values: Sequence[int]):
 
 
 class CacheManager:
-    def __init__(self, groups: Sequence[CacheGroup], n_slots: int):
+    def __init__(self, groups: Sequence[CacheGroup], n_slots: int, can_truncate: bool = True):
+        """``can_truncate``: whether all that the model keeps for a request can be cut back to a
+        shorter length (pages can, a state of fixed size cannot); if not, ``truncate`` to less than
+        a request holds raises."""
         self.groups = list(groups)
+        self.can_truncate = bool(can_truncate)
         self.n_slots = int(n_slots)
         self._lib = _lib()
         self._h = ctypes.c_void_p(self._lib.lcu_cache_create(
             len(self.groups), _ints([g.num_pages for g in self.groups]), _ints([g.page_size for g in self.groups]),
-            _ints([g.window for g in self.groups]), self.n_slots))
+            _ints([g.window for g in self.groups]), self.n_slots, int(self.can_truncate)))
         if not self._h:
             raise CacheError("cache manager: bad group description")
 

@@ -11,14 +11,15 @@ using namespace lcu;
 
 #define API extern "C" __attribute__((visibility("default")))
 
-API void *lcu_cache_create(int n_groups, const int *num_pages, const int *page_size, const int *window, int n_slots) {
+API void *lcu_cache_create(int n_groups, const int *num_pages, const int *page_size, const int *window, int n_slots,
+                           int can_truncate) {
     std::vector<GroupDesc> g;
     for (int i = 0; i < n_groups; ++i) {
         if (num_pages[i] < 0 || page_size[i] <= 0 || window[i] < 0) return nullptr;
         g.push_back({num_pages[i], page_size[i], window[i]});
     }
     if (n_slots < 0) return nullptr;
-    return new CacheManager(g, n_slots);
+    return new CacheManager(g, n_slots, can_truncate != 0);
 }
 API void lcu_cache_destroy(void *h) { delete (CacheManager *)h; }
 API int lcu_cache_add(void *h, long long id) { return ((CacheManager *)h)->add(id); }

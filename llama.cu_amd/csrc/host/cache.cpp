@@ -24,7 +24,8 @@ bool PagePool::give(int page) {
     return true;
 }
 
-CacheManager::CacheManager(const std::vector<GroupDesc> &groups, int n_slots) : groups_(groups), n_slots_(n_slots) {
+CacheManager::CacheManager(const std::vector<GroupDesc> &groups, int n_slots, bool can_truncate)
+    : groups_(groups), n_slots_(n_slots), can_truncate_(can_truncate) {
     for (const auto &g : groups_) pools_.emplace_back(g.num_pages);
     for (int i = n_slots - 1; i >= 0; --i) free_slots_.push_back(i);
 }
@@ -109,6 +110,7 @@ int CacheManager::truncate(int64_t id, int new_len) {
     if (it == reqs_.end()) return CACHE_UNKNOWN_REQUEST;
     RequestCache &rc = it->second;
     if (new_len < 0 || new_len > rc.len) return CACHE_BAD_ARGUMENT;
+    if (new_len < rc.len && !can_truncate_) return CACHE_CANNOT_TRUNCATE;
     // a windowed group must still hold what the query at new_len will see
     for (size_t g = 0; g < groups_.size(); ++g) {
         const int w = groups_[g].window;

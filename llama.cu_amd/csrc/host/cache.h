@@ -52,11 +52,15 @@ enum CacheStatus {
     CACHE_BAD_ARGUMENT = -3,
     CACHE_WINDOW_PASSED = -4, // truncate below what a window has already given back
     CACHE_CORRUPT = -5,
+    CACHE_CANNOT_TRUNCATE = -6,   // the model keeps per-request state that cannot be cut back to a shorter length
 };
 
 class CacheManager {
   public:
-    CacheManager(const std::vector<GroupDesc> &groups, int n_slots);
+    // can_truncate: whether everything that the model keeps for a request can be cut back to a
+    // shorter length.  Pages can; a state of fixed size that has folded tokens in cannot, and
+    // then `truncate` to less than the request holds is refused.
+    CacheManager(const std::vector<GroupDesc> &groups, int n_slots, bool can_truncate = true);
 
     int add(int64_t id);                       // CACHE_OK and a slot taken, or an error
     int reserve(int64_t id, int new_len);      // pages for tokens [len, new_len) in every group, all or nothing
@@ -71,6 +75,7 @@ class CacheManager {
     int free_pages(int g) const { return pools_[g].free_count(); }
     int free_slots() const { return (int)free_slots_.size(); }
     int n_slots() const { return n_slots_; }
+    bool can_truncate() const { return can_truncate_; }
     int live_requests() const { return (int)reqs_.size(); }
     // pages that `reserve(id, new_len)` would take from group g
     int pages_needed(int64_t id, int g, int new_len) const;
@@ -94,6 +99,7 @@ class CacheManager {
     std::vector<PagePool> pools_;
     std::vector<int> free_slots_;
     int n_slots_;
+    bool can_truncate_;
     std::unordered_map<int64_t, RequestCache> reqs_;
 };
 

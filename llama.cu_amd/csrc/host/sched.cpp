@@ -223,7 +223,14 @@ int Scheduler::finish_now(int64_t id, int reason, int n_tokens) {
         r.tokens.resize(n_tokens);
         if (r.computed > n_tokens - 1) {
             r.computed = n_tokens - 1;
-            if (cache_->has(id) && cache_->get(id)->len > r.computed) cache_->truncate(id, r.computed);
+            if (cache_->has(id) && cache_->get(id)->len > r.computed && cache_->truncate(id, r.computed) != CACHE_OK) {
+                // What was computed beyond the end cannot be taken back: a window has given back a page
+                // that the shorter request would still see, or the model keeps a state that has folded
+                // the tokens in.  The request loses its cache; if it goes on (a kept request's next
+                // turn), it is computed again from its tokens.
+                cache_->release(id);
+                r.computed = 0;
+            }
         }
     }
     if (r.reason == NOT_FINISHED) finish(r, reason);

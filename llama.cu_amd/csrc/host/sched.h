@@ -76,7 +76,9 @@ class Scheduler {
     // End a request from outside (an end-of-sequence token learned late): its tokens are cut to
     // n_tokens (if that is not negative) and a kept cache to what precedes the last of them, as if
     // the request had ended when that token was appended.  A request that ended by count at the
-    // same token takes the new reason.
+    // same token takes the new reason.  Where the cache cannot be cut back (a window has passed a
+    // page that the shorter request would see, or the model keeps a state of fixed size), the
+    // request's cache is given back instead and a later turn computes it again from its tokens.
     int finish_now(int64_t id, int reason, int n_tokens);
 
     const SchedRequest *get(int64_t id) const;

@@ -675,7 +675,7 @@ attention_prefill_kernel(const bf16_t *__restrict__ q, int q_stride, bf16_t *__r
     // a workgroup takes tasks_per_wg tasks one after the other (the host pairs a long one with
     // a short one, so that workgroups take about equally long)
     for (int task = blockIdx.x * tasks_per_wg; task < (blockIdx.x + 1) * tasks_per_wg && task < n_tasks; ++task) {
-    __syncthreads();                               // the last task's use of LDS is over (and its copies have landed)
+    __syncthreads();                               // the last task's use of LDS is over (its copies landed before its merge)
     const int l16 = lane & 15, grp = lane >> 4;
     const int g = nh / nkvh;
     const int chunks = (g + 15) / 16;
@@ -740,7 +740,11 @@ attention_prefill_kernel(const bf16_t *__restrict__ q, int q_stride, bf16_t *__r
         fill = fill + 1 == PRE_RING ? 0 : fill + 1;
     }
     // ---- the second half hands its state to the first, which merges and writes
-    __syncthreads();                               // every copy has landed, every wave is done with the buffers
+    // The last copies into the ring (two double steps that nobody reads) may still be on their way: a
+    // barrier does not wait for a wave's copies from memory into LDS, and the states below overlay the
+    // ring.  So every wave waits for its own copies first; after the barrier none is in flight.
+    wait_loads<0>();
+    __syncthreads();                               // every wave is done with the buffers
     float *xch = (float *)lds_ring;                // [value][query wave][lane]
     constexpr int NV = QB * (2 + (DH / 16) * 4);
     if (half == 1) {

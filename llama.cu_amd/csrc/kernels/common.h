@@ -38,6 +38,17 @@ __device__ __forceinline__ uint32_t pack2_bf16(float lo, float hi) {
 
 constexpr int WAVE = 64;
 
+// The rotation of one pair (a, b) by an angle with cosine c and sine s, rounded the same way in
+// every kernel that rotates: one product rounded, the other fused into the sum, written out so
+// that the compiler has no choice of its own.  A token's rotated values then do not depend on
+// which kernel its batch was given to.
+__device__ inline void rotate_pair(float a, float b, float c, float s, float &ra, float &rb) {
+#pragma clang fp contract(off)
+    const float bs = b * s, bc = b * c;
+    ra = __builtin_fmaf(a, c, -bs);
+    rb = __builtin_fmaf(a, s, bc);
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, WAVE);

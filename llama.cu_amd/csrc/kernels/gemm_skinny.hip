@@ -260,11 +260,14 @@ gemm_skinny_kernel(const bf16_t *__restrict__ X, int ldx, const bf16_t *__restri
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int i = 16 * rope_c + 4 * grp + r;
-                float a = acc[0][m][r], b = acc[NT - 1][m][r];
+                // rounded to bfloat16 before the rotation, as the product's plain epilogue stores them for
+                // the rotation kernel: a token's query and key are the same bits whichever way they are made
+                float a = to_f32(from_f32<bf16_t>(acc[0][m][r])), b = to_f32(from_f32<bf16_t>(acc[NT - 1][m][r]));
                 if (is_q || is_k) {
                     float c = __uint_as_float(0x7fc00000u), sn = c;         // a position outside the table gives NaN
                     if (in_table) { c = ex.cos_t[(size_t)pos * half_dim + i]; sn = ex.sin_t[(size_t)pos * half_dim + i]; }
-                    const float ra = a * c - b * sn, rb = a * sn + b * c;
+                    float ra, rb;
+                    rotate_pair(a, b, c, sn, ra, rb);
                     a = ra; b = rb;
                 }
                 const bf16_t va = from_f32<bf16_t>(a), vb = from_f32<bf16_t>(b);

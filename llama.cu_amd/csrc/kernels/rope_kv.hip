@@ -11,16 +11,6 @@
 
 // One block per (token, head): query heads are rotated in place, key heads are rotated into
 // the cache, value heads are copied into the cache.
-// One rotation, rounded the same way in every kernel of this file: one product rounded, the
-// other fused into the sum, written out so that the compiler has no choice of its own.  A
-// token's rotated values then do not depend on which kernel its batch was given to.
-__device__ inline void rotate_pair(float a, float b, float c, float s, float &ra, float &rb) {
-#pragma clang fp contract(off)
-    const float bs = b * s, bc = b * c;
-    ra = __builtin_fmaf(a, c, -bs);
-    rb = __builtin_fmaf(a, s, bc);
-}
-
 template <class T>
 __global__ void rope_kv_store_kernel(T *__restrict__ qkv, int row_stride, const int *__restrict__ positions,
                                      const int *__restrict__ slots, const float *__restrict__ cos_t,

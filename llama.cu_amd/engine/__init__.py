@@ -1,5 +1,6 @@
 """The step function, the scheduler above it, and the engine that ties them to sampling."""
 from .batch import BatchBuilder, StepContext
-from .runner import LayerCache, ModelRunner
+from ..parts.base import LayerCache
+from .runner import ModelRunner
 
 __all__ = ["BatchBuilder", "StepContext", "LayerCache", "ModelRunner"]

@@ -17,24 +17,12 @@ import torch
 
 from ..cache import CacheGroup, CacheManager, OutOfPages
 from ..config import load_config
-from ..parts import BuildContext, DecoderModel, ModelSpec, PagedKV, SlotState
+from ..parts import BuildContext, CacheNeed, DecoderModel, LayerCache, ModelSpec
 from ..weights import load_weights, open_safetensors, random_tensors
 from .batch import BatchBuilder, StepContext
 
 DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "f32": torch.float32,
           "fp32": torch.float32, torch.bfloat16: torch.bfloat16, torch.float32: torch.float32}
-
-
-@dataclass
-class LayerCache:
-    """What one entry of the run order gets: the pages of its layer (``pages``,
-    ``[num_pages, 2, kv_heads * head_dim * page_size]``) with the group whose block tables
-    index them, whether the entry writes them, and/or its per-request state
-    (``state``, ``[slots, *shape]``)."""
-    group: int = -1
-    pages: Optional[torch.Tensor] = None
-    writes: bool = True
-    state: Optional[torch.Tensor] = None
 
 
 def require_gpu(device) -> torch.device:
@@ -70,38 +58,38 @@ class ModelRunner:
         build = BuildContext(self.dtype, self.device, spec.max_positions, self.page_size, self.pack_weights)
         self.model.load(tensors, build)
 
-        # cache groups: one per distinct window among the layers that page keys and values
+        # cache groups: one per distinct pool that the layers' needs name (for keys and values in pages:
+        # one per window); what a need is made of is the need's own business (parts.base.CacheNeed)
         needs = self.model.cache_needs()
-        windows = sorted({n.window for n in needs if isinstance(n, PagedKV)})
+        for i, need in enumerate(needs):
+            if need is not None and not isinstance(need, CacheNeed):
+                raise ValueError(f"run order entry {i}: {need!r} is no cache need (parts.base.CacheNeed)")
+        pools = sorted({n.pool() for n in needs if n is not None and n.pool() is not None})
+        elem = torch.empty(0, dtype=self.dtype).element_size()
         if num_pages is None and max_tokens is not None:
             num_pages = (int(max_tokens) + self.page_size - 1) // self.page_size
         if num_pages is None:
             # what the free memory holds, and no more than every slot filled to the limit
-            elem = torch.empty(0, dtype=self.dtype).element_size()
-            page_bytes = sum(2 * n.kv_heads * n.head_dim * self.page_size * elem for n in needs if isinstance(n, PagedKV))
+            page_bytes = sum(n.page_bytes(self.page_size, elem) for n in needs if n is not None)
             free, _ = torch.cuda.mem_get_info(self.device)
             by_memory = int(free * kv_fraction) // max(page_bytes, 1)
             by_need = self.max_seqs * ((self.max_model_len + self.page_size - 1) // self.page_size)
             num_pages = max(1, min(by_memory, by_need))
         self.num_pages = int(num_pages)
-        self.groups = [CacheGroup(self.num_pages, self.page_size, w) for w in windows]
-        self.cache = CacheManager(self.groups, self.max_seqs)
+        self.groups = [CacheGroup(self.num_pages, self.page_size, p[0]) for p in pools]
+        # a request's cache can be cut back to a shorter length only if every need's can
+        self.can_truncate = all(n.can_truncate for n in needs if n is not None)
+        self.cache = CacheManager(self.groups, self.max_seqs, can_truncate=self.can_truncate)
         self.caches: List[LayerCache] = []
         for i, (entry, need) in enumerate(zip(spec.run_order, needs)):
             if entry.cache_of is not None:
                 src = self.caches[entry.cache_of]
                 self.caches.append(LayerCache(group=src.group, pages=src.pages, writes=False, state=src.state))
-            elif isinstance(need, PagedKV):
-                pages = torch.zeros((self.num_pages, 2, need.kv_heads * need.head_dim * self.page_size),
-                                    dtype=self.dtype, device=self.device)
-                self.caches.append(LayerCache(group=windows.index(need.window), pages=pages))
-            elif isinstance(need, SlotState):
-                state = torch.zeros((self.max_seqs,) + tuple(need.shape), dtype=need.dtype, device=self.device)
-                self.caches.append(LayerCache(state=state))
             elif need is None:
                 self.caches.append(LayerCache())
             else:
-                raise ValueError(f"run order entry {i}: unknown cache need {need!r}")
+                group = pools.index(need.pool()) if need.pool() is not None else -1
+                self.caches.append(need.allocate(group, self.num_pages, self.page_size, self.max_seqs, self.dtype, self.device))
         max_pages = [(self.max_model_len + self.page_size - 1) // self.page_size for _ in self.groups]
         self.builder = BatchBuilder(self.cache, self.max_batch_tokens, self.max_seqs, max_pages, self.device)
         # captured decode steps, by batch size: (graph, its logits tensor)
@@ -195,12 +183,13 @@ class ModelRunner:
         return logits
 
     def _decode_splits(self, batch: int, max_ctx_len: int) -> int:
-        from ..kernels.ops import decode_splits
+        """Into how many parts the layers' mixers want a decoding request's keys cut (the most any of
+        them asks for; a mixer without keys asks for nothing)."""
         best = 1
-        for need in self.model.cache_needs():
-            if isinstance(need, PagedKV):
-                heads = getattr(self.model.layers[0].mixer, "heads", need.kv_heads)
-                best = max(best, decode_splits(batch, heads, need.kv_heads, max_ctx_len))
+        for layer in self.model.layers:
+            ask = getattr(layer, "decode_splits", None)
+            if callable(ask):
+                best = max(best, int(ask(batch, max_ctx_len)))
         return best
 
     def step(self, req_ids: Sequence[int], tokens: Sequence[Sequence[int]],

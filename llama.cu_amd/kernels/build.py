@@ -23,17 +23,18 @@ from typing import Dict, List
 _CSRC = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "csrc")
 _KERNEL_DIR = os.path.join(_CSRC, "kernels")
 _HOST_DIR = os.path.join(_CSRC, "host")
+_SHARED_DIR = os.path.join(_CSRC, "shared")       # headers that the host library and kernels both compile
 
 # packed 32-bit float instructions stay off for all device code
 HIP_FLAGS = ["-O3", "--offload-arch=gfx950", "-std=c++17", "-shared", "-fPIC",
              "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
              "-Wno-unused-command-line-argument"]
-HOST_FLAGS = ["-O2", "-std=c++17", "-shared", "-fPIC", "-Wall"]
+HOST_FLAGS = ["-O2", "-std=c++17", "-shared", "-fPIC", "-Wall", "-pthread", "-ffp-contract=off"]
 # extra flags for experiments (they enter the hash in the libraries' names)
 HIP_FLAGS += os.environ.get("LCU_HIP_FLAGS", "").split()
 
 KERNEL_LIBRARIES = ["elementwise", "rope_kv", "attention_generic", "attention_mfma", "gemm_generic", "gemm_skinny",
-                    "gemm_mid", "sampling"]
+                    "gemm_mid", "sampling", "random_fill"]
 HOST_LIBRARY = "host"
 
 _loaded: Dict[str, ctypes.CDLL] = {}
@@ -59,7 +60,7 @@ def _sources(name: str) -> List[str]:
 
 def _headers(name: str) -> List[str]:
     d = _HOST_DIR if name == HOST_LIBRARY else _KERNEL_DIR
-    return sorted(os.path.join(d, f) for f in os.listdir(d) if f.endswith(".h"))
+    return sorted(os.path.join(x, f) for x in (d, _SHARED_DIR) for f in os.listdir(x) if f.endswith(".h"))
 
 
 def _digest(name: str) -> str:

@@ -214,6 +214,18 @@ def feed_tokens(tokens: torch.Tensor, sampled: torch.Tensor, src: torch.Tensor, 
                                src.numel(), _stream()), "feed_tokens")
 
 
+def random_fill(out: torch.Tensor, key: int, std: float, shift: float = 0.0, first: int = 0) -> torch.Tensor:
+    """``out[i] = normal(key, first + i) * std + shift`` over the flattened ``out`` (float32 or bfloat16):
+    the counter-based generator that the host library has too (weights.random)."""
+    _gpu(out)
+    _contig(out, "random_fill out")
+    lib = build.load("random_fill")
+    _check(lib.lcu_random_fill(_ptr(out), _type(out, "random_fill out"), ctypes.c_longlong(out.numel()),
+                               ctypes.c_ulonglong(key & ((1 << 64) - 1)), ctypes.c_longlong(first), ctypes.c_float(std),
+                               ctypes.c_float(shift), _stream()), "random_fill")
+    return out
+
+
 # ------------------------------------------------------------------ rotation and cache write
 
 

@@ -49,6 +49,11 @@ class Attention(Part):
     def cache_need(self):
         return PagedKV(self.kv_heads, self.head_dim, self.window)
 
+    def decode_splits(self, batch: int, max_ctx_len: int) -> int:
+        """Into how many parts the decode kernel should cut each request's keys when ``batch``
+        requests decode over at most ``max_ctx_len`` keys (a captured graph fixes the number)."""
+        return ops.decode_splits(batch, self.heads, self.kv_heads, max_ctx_len)
+
     def load(self, tensors, build: BuildContext) -> None:
         if self.shares_kv:
             self.w_qkv = Weight(tensors["q_proj.weight"], build)

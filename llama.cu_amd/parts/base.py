@@ -72,19 +72,74 @@ class ModelSpec:
 # ------------------------------------------------------------------ cache needs
 
 
+@dataclass
+class LayerCache:
+    """What one entry of the run order gets: the pages of its layer (``pages``,
+    ``[num_pages, 2, kv_heads * head_dim * page_size]``) with the group whose block tables
+    index them, whether the entry writes them, and/or its per-request state
+    (``state``, ``[slots, *shape]``)."""
+    group: int = -1
+    pages: Optional[torch.Tensor] = None
+    writes: bool = True
+    state: Optional[torch.Tensor] = None
+
+
+class CacheNeed:
+    """What a mixer asks of the cache manager.  The engine knows no kind of need by name: it asks
+    every need these questions.
+
+    ``pool()``        None, or ``(window,)``: the need is pages of keys and values, and needs with
+                      an equal answer share one pool of page ids and one block table per request
+                      (``window`` 0: every token is kept; w: pages that a window of w tokens has
+                      passed are given back);
+    ``page_bytes(page_size, elem_size)``   bytes of one page of this need (0 if it has no pages);
+    ``allocate(group, num_pages, page_size, slots, dtype, device)``   the memory, as a LayerCache;
+    ``can_truncate``  whether what the need holds for a request can be cut back to a shorter
+                      length (pages can; a state that has folded tokens in cannot).  A request
+                      whose cache cannot be cut back and has to be (an end-of-sequence token
+                      learned after more was computed) loses its cache and is computed again from
+                      its tokens when it goes on.
+    """
+    can_truncate = True
+
+    def pool(self):
+        return None
+
+    def page_bytes(self, page_size: int, elem_size: int) -> int:
+        return 0
+
+    def allocate(self, group: int, num_pages: int, page_size: int, slots: int, dtype, device) -> LayerCache:
+        return LayerCache()
+
+
 @dataclass(frozen=True)
-class PagedKV:
+class PagedKV(CacheNeed):
     """Keys and values of every token (or of the last ``window`` tokens), in pages."""
     kv_heads: int
     head_dim: int
     window: int = 0          # 0: all tokens
 
+    def pool(self):
+        return (self.window,)
+
+    def page_bytes(self, page_size: int, elem_size: int) -> int:
+        return 2 * self.kv_heads * self.head_dim * page_size * elem_size
+
+    def allocate(self, group, num_pages, page_size, slots, dtype, device) -> LayerCache:
+        pages = torch.zeros((num_pages, 2, self.kv_heads * self.head_dim * page_size), dtype=dtype, device=device)
+        return LayerCache(group=group, pages=pages)
+
 
 @dataclass(frozen=True)
-class SlotState:
-    """A state of fixed size per request (``shape`` without the slot axis)."""
+class SlotState(CacheNeed):
+    """A state of fixed size per request (``shape`` without the slot axis).  The mixer that owns
+    it starts it anew when a request's first token (position 0) comes."""
     shape: Tuple[int, ...]
     dtype: torch.dtype = torch.float32
+    can_truncate = False
+
+    def allocate(self, group, num_pages, page_size, slots, dtype, device) -> LayerCache:
+        return LayerCache(state=torch.zeros((slots,) + tuple(self.shape), dtype=self.dtype, device=device))
 
 
 # ------------------------------------------------------------------ building

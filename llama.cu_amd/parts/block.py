@@ -46,6 +46,10 @@ class PreNormBlock(Part):
     def cache_need(self):
         return self.mixer.cache_need()
 
+    def decode_splits(self, batch: int, max_ctx_len: int) -> int:
+        ask = getattr(self.mixer, "decode_splits", None)
+        return int(ask(batch, max_ctx_len)) if callable(ask) else 1
+
     ends_in_next_norm = True     # forward takes ``next_norm``
     ends_in_planes = True        # forward takes ``planes_ok``
 

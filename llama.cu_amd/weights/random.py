@@ -1,10 +1,17 @@
 """Random weights from a configuration and a seed: matrices N(0, std), norm weights
-1 + N(0, std), each tensor from its own stream (seed and tensor name), so a tensor's
-values do not depend on which other tensors the model has.  The reference has no such
-mode; it exists so that the engine can be tested and measured without any file."""
+1 + N(0, std).  The reference has no such mode; it exists so that the engine can be tested
+against a plain implementation and measured without any file.
+
+One generator for the host and the GPU (csrc/shared/random_normal.h, compiled into the host
+library and into the kernel of csrc/kernels/random_fill.hip): element ``i`` of a tensor is a
+function of (seed, tensor name, i) alone, so a model that is made on the GPU from a seed is,
+bit for bit, the model that ``write_random_model`` writes to a folder from the same seed, and a
+tensor's values do not depend on which other tensors the model has.  Tensors are made under the
+names that files use, before anything is fused.
+"""
 from __future__ import annotations
 
-import hashlib
+import ctypes
 import json
 import os
 from typing import Dict
@@ -14,31 +21,68 @@ import torch
 from ..parts.base import TensorSpec
 from .safetensors_io import write_safetensors
 
+_MASK = (1 << 64) - 1
+_GOLDEN = 0x9E3779B97F4A7C15
 
-def _stream_seed(seed: int, name: str) -> int:
-    h = hashlib.sha256(f"{seed}:{name}".encode()).digest()
-    return int.from_bytes(h[:8], "little") & 0x7FFFFFFFFFFFFFFF
+
+def _mix64(z: int) -> int:
+    z &= _MASK
+    z ^= z >> 30
+    z = (z * 0xBF58476D1CE4E5B9) & _MASK
+    z ^= z >> 27
+    z = (z * 0x94D049BB133111EB) & _MASK
+    z ^= z >> 31
+    return z
+
+
+def _fnv1a64(text: str) -> int:
+    h = 0xCBF29CE484222325
+    for b in text.encode():
+        h = ((h ^ b) * 0x100000001B3) & _MASK
+    return h
+
+
+def stream_key(seed: int, name: str) -> int:
+    """The key of the stream of tensor ``name`` under ``seed``."""
+    return _mix64(_mix64(int(seed) & _MASK) ^ _fnv1a64(name))
+
+
+def fill_normal(out: torch.Tensor, key: int, std: float, shift: float = 0.0) -> torch.Tensor:
+    """``out[i] = normal(key, i) * std + shift`` over the flattened, contiguous tensor ``out``
+    (float32 or bfloat16), on the host or on the GPU: the same bits on both."""
+    if out.dtype not in (torch.float32, torch.bfloat16) or not out.is_contiguous():
+        raise ValueError("fill_normal: a contiguous float32 or bfloat16 tensor is needed")
+    if out.is_cuda:
+        from ..kernels import ops
+        return ops.random_fill(out, key, std, shift)
+    from ..kernels import build
+    lib = build.load(build.HOST_LIBRARY)
+    st = lib.lcu_random_fill_host(ctypes.c_void_p(out.data_ptr()), 0 if out.dtype == torch.float32 else 1,
+                                  ctypes.c_longlong(out.numel()), ctypes.c_ulonglong(key), ctypes.c_longlong(0),
+                                  ctypes.c_float(std), ctypes.c_float(shift), min(8, os.cpu_count() or 1))
+    if st:
+        raise ValueError(f"fill_normal: the host library refused its arguments ({st})")
+    return out
 
 
 def random_tensors(expected: Dict[str, TensorSpec], seed: int, dtype: torch.dtype = torch.bfloat16,
                    std: float = 0.02, device="cpu", vector_dtype=None) -> Dict[str, torch.Tensor]:
     """A tensor for every expected name that the random mode makes (a tied model gets no
-    output matrix).  ``vector_dtype`` (default: ``dtype``)
-    is the type of 1-d tensors (norm weights)."""
+    output matrix).  ``vector_dtype`` (default: ``dtype``) is the type of 1-d tensors (norm
+    weights).  Values are made in 32-bit and rounded once to the tensor's type."""
     out = {}
     dev = torch.device(device)
     for name, spec in expected.items():
         if not spec.random:
             continue
-        g = torch.Generator(device=dev).manual_seed(_stream_seed(seed, name))
         if spec.integer:
             out[name] = torch.zeros(spec.shape, dtype=torch.int32, device=dev)
             continue
-        t = torch.randn(spec.shape, generator=g, dtype=torch.float32, device=dev) * std
-        if spec.init == "one_plus_normal":
-            t = t + 1.0
         dt = (vector_dtype or dtype) if len(spec.shape) == 1 else dtype
-        out[name] = t.to(dt)
+        made = dt if dt in (torch.float32, torch.bfloat16) else torch.float32
+        t = torch.empty(spec.shape, dtype=made, device=dev)
+        fill_normal(t, stream_key(seed, name), std, 1.0 if spec.init == "one_plus_normal" else 0.0)
+        out[name] = t if made == dt else t.to(dt)
     return out
 
 

@@ -176,3 +176,15 @@ def test_random_orders_keep_the_invariants(seed):
     for r in list(live):
         m.release(r)
     assert m.free_pages(0) == 24 and m.free_pages(1) == 10 and m.free_slots() == 5
+
+
+def test_a_cache_with_state_that_cannot_be_cut_back_refuses_to_truncate():
+    m = CacheManager([CacheGroup(8, 16)], 2, can_truncate=False)
+    m.add(1); m.reserve(1, 40); m.commit(1)
+    m.reserve(1, 70)
+    m.truncate(1, 40)                      # giving back what was reserved and not written is no cut
+    assert m.length(1) == 40 and m.reserved(1) == 40 and m.free_pages() == 5
+    with pytest.raises(CacheError, match="cannot be cut back"):
+        m.truncate(1, 39)
+    assert m.length(1) == 40
+    m.check()

@@ -697,6 +697,34 @@ def test_gemm_skinny_q_k_v_with_rotation_and_cache_write(m, k, nh, nkv, dh, page
                                  2, 1, 48, page)
 
 
+@pytest.mark.parametrize("m", [1, 17, 32])
+@pytest.mark.parametrize("packed,scaled", [(False, False), (True, True)])
+def test_q_k_v_epilogue_leaves_the_same_bits_as_product_then_rotation_kernel(m, packed, scaled):
+    """A token's query and its key and value in the cache are the same bits whether the product's
+    epilogue rotates and stores them or the product stores bfloat16 rows and the rotation kernel
+    follows: both round the product to bfloat16 first and rotate with one formula."""
+    from llama_cu_amd.kernels import ops
+    from llama_cu_amd.parts.position import Rotary
+    k, nh, nkv, dh, page, max_pos, pages = 384, 6, 2, 64, 16, 500, 9
+    cos, sin = (torch.from_numpy(t).cuda() for t in Rotary(dh, 500000.0, max_pos).host_tables())
+    x = rnd(m, k, seed=m).to(torch.bfloat16).cuda()
+    w = rnd((nh + 2 * nkv) * dh, k, seed=5, scale=0.3).to(torch.bfloat16).cuda()
+    wg = ops.pack_weight(w) if packed else w
+    pos = torch.tensor(random.Random(3).sample(range(max_pos), m), dtype=torch.int32).cuda()
+    slots = torch.tensor(random.Random(4).sample(range(pages * page), m), dtype=torch.int32).cuda()
+    kw = {}
+    if scaled:
+        kw = dict(row_sumsq=(rnd(m, 3, seed=9).abs() * 40.0).cuda(), norm_width=k, eps=1e-5)
+    cache_a = torch.zeros((pages, 2, nkv * dh * page), dtype=torch.bfloat16).cuda()
+    cache_b = torch.zeros_like(cache_a)
+    q_a = ops.gemm_skinny_qkv_rope(x, wg, pos, slots, cos, sin, cache_a, nh, nkv, dh, page, packed=packed, **kw)
+    qkv = ops.gemm_skinny(x, wg, tiles=2, waves=8, packed=packed, **kw)
+    ops.rope_kv_store(qkv, pos, nh, nkv, dh, cos, sin, dh, 0, cache_b, slots, page)
+    assert torch.equal(q_a, qkv[:, :nh * dh])
+    assert torch.equal(cache_a, cache_b)
+    assert float(cache_a.float().abs().max()) > 0
+
+
 def test_gemm_skinny_add_norm_refuses_what_it_cannot_take():
     from llama_cu_amd.kernels import ops
     x = rnd(33, 64).to(torch.bfloat16).cuda()

@@ -426,3 +426,104 @@ def test_a_toy_routed_feed_forward_and_a_toy_position_encoding_are_registered_an
         got = common.collect(steps, outputs, 256)
         common.assert_matches_plain(got, want, "float32", "toy parts")
     runner.cache.check()
+
+
+def _engine_turns(engine, prompt, eos, more, steps):
+    """A kept request: one turn until the end-of-sequence token, then a turn with ``more``."""
+    from llama_cu_amd.sampling import GREEDY
+    engine.eos = {eos} if eos is not None else set()
+    rid = engine.add_request(prompt, GREEDY, steps, keep=True, ignore_eos=eos is None)
+    turns = []
+    for turn in range(2):
+        toks, why = [], None
+        while not engine.idle:
+            for o in engine.step():
+                if o.token is not None:
+                    toks.append(o.token)
+                why = o.finished or why
+        turns.append((toks, why))
+        if turn == 0:
+            engine.continue_request(rid, more, steps)
+    engine.drop(rid)
+    engine.runner.cache.check()
+    assert engine.runner.cache.free_slots() == engine.runner.max_seqs
+    assert all(engine.runner.cache.free_pages(g) == engine.runner.num_pages for g in range(len(engine.runner.groups)))
+    return turns
+
+
+@pytest.mark.parametrize("kind", ["state", "window"])
+def test_an_end_learned_late_with_a_cache_that_cannot_be_cut_back(kind):
+    """A toy mixer that folds every token into a state of fixed size, and an attention layer whose
+    window of 4 tokens gives a page back with every fourth token, each in layer 1 of Tiny A, through
+    the engine that runs ahead: when the end-of-sequence token is learned, one token more has gone
+    into the state (or the window has passed a page that the shorter request would see).  The kept
+    request's next turn must continue as if that token had never been computed: the tokens of the
+    engine that runs ahead equal those of the engine that works in turn, and both equal a request
+    that is given the whole context at once."""
+    import llama_cu_amd
+    from llama_cu_amd.config import LlamaConfig
+    from llama_cu_amd.engine.engine import Engine
+    from llama_cu_amd.models.llama import llama_spec
+    from llama_cu_amd.parts import Part, PartSpec, SlotState, TensorSpec, register_part
+
+    class DecayingSum(Part):
+        """state <- 0.5 state + h; out = state @ W (a state that cannot be cut back)."""
+        def __init__(self, hidden_size):
+            self.d = hidden_size
+
+        def tensors(self):
+            return {"mix.weight": TensorSpec((self.d, self.d))}
+
+        def cache_need(self):
+            return SlotState((self.d,), torch.float32)
+
+        def load(self, tensors, build):
+            self.w = tensors["mix.weight"].float()
+
+        def forward(self, h, step, cache):
+            out = torch.empty_like(h)
+            start = 0
+            for r, n in enumerate(step.q_lens):
+                slot = step.state_slots[r]
+                if step.ctx_lens[r] - n == 0:
+                    cache.state[slot].zero_()
+                st = cache.state[slot].clone()
+                for i in range(n):
+                    st = 0.5 * st + h[start + i].float()
+                    out[start + i] = (st @ self.w.T).to(h.dtype)
+                cache.state[slot] = st
+                start += n
+            return out
+
+    register_part("mixer", "decaying_sum", DecayingSum, replace=True)
+    spec = llama_spec(LlamaConfig.from_dict(dict(common.TINY_A)))
+    if kind == "state":
+        spec.layers[1].params["mixer"] = PartSpec("decaying_sum", {"hidden_size": 64}, "toy")
+    else:
+        spec.layers[1].params["mixer"].params["window"] = 4
+    prompt = list(common.random_requests(256, [9], seed=3).values())[0]
+    more = [7, 8, 9]
+
+    def engine(run_ahead):
+        runner, _ = runner_for(spec, 4, "float32", max_tokens=256, max_seqs=2, page_size=8)
+        assert runner.can_truncate == (kind == "window")
+        return Engine(runner, run_ahead=run_ahead)
+
+    probe = _engine_turns(engine(False), prompt, None, more, 10)[0][0]
+    assert len(probe) == 10
+    # every place of the end-of-sequence token among the first tokens: with pages of 8 and a window
+    # of 4 some of them fall on the step that gives a page back
+    for at in range(1, 8):
+        eos = probe[at]
+        if eos in probe[:at]:
+            continue
+        want = _engine_turns(engine(False), prompt, eos, more, 10)
+        assert want[0] == (probe[:at + 1], "eos")
+        e = engine(True)
+        got = _engine_turns(e, prompt, eos, more, 10)
+        assert got == want, f"end-of-sequence token at {at}"
+        # the second turn is what a fresh request with the whole context generates
+        fresh = engine(False)
+        whole = fresh.generate([prompt + probe[:at + 1] + more], max_steps=len(want[1][0]), ignore_eos=True)[0]
+        stop = want[1][0].index(eos) + 1 if eos in want[1][0] else len(want[1][0])
+        assert want[1][0][:stop] == whole[:stop]

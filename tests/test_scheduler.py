@@ -260,3 +260,48 @@ def test_an_end_by_count_at_the_same_token_takes_the_late_reason():
     assert s.finish(0, "eos", 4) == "eos" and s.info(0).reason == "eos"
     cache.check()
     assert cache.free_pages(0) == 64
+
+
+def test_an_end_learned_late_at_a_windows_edge_gives_the_cache_back_and_the_next_turn_recomputes():
+    """Window 4, pages of 4: once token 7 is in the cache, page 0 is given back (the next query, at
+    8, sees keys 5..8).  If the request is then cut back to 6 tokens, the next query, at 6, would
+    see keys 3..6, and key 3 lay in page 0, which is gone.  The scheduler then gives the whole
+    cache back and a later turn starts at token 0."""
+    cache = CacheManager([CacheGroup(16, 4, window=4)], 4)
+    s = Scheduler(cache, 4, 64, 32, 512)
+    s.add(0, list(range(6)), 10, keep=True)
+    run_round(s, next_token=lambda req, n: 0)            # tokens 0..5 computed, placeholder 6
+    run_round(s, next_token=lambda req, n: 0)            # token 6 computed, placeholder 7
+    run_round(s, next_token=lambda req, n: 0)            # token 7 computed: page 0 is given back
+    assert cache.length(0) == 8 and cache.table(0)[0] == -1
+    # the token at index 6 was the end of the sequence: 7 tokens remain, 6 of them in the cache
+    assert s.finish(0, "eos", 7) == "eos"
+    assert not cache.has(0) and s.info(0).computed == 0
+    assert cache.free_pages(0) == 16
+    cache.check()
+    s.extend(0, [5, 6], 3)
+    plan = s.plan()
+    assert [(e.req, e.start, e.count) for e in plan] == [(0, 0, 9)]
+    s.commit()
+    s.abort(0); s.drop(0)
+    cache.check()
+
+
+def test_an_end_learned_late_with_state_that_cannot_be_cut_back_recomputes_the_next_turn():
+    cache = CacheManager([CacheGroup(16, 4)], 4, can_truncate=False)
+    s = Scheduler(cache, 4, 64, 32, 512)
+    s.add(0, list(range(7)), 10, keep=True)
+    s.add(1, list(range(3)), 2, keep=True)
+    run_round(s, next_token=lambda req, n: 0)
+    run_round(s, next_token=lambda req, n: 0)
+    run_round(s, next_token=lambda req, n: 0)
+    assert cache.length(0) == 9
+    assert s.finish(0, "eos", 8) == "eos"                 # one token computed beyond the end
+    assert not cache.has(0) and s.info(0).computed == 0
+    # request 1 ended by count with nothing computed beyond its end: its cache stays
+    assert s.info(1).reason == "max_steps" and cache.has(1) and cache.length(1) == 4
+    s.extend(0, [5], 2)
+    s.extend(1, [5], 2)
+    plan = s.plan()
+    assert sorted((e.req, e.start, e.count) for e in plan) == [(0, 0, 9), (1, 4, 2)]
+    cache.check()
