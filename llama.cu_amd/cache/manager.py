@@ -143,6 +143,14 @@ class CacheManager:
                 return list(buf[:n])
             cap = n
 
+    def page_owners(self, group: int = 0) -> List[int]:
+        """For every page of ``group`` the request that holds it, -1 for a free page."""
+        n = self.groups[group].num_pages
+        buf = (ctypes.c_longlong * max(n, 1))()
+        if self._lib.lcu_cache_page_owners(self._h, group, buf, n) != n:
+            raise CacheError(f"page owners of group {group}: unknown group")
+        return list(buf[:n])
+
     def check(self) -> None:
         """Raise if a page or slot is lost, held twice, or both free and held."""
         why = ctypes.create_string_buffer(256)

@@ -13,74 +13,97 @@ from typing import List, Optional
 
 
 def _base(p: argparse.ArgumentParser) -> None:
-    p.add_argument("model", metavar="MODEL", help="model folder (config.json, model.safetensors[, tokenizer.json])")
+    p.add_argument("model", metavar="MODEL", help="model folder (config.json, model.safetensors[, tokenizer.json]); with "
+                   "--random-weights a folder that holds config.json, or a config.json itself, is enough")
     p.add_argument("--max-steps", type=int, default=1000, help="most tokens to generate (default 1000)")
     p.add_argument("--dtype", choices=["bfloat16", "float32"], default="bfloat16")
+    p.add_argument("--random-weights", type=int, default=None, metavar="SEED",
+                   help="make the weights from SEED on the GPU instead of reading model.safetensors")
     p.add_argument("--temperature", type=float, default=0.0)
     p.add_argument("--top-p", type=float, default=1.0)
     p.add_argument("--top-k", type=int, default=None)
     p.add_argument("--seed", type=int, default=0)
-    p.add_argument("--max-tokens", type=int, default=None, help="size of the cache pool in tokens (default: from free memory)")
+    p.add_argument("--page-size", type=int, default=16, help="tokens per page of the cache (default 16)")
+    p.add_argument("--num-pages", type=int, default=None, help="pages in the cache pool (default: from free memory)")
+    p.add_argument("--max-tokens", type=int, default=None, help="size of the cache pool in tokens, instead of --num-pages")
+    p.add_argument("--max-seqs", type=int, default=4, help="most requests that run at a time (default 4)")
+
+
+def model_folder(path: str) -> str:
+    """The folder of MODEL: MODEL itself, or the folder of a config.json that was named."""
+    import os
+    return os.path.dirname(os.path.abspath(path)) if os.path.isfile(path) else path
 
 
 def _engine(args):
+    from . import models  # noqa: F401  (registers the architectures)
     from . import text
+    from .config import load_config
     from .engine.engine import Engine
     from .sampling import SamplingParams, TOP_K_ALL
-    kw = {}
-    if args.max_tokens:
+    kw = dict(page_size=args.page_size, max_seqs=args.max_seqs)
+    if args.num_pages:
+        kw["num_pages"] = args.num_pages
+    elif args.max_tokens:
         kw["max_tokens"] = args.max_tokens
+    folder = model_folder(args.model)
     t0 = time.time()
-    engine = Engine.from_folder(args.model, dtype=args.dtype, max_seqs=4, **kw)
+    if args.random_weights is not None:
+        _, cfg = load_config(folder)
+        engine = Engine.from_config(cfg, args.random_weights, dtype=args.dtype, **kw)
+    else:
+        engine = Engine.from_folder(folder, dtype=args.dtype, **kw)
     print(f"[info] model ready in {time.time() - t0:.2f} s", file=sys.stderr)
     params = SamplingParams(args.temperature, args.top_p, args.top_k or TOP_K_ALL, args.seed)
-    tok = text.load_tokenizer(args.model, engine.runner.spec.vocab_size)
-    return engine, params, tok
+    tok = text.load_tokenizer(folder, engine.runner.spec.vocab_size)
+    return engine, params, tok, folder
 
 
 def _stream(engine, rid: int, decoder, out=sys.stdout):
-    """Run rounds until request ``rid`` ends; print its text as it comes.  Returns (time of
-    the first round, time of the later rounds, tokens)."""
-    prefill = decode = 0.0
+    """Run rounds until request ``rid`` ends; print its text as it comes.  Returns (prefill,
+    decode, tokens) as the reference counts them (llama.cu/xtask/src/generate.rs:41-52): prefill
+    is the time until the first token has been received, decode all the time after that.  The
+    engine runs ahead, so a call of ``step`` returns the tokens of the round before the one it
+    launches; the clock therefore runs over calls, not per call."""
+    start = time.time()
+    first_at = None
     ntoks = 0
-    first = True
     while True:
-        t = time.time()
         results = engine.step()
-        dt = time.time() - t
-        if first:
-            prefill, first = dt, False
-        else:
-            decode += dt
         done = False
         for o in results:
             if o.req != rid:
                 continue
             if o.token is not None:
+                if first_at is None:
+                    first_at = time.time()
                 ntoks += 1
                 out.write(decoder.push(o.token))
                 out.flush()
             done = done or o.finished is not None
         if done or engine.idle:
-            return prefill, decode, ntoks
+            end = time.time()
+            if first_at is None:
+                first_at = end
+            return first_at - start, end - first_at, ntoks
 
 
 def generate(args) -> int:
     """llama.cu/xtask/src/generate.rs:16-69: echo the prompt, stream the continuation, then
     report prefill time, decode time, tokens, time per token and tokens per second."""
     from . import text
-    engine, params, tok = _engine(args)
+    engine, params, tok, folder = _engine(args)
     prompt = args.prompt if args.prompt is not None else "Once upon a time,"
     sys.stdout.write(prompt)
     sys.stdout.flush()
     if args.use_template:
-        prompt = text.load_chat_template(args.model).render([text.user(prompt)])
+        prompt = text.load_chat_template(folder).render([text.user(prompt)])
     rid = engine.add_request(tok.encode(prompt), params, args.max_steps)
     prefill, decode, ntoks = _stream(engine, rid, text.StreamDecoder(tok))
     print()
     print(f"[info] prefill = {prefill * 1e3:.2f} ms, decode = {decode * 1e3:.2f} ms", file=sys.stderr)
-    if ntoks > 1 and decode > 0:
-        per = decode / (ntoks - 1)
+    if ntoks > 0 and decode > 0:
+        per = decode / ntoks              # as the reference: over all tokens, the first included (generate.rs:63)
         print(f"[info] n toks = {ntoks}, perf: {per * 1e3:.3f} ms/tok, {1 / per:.1f} tok/s", file=sys.stderr)
     return 0
 
@@ -88,8 +111,8 @@ def generate(args) -> int:
 def chat(args) -> int:
     """llama.cu/xtask/src/chat/mod.rs:38-77: one session whose cache lives across turns."""
     from . import text
-    engine, params, tok = _engine(args)
-    template = text.load_chat_template(args.model)
+    engine, params, tok, folder = _engine(args)
+    template = text.load_chat_template(folder)
     rid: Optional[int] = None
     while True:
         line = ""

@@ -59,6 +59,15 @@ API int lcu_cache_fill_batch(void *h, int n_req, const long long *ids, const int
     return ((CacheManager *)h)->fill_batch(n_req, (const int64_t *)ids, n_new, positions, req_of_token, q_start,
                                            ctx_len, state_slot, block_tables, max_pages, slots);
 }
+// owners[p] = the request that holds page p of group g, -1 if it is free; returns the number of
+// pages of the group (-1 for a bad group, and nothing is written if cap is too small).
+API int lcu_cache_page_owners(void *h, int g, long long *owners, int cap) {
+    CacheManager *m = (CacheManager *)h;
+    if (g < 0 || g >= m->n_groups()) return -1;
+    const int n = m->group(g).num_pages;
+    if (n <= cap) m->page_owners(g, (int64_t *)owners);
+    return n;
+}
 API int lcu_cache_check(void *h, char *why, int cap) {
     std::string w;
     const int st = ((CacheManager *)h)->check(&w);

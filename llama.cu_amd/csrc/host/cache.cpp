@@ -179,6 +179,13 @@ int CacheManager::fill_batch(int n_req, const int64_t *ids, const int *n_new, in
     return CACHE_OK;
 }
 
+void CacheManager::page_owners(int g, int64_t *owners) const {
+    for (int p = 0; p < pools_[g].size(); ++p) owners[p] = -1;
+    for (const auto &kv : reqs_)
+        for (int p : kv.second.tables[g])
+            if (p >= 0 && p < pools_[g].size()) owners[p] = kv.first;
+}
+
 int CacheManager::check(std::string *why) const {
     auto fail = [&](const std::string &m) {
         if (why) *why = m;

@@ -90,6 +90,10 @@ class CacheManager {
                    int *q_start, int *ctx_len, int *state_slot, int *const *block_tables, const int *max_pages,
                    int *const *slots) const;
 
+    // owners[p] = the request that holds page p of group g, or -1 for a free page (owners has
+    // room for the group's pages).
+    void page_owners(int g, int64_t *owners) const;
+
     // Every page is free or held by exactly one table entry; every slot likewise.
     int check(std::string *why = nullptr) const;
 

@@ -19,6 +19,7 @@ from ..cache import CacheGroup, CacheManager, OutOfPages
 from ..config import load_config
 from ..parts import BuildContext, CacheNeed, DecoderModel, LayerCache, ModelSpec
 from ..weights import load_weights, open_safetensors, random_tensors
+from ..weights.loader import convert
 from .batch import BatchBuilder, StepContext
 
 DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "f32": torch.float32,
@@ -37,7 +38,8 @@ class ModelRunner:
     def __init__(self, spec: ModelSpec, tensors: Dict[str, torch.Tensor], dtype, device="cuda:0",
                  page_size: int = 16, max_tokens: Optional[int] = None, num_pages: Optional[int] = None,
                  max_seqs: int = 8, max_batch_tokens: int = 2048, max_model_len: Optional[int] = None,
-                 kv_fraction: float = 0.85, use_graphs: bool = True, pack_weights: Optional[bool] = None):
+                 kv_fraction: float = 0.85, use_graphs: bool = True, pack_weights: Optional[bool] = None,
+                 poison_freed: bool = False):
         self.device = require_gpu(device)
         self.dtype = DTYPES[dtype]
         self.spec = spec
@@ -92,6 +94,10 @@ class ModelRunner:
                 self.caches.append(need.allocate(group, self.num_pages, self.page_size, self.max_seqs, self.dtype, self.device))
         max_pages = [(self.max_model_len + self.page_size - 1) // self.page_size for _ in self.groups]
         self.builder = BatchBuilder(self.cache, self.max_batch_tokens, self.max_seqs, max_pages, self.device)
+        # a debugging aid: pages that were given back, or went to another request, since the last step are
+        # filled with NaN before the step runs, so that a read of memory that its request does not own shows
+        self.poison_freed = bool(poison_freed)
+        self._owners: Optional[List[List[int]]] = None
         # captured decode steps, by batch size: (graph, its logits tensor)
         self.use_graphs = bool(use_graphs) and self.model.graph_safe
         self._graphs: Dict[tuple, Any] = {}        # (batch size, key parts) -> (graph, its logits)
@@ -112,13 +118,19 @@ class ModelRunner:
         return runner
 
     @classmethod
-    def from_config(cls, cfg, seed: int, dtype="bfloat16", device="cuda:0", std: float = 0.02, **kw) -> "ModelRunner":
-        """Random weights made on the device (nothing is written or read)."""
+    def from_config(cls, cfg, seed: int, dtype="bfloat16", device="cuda:0", std: float = 0.02, stored=None,
+                    **kw) -> "ModelRunner":
+        """Random weights made on the device from ``seed`` (nothing is written or read): bit for
+        bit the weights that ``write_random_model`` writes for the same seed.  ``stored``: the
+        type that a file would hold them in, if not the compute type (``"bfloat16"`` with the
+        float32 compute type gives the float32 engine weights that bfloat16 holds exactly)."""
         from .. import models  # noqa: F401
         from ..config import architecture_of
         device = require_gpu(device)
         spec = architecture_of(cfg.to_dict()).build_spec(cfg)
-        tensors = random_tensors(DecoderModel(spec).tensors(), seed, dtype=DTYPES[dtype], std=std, device=device)
+        expected = DecoderModel(spec).tensors()
+        tensors = random_tensors(expected, seed, dtype=DTYPES[stored or dtype], std=std, device=device)
+        tensors = {n: convert(t, expected[n], DTYPES[dtype]) for n, t in tensors.items()}
         runner = cls(spec, tensors, dtype, device, **kw)
         runner.config = cfg
         return runner
@@ -148,7 +160,26 @@ class ModelRunner:
             for rid in added:
                 self.cache.release(rid)
             raise
+        if self.poison_freed:
+            self._poison_pages_that_changed_hands()
         return self.builder.build(req_ids, tokens, want, self.spec.vocab_size, feed)
+
+    def _poison_pages_that_changed_hands(self) -> None:
+        """Called when a step's pages are reserved and nothing of it has run: every page that a request
+        held at the last call and that is free now, or another request's (who has written nothing to it
+        yet), is filled with NaN."""
+        now = [self.cache.page_owners(g) for g in range(len(self.groups))]
+        before, self._owners = self._owners, now
+        if before is None:
+            return
+        for g in range(len(self.groups)):
+            gone = [p for p, (a, b) in enumerate(zip(before[g], now[g])) if a >= 0 and a != b]
+            if not gone:
+                continue
+            index = torch.tensor(gone, dtype=torch.long, device=self.device)
+            for c in self.caches:
+                if c.group == g and c.writes and c.pages is not None:
+                    c.pages.index_fill_(0, index, float("nan"))
 
     GRAPH_AFTER = 2          # a batch size is captured when it comes for the third time
     GRAPH_MAX_BATCH = 256

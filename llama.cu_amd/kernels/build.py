@@ -23,6 +23,7 @@ from typing import Dict, List
 _CSRC = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "csrc")
 _KERNEL_DIR = os.path.join(_CSRC, "kernels")
 _HOST_DIR = os.path.join(_CSRC, "host")
+_REF_DIR = os.path.join(_CSRC, "ref")               # plain C++ references of the kernels, part of the host library
 _SHARED_DIR = os.path.join(_CSRC, "shared")       # headers that the host library and kernels both compile
 
 # packed 32-bit float instructions stay off for all device code
@@ -51,7 +52,7 @@ def _say(msg: str) -> None:
 
 def _sources(name: str) -> List[str]:
     if name == HOST_LIBRARY:
-        return sorted(os.path.join(_HOST_DIR, f) for f in os.listdir(_HOST_DIR) if f.endswith(".cpp"))
+        return sorted(os.path.join(d, f) for d in (_HOST_DIR, _REF_DIR) for f in os.listdir(d) if f.endswith(".cpp"))
     path = os.path.join(_KERNEL_DIR, name + ".hip")
     if not os.path.isfile(path):
         raise BuildError(f"no kernel source {path}")

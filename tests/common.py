@@ -67,29 +67,36 @@ def ceil64(n: int) -> int:
     return (n + 63) // 64 * 64
 
 
-def trace_whole(reqs):
+def _want(name, first, n, keep):
+    """The places among tokens first .. first + n - 1 of request ``name`` whose logits are wanted:
+    all, or those whose position ``keep(name, position)`` accepts."""
+    return [k for k in range(n) if keep is None or keep(name, first + k)]
+
+
+def trace_whole(reqs, keep=None):
     """Each request alone and whole: one step with all its tokens, all logits wanted."""
     steps = []
     for name, toks in reqs.items():
-        steps.append({"step": len(steps), "entries": [{"id": name, "tokens": toks, "want": list(range(len(toks)))}],
+        steps.append({"step": len(steps), "entries": [{"id": name, "tokens": toks, "want": _want(name, 0, len(toks), keep)}],
                       "end": [name]})
     return steps, max(ceil64(len(t)) for t in reqs.values())
 
 
-def trace_tail_decode(reqs, tail=32):
+def trace_tail_decode(reqs, tail=32, keep=None):
     """Most of a request in one step, its last ``tail`` tokens one by one."""
     steps = []
     for name, toks in reqs.items():
         head = max(len(toks) - tail, 0)
         if head:
-            steps.append({"step": len(steps), "entries": [{"id": name, "tokens": toks[:head], "want": list(range(head))}], "end": []})
+            steps.append({"step": len(steps), "entries": [{"id": name, "tokens": toks[:head], "want": _want(name, 0, head, keep)}],
+                          "end": []})
         for i in range(head, len(toks)):
-            steps.append({"step": len(steps), "entries": [{"id": name, "tokens": [toks[i]], "want": [0]}],
+            steps.append({"step": len(steps), "entries": [{"id": name, "tokens": [toks[i]], "want": _want(name, i, 1, keep)}],
                           "end": [name] if i == len(toks) - 1 else []})
     return steps, max(ceil64(len(t)) for t in reqs.values())
 
 
-def trace_portions(reqs, sizes=(7, 2, 16, 3, 48, 2, 1, 33, 5, 2)):
+def trace_portions(reqs, sizes=(7, 2, 16, 3, 48, 2, 1, 33, 5, 2), keep=None):
     """Portions of changing size, down to two tokens (and one), across page edges."""
     steps = []
     k = 0
@@ -98,16 +105,17 @@ def trace_portions(reqs, sizes=(7, 2, 16, 3, 48, 2, 1, 33, 5, 2)):
         while fed < len(toks):
             n = min(sizes[k % len(sizes)], len(toks) - fed)
             k += 1
-            steps.append({"step": len(steps), "entries": [{"id": name, "tokens": toks[fed:fed + n], "want": list(range(n))}],
+            steps.append({"step": len(steps), "entries": [{"id": name, "tokens": toks[fed:fed + n], "want": _want(name, fed, n, keep)}],
                           "end": [name] if fed + n == len(toks) else []})
             fed += n
     return steps, max(ceil64(len(t)) for t in reqs.values())
 
 
-def trace_mixed(reqs, seed=0, max_live=4, tail=12):
+def trace_mixed(reqs, seed=0, max_live=4, tail=12, sizes=(2, 2, 3, 5, 7, 16, 17, 31, 48), keep=None, preempt=0.0):
     """Up to ``max_live`` requests at a time: portions of some beside single tokens of
-    others; requests sit steps out; finished requests' pages go to the next ones.  Returns
-    the steps and the smallest ``--max-tokens`` that holds them."""
+    others; requests sit steps out; finished requests' pages go to the next ones.  ``preempt``:
+    the chance per step that one live request loses its pages (it is computed again when it next
+    appears).  Returns the steps and the smallest ``--max-tokens`` that holds them."""
     rng = random.Random(seed)
     pending = list(reqs.items())
     live: Dict[str, int] = {}
@@ -127,20 +135,23 @@ def trace_mixed(reqs, seed=0, max_live=4, tail=12):
             if remaining <= tail:
                 n = 1
             else:
-                n = min(remaining - tail, rng.choice([2, 2, 3, 5, 7, 16, 17, 31, 48]))
-            entries.append({"id": name, "tokens": toks[fed:fed + n], "want": list(range(n))})
+                n = min(remaining - tail, rng.choice(list(sizes)))
+            entries.append({"id": name, "tokens": toks[fed:fed + n], "want": _want(name, fed, n, keep)})
             live[name] = fed + n
         if not entries:
             name = names[0]
             toks, fed = reqs[name], live[name]
-            entries.append({"id": name, "tokens": toks[fed:fed + 1], "want": [0]})
+            entries.append({"id": name, "tokens": toks[fed:fed + 1], "want": _want(name, fed, 1, keep)})
             live[name] = fed + 1
         need = max(need, sum(ceil64(v) for v in live.values()))
         for name in list(live):
             if live[name] == len(reqs[name]):
                 end.append(name)
                 del live[name]
-        steps.append({"step": len(steps), "entries": entries, "end": end})
+        step = {"step": len(steps), "entries": entries, "end": end}
+        if preempt and live and rng.random() < preempt:
+            step["preempt"] = [rng.choice(sorted(live))]
+        steps.append(step)
     return steps, need
 
 
@@ -162,11 +173,15 @@ def collect(steps, outputs: Dict[int, np.ndarray], vocab: int) -> Dict[str, Dict
     return got
 
 
-def run_trace_inprocess(folder: str, dtype: str, steps, max_tokens: int) -> Dict[int, np.ndarray]:
+def run_trace_inprocess(folder: str, dtype: str, steps, max_tokens: int, stats: Optional[dict] = None, **kw) -> Dict[int, np.ndarray]:
+    """Replay in this process.  Pages that are given back are filled with NaN, so a read of memory
+    that no live request owns shows.  ``stats``: takes ``pages_used_again`` (pages that more than
+    one request held) and ``mixed_steps`` (steps with a portion of several tokens beside a single
+    token)."""
     sys.path.insert(0, ROOT)
     import llama_cu_amd  # noqa: F401
     from llama_cu_amd.engine.trace import TraceReplayer
-    rep = TraceReplayer(folder, dtype, max_tokens)
+    rep = TraceReplayer.open(folder, dtype, max_tokens, poison_freed=True, **kw)
     outputs = {}
     for st in steps:
         out = rep.step(st)
@@ -175,15 +190,18 @@ def run_trace_inprocess(folder: str, dtype: str, steps, max_tokens: int) -> Dict
     rep.runner.cache.check()
     assert rep.runner.cache.live_requests() == 0
     assert rep.runner.cache.free_pages(0) == rep.runner.num_pages
+    if stats is not None:
+        stats["pages_used_again"] = rep.pages_used_again(0)
+        stats["mixed_steps"] = rep.mixed_steps
     return outputs
 
 
-def run_trace_program(folder: str, dtype: str, steps, max_tokens: int, vocab: int) -> Dict[int, np.ndarray]:
+def run_trace_program(folder: str, dtype: str, steps, max_tokens: int, vocab: int, extra: Sequence[str] = ()) -> Dict[int, np.ndarray]:
     """Through ``bin/trace_run`` as a user runs it."""
     out_dir = tempfile.mkdtemp(prefix="lcu_trace_")
     text = "".join(json.dumps(s) + "\n" for s in steps)
     proc = subprocess.run([os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", dtype, "--out", out_dir,
-                           "--max-tokens", str(max_tokens)], input=text, capture_output=True, text=True, timeout=600)
+                           "--max-tokens", str(max_tokens)] + list(extra), input=text, capture_output=True, text=True, timeout=600)
     assert proc.returncode == 0, proc.stderr[-2000:]
     done = [l for l in proc.stdout.splitlines() if l.startswith("done ")]
     assert done == [f"done {s['step']}" for s in steps]

@@ -89,15 +89,16 @@ def rope(x: torch.Tensor, pos: Sequence[int], sin: torch.Tensor, cos: torch.Tens
     n, heads, dh = x.shape
     half = dh // 2
     out = torch.empty_like(x)
+    # pair i is (x[2i], x[2i+1]) or (x[i], x[i + half])
+    ia = [2 * i if pairing == "adjacent" else i for i in range(half)]
+    ib = [2 * i + 1 if pairing == "adjacent" else i + half for i in range(half)]
     for t in range(n):
         s = sin[int(pos[t])]
         c = cos[int(pos[t])]
-        for i in range(half):
-            ia, ib = (2 * i, 2 * i + 1) if pairing == "adjacent" else (i, i + half)
-            a = x[t, :, ia]
-            b = x[t, :, ib]
-            out[t, :, ia] = a * c[i] - b * s[i]
-            out[t, :, ib] = a * s[i] + b * c[i]
+        a = x[t][:, ia]                    # [heads, half]: the first element of every pair
+        b = x[t][:, ib]
+        out[t][:, ia] = a * c - b * s
+        out[t][:, ib] = a * s + b * c
     return out
 
 
@@ -211,8 +212,11 @@ def feed_forward(w: Dict[str, torch.Tensor], prefix: str, x2: torch.Tensor) -> t
     return linear(swiglu(gate, up), w[prefix + "mlp.down_proj.weight"])
 
 
-def forward(cfg: PlainConfig, w: Dict[str, torch.Tensor], tokens: Sequence[int]) -> torch.Tensor:
-    """Logits ``[n, vocab]`` at every position of one whole sequence that starts at 0.
+def forward(cfg: PlainConfig, w: Dict[str, torch.Tensor], tokens: Sequence[int],
+            logits_at: Optional[Sequence[int]] = None) -> torch.Tensor:
+    """Logits ``[n, vocab]`` at every position of one whole sequence that starts at 0
+    (``logits_at``: at these positions only, ``[len(logits_at), vocab]``: the output selects
+    its rows before the final norm, llama.cu/src/exec/output_head.rs:74-78).
 
     Block: ``x += attn(norm1(x)); x += ffn(norm2(x))``
     (llama.cu/src/model/mod.rs:100-157: ``TransformerBlk::new(norm, attention, norm, mlp)``,
@@ -238,6 +242,8 @@ def forward(cfg: PlainConfig, w: Dict[str, torch.Tensor], tokens: Sequence[int])
         kept.append(made[0] if cache_of is None else None)
         x2 = rms_norm(x, w[p + "post_attention_layernorm.weight"], cfg.rms_norm_eps)
         x = x + feed_forward(w, p, x2)
+    if logits_at is not None:
+        x = x[list(logits_at)]
     y = rms_norm(x, w["model.norm.weight"], cfg.rms_norm_eps)
     head = w["model.embed_tokens.weight"] if (cfg.tie_word_embeddings or "lm_head.weight" not in w) \
         else w["lm_head.weight"]

@@ -114,7 +114,7 @@ def test_generate_command_line(folder_a):
     """``generate MODEL --max-steps N -p PROMPT`` prints the prompt, then the continuation."""
     root = common.ROOT
     proc = subprocess.run([os.path.join(root, "bin", "llama.cu_amd"), "generate", folder_a, "--max-steps", "8",
-                           "-p", "Hi there", "--dtype", "float32", "--max-tokens", "256"],
+                           "-p", "Hi there", "--dtype", "float32", "--num-pages", "16", "--max-seqs", "2"],
                           capture_output=True, timeout=300)
     assert proc.returncode == 0, proc.stderr.decode()[-2000:]
     assert proc.stdout.startswith(b"Hi there")
@@ -124,6 +124,53 @@ def test_generate_command_line(folder_a):
     shown = bytes(t for t in want if t < 256).decode("utf-8", errors="replace")
     # the byte tokenizer shows what decodes; compare what is printable
     assert proc.stdout[len(b"Hi there"):].decode("utf-8", errors="replace").rstrip("\n").replace("�", "") == shown.replace("�", "")
+
+
+def test_generate_reports_the_time_to_the_first_token_as_prefill(folder_b):
+    """The report of ``generate`` as the reference counts it (llama.cu/xtask/src/generate.rs:41-52):
+    prefill is the time until the first token has been received, decode the time after it.  With a
+    prompt of 200 tokens in 32-bit and 3 generated tokens the prefill takes longer than a decode
+    step; an engine that runs ahead and times its calls would report the opposite."""
+    import io
+    from llama_cu_amd import cli, text
+    from llama_cu_amd.engine.engine import Engine
+    prompt = list(common.random_requests(384, [200], seed=4).values())[0]
+    engine = Engine.from_folder(folder_b, dtype="float32", max_tokens=512, max_seqs=2, use_graphs=False)
+    engine.generate([prompt[:5]], max_steps=3, ignore_eos=True)          # everything is built and loaded
+    rid = engine.add_request(prompt, max_steps=24, ignore_eos=True)
+    out = io.StringIO()
+    prefill, decode, ntoks = cli._stream(engine, rid, text.StreamDecoder(text.ByteTokenizer(384)), out=out)
+    assert ntoks == 24
+    assert prefill > 0 and decode > 0
+    assert prefill > decode / 23, (prefill, decode)                      # more than one decode step
+
+
+def test_chat_command_two_turns_over_stdin(folder_b):
+    """``chat MODEL``: two user lines over standard input; the session's cache lives across the
+    turns (llama.cu/xtask/src/chat/mod.rs:38-77), so the second answer is what the plain
+    implementation generates from the whole conversation so far."""
+    from llama_cu_amd import text
+    root = common.ROOT
+    lines = ["Hi", "And then?"]
+    proc = subprocess.run([os.path.join(root, "bin", "llama.cu_amd"), "chat", folder_b, "--max-steps", "6",
+                           "--dtype", "float32", "--max-tokens", "256", "--max-seqs", "2", "--page-size", "32"],
+                          input="".join(l + "\n" for l in lines).encode(), capture_output=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr.decode()[-2000:]
+    shown = proc.stdout.decode("utf-8", errors="replace")
+    assert shown.count("user> ") == 3 and shown.count("assistant> ") == 2 and shown.count("=== over ===") == 2
+    cfg, w = plain.load_folder(folder_b)
+    template = text.load_chat_template(folder_b)
+    tok = text.ByteTokenizer(384)
+    context, answers = [], []
+    for line in lines:
+        context += tok.encode(template.render([text.user(line)]))
+        reply = plain.greedy_generate(cfg, w, context, 6)
+        answers.append(reply)
+        context += reply
+    got = shown.split("assistant> ")[1:]
+    for reply, part in zip(answers, got):
+        want = bytes(t for t in reply if t < 256).decode("utf-8", errors="replace").replace("�", "")
+        assert part.split("\n=== over ===")[0].replace("�", "") == want
 
 
 def test_smoke_entry():

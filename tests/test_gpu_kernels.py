@@ -779,3 +779,36 @@ def test_feed_tokens():
     ops.feed_tokens(got2, sampled.cuda(), torch.tensor([9, -1, 2], dtype=torch.int32).cuda(),
                     torch.tensor([0, 1, 37], dtype=torch.int32).cuda())
     assert torch.equal(got2.cpu(), tokens)
+
+
+# ------------------------------------------------------------------ random weights
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_random_weights_are_the_same_bits_on_the_host_and_on_the_gpu(dtype):
+    """One generator for both: every tensor of Tiny B and one matrix of the Llama-3-8B shape
+    (4096 x 14336) made on the GPU equal, bit for bit, the ones made on the host from the same
+    seed; other names and other seeds give other streams."""
+    import common
+    from llama_cu_amd.config import LlamaConfig
+    from llama_cu_amd.models.llama import llama_spec
+    from llama_cu_amd.parts import DecoderModel, TensorSpec
+    from llama_cu_amd.weights import fill_normal, random_tensors, stream_key
+    expected = DecoderModel(llama_spec(LlamaConfig.from_dict(common.TINY_B))).tensors()
+    host = random_tensors(expected, 11, dtype=DT[dtype], device="cpu")
+    dev = random_tensors(expected, 11, dtype=DT[dtype], device="cuda")
+    assert set(host) == set(dev) and len(host) > 20
+    for name in host:
+        assert torch.equal(host[name], dev[name].cpu()), name
+    other = random_tensors(expected, 12, dtype=DT[dtype], device="cuda")
+    assert not torch.equal(other["model.norm.weight"], dev["model.norm.weight"])
+    assert not torch.equal(dev["model.layers.0.mlp.up_proj.weight"], dev["model.layers.0.mlp.gate_proj.weight"])
+    big = {"model.layers.31.mlp.down_proj.weight": TensorSpec((4096, 14336))}
+    h = random_tensors(big, 3, dtype=DT[dtype], device="cpu")["model.layers.31.mlp.down_proj.weight"]
+    g = random_tensors(big, 3, dtype=DT[dtype], device="cuda")["model.layers.31.mlp.down_proj.weight"]
+    assert torch.equal(h, g.cpu())
+    assert abs(float(h.float().std()) - 0.02) < 1e-4 and abs(float(h.float().mean())) < 1e-4
+    # a part of a stream made alone
+    from llama_cu_amd.kernels import ops
+    key = stream_key(3, "x")
+    whole = fill_normal(torch.empty(5000, dtype=DT[dtype]), key, 1.0)
+    part = ops.random_fill(torch.empty(777, dtype=DT[dtype], device="cuda"), key, 1.0, first=1234)
+    assert torch.equal(part.cpu(), whole[1234:1234 + 777])

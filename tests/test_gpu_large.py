@@ -17,21 +17,117 @@ SHAPE = dict(architectures=["LlamaForCausalLM"], num_hidden_layers=2, hidden_siz
              max_position_embeddings=8192, rope_theta=500000.0, rms_norm_eps=1e-5, tie_word_embeddings=False)
 
 
+SEED = 41
+
+
+def config():
+    from llama_cu_amd.config import LlamaConfig
+    return LlamaConfig.from_dict(SHAPE)
+
+
+def host_weights():
+    """The weights of seed SEED as a bfloat16 file would hold them, made on the host.  The engine
+    makes its own on the GPU from the same seed (the same bits, as the kernels' tests show); with
+    ``stored="bfloat16"`` the 32-bit engine gets the same values widened, so that one plain
+    computation serves both compute types."""
+    from llama_cu_amd.models.llama import llama_spec
+    from llama_cu_amd.parts import DecoderModel
+    from llama_cu_amd.weights import random_tensors
+    return random_tensors(DecoderModel(llama_spec(config())).tensors(), SEED, dtype=torch.bfloat16, device="cpu")
+
+
+def runner_for(dtype, **kw):
+    from llama_cu_amd.engine.runner import ModelRunner
+    return ModelRunner.from_config(config(), SEED, dtype=dtype, stored="bfloat16", **kw)
+
+
 @pytest.fixture(scope="module")
 def big():
-    out = {}
     reqs = common.random_requests(SHAPE["vocab_size"], [70, 33], seed=3)
-    for dtype, tdt, std in (("float32", torch.float32, 0.02), ("bfloat16", torch.bfloat16, 0.02)):
-        folder = common.make_folder(SHAPE, seed=41, dtype=tdt, std=std)
-        out[dtype] = (folder, reqs, common.plain_logits(folder, reqs))
-    return out
+    w = host_weights()
+    pcfg = plain.PlainConfig.from_dict(SHAPE)
+    want = {name: plain.forward(pcfg, w, toks) for name, toks in reqs.items()}
+    return {dtype: (None, reqs, want) for dtype in ("float32", "bfloat16")}
+
+
+# ------------------------------------------------------------------ long contexts through the four traces
+LONG = [100, 1300, 2500, 600]
+
+
+def _kept(name, pos, lens):
+    """The positions whose logits are compared: the first and the last 40 of a request, every 61st,
+    and the ones around the places where the number of key parts of the decode kernel and the
+    pages of a portion change."""
+    n = lens[name]
+    return pos < 3 or pos >= n - 40 or pos % 61 == 0 or pos in (511, 512, 1023, 1024, 1025, 2047, 2048)
+
+
+@pytest.fixture(scope="module")
+def long_requests():
+    reqs = common.random_requests(SHAPE["vocab_size"], LONG, seed=8)
+    lens = {k: len(v) for k, v in reqs.items()}
+    keep = lambda name, pos: _kept(name, pos, lens)
+    w = host_weights()
+    pcfg = plain.PlainConfig.from_dict(SHAPE)
+    want = {}
+    for name, toks in reqs.items():
+        at = [p for p in range(len(toks)) if keep(name, p)]
+        print(f"plain: request {name}, {len(toks)} tokens, logits at {len(at)} positions", flush=True)
+        want[name] = (at, plain.forward(pcfg, w, toks, logits_at=at))
+    return reqs, keep, want
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("mode", ["whole", "tail", "portions", "mixed"])
+def test_long_requests_at_full_layer_sizes_through_the_four_traces(long_requests, dtype, mode):
+    """Two layers of the Llama-3-8B shape with random weights from a seed, requests of 100, 1,300,
+    2,500 and 600 tokens: whole; with the last 32 tokens decoded one by one (the decode kernel cuts
+    2,500 keys into parts, and its steps are replayed from a captured graph); in portions of 1 to
+    700 tokens (prefill over a history of up to 2,000 keys); and mixed, four live requests with a
+    pool so small that pages are used again, one of them losing its pages on the way and computed
+    again.  Logits at the kept positions against the plain implementation."""
+    from llama_cu_amd.engine.trace import TraceReplayer
+    reqs, keep, want = long_requests
+    if mode == "whole":
+        steps, max_tokens = common.trace_whole(reqs, keep=keep)
+    elif mode == "tail":
+        steps, max_tokens = common.trace_tail_decode(reqs, keep=keep)
+    elif mode == "portions":
+        steps, max_tokens = common.trace_portions(reqs, sizes=(300, 2, 700, 17, 1, 512, 64, 5), keep=keep)
+    else:
+        steps, max_tokens = common.trace_mixed(reqs, seed=2, tail=20, sizes=(2, 3, 17, 48, 130, 300, 640), keep=keep,
+                                               preempt=0.04)
+    print(f"{mode} {dtype}: {len(steps)} steps, max-tokens {max_tokens}", flush=True)
+    rep = TraceReplayer(runner_for(dtype, page_size=16, max_tokens=max_tokens, max_seqs=8,
+                                   max_batch_tokens=max_tokens, poison_freed=True))
+    outputs = {}
+    for st in steps:
+        out = rep.step(st)
+        if out is not None:
+            outputs[st["step"]] = out
+    rep.runner.cache.check()
+    assert rep.runner.cache.free_pages(0) == rep.runner.num_pages
+    got = common.collect(steps, outputs, SHAPE["vocab_size"])
+    if mode == "mixed":
+        assert rep.pages_used_again(0) > 0 and rep.mixed_steps > 0
+        assert any(st.get("preempt") for st in steps)
+    if mode == "tail" and dtype == "bfloat16":
+        assert any(key[0] == 1 and key[1] > 1 for key in rep.runner._graphs), rep.runner._graphs.keys()   # split keys, captured
+    rel = common.REL_TOL[dtype]
+    for name, (at, ref) in want.items():
+        ref = ref.numpy()
+        scale = float(np.abs(ref).max())
+        assert set(got[name]) == set(at), f"{mode}: request {name}: positions differ"
+        for row, pos in enumerate(at):
+            err = float(np.abs(got[name][pos].astype(np.float64) - ref[row]).max())
+            assert np.isfinite(err) and err <= rel * scale, \
+                f"{mode}/{dtype}: request {name}, first wrong position {pos}: error {err:.3e} > {rel * scale:.3e}"
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_whole_portions_and_decoding_at_full_layer_sizes(big, dtype):
-    from llama_cu_amd.engine.runner import ModelRunner
-    folder, reqs, want = big[dtype]
-    runner = ModelRunner.from_folder(folder, dtype=dtype, max_tokens=512, max_seqs=4)
+    _, reqs, want = big[dtype]
+    runner = runner_for(dtype, max_tokens=512, max_seqs=4)
     names = list(reqs)
     ids = {n: i for i, n in enumerate(names)}
     got = {n: {} for n in names}
@@ -68,8 +164,8 @@ def test_steps_of_33_to_64_rows_at_full_layer_sizes(big, dtype, monkeypatch):
         calls["swiglu" if kw.get("swiglu") else "planes"] += 1
         return real(*a, **kw)
     monkeypatch.setattr(ops, "gemm_mid", counted)
-    folder, reqs, want = big[dtype]
-    runner = ModelRunner.from_folder(folder, dtype=dtype, max_tokens=512, max_seqs=4)
+    _, reqs, want = big[dtype]
+    runner = runner_for(dtype, max_tokens=512, max_seqs=4)
     r0, r1 = reqs["r0"], reqs["r1"]
     got = {"r0": {}, "r1": {}}
     logits = runner.step([0], [r0[:40]], [list(range(40))]).cpu().numpy()                    # 40 rows
@@ -97,13 +193,12 @@ def test_captured_steps_of_36_requests_equal_eager_ones(big):
     64 rows and its planes of partial sums inside it) give the bits of eager steps on every replay,
     with eager work between the replays."""
     from llama_cu_amd.engine.runner import ModelRunner
-    folder = big["bfloat16"][0]
     rng = np.random.default_rng(5)
     prompts = [[int(t) for t in rng.integers(SHAPE["vocab_size"], size=3 + i % 5)] for i in range(36)]
     feeds = [[[int(t)] for t in rng.integers(SHAPE["vocab_size"], size=36)] for _ in range(6)]
 
     def decode(use_graphs):
-        runner = ModelRunner.from_folder(folder, dtype="bfloat16", max_tokens=36 * 32 + 64, max_seqs=40, use_graphs=use_graphs)
+        runner = runner_for("bfloat16", max_tokens=36 * 32 + 64, max_seqs=40, use_graphs=use_graphs)
         ids = list(range(36))
         runner.step(ids, prompts)
         outs = []

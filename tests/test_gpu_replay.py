@@ -42,9 +42,13 @@ def test_replay_matches_plain(models, name, dtype, mode, monkeypatch):
         from llama_cu_amd.kernels import ops
         real = ops.gemm_mid
         monkeypatch.setattr(ops, "gemm_mid", lambda *a, **kw: (calls.append(a[0].shape[0]), real(*a, **kw))[1])
-    outputs = common.run_trace_inprocess(folder, dtype, steps, max_tokens)
+    stats = {}
+    outputs = common.run_trace_inprocess(folder, dtype, steps, max_tokens, stats=stats)
     got = common.collect(steps, outputs, vocab)
     common.assert_matches_plain(got, want, dtype, f"{name}/{dtype}/{mode}")
+    if mode == "mixed":
+        # the pool is so small that pages went from one request to another, and portions stood beside single tokens
+        assert stats["pages_used_again"] > 0 and stats["mixed_steps"] > 0, stats
     if name == "D" and dtype == "bfloat16" and mode in ("whole", "mixed"):
         assert calls and all(32 < rows <= 128 for rows in calls), calls      # the planes of partial sums were in it
 
@@ -57,6 +61,48 @@ def test_trace_run_program(models, dtype):
     outputs = common.run_trace_program(folder, dtype, steps, max_tokens, common.TINY_A["vocab_size"])
     got = common.collect(steps, outputs, common.TINY_A["vocab_size"])
     common.assert_matches_plain(got, want, dtype, f"trace_run/{dtype}")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_replay_with_requests_that_lose_their_pages_and_are_computed_again(models, dtype):
+    """``"preempt": [name]`` in a step: the request's pages are given back, and the next step that
+    names it computes all its earlier tokens again beside its new ones, in one batch with the
+    other requests.  The logits are those of the plain implementation all the same."""
+    folder, reqs, want = models[("B", dtype)]
+    steps, max_tokens = common.trace_mixed(reqs, seed=7, preempt=0.2)
+    assert sum(len(s.get("preempt", [])) for s in steps) >= 3
+    stats = {}
+    outputs = common.run_trace_inprocess(folder, dtype, steps, max_tokens, stats=stats)
+    got = common.collect(steps, outputs, common.TINY_B["vocab_size"])
+    common.assert_matches_plain(got, want, dtype, f"preempted/{dtype}")
+    assert stats["pages_used_again"] > 0
+
+
+def test_trace_run_program_with_weights_from_a_seed_and_its_own_pages(tmp_path):
+    """``--random-weights SEED``: the folder holds config.json only and the weights are made on the
+    GPU; the plain implementation gets the weights of the same seed made on the host.  Pages of 32
+    tokens and a pool given in pages."""
+    import json
+    import os
+    import plain
+    from llama_cu_amd.config import LlamaConfig
+    from llama_cu_amd.models.llama import llama_spec
+    from llama_cu_amd.parts import DecoderModel
+    from llama_cu_amd.weights import random_tensors
+    with open(tmp_path / "config.json", "w") as f:
+        json.dump(common.TINY_B, f)
+    spec = llama_spec(LlamaConfig.from_dict(common.TINY_B))
+    w = random_tensors(DecoderModel(spec).tensors(), 5, dtype=torch.float32, device="cpu", std=0.02)
+    reqs = common.random_requests(common.TINY_B["vocab_size"], [40, 97, 130, 66], seed=9)
+    pcfg = plain.PlainConfig.from_dict(common.TINY_B)
+    want = {name: plain.forward(pcfg, w, toks) for name, toks in reqs.items()}
+    steps, max_tokens = common.trace_mixed(reqs, seed=4)
+    outputs = common.run_trace_program(str(tmp_path), "float32", steps, max_tokens, common.TINY_B["vocab_size"],
+                                       extra=["--random-weights", "5", "--page-size", "32", "--num-pages", str(max_tokens // 32),
+                                              "--max-live", "4", "--poison-freed"])
+    got = common.collect(steps, outputs, common.TINY_B["vocab_size"])
+    common.assert_matches_plain(got, want, "float32", "trace_run --random-weights")
+    assert not os.path.exists(tmp_path / "model.safetensors")
 
 
 def test_float32_does_not_depend_on_cutting(models):

@@ -50,3 +50,24 @@ def test_byte_tokenizer_and_streaming():
     import pytest
     with pytest.raises(ValueError):
         text.ByteTokenizer(100)
+
+
+def test_a_tokenizer_file_is_read_and_round_trips(tmp_path):
+    """A small word-level ``tokenizer.json`` made with the ``tokenizers`` package: a folder that
+    holds one gets it, and text goes to ids and back."""
+    import pytest
+    tokenizers = pytest.importorskip("tokenizers")
+    from tokenizers import Tokenizer, decoders, models, pre_tokenizers
+    vocab = {"[UNK]": 0, "hello": 1, "world": 2, "once": 3, "upon": 4, "a": 5, "time": 6, ",": 7}
+    tk = Tokenizer(models.WordLevel(vocab, unk_token="[UNK]"))
+    tk.pre_tokenizer = pre_tokenizers.Whitespace()
+    tk.decoder = decoders.Fuse()
+    tk.save(str(tmp_path / "tokenizer.json"))
+    tok = text.load_tokenizer(str(tmp_path), 8)
+    assert isinstance(tok, text.FileTokenizer)
+    ids = tok.encode("once upon a time, hello")
+    assert ids == [3, 4, 5, 6, 7, 1]
+    assert tok.encode("hello zebra") == [1, 0]                    # what the file does not know
+    assert tok.decode([1, 2]).replace(" ", "") == "helloworld"
+    dec = text.StreamDecoder(tok)
+    assert "".join(dec.push(i) for i in [3, 4]).replace(" ", "") == "onceupon"

@@ -172,3 +172,38 @@ def test_random_model_command_writes_a_folder_that_loads(tmp_path):
     names = {n for f in files for n in f.names()}
     assert "model.embed_tokens.weight" in names and "model.layers.1.mlp.down_proj.weight" in names
 
+
+
+def test_the_generator_is_a_function_of_seed_name_and_index_and_is_normal():
+    """Element i of a tensor depends on (seed, name, i) alone; the values are Box-Muller normals:
+    a plain formula with the library's logarithm and cosine gives the same numbers to within the
+    polynomials' error, and the moments of a million of them are those of N(0, 1)."""
+    import math
+    from llama_cu_amd.weights import fill_normal, stream_key
+    key = stream_key(7, "model.embed_tokens.weight")
+    assert key != stream_key(8, "model.embed_tokens.weight") and key != stream_key(7, "model.embed_tokens.weigh")
+    assert stream_key(0, "a") != stream_key(1, "a") != stream_key(2, "a")
+    t = fill_normal(torch.empty(1 << 20), key, 1.0)
+    short = fill_normal(torch.empty(1000), key, 1.0)
+    assert torch.equal(short, t[:1000])                              # a prefix of the same stream
+    mask = (1 << 64) - 1
+
+    def mix(z):
+        z &= mask; z ^= z >> 30; z = z * 0xBF58476D1CE4E5B9 & mask; z ^= z >> 27; z = z * 0x94D049BB133111EB & mask
+        return z ^ (z >> 31)
+    for i in (0, 1, 2, 999, 12345, (1 << 20) - 1):
+        z = mix(key + (i + 1) * 0x9E3779B97F4A7C15)
+        u1, u2 = ((z >> 32) + 0.5) / 2 ** 32, ((z & 0xFFFFFFFF) + 0.5) / 2 ** 32
+        want = math.sqrt(-2 * math.log(u1)) * math.cos(2 * math.pi * u2)
+        assert abs(float(t[i]) - want) <= 1e-6 * max(1.0, abs(want)), (i, float(t[i]), want)
+    d = t.double()
+    assert abs(float(d.mean())) < 4e-3 and abs(float(d.std()) - 1) < 4e-3
+    assert abs(float((d ** 3).mean())) < 2e-2 and abs(float((d ** 4).mean()) - 3) < 5e-2
+    assert 4.0 < float(d.abs().max()) < 6.5                           # tails are there, and finite
+    assert abs(float((d[1:] * d[:-1]).mean())) < 4e-3                  # neighbours are uncorrelated
+    # scale and shift in 32-bit, one rounding to bfloat16
+    f = fill_normal(torch.empty(4096), key, 0.02, 1.0)
+    assert torch.equal(f, t[:4096] * 0.02 + 1.0)
+    assert torch.equal(fill_normal(torch.empty(4096, dtype=torch.bfloat16), key, 0.02, 1.0), f.to(torch.bfloat16))
+    with pytest.raises(ValueError):
+        fill_normal(torch.empty(4, dtype=torch.float16), key, 1.0)
