@@ -27,6 +27,9 @@
 //   prefill kernel  any number of tokens per request (also one).  A workgroup of 8 waves
 //                   takes consecutive tokens of one request; the keys and values of a step
 //                   are copied to LDS once and shared by the waves.
+#include <mutex>
+
+#include "attention_static.h"
 #include "common.h"
 #include "kv_layout.h"
 
@@ -535,6 +538,66 @@ LCU_API int lcu_attention_decode_bf16(const void *q, int q_stride, void *out, in
     if (dh == 32) GO(32);
 #undef GO
     return LCU_UNSUPPORTED;
+}
+
+// ---------------------------------------------------------------------------- no allocation
+// The decode entry point for callers that cannot allocate (see attention_static.h): the parts'
+// partial results go to a buffer in the library's own device image.  In host code `scratch` is
+// only the symbol's stand-in; its address on a device is what hipGetSymbolAddress gives there.
+static __device__ __align__(256) unsigned char scratch[LCU_ATTENTION_STATIC_SCRATCH_BYTES];
+
+constexpr int STATIC_MAX_DEVICES = 64;
+static void *scratch_on_device[STATIC_MAX_DEVICES];     // per device: each holds its own copy at its own address
+static std::mutex scratch_lock;
+
+// The buffer's address on the current device, looked up at the first call there.
+static int static_scratch(void **ptr) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= STATIC_MAX_DEVICES) return LCU_UNSUPPORTED;
+    std::lock_guard<std::mutex> guard(scratch_lock);
+    if (!scratch_on_device[dev]) {
+        void *p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return (int)e;
+        if (!p) return LCU_UNSUPPORTED;
+        scratch_on_device[dev] = p;
+    }
+    *ptr = scratch_on_device[dev];
+    return LCU_OK;
+}
+
+LCU_API int lcu_attention_static_init(void) {
+    void *p = nullptr;
+    return static_scratch(&p);
+}
+
+LCU_API long long lcu_attention_static_scratch_bytes(void) { return (long long)LCU_ATTENTION_STATIC_SCRATCH_BYTES; }
+
+LCU_API long long lcu_attention_static_scratch_needed(int n_req, int nh, int dh, int n_splits) {
+    if (n_req <= 0 || nh <= 0 || dh <= 0 || n_splits <= 1) return 0;
+    return (long long)n_req * nh * n_splits * (dh + 2) * (long long)sizeof(float);
+}
+
+LCU_API int lcu_attention_decode_bf16_static(const void *q, int q_stride, void *out, int out_stride, const void *cache,
+                                             const int *block_table, int max_pages, const int *q_start, const int *ctx_len,
+                                             const int *req_list, int n_req, int nh, int nkvh, int dh, int page, float scale,
+                                             int window, int n_splits, hipStream_t stream) {
+    if (n_req <= 0) return LCU_OK;
+    float *part_o = nullptr, *part_ml = nullptr;
+    if (n_splits > 1) {
+        if (nh <= 0 || dh <= 0 || dh % 4) return LCU_BAD_ARGUMENT;
+        if (lcu_attention_static_scratch_needed(n_req, nh, dh, n_splits) > (long long)LCU_ATTENTION_STATIC_SCRATCH_BYTES)
+            return LCU_SCRATCH_EXCEEDED;
+        void *base = nullptr;
+        const int st = static_scratch(&base);
+        if (st != LCU_OK) return st;
+        part_o = (float *)base;                                            // [n_req * nh * n_splits * dh]
+        part_ml = part_o + (size_t)n_req * nh * n_splits * dh;            // [n_req * nh * n_splits * 2]
+    }
+    return lcu_attention_decode_bf16(q, q_stride, out, out_stride, cache, block_table, max_pages, q_start, ctx_len, req_list,
+                                     n_req, nh, nkvh, dh, page, scale, window, n_splits, part_o, part_ml, stream);
 }
 
 // ============================================================================ prefill
