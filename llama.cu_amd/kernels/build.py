@@ -12,6 +12,7 @@ from __future__ import annotations
 import ctypes
 import hashlib
 import os
+import re
 import shutil
 import subprocess
 import sys
@@ -59,9 +60,25 @@ def _sources(name: str) -> List[str]:
     return [path]
 
 
+_INCLUDE = re.compile(r'^\s*#\s*include\s+"([^"]+)"', re.M)
+
+
 def _headers(name: str) -> List[str]:
-    d = _HOST_DIR if name == HOST_LIBRARY else _KERNEL_DIR
-    return sorted(os.path.join(x, f) for x in (d, _SHARED_DIR) for f in os.listdir(x) if f.endswith(".h"))
+    """The project's own headers that the library's sources include, directly or through one
+    another (``#include "..."``, relative to the file that names them): a change of one of them
+    builds the library again, a change of any other header does not."""
+    seen: Dict[str, None] = {}
+    todo = list(_sources(name))
+    while todo:
+        path = todo.pop()
+        with open(path) as f:
+            text = f.read()
+        for inc in _INCLUDE.findall(text):
+            h = os.path.normpath(os.path.join(os.path.dirname(path), inc))
+            if h not in seen and os.path.isfile(h):
+                seen[h] = None
+                todo.append(h)
+    return sorted(seen)
 
 
 def _digest(name: str) -> str:
