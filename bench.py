@@ -84,14 +84,20 @@ def run_decode(engine, cfg, batch, steps, warmup, rng, sync, prompt_len=PROMPT_L
         engine.step()
     for _ in range(warmup):
         engine.step()
+    import torch
     ctx0 = engine.sched.info(ids[0]).n_tokens
     sync()
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
+    marks[0].record()
     t0 = time.perf_counter()
     produced = 0
-    for _ in range(steps):
+    for k in range(steps):
         produced += sum(1 for o in engine.step() if o.token is not None)
+        marks[k + 1].record()                       # on the stream, after the step's kernels
     sync()
     dt = time.perf_counter() - t0
+    per_step = sorted(marks[k].elapsed_time(marks[k + 1]) for k in range(steps))
+    run_decode.median_ms = per_step[len(per_step) // 2]
     ctx1 = engine.sched.info(ids[0]).n_tokens
     for i in ids:
         engine.abort(i)
@@ -118,6 +124,44 @@ def run_prefill(engine, cfg, rng, sync, repeats=3, history=0):
         if k > 0:                                   # the first run warms up
             best = dt if best is None else min(best, dt)
     return best
+
+
+def run_mixed(engine, cfg, n_requests, rng, sync, new_tokens=128, lo=16, hi=2048):
+    """The mixed batch of BASELINE's Llama-2-7B workload: ``n_requests`` requests at once, prompt
+    lengths uniform in [lo, hi], ``new_tokens`` greedy tokens each, through the scheduler under its
+    token budget (prompt portions beside decoding requests).  Returns a dict of what was measured:
+    the reference's bench prints the same (llama.cu/xtask/src/bench.rs:63-80: time to the first
+    answer, tokens, time per token, steps, time per step)."""
+    import torch
+    from llama_cu_amd.sampling import GREEDY
+    lens = [rng.randrange(lo, hi + 1) for _ in range(n_requests)]
+    ids = [engine.add_request([rng.randrange(cfg.vocab_size) for _ in range(n)], GREEDY, max_steps=new_tokens, ignore_eos=True)
+           for n in lens]
+    sync()
+    marks = [torch.cuda.Event(enable_timing=True)]
+    marks[0].record()
+    t0 = time.perf_counter()
+    produced = steps = 0
+    first_all = first_steps = None
+    while not engine.idle:
+        outs = engine.step()
+        steps += 1
+        marks.append(torch.cuda.Event(enable_timing=True))
+        marks[-1].record()
+        produced += sum(1 for o in outs if o.token is not None)
+        if first_all is None and all(engine.sched.info(i).generated > 0 for i in ids):
+            sync()
+            first_all, first_steps = time.perf_counter() - t0, steps
+    sync()
+    dt = time.perf_counter() - t0
+    for i in ids:
+        engine.drop(i)
+    assert produced == n_requests * new_tokens, (produced, n_requests, new_tokens)
+    per_step = [marks[k].elapsed_time(marks[k + 1]) for k in range(steps)]
+    decode_steps = sorted(per_step[first_steps:]) or [0.0]
+    return {"requests": n_requests, "prompt_tokens": sum(lens), "new_tokens": produced, "seconds": dt,
+            "all_prompts_in_ms": first_all * 1e3, "prefill_steps": first_steps, "steps": steps,
+            "decode_step_median_ms": decode_steps[len(decode_steps) // 2], "preemptions": engine.sched.preemptions}
 
 
 def kernel_summary(db: str, steps: int) -> int:
@@ -164,6 +208,10 @@ def main() -> int:
                          "limit grows with it)")
     ap.add_argument("--dtype", choices=["bfloat16", "float32"], default="bfloat16")
     ap.add_argument("--page-size", type=int, default=16, help="tokens in a page of the cache (a multiple of 16)")
+    ap.add_argument("--workload", choices=["decode", "mixed"], default="decode",
+                    help="decode: --batch requests decode together after prompts of --prompt-len (the default); mixed: "
+                         "--batch requests at once with prompt lengths uniform in [16, 2048], 128 tokens each, through the "
+                         "scheduler (BASELINE's Llama-2-7B workload: --shape llama2-7b --batch 64)")
     ap.add_argument("--no-points", action="store_true", help="skip decoding at batch 1 and 64 and the prefill")
     ap.add_argument("--only-prefill", action="store_true", help="time the 2048-token prefill alone (for profiles)")
     ap.add_argument("--prefill-history", type=int, default=0,
@@ -197,13 +245,28 @@ def main() -> int:
     rng = random.Random(0)
     sync = torch.cuda.synchronize
     page = args.page_size
-    biggest = max(args.batch, 1 if (args.no_points or args.only_prefill) else 64)
+    biggest = max(args.batch, 1 if (args.no_points or args.only_prefill or args.workload == "mixed") else 64)
     # a request decodes while later ones still prefill: room for that too
     per_req = max(args.prompt_len, PROMPT_LEN) + grow
     engine = Engine.from_config(cfg, seed=0, dtype=args.dtype, page_size=page,
                                 max_tokens=biggest * ((per_req + page - 1) // page * page) + args.prefill_history + PREFILL_TOKENS + page,
                                 max_seqs=biggest + 2, max_batch_tokens=max(PREFILL_TOKENS, biggest), prefill_chunk=PREFILL_TOKENS)
 
+    if args.workload == "mixed":
+        run_mixed(engine, cfg, min(args.batch, 8), rng, sync, new_tokens=8)          # builds, loads and captures
+        m = run_mixed(engine, cfg, args.batch, rng, sync)
+        print(json.dumps({
+            "metric": f"generated tok/s ({shape_name} shape, mixed batch: {args.batch} requests at once, prompts uniform in "
+                      f"[16, 2048], 128 tokens each)", "value": round(m["new_tokens"] / m["seconds"], 1), "unit": "tok/s",
+            "n_gpus": 1, "steps": m["steps"], "warmup": 0, "ms_per_step": round(m["seconds"] / m["steps"] * 1e3, 3),
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": dt_name, "data": "synthetic",
+            "config": {"model": f"{shape_name} shape, random weights", "global_batch": args.batch, "parallelism": "none (1 GPU)",
+                       "layers": cfg.num_hidden_layers, "layers_of_shape": full_layers, "kv_heads": cfg.num_key_value_heads,
+                       "intermediate_size": cfg.intermediate_size, "vocab_size": cfg.vocab_size, "page_size": page,
+                       "token_budget": PREFILL_TOKENS, "sampling": "greedy"},
+            "mixed": {k: (round(v, 3) if isinstance(v, float) else v) for k, v in m.items()},
+            "total_tok_s": round((m["prompt_tokens"] + m["new_tokens"]) / m["seconds"], 1)}), flush=True)
+        return 0
     if args.only_prefill:
         pt = run_prefill(engine, cfg, rng, sync, repeats=args.steps, history=args.prefill_history)
         flops = prefill_flops(cfg, PREFILL_TOKENS, args.prefill_history)
@@ -212,12 +275,14 @@ def main() -> int:
         return 0
     seconds, produced, mean_ctx = run_decode(engine, cfg, args.batch, args.steps, args.warmup, rng, sync, args.prompt_len)
     ms_per_step = seconds / args.steps * 1e3
+    median_ms = run_decode.median_ms                # of the steps' times on the GPU (events), beside the mean of the wall time
     value = produced / seconds
     step_bytes = weight_bytes(cfg, elem) + args.batch * mean_ctx * kv_bytes_per_token(cfg, elem)
     achieved = step_bytes / (seconds / args.steps)
     line = {
         "metric": f"decode tok/s ({shape_name} shape, prompts of {args.prompt_len} tokens)", "value": round(value, 2), "unit": "tok/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
+        "ms_per_step_median": round(median_ms, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": dt_name, "data": "synthetic",
         "config": {"model": f"{shape_name} shape, random weights", "global_batch": args.batch, "seq_len": args.prompt_len,
                    "parallelism": "none (1 GPU)", "context": cfg.max_position_embeddings,

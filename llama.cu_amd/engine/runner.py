@@ -10,6 +10,7 @@ sampled ids instead of logits.)
 """
 from __future__ import annotations
 
+import sys
 from dataclasses import dataclass
 from typing import Any, Dict, List, Optional, Sequence
 
@@ -112,7 +113,9 @@ class ModelRunner:
         arch, cfg = load_config(folder)
         spec = arch.build_spec(cfg)
         files = open_safetensors(folder)
-        tensors = load_weights(files, DecoderModel(spec).tensors(), DTYPES[dtype], device)
+        model = DecoderModel(spec)
+        tensors = load_weights(files, model.tensors(), DTYPES[dtype], device, groups=model.fused_groups(DTYPES[dtype], device),
+                               log=lambda line: print(f"[llama.cu_amd] {line}", file=sys.stderr, flush=True))
         runner = cls(spec, tensors, dtype, device, **kw)
         runner.config = cfg
         return runner

@@ -18,6 +18,7 @@ from .base import BuildContext, PagedKV, Part, PartSpec, ScaledRows, TensorSpec,
 from .linear import (Weight, linear, linear_into_norm, linear_planes, linear_qkv_rope, linear_scaled, mid_takes,
                      skinny_takes)
 from .position import NoPosition
+from ..weights.loader import fused_rows
 
 
 class Attention(Part):
@@ -46,6 +47,9 @@ class Attention(Part):
             t["v_proj.weight"] = TensorSpec((nkv * dh, d))
         return t
 
+    def fused_groups(self, dtype, device):
+        return [] if self.shares_kv else [(("q_proj.weight", "k_proj.weight", "v_proj.weight"), 0)]
+
     def cache_need(self):
         return PagedKV(self.kv_heads, self.head_dim, self.window)
 
@@ -58,10 +62,8 @@ class Attention(Part):
         if self.shares_kv:
             self.w_qkv = Weight(tensors["q_proj.weight"], build)
         else:
-            parts = [tensors["q_proj.weight"], tensors["k_proj.weight"], tensors["v_proj.weight"]]
-            if len({p.dtype for p in parts}) != 1:
-                parts = [p.float() for p in parts]
-            self.w_qkv = Weight(torch.cat(parts, dim=0), build)
+            # one matrix with the rows of q, then k, then v: in place where the loader laid them out so
+            self.w_qkv = Weight(fused_rows([tensors["q_proj.weight"], tensors["k_proj.weight"], tensors["v_proj.weight"]]), build)
         self.w_o = Weight(tensors["o_proj.weight"], build)
         self.position.load({}, build)
         # a position encoding that is its rotation tables alone (apply() does nothing of its own)

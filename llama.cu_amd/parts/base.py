@@ -182,6 +182,12 @@ class Part:
     def load(self, tensors: Dict[str, torch.Tensor], build: BuildContext) -> None:
         pass
 
+    def fused_groups(self, dtype: torch.dtype, device: torch.device) -> List[Tuple[Tuple[str, ...], int]]:
+        """Tensors that this part multiplies as one matrix: ``[(names in row order, rows to which each
+        is filled up with zeros, or 0)]``.  The weight loader lays such tensors out one after the other,
+        so that the part finds the fused matrix in place (``weights.loader.fused_rows``)."""
+        return []
+
 
 _REGISTRIES: Dict[str, Dict[str, Callable[..., Part]]] = {
     "norm": {}, "mixer": {}, "ffn": {}, "position": {}, "block": {}, "embedding": {}, "head": {}}

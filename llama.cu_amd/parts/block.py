@@ -43,6 +43,12 @@ class PreNormBlock(Part):
             pre = name + "." if name else ""
             part.load({k[len(pre):]: v for k, v in tensors.items() if k.startswith(pre)}, build)
 
+    def fused_groups(self, dtype, device):
+        out = []
+        for name, part in self._children():
+            out += [(tuple(prefixed(name, n) for n in names), pad) for names, pad in part.fused_groups(dtype, device)]
+        return out
+
     def cache_need(self):
         return self.mixer.cache_need()
 

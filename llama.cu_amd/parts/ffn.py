@@ -13,6 +13,7 @@ import torch
 
 from ..kernels import ops
 from .base import BuildContext, Part, ScaledRows, TensorSpec, register_part
+from ..weights.loader import fused_rows
 from .linear import (Weight, library_friendly_rows, linear, linear_into_norm, linear_planes, linear_swiglu,
                      linear_swiglu_mid, mid_swiglu_takes, mid_takes, skinny_row_limit, skinny_takes)
 
@@ -29,21 +30,29 @@ class SwiGLU(Part):
         return {"gate_proj.weight": TensorSpec((di, d)), "up_proj.weight": TensorSpec((di, d)),
                 "down_proj.weight": TensorSpec((d, di))}
 
+    def _padded_rows(self, dtype, device) -> int:
+        """Rows of each half of the plain gate/up matrix: more than ``intermediate_size`` where the library's
+        product of many rows is faster with rows of zeros behind each half (``library_friendly_rows``)."""
+        if dtype == torch.bfloat16 and torch.device(device).type == "cuda":
+            return library_friendly_rows(self.intermediate_size, self.hidden_size, device)
+        return self.intermediate_size
+
+    def fused_groups(self, dtype, device):
+        rows = self._padded_rows(dtype, device)
+        return [(("gate_proj.weight", "up_proj.weight"), rows if rows != self.intermediate_size else 0)]
+
     def load(self, tensors, build: BuildContext) -> None:
         g, u = tensors["gate_proj.weight"], tensors["up_proj.weight"]
-        if g.dtype != u.dtype:
-            g, u = g.float(), u.float()
-        both = torch.cat([g, u], dim=0)
         rows = self.intermediate_size
-        if build.dtype == torch.bfloat16 and both.dtype == torch.bfloat16 and both.is_cuda:
-            rows = library_friendly_rows(self.intermediate_size, self.hidden_size, both.device)
+        if build.dtype == torch.bfloat16 and g.dtype == u.dtype == torch.bfloat16 and g.is_cuda:
+            rows = self._padded_rows(build.dtype, g.device)
         if rows != self.intermediate_size:
-            # the plain copy, which the library multiplies, gets rows of zeros behind each half; the
+            # the plain copy, which the library multiplies, has rows of zeros behind each half; the
             # copy that the decode kernels stream does not
-            zeros = torch.zeros((rows - self.intermediate_size, self.hidden_size), dtype=both.dtype, device=both.device)
-            self.w_gate_up = Weight(torch.cat([g, zeros, u, zeros], dim=0), build, packed_from=both)
+            plain = fused_rows([g, u], pad_rows_to=rows)
+            self.w_gate_up = Weight(plain, build, packed_from=torch.cat([g, u], dim=0) if build.pack_weights else None)
         else:
-            self.w_gate_up = Weight(both, build)
+            self.w_gate_up = Weight(fused_rows([g, u]), build)
         self.w_down = Weight(tensors["down_proj.weight"], build)
         self.dtype = build.dtype
 

@@ -14,6 +14,7 @@ Which routine multiplies is decided here and nowhere else:
 """
 from __future__ import annotations
 
+import sys
 from typing import Optional, Union
 
 import torch
@@ -130,6 +131,11 @@ def library_friendly_rows(di: int, d: int, device) -> int:
             del w
         best = min(times, key=times.get)
         _friendly_rows[key] = best if times[best] <= 0.85 * times[di] else di
+        # the choice enters the log: it rests on a timing, and a run should say what it chose
+        took = ", ".join(f"{rows}: {t / 4 * 1e3:.0f} us" for rows, t in sorted(times.items()))
+        print(f"[llama.cu_amd] gate/up product of 2,048 rows with halves of {di} x {d}: the library takes {took} per "
+              f"half size; each half of the plain copy is {'filled up to ' + str(_friendly_rows[key]) + ' rows' if _friendly_rows[key] != di else 'left as it is'}",
+              file=sys.stderr, flush=True)
     return _friendly_rows[key]
 
 

@@ -105,6 +105,14 @@ class DecoderModel:
                 out[prefixed(prefix, k)] = v
         return out
 
+    def fused_groups(self, dtype, device):
+        """The parts' fused groups under their full tensor names, as the weight loader takes them."""
+        from ..weights.loader import FusedGroup
+        out = []
+        for prefix, part in self._named_parts():
+            out += [FusedGroup(tuple(prefixed(prefix, n) for n in names), pad) for names, pad in part.fused_groups(dtype, device)]
+        return out
+
     def load(self, tensors: Dict[str, torch.Tensor], build: BuildContext) -> None:
         for prefix, part in self._named_parts():
             pre = prefix + "." if prefix else ""

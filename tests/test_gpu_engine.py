@@ -97,6 +97,85 @@ def test_long_decoding_matches_plain(folder_a):
     assert got == plain.greedy_generate(cfg, w, prompt, 100)
 
 
+@pytest.mark.parametrize("name", ["B", "D"])
+@pytest.mark.parametrize("run_ahead", [False, True])
+def test_greedy_generation_in_bfloat16_through_scheduler_and_sampler(name, run_ahead):
+    """The bfloat16 path through the whole engine (portions of prompts, a pool so small that a
+    request is preempted and computed again, captured decode steps, the arg-max kernel): every
+    generated token is the plain implementation's arg-max given the same tokens before it, or,
+    where the plain implementation's two best logits lie within the bfloat16 tolerance of each
+    other, one whose plain logit lies within that tolerance of the best.  Most tokens must be
+    the arg-max itself."""
+    from llama_cu_amd.engine.engine import Engine
+    cfg_d = common.TINY[name]
+    folder = common.make_folder(cfg_d, seed=31, dtype=torch.bfloat16, std=0.1)
+    prompts = list(common.random_requests(cfg_d["vocab_size"], [3, 40, 77, 21, 60], seed=5).values())
+    engine = Engine.from_folder(folder, dtype="bfloat16", max_tokens=224, max_seqs=4, max_batch_tokens=48, prefill_chunk=32,
+                                run_ahead=run_ahead)
+    steps = 40
+    got = engine.generate(prompts, max_steps=steps, ignore_eos=True)
+    assert engine.sched.preemptions > 0                                # the pool was too small for all of them
+    assert any(key[0] > 1 for key in engine.runner._graphs)            # decode steps were replayed from graphs
+    engine.runner.cache.check()
+    cfg, w = plain.load_folder(folder)
+    exact = total = 0
+    for prompt, out in zip(prompts, got):
+        assert len(out) == steps
+        logits = plain.forward(cfg, w, prompt + out[:-1])[len(prompt) - 1:]
+        tol = common.REL_TOL["bfloat16"] * float(logits.abs().max())
+        for i, tok in enumerate(out):
+            best = float(logits[i].max())
+            assert float(logits[i][tok]) >= best - tol, f"token {i} of a request: logit {float(logits[i][tok])} against the best {best}"
+            exact += int(tok == int(torch.argmax(logits[i])))
+            total += 1
+    assert exact >= 0.7 * total, (exact, total)
+
+
+@pytest.mark.parametrize("stored", [torch.float16, torch.float32])
+def test_loading_takes_no_more_memory_than_the_weights_and_one_tensor(stored, tmp_path):
+    """A folder whose file stores float16 (converted on the device) or float32 (kept) loads into one
+    allocation through pinned staging: the most device memory ever held while loading is the weights
+    plus one tensor as the file holds it, and the engine built on them (no second, packed copy) adds
+    only its cache; its logits are the plain implementation's."""
+    from llama_cu_amd.config import LlamaConfig
+    from llama_cu_amd.engine.runner import ModelRunner
+    from llama_cu_amd.models.llama import llama_spec
+    from llama_cu_amd.parts import DecoderModel
+    from llama_cu_amd.weights import load_weights, open_safetensors, write_random_model
+    cfg_d = dict(common.TINY_D, hidden_size=512, intermediate_size=2048, vocab_size=4000, num_hidden_layers=3)
+    cfg = LlamaConfig.from_dict(cfg_d)
+    folder = write_random_model(str(tmp_path / "m"), cfg, seed=2, dtype=stored, std=0.05)
+    model = DecoderModel(llama_spec(cfg))
+    compute = torch.bfloat16 if stored == torch.float16 else torch.float32
+    dev = torch.device("cuda:0")
+    torch.cuda.synchronize()
+    torch.cuda.empty_cache()
+    torch.cuda.reset_peak_memory_stats(dev)
+    before = torch.cuda.memory_allocated(dev)
+    lines = []
+    t = load_weights(open_safetensors(folder), model.tensors(), compute, dev, groups=model.fused_groups(compute, dev),
+                     log=lines.append)
+    peak = torch.cuda.max_memory_allocated(dev) - before
+    held = torch.cuda.memory_allocated(dev) - before
+    elem = 2 if compute == torch.bfloat16 else 4
+    weights = sum(v.numel() for v in t.values()) * elem
+    largest = max(v.numel() for v in t.values()) * (2 if stored == torch.float16 else 4)
+    assert weights <= held <= weights + 256 * len(t) + 4096
+    assert peak <= held + largest + 4096, (peak, held, largest)
+    assert "GB/s" in lines[0]
+    del t
+    name = "bfloat16" if compute == torch.bfloat16 else "float32"
+    runner = ModelRunner.from_folder(folder, dtype=name, max_tokens=256, max_seqs=2, pack_weights=False)
+    assert runner.model.layers[0].mixer.w_qkv.plain.data_ptr() == runner.model.layers[0].mixer.w_qkv.plain.untyped_storage().data_ptr() \
+        or runner.model.layers[0].mixer.w_qkv.plain.storage_offset() > 0          # a view of the allocation, not a copy
+    toks = list(common.random_requests(4000, [50], seed=1).values())[0]
+    got = runner.step([0], [toks], [list(range(50))]).cpu()
+    pcfg, pw = plain.load_folder(folder)
+    want = plain.forward(pcfg, pw, toks)
+    err = float((got.double() - want).abs().max())
+    assert err <= common.REL_TOL[name] * float(want.abs().max())
+
+
 def test_context_limit_ends_a_request(folder_a):
     from llama_cu_amd.engine.engine import Engine
     engine = Engine.from_folder(folder_a, dtype="float32", max_tokens=512, max_seqs=2)

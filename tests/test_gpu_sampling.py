@@ -93,6 +93,37 @@ def test_sample_frequencies_follow_the_cut_softmax():
     assert freq[[i for i in range(vocab) if i not in keep]].sum() == 0
 
 
+def test_sample_frequencies_with_a_top_p_cut_inside_the_support():
+    """top_p cuts the cumulative weights of the sorted tokens at ``top_p`` of their total
+    (llama.cu/src/op/random_sample/sample.cuh:71-87: the drawn number is scaled by
+    ``min(top_p * c[n-1], c[top_k-1])``): tokens wholly below the cut keep their weight, the token
+    that the cut falls into keeps only the part below the cut, and nothing beyond it is ever drawn.
+    (The usual nucleus rule would keep that token whole: the frequencies tell the two apart.)"""
+    from llama_cu_amd.sampling import sample_rows
+    vocab, n, T, top_p = 30, 40000, 1.1, 0.62
+    l = _logits(1, vocab, 11, scale=1.2)[0]
+    rng = np.random.default_rng(3)
+    u = [float(x) for x in rng.random(n)]
+    got = sample_rows(l.repeat(n, 1).cuda(), [T] * n, [top_p] * n, [10 ** 9] * n, u).cpu().numpy()
+    p = torch.softmax(l.double() / T, 0).numpy()
+    order = np.argsort(-p, kind="stable")
+    c = np.cumsum(p[order])
+    q = np.zeros(vocab)
+    below = 0.0
+    for rank, tok in enumerate(order):
+        q[tok] = max(0.0, min(c[rank], top_p) - below) / top_p
+        below = c[rank]
+    cut = int(np.searchsorted(c, top_p))                       # the rank the cut falls into
+    assert 2 <= cut < vocab - 3                                 # strictly inside the support
+    part = q[order[cut]] * top_p / p[order[cut]]
+    assert 0.15 < part < 0.85                                   # a real part of that token, neither none nor all of it
+    freq = np.bincount(got, minlength=vocab) / n
+    assert np.abs(freq - q).max() < 0.01
+    assert freq[order[cut + 1:]].sum() == 0                     # nothing beyond the cut
+    whole = p[order[cut]] / c[cut]                              # what the token would get if it were kept whole
+    assert abs(freq[order[cut]] - q[order[cut]]) < 0.01 < abs(whole - q[order[cut]])
+
+
 def test_per_row_parameters_and_sampler_mix():
     from llama_cu_amd.sampling import Sampler, SamplingParams, uniform
     l = _logits(4, 500, 9)

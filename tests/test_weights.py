@@ -207,3 +207,47 @@ def test_the_generator_is_a_function_of_seed_name_and_index_and_is_normal():
     assert torch.equal(fill_normal(torch.empty(4096, dtype=torch.bfloat16), key, 0.02, 1.0), f.to(torch.bfloat16))
     with pytest.raises(ValueError):
         fill_normal(torch.empty(4, dtype=torch.float16), key, 1.0)
+
+
+def test_weights_lie_in_one_allocation_and_fused_tensors_stand_in_place(tmp_path):
+    """All tensors are views of one allocation; q, k, v and gate, up stand one after the other, so
+    that the fused matrices are views too (nothing is concatenated), also when the file stores
+    another type than the engine keeps; with rows of zeros behind each member where asked for."""
+    from llama_cu_amd.models.llama import llama_spec
+    from llama_cu_amd.parts import DecoderModel
+    from llama_cu_amd.weights.loader import FusedGroup, fused_rows, plan_arena
+    cfg = LlamaConfig.from_dict(common.TINY_B)
+    model = DecoderModel(llama_spec(cfg))
+    groups = model.fused_groups(torch.bfloat16, torch.device("cpu"))
+    assert FusedGroup(("model.layers.1.self_attn.q_proj.weight", "model.layers.1.self_attn.k_proj.weight",
+                       "model.layers.1.self_attn.v_proj.weight"), 0) in groups
+    assert FusedGroup(("model.layers.2.mlp.gate_proj.weight", "model.layers.2.mlp.up_proj.weight"), 0) in groups
+    lines = []
+    for stored, compute in ((torch.float16, torch.bfloat16), (torch.float32, torch.float32), (torch.bfloat16, torch.bfloat16)):
+        folder = write_random_model(str(tmp_path / f"m{len(lines)}"), cfg, seed=3, dtype=stored, vector_dtype=torch.float32)
+        t = load_weights(open_safetensors(folder), model.tensors(), compute, torch.device("cpu"), groups=groups, log=lines.append)
+        base = {v.untyped_storage().data_ptr() for v in t.values()}
+        assert len(base) == 1                                                # one allocation
+        start = next(iter(base))
+        assert all((v.data_ptr() - start) % 256 == 0 or "k_proj" in n or "v_proj" in n or "up_proj" in n for n, v in t.items())
+        p = "model.layers.0."
+        q, k, v = (t[p + f"self_attn.{x}_proj.weight"] for x in "qkv")
+        qkv = fused_rows([q, k, v])
+        assert qkv.data_ptr() == q.data_ptr() and qkv.shape == (q.shape[0] + k.shape[0] + v.shape[0], 128)
+        assert torch.equal(qkv, torch.cat([q, k, v]))
+        gu = fused_rows([t[p + "mlp.gate_proj.weight"], t[p + "mlp.up_proj.weight"]])
+        assert gu.data_ptr() == t[p + "mlp.gate_proj.weight"].data_ptr()
+        assert t["model.norm.weight"].dtype == torch.float32                 # stored in 32-bit: stays so
+        assert q.dtype == compute
+        # the values are the file's, converted once
+        raw = open_safetensors(folder)[0].tensor(p + "self_attn.k_proj.weight")
+        assert torch.equal(k, raw.to(compute))
+    assert len(lines) == 3 and "GB/s" in lines[0] and "one allocation" in lines[0]
+    # tensors that do not stand together are concatenated, with the same result
+    a, b = torch.randn(3, 8), torch.randn(5, 8)
+    assert torch.equal(fused_rows([a, b]), torch.cat([a, b]))
+    assert fused_rows([a, b], pad_rows_to=6).shape == (12, 8) and bool((fused_rows([a, b], pad_rows_to=6)[3:6] == 0).all())
+    # rows of zeros behind each member of a group
+    expected = {"g": TensorSpec((5, 8)), "u": TensorSpec((5, 8)), "x": TensorSpec((3,))}
+    place, total = plan_arena(expected, {n: torch.bfloat16 for n in expected}, torch.bfloat16, [FusedGroup(("g", "u"), 8)])
+    assert place["u"][0] - place["g"][0] == 8 * 8 * 2 and place["x"][0] >= place["u"][0] + 8 * 8 * 2 and total % 256 == 0
