@@ -10,6 +10,10 @@ from .parts import register_part
 
 from .sampling import SamplingParams
 
+import os
+
+_engines: dict = {}
+
 
 def Engine(model: str, dtype: str = "bfloat16", device: str = "cuda:0", **kw):
     """The engine for the model folder ``model`` (see engine.engine.Engine)."""
@@ -23,7 +27,11 @@ def generate(model: str, prompts, sampling: SamplingParams = SamplingParams(), m
     encodes) with the model of the folder ``model``; returns token ids, or strings for
     string prompts."""
     from . import text
-    engine = Engine(model, dtype=dtype, device=device, **kw)
+    key = (os.path.abspath(model), dtype, str(device), tuple(sorted(kw.items())))
+    engine = _engines.get(key)
+    if engine is None:                       # a model is loaded once per process and set of options
+        _engines.clear()
+        engine = _engines[key] = Engine(model, dtype=dtype, device=device, **kw)
     as_text = len(prompts) > 0 and isinstance(prompts[0], str)
     tok = text.load_tokenizer(model, engine.runner.spec.vocab_size) if as_text else None
     ids = [tok.encode(p) for p in prompts] if as_text else [list(p) for p in prompts]

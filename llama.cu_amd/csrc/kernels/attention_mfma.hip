@@ -2,31 +2,29 @@
 //
 // Both kernels work on the transposed problem, so that nothing has to move between
 // lanes or through LDS between the two matrix products:
-//   S^T[key, q] = K[key, :] . Q[q, :]      v_mfma_f32_16x16x32_bf16, A = K (a lane holds 8
-//                                          dims of one key: one 16-byte load in the cache's
-//                                          key layout), B = Q (kept in registers)
-//   O^T[dim, q] += V^T[dim, key] . P^T[key, q]   A = V^T (a lane holds tokens of one dim:
-//                                          8-byte loads in the cache's value layout),
-//                                          B = P^T: exactly the lane's own S^T values
-// In S^T a lane owns one query row (lane % 16) and 8 of each 32 keys, so the softmax's
-// maximum and sum run over a lane's registers and two cross-lane steps.  Which 8 keys is the
-// kernel's choice, by the order in which it feeds the keys' rows to the first product: the decode
-// kernel, which loads from the pages, takes 4 keys of each tile of 16 (keys of a tile are
-// neighbours in memory); the prefill kernel, which reads from its copy in LDS, takes 8 keys in a
-// row (its values are then one 16-byte read).  Scores, the running maximum and sum and the
-// output are 32-bit; P is rounded to bfloat16 for the second product.
+//   S^T[key, q] = K[key, :] . Q[q, :]      A = K (a lane holds 8 dims of one key: one 16-byte
+//                                          load in the cache's key layout), B = Q (kept in registers)
+//   O^T[dim, q] += V^T[dim, key] . P^T[key, q]   A = V^T (a lane holds tokens of one dim, as the
+//                                          cache's value layout has them), B = P^T: exactly the
+//                                          lane's own S^T values
+// so the softmax's maximum and sum run over a lane's registers and one or two cross-lane steps.
+// Which keys a lane holds is the kernel's choice, by the order in which it feeds the keys' rows
+// to the first product.  Scores, the running maximum and sum and the output are 32-bit; P is
+// rounded to bfloat16 for the second product.
 //
-// A "row" is one (token, head) pair; 16 rows that share a request and a key/value head
-// form a block: the heads of a group for one token, for several tokens if the group is
-// small.
+// A "row" is one (token, head) pair; the rows of a block share a request and a key/value head:
+// the heads of a group for one token, for several tokens if the group is small.
 //
-//   decode kernel   one token per request.  A workgroup of 4 waves takes one request and
+//   decode kernel   one token per request, v_mfma_f32_16x16x32_bf16 (blocks of 16 rows; a lane
+//                   owns row lane % 16 and 8 of each 32 keys, 4 of each tile of 16, which are
+//                   neighbours in memory).  A workgroup of 4 waves takes one request and
 //                   key/value head and one of `n_splits` equal parts of its keys; the
 //                   waves take 32-key steps in turn and merge through LDS; parts are
 //                   merged by a second kernel.
-//   prefill kernel  any number of tokens per request (also one).  A workgroup of 8 waves
-//                   takes consecutive tokens of one request; the keys and values of a step
-//                   are copied to LDS once and shared by the waves.
+//   prefill kernel  any number of tokens per request (also one), v_mfma_f32_32x32x16_bf16 (blocks
+//                   of 32 rows; a lane owns row lane % 32 and 16 of each 32 keys).  A workgroup of
+//                   8 waves takes consecutive tokens of one request; the keys and values of a
+//                   step are copied to LDS once and shared by the waves.
 #include <mutex>
 
 #include "attention_static.h"
@@ -170,9 +168,8 @@ __device__ __forceinline__ float max_over_groups(float x) {
 
 // The softmax of the step, online: new maxima and sums, the output rescaled, the weights as
 // bfloat16 operands.
-// PERM: the lane's eight scores are the keys k0 + 8 grp .. + 7 in a row (the prefill kernel reads
-// its key tiles from LDS in that order); else four keys of each tile, k0 + 16 t + 4 grp .. + 3.
-template <int DH, int QB, bool MASK, bool PERM = false>
+// The lane's eight scores are four keys of each tile, k0 + 16 t + 4 grp .. + 3.
+template <int DH, int QB, bool MASK>
 __device__ __forceinline__ void attn_softmax(const f32x4 (&s)[QB][2], int k0, AttnState<DH, QB> &st, const int (&p_row)[QB],
                                              const int (&lo_row)[QB], float scale_log2, int grp, u32x4 (&pb)[QB]) {
 #pragma unroll
@@ -183,7 +180,7 @@ __device__ __forceinline__ void attn_softmax(const f32x4 (&s)[QB][2], int k0, At
         if (MASK) {
 #pragma unroll
             for (int r = 0; r < 8; ++r) {
-                const int j = PERM ? k0 + 8 * grp + r : k0 + 16 * (r / 4) + 4 * grp + (r % 4);
+                const int j = k0 + 16 * (r / 4) + 4 * grp + (r % 4);
                 if (j > p_row[b] || j < lo_row[b]) v[r] = -INFINITY;
             }
         }
@@ -238,29 +235,6 @@ __device__ __forceinline__ void attn_mix(const u32x2 (&v)[DH / 16][2], const u32
     }
 }
 
-// The same with the lane's values being the keys k0 + 8 grp .. + 7 of dim 16 dt + lane % 16, as one
-// 16-byte chunk of the page holds them.
-template <int DH, int QB, bool MASK>
-__device__ __forceinline__ void attn_mix_perm(const u32x4 (&v)[DH / 16], const u32x4 (&pb)[QB], int k0, int p_max, int lo_min,
-                                              int grp, AttnState<DH, QB> &st) {
-    uint32_t keep[4] = {0xffffffffu, 0xffffffffu, 0xffffffffu, 0xffffffffu};
-    if (MASK) {
-        // values of keys that no row sees are taken as zero: their memory may hold anything
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            const int j = k0 + 8 * grp + e;
-            if (j > p_max || j < lo_min) keep[e / 2] &= (e & 1) ? 0x0000ffffu : 0xffff0000u;   // clears element e of its dword
-        }
-    }
-#pragma unroll
-    for (int dt = 0; dt < DH / 16; ++dt) {
-        u32x4 a = v[dt];
-        if (MASK) { a.x &= keep[0]; a.y &= keep[1]; a.z &= keep[2]; a.w &= keep[3]; }
-#pragma unroll
-        for (int b = 0; b < QB; ++b) st.o[b][dt] = mfma16(a, pb[b], st.o[b][dt]);
-    }
-}
-
 template <int DH, int QB, bool MASK>
 __device__ __forceinline__ void attn_compute(const KVFrag<DH> &f, int k0, const u32x4 (&q)[QB][DH / 32],
                                              AttnState<DH, QB> &st, const int (&p_row)[QB], const int (&lo_row)[QB],
@@ -270,38 +244,6 @@ __device__ __forceinline__ void attn_compute(const KVFrag<DH> &f, int k0, const 
     u32x4 pb[QB];
     attn_softmax<DH, QB, MASK>(s, k0, st, p_row, lo_row, scale_log2, grp, pb);
     attn_mix<DH, QB, MASK>(f.v, pb, k0, p_max, lo_min, grp, st);
-}
-
-// The same step with the operands taken from a copy in LDS (the layout that stage_issue
-// makes): first the keys alone, so that the values do not hold registers while the scores
-// are made; the values are asked for before the softmax's arithmetic and are there after it.
-template <int DH, int QB, bool MASK>
-__device__ __forceinline__ void attn_compute_lds(const u32x4 *__restrict__ buf, int k0, const u32x4 (&q)[QB][DH / 32],
-                                                 AttnState<DH, QB> &st, const int (&p_row)[QB], const int (&lo_row)[QB],
-                                                 int p_max, int lo_min, float scale_log2, int l16, int grp) {
-    // Row i of the matrix instruction's key tile t is key 8 (i / 4) + 4 t + i % 4 of the step, so that a
-    // lane's eight scores (rows 4 grp .. + 3 of both tiles) are eight keys in a row, and with them its
-    // values one chunk of 16 bytes: one read, the operand as it arrives.  In LDS key tile i / 8 holds
-    // that key at place i % 8 + 8 t of its row (stage_issue orders the tokens so): the lanes of a read
-    // take neighbouring bytes.
-    f32x4 s[QB][2];
-    {
-        u32x4 k[2][DH / 32];
-        const u32x4 *kb0 = buf + (l16 >> 3) * 2 * DH + grp * 16 + (l16 & 7);
-#pragma unroll
-        for (int t = 0; t < 2; ++t)
-#pragma unroll
-            for (int kb = 0; kb < DH / 32; ++kb) k[t][kb] = kb0[4 * kb * 16 + 8 * t];
-        attn_scores<DH, QB>(k, q, s);
-    }
-    __builtin_amdgcn_sched_barrier(0);             // the values' reads stay below the scores
-    u32x4 v[DH / 16];
-    const u32x4 *vb = buf + 4 * DH + (grp >> 1) * 2 * DH + (grp & 1) * 16 + l16;
-#pragma unroll
-    for (int dt = 0; dt < DH / 16; ++dt) v[dt] = vb[32 * dt];
-    u32x4 pb[QB];
-    attn_softmax<DH, QB, MASK, true>(s, k0, st, p_row, lo_row, scale_log2, grp, pb);
-    attn_mix_perm<DH, QB, MASK>(v, pb, k0, p_max, lo_min, grp, st);
 }
 
 // Masks only where a row needs them (the choice is the same for the whole wave).
@@ -601,76 +543,13 @@ LCU_API int lcu_attention_decode_bf16_static(const void *q, int q_stride, void *
 }
 
 // ============================================================================ prefill
-#ifndef LCU_PRE_QB
-#define LCU_PRE_QB 2
-#endif
 #ifndef LCU_PRE_MIN_WAVES
 #define LCU_PRE_MIN_WAVES 2
 #endif
 constexpr int PRE_QWAVES = 4;             // waves of a workgroup that hold different rows
 constexpr int PRE_HALVES = 2;             // wave groups that share the rows and take every second step of 32 keys
 constexpr int PRE_WAVES = PRE_QWAVES * PRE_HALVES;
-constexpr int PRE_QB = LCU_PRE_QB;
 constexpr int PRE_RING = 3;               // buffers of 64 keys in LDS: one is read, two are on their way
-
-// The keys and values of two steps of 32, copied into LDS in chunks of 16 bytes: per step and
-// tile of 16 keys first the keys as they lie in their page, [dim/8][token][8], then (after both
-// key tiles) the values, whose page holds [dim][token]: a chunk is 8 tokens of one dim, and of
-// every 16 dims first come the 16 chunks of tokens 0..7, then those of tokens 8..15 (the lanes that
-// read one half of 16 dims then read neighbouring bytes; with the page's own order four of them
-// fell into one bank, and the bank conflicts took a quarter of the kernel's time).  A step holds
-// 8*DH chunks: [K tile 0 | K tile 1 | V tile 0 | V tile 1], 2*DH chunks each; a buffer holds two
-// steps.  A thread of the workgroup copies chunks tid, tid + 512, ...
-//
-// The copy goes from memory straight into LDS (global_load_lds_dwordx4: no registers hold the
-// data on its way, lane l of a wave writes the 16 bytes l of the wave's 1 KB), so the loads of
-// two buffers can be in flight while one is computed.  The page of a chunk is the same for a
-// whole wave (2*DH chunks of a region are a multiple of 64), so the block table is read with
-// scalar loads, which do not make the wave wait for the vector loads in flight.
-// Steps beyond the end of the keys are copied all the same, from the pages that the clamped
-// block table names (valid memory), into a buffer that nobody reads: no branch around a load.
-// The address of a chunk is a wave-uniform base (page, token) plus a small per-lane offset.
-// A page holds less than 4 GiB (the host checks).
-template <int DH>
-__device__ __forceinline__ void stage_issue(u32x4 *__restrict__ buf, const bf16_t *__restrict__ cache,
-                                            const int *__restrict__ bt, int max_pages, int page, uint32_t tile_magic,
-                                            size_t page_elems, int nkvh, int kvh, int k0, int wave_id) {
-    // Everything but the lane's offset is made in scalar registers from the wave's number: a wave's
-    // 64 chunks lie in one region of one step (regions are multiples of 64 chunks), and a tile of 16
-    // keys lies in one page.  Tile T is in page T / (page / 16): with tile_magic =
-    // floor(2^32 / (page / 16)) + 1 the quotient is the high word of T * tile_magic (exact while
-    // T * page / 16 < 2^32; 0 stands for pages of 16 keys, where the page is the tile).
-    constexpr uint32_t E = sizeof(bf16_t);
-    const int tiles_per_page = page / 16;
-    int tid = threadIdx.x;
-    asm volatile("" : "+v"(tid));                  // made anew in every step, not kept in registers across the loop
-    const int lane = tid & (WAVE - 1);
-    // keys [dim/8][token][8]; place p of a row of 16 takes token p with bits 2 and 3 swapped (0-3, 8-11,
-    // 4-7, 12-15: the order in which attn_compute_lds reads them)
-    const uint32_t k_tok = (lane & 3) | ((lane & 4) << 1) | ((lane & 8) >> 1);
-    const uint32_t k_lane = ((uint32_t)(lane >> 4) * page + k_tok) * 8 * E;
-    // values [dim][token]: of 16 dims first the chunks with tokens 0..7, then those with tokens 8..15
-    // (so that the 32 lanes that read one half of 16 dims read 256 bytes in a row: no two in one bank)
-    const uint32_t v_lane = ((uint32_t)(16 * (lane >> 5) + (lane & 15)) * page + ((lane >> 4) & 1) * 8) * E;
-#pragma unroll
-    for (int i = 0; i < DH / 32; ++i) {
-        const int cw = wave_id * WAVE + 512 * i;                  // the wave's first chunk
-        const int sub = cw / (8 * DH), c = cw % (8 * DH);
-        const int region = c / (2 * DH), w0 = c % (2 * DH), t = region & 1;
-        const uint32_t tile = (uint32_t)(k0 >> 4) + 2 * sub + t;
-        int pi = tile_magic ? (int)__umulhi(tile, tile_magic) : (int)tile;
-        const uint32_t tok0 = (tile - (uint32_t)pi * tiles_per_page) * 16;
-        pi = pi < max_pages ? pi : max_pages - 1;
-        const int page_id = bt[pi];
-        const uint32_t s_off = region < 2 ? ((uint32_t)(kvh * (DH / 8) + w0 / 16) * page + tok0) * 8 * E
-                                          : ((uint32_t)((nkvh + kvh) * DH + w0 / 2) * page + tok0) * E;
-        // a buffer load whose buffer is the page: all of the address but the lane's offset is scalar
-        const __amdgpu_buffer_rsrc_t pg = __builtin_amdgcn_make_buffer_rsrc(
-            const_cast<bf16_t *>(cache + (size_t)page_id * page_elems), 0, (uint32_t)(page_elems * E), 0x00020000);
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(pg, (__attribute__((address_space(3))) void *)(buf + 512 * i + WAVE * wave_id), 16,
-                                                 region < 2 ? k_lane : v_lane, s_off, 0, 0);
-    }
-}
 
 // Wait until at most `left` of this wave's vector memory operations are outstanding.
 template <int LEFT>
@@ -679,88 +558,234 @@ __device__ __forceinline__ void wait_loads() {
     __builtin_amdgcn_s_waitcnt((LEFT & 15) | ((LEFT >> 4) << 14) | (7 << 4) | (15 << 8));
 }
 
-// One turn of the ring: this wave's step of 32 keys from the buffer `src`, and the workgroup's
-// copy of a later double step into the buffer `dst`.  The two are different buffers of the
-// ring, which the qualifiers say: a read from LDS otherwise waits for every copy in flight,
-// the one into `dst` included, as if it read what that copy writes.
-template <int DH, int QB>
-__device__ __forceinline__ void ring_step(const u32x4 *__restrict__ src, u32x4 *__restrict__ dst,
-                                          const bf16_t *__restrict__ cache, const int *__restrict__ bt, int max_pages, int page,
-                                          uint32_t tile_magic, size_t page_elems, int nkvh, int kvh, int k0_copy, int wave_id,
-                                          int blk, int blk_end,
-                                          bool wave_has, int p_max, int p_min, int lo_min, int lo_max,
-                                          const int (&tok_row)[QB], int pos_of_tok, int window, const u32x4 (&qv)[QB][DH / 32],
-                                          AttnState<DH, QB> &st, float scale_log2) {
-    stage_issue<DH>(dst, cache, bt, max_pages, page, tile_magic, page_elems, nkvh, kvh, k0_copy, wave_id);
-    const int k0 = blk * 32;
-    // the lane's coordinates are made anew in every step: kept across the loop they would
-    // be spilled, and a reload from scratch waits for all the copies in flight
+// The prefill kernel's arithmetic on v_mfma_f32_32x32x16_bf16.  A wave holds 32 rows (lane % 32 is the
+// row, both for Q as the B operand and for S^T and O^T as results), so every lane owns ONE row: its
+// 16 scores of a step of 32 keys lie in its own registers, the row's maximum crosses lanes once
+// (lane and lane + 32), and maximum, sum and rescaling are kept once per lane.
+//   S^T[key, row] = K[key, :] . Q[row, :]     A = K: lane holds 8 dims (16 sidx + 8 hi ..) of the key in
+//                                             slot lane % 32: one 16-byte read of the keys' copy in LDS
+//   O^T[dim, row] += V^T[dim, key] . P^T[key, row]   A = V^T: lane holds 8 keys of dim 32 t + lane % 32,
+//                                             B = P^T: the lane's own scores
+// Result element i of a lane (hi = lane / 32) is row 8 (i / 4) + 4 hi + i % 4 of the instruction.  The
+// keys' copy in LDS stands so (stage_issue) that row m of the first product is key
+// 16 (m / 16) + (m % 16 with bits 2 and 3 swapped) of the step: a lane's elements 8 kk .. 8 kk + 7 are then
+// the keys 16 kk + 8 hi .. + 7 in a row, which is what its 16-byte read of the values' copy holds.
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+
+__device__ __forceinline__ f32x16 mfma32(u32x4 a, u32x4 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+}
+
+template <int DH>
+struct PrefillState {
+    f32x16 o[DH / 32];      // O^T: lane = (row lane % 32, dims 32 t + 8 (i / 4) + 4 hi + i % 4)
+    float m;                // running maximum (in units of log2), the same in the row's two lanes
+    float l;                // running sum over the lane's own keys only
+};
+
+// The key of the step that a lane's score i belongs to (k0: the step's first key).
+__device__ __forceinline__ int key_of_score(int k0, int i, int hi) { return k0 + 16 * (i / 8) + 8 * hi + (i % 8); }
+
+// The larger of the values that lane l and lane l ^ 32 hold, in both.
+__device__ __forceinline__ float max_over_halves(float x) {
+    const unsigned u = __float_as_uint(x);
+    const auto b = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+
+// The keys and values of two steps of 32 keys, copied into LDS in chunks of 16 bytes.  Per step 8 * DH
+// chunks: [K tile 0 | K tile 1 | V tile 0 | V tile 1], 2 * DH chunks per tile of 16 keys; a buffer holds two
+// steps.  Keys as the page holds them, [dim / 8][slot 16], the token in slot p being p with bits 2 and 3
+// swapped.  Values: [half][dim], the chunk of tokens 8 half .. + 7 of the tile for every dim (the page holds
+// [dim][token]).  With these orders the lanes of every read of an operand take neighbouring bytes: no bank
+// conflicts (with the values as their page has them four lanes of a read fell into one bank, and the
+// conflicts took a quarter of the kernel's time).  A thread of the workgroup copies chunks tid, tid + 512, ...
+//
+// The copy goes from memory straight into LDS (buffer_load ... lds: no registers hold the data on its way,
+// lane l of a wave writes the 16 bytes l of the wave's 1 KB), so the loads of two buffers can be in flight
+// while one is computed.  Everything but the lane's offset is made in scalar registers from the wave's
+// number: a wave's 64 chunks lie in one region of one step (regions are multiples of 64 chunks), and a
+// tile of 16 keys lies in one page, whose number is read through the scalar unit (which does not make
+// the wave wait for the vector loads in flight); the buffer of the load is the page.  Tile T is in page
+// T / (page / 16): with tile_magic = floor(2^32 / (page / 16)) + 1 the quotient is the high word of
+// T * tile_magic (exact while T * page / 16 < 2^32; 0 stands for pages of 16 keys, where the page is the
+// tile).  Steps beyond the end of the keys are copied all the same, from the pages that the clamped block
+// table names (valid memory), into a buffer that nobody reads: no branch around a load.  A page holds
+// less than 2 GiB (the host checks).
+template <int DH>
+__device__ __forceinline__ void stage_issue(u32x4 *__restrict__ buf, const bf16_t *__restrict__ cache,
+                                              const int *__restrict__ bt, int max_pages, int page, uint32_t tile_magic,
+                                              size_t page_elems, int nkvh, int kvh, int k0, int wave_id) {
+    constexpr uint32_t E = sizeof(bf16_t);
+    const int tiles_per_page = page / 16;
     int tid = threadIdx.x;
-    asm volatile("" : "+v"(tid));
-    const int l16 = tid & 15, grp = (tid >> 4) & 3;
-    if (wave_has && blk < blk_end && k0 <= p_max && k0 + 31 >= lo_min) {
-        if (k0 + 31 > p_min || k0 < lo_max) {
-            // the rows' limits are made here, where a step needs them, not kept in registers
-            int p_row[QB], lo_row[QB];
+    asm volatile("" : "+v"(tid));                  // made anew in every step, not kept in registers across the loop
+    const int lane = tid & (WAVE - 1);
+    const uint32_t k_tok = (lane & 3) | ((lane & 4) << 1) | ((lane & 8) >> 1);
+    const uint32_t k_lane = ((uint32_t)(lane >> 4) * page + k_tok) * 8 * E;      // a wave: 4 dim chunks x 16 slots
 #pragma unroll
-            for (int b = 0; b < QB; ++b) {
-                p_row[b] = tok_row[b] < 0 ? -1 : tok_row[b] + pos_of_tok;
-                lo_row[b] = tok_row[b] >= 0 && window > 0 && p_row[b] - window + 1 > 0 ? p_row[b] - window + 1 : 0;
-            }
-            attn_compute_lds<DH, QB, true>(src, k0, qv, st, p_row, lo_row, p_max, lo_min, scale_log2, l16, grp);
-        } else {
-            const int none[QB] = {};
-            attn_compute_lds<DH, QB, false>(src, k0, qv, st, none, none, p_max, lo_min, scale_log2, l16, grp);
-        }
+    for (int i = 0; i < DH / 32; ++i) {
+        const int cw = wave_id * WAVE + 512 * i;                  // the wave's first chunk
+        const int sub = cw / (8 * DH), c = cw % (8 * DH);
+        const int region = c / (2 * DH), w0 = c % (2 * DH), t = region & 1;
+        // values: the lane's chunk is number w0 + lane of [half][dim] (a wave may hold the end of one half
+        // and the start of the other where head_dim is no multiple of 64)
+        const uint32_t v_at = (uint32_t)(w0 + lane), v_half = v_at / DH, v_dim = v_at - v_half * DH;
+        const uint32_t v_lane = (v_dim * page + 8 * v_half) * E;
+        const uint32_t tile = (uint32_t)(k0 >> 4) + 2 * sub + t;
+        int pi = tile_magic ? (int)__umulhi(tile, tile_magic) : (int)tile;
+        const uint32_t tok0 = (tile - (uint32_t)pi * tiles_per_page) * 16;
+        pi = pi < max_pages ? pi : max_pages - 1;
+        const int page_id = bt[pi];
+        // keys: dim chunks w0 / 16 .. + 3
+        const uint32_t s_off = region < 2 ? ((uint32_t)(kvh * (DH / 8) + w0 / 16) * page + tok0) * 8 * E
+                                          : ((uint32_t)((nkvh + kvh) * DH) * page + tok0) * E;
+        const __amdgpu_buffer_rsrc_t pg = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<bf16_t *>(cache + (size_t)page_id * page_elems), 0, (uint32_t)(page_elems * E), 0x00020000);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(pg, (__attribute__((address_space(3))) void *)(buf + 512 * i + WAVE * wave_id), 16,
+                                                 region < 2 ? k_lane : v_lane, s_off, 0, 0);
     }
 }
 
-// A task is a block of consecutive tokens of one request: a workgroup has PRE_QWAVES x 2 waves;
-// wave q of either half takes QB blocks of 16 rows (tokens x the heads of one chunk of a
-// group), so a task covers 4 * QB * (16 / heads per chunk) tokens, starting at batch index
-// task_tok0[t].  The workgroup walks the keys that any of its rows sees, 64 at a time: the
-// first half of the waves takes the first 32 of them, the second half the other 32, each
-// with an online softmax of its own, and the two are merged at the end.  So a compute unit
-// holds two waves per SIMD that work on one task (while one waits for the softmax's
-// arithmetic the other feeds the matrix cores), however few tasks there are.  The keys and
-// values are copied to LDS once per workgroup, two buffers ahead of the one that is read.
-template <int DH, int QB>
+// One step of 32 keys for the wave's 32 rows, operands from the copy in LDS (`buf`: the step's 8 * DH
+// chunks).  p_row / lo_row: the last and first key that the lane's row may see; MASK: some row of
+// the wave does not see all 32 keys; p_max / lo_min bound what any row of the wave sees (values of
+// keys outside are not used at all, whatever the memory holds).
+template <int DH, bool MASK>
+__device__ __forceinline__ void attn_compute_lds(const u32x4 *__restrict__ buf, int k0, const u32x4 (&q)[DH / 16],
+                                               PrefillState<DH> &st, int p_row, int lo_row, int p_max, int lo_min,
+                                               float scale_log2, int n, int hi) {
+    f32x16 s;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) s[i] = 0.f;
+    {
+        // row m = n of the instruction: key tile n / 16, slot n % 16; dims 16 sidx + 8 hi ..: dim chunk 2 sidx + hi
+        const u32x4 *kb = buf + (n >> 4) * 2 * DH + hi * 16 + (n & 15);
+        u32x4 k[DH / 16];
+#pragma unroll
+        for (int sidx = 0; sidx < DH / 16; ++sidx) k[sidx] = kb[32 * sidx];
+#pragma unroll
+        for (int sidx = 0; sidx < DH / 16; ++sidx) s = mfma32(k[sidx], q[sidx], s);
+    }
+    __builtin_amdgcn_sched_barrier(0);             // the values' reads stay below the scores
+    // dim 32 t + n, keys 16 kk + 8 hi .. + 7: V tile kk, half hi
+    u32x4 v[DH / 32][2];
+    const u32x4 *vb = buf + 4 * DH + hi * DH + n;
+#pragma unroll
+    for (int t = 0; t < DH / 32; ++t)
+#pragma unroll
+        for (int kk = 0; kk < 2; ++kk) v[t][kk] = vb[kk * 2 * DH + 32 * t];
+    float x[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) x[i] = s[i];
+    if (MASK) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int j = key_of_score(k0, i, hi);
+            if (j > p_row || j < lo_row) x[i] = -INFINITY;
+        }
+    }
+    float mx = fmaxf(fmaxf(x[0], x[1]), x[2]);
+#pragma unroll
+    for (int i = 3; i < 15; i += 2) mx = fmaxf(fmaxf(mx, x[i]), x[i + 1]);
+    mx = fmaxf(mx, x[15]);
+    mx = max_over_halves(mx);
+    // the reference point of the exponentials moves only when the maximum has grown by more than
+    // 2^RESCALE_SLACK (see attn_softmax)
+    const float m_true = fmaxf(st.m, mx * scale_log2);
+    const float m_new = m_true - st.m <= RESCALE_SLACK ? st.m : m_true;       // false for the first keys (-inf)
+    const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+    const float alpha = fast_exp2(st.m - m_safe);
+    float p[16], sum = 0.f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        p[i] = fast_exp2(fmaf(x[i], scale_log2, -m_safe));
+        sum += p[i];
+    }
+    st.l = st.l * alpha + sum;
+    st.m = m_new;
+    if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+#pragma unroll
+        for (int t = 0; t < DH / 32; ++t) st.o[t] *= alpha;
+    }
+    u32x4 pb[2];
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk)
+        pb[kk] = u32x4{pack_bf16(p[8 * kk], p[8 * kk + 1]), pack_bf16(p[8 * kk + 2], p[8 * kk + 3]),
+                       pack_bf16(p[8 * kk + 4], p[8 * kk + 5]), pack_bf16(p[8 * kk + 6], p[8 * kk + 7])};
+    uint32_t keep[2][4];
+    if (MASK) {
+        // values of keys that no row sees are taken as zero: their memory may hold anything
+#pragma unroll
+        for (int kk = 0; kk < 2; ++kk) {
+#pragma unroll
+            for (int w = 0; w < 4; ++w) keep[kk][w] = 0xffffffffu;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const int j = k0 + 16 * kk + 8 * hi + e;
+                if (j > p_max || j < lo_min) keep[kk][e / 2] &= (e & 1) ? 0x0000ffffu : 0xffff0000u;
+            }
+        }
+    }
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+        for (int t = 0; t < DH / 32; ++t) {
+            u32x4 a = v[t][kk];
+            if (MASK) { a.x &= keep[kk][0]; a.y &= keep[kk][1]; a.z &= keep[kk][2]; a.w &= keep[kk][3]; }
+            st.o[t] = mfma32(a, pb[kk], st.o[t]);
+        }
+}
+
+// A task is a block of consecutive tokens of one request: a workgroup has PRE_QWAVES x 2 waves; wave q of
+// either half takes 32 rows (tokens x the heads of one chunk of a group), so a task covers
+// 4 * (32 / heads per chunk) tokens, starting at batch index task_tok0[t].  The workgroup walks the keys
+// that any of its rows sees, 64 at a time: the first half of the waves takes the first 32 of them, the
+// second half the other 32, each with an online softmax of its own, and the two are merged at the end.
+// So a compute unit holds two waves per SIMD that work on one task (while one waits for the softmax's
+// arithmetic the other feeds the matrix cores), however few tasks there are.  The keys and values are
+// copied to LDS once per workgroup, two buffers ahead of the one that is read: before a double step every
+// wave waits for its own part of its copy, then a barrier (which waits for LDS only) makes the whole copy
+// visible and says that the buffer of the double step before is free for the one two ahead.
+template <int DH>
 __global__ void __launch_bounds__(PRE_WAVES *WAVE, LCU_PRE_MIN_WAVES)
 attention_prefill_kernel(const bf16_t *__restrict__ q, int q_stride, bf16_t *__restrict__ out, int out_stride,
-                         const bf16_t *__restrict__ cache, const int *__restrict__ block_table, int max_pages,
-                         const int *__restrict__ q_start, const int *__restrict__ ctx_len,
-                         const int *__restrict__ task_req, const int *__restrict__ task_tok0, int n_tasks,
-                         int tasks_per_wg, int nh, int nkvh, int page, uint32_t tile_magic, float scale_log2, int window) {
+                           const bf16_t *__restrict__ cache, const int *__restrict__ block_table, int max_pages,
+                           const int *__restrict__ q_start, const int *__restrict__ ctx_len,
+                           const int *__restrict__ task_req, const int *__restrict__ task_tok0, int n_tasks,
+                           int tasks_per_wg, int nh, int nkvh, int page, uint32_t tile_magic, float scale_log2, int window) {
     extern __shared__ u32x4 lds_ring[];            // [PRE_RING][16 * DH]; at the end the halves' states
-    // the wave's number as a scalar: what follows from it (its rows' limits) then lives in scalar registers
     const int wave_id = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
     const int lane = threadIdx.x & (WAVE - 1), wave = wave_id % PRE_QWAVES, half = wave_id / PRE_QWAVES;
-    // a workgroup takes tasks_per_wg tasks one after the other (the host pairs a long one with
-    // a short one, so that workgroups take about equally long)
-    for (int task = blockIdx.x * tasks_per_wg; task < (blockIdx.x + 1) * tasks_per_wg && task < n_tasks; ++task) {
-    __syncthreads();                               // the last task's use of LDS is over (its copies landed before its merge)
-    const int l16 = lane & 15, grp = lane >> 4;
+    // Workgroups go to the chip's eight dies in turn (workgroup i to die i % 8), and each die has an L2 of
+    // its own.  The key/value head is the fastest index of the grid, so that the workgroups of one head
+    // (with 8 heads, or a multiple or a divisor of 8) all run on one die, whose L2 then holds that head's keys and
+    // values for all of them: with the task as the fastest index every die read every head's keys.
     const int g = nh / nkvh;
     const int chunks = (g + 15) / 16;
-    const int kvh = blockIdx.y / chunks, chunk = blockIdx.y % chunks;
+    const int head_chunk = blockIdx.x % (nkvh * chunks), wg = blockIdx.x / (nkvh * chunks);
+    for (int task = wg * tasks_per_wg; task < (wg + 1) * tasks_per_wg && task < n_tasks; ++task) {
+    __syncthreads();                               // the last task's use of LDS is over (its copies landed before its merge)
+    const int n = lane & 31, hi = lane >> 5;
+    const int kvh = head_chunk / chunks, chunk = head_chunk % chunks;
     const int hc = (g - 16 * chunk) < 16 ? (g - 16 * chunk) : 16;      // heads of this chunk
-    const int tokens_per_block = 16 / hc;                               // tokens in 16 rows
-    const int tokens_per_wave = QB * tokens_per_block;
+    const int tokens_per_wave = 32 / hc;                                // tokens in 32 rows
     const int r = task_req[task], task_tok = task_tok0[task];
     const int q_end = q_start[r + 1];
     const int ctx = ctx_len[r];
     const int head0 = kvh * g + 16 * chunk;
     const int tok0 = task_tok + wave * tokens_per_wave;                 // this wave's first token
-
-    u32x4 qv[QB][DH / 32];
-    int tok_row[QB];
     const int pos_of_tok = ctx - q_end;                                 // a token's position = its batch index + this
+
+    const int tok = tok0 + n / hc;
+    const bool valid = n < tokens_per_wave * hc && tok < q_end;
+    const int tok_row = valid ? tok : -1;
+    u32x4 qv[DH / 16];
+    {
+        const bf16_t *qrow = q + (size_t)(valid ? tok : task_tok) * q_stride + (size_t)(head0 + n % hc) * DH;
 #pragma unroll
-    for (int b = 0; b < QB; ++b) {
-        const int tok = tok0 + b * tokens_per_block + l16 / hc;
-        const bool valid = l16 < tokens_per_block * hc && tok < q_end;
-        tok_row[b] = valid ? tok : -1;
-        load_q<DH>(q + (size_t)(valid ? tok : task_tok) * q_stride + (size_t)(head0 + l16 % hc) * DH, valid, qv[b], grp);
+        for (int sidx = 0; sidx < DH / 16; ++sidx)
+            qv[sidx] = valid ? *(const u32x4 *)(qrow + 16 * sidx + 8 * hi) : u32x4{0u, 0u, 0u, 0u};
     }
     // what this wave sees (the same in all its lanes), and what the workgroup sees
     const bool wave_has = tok0 < q_end;
@@ -777,101 +802,109 @@ attention_prefill_kernel(const bf16_t *__restrict__ q, int q_stride, bf16_t *__r
     const int wg_p_min = ctx - (q_end - task_tok);
     const int wg_lo_min = window > 0 && wg_p_min - window + 1 > 0 ? wg_p_min - window + 1 : 0;
 
-    AttnState<DH, QB> st;
-    attn_init(st);
+    PrefillState<DH> st;
+    st.m = -INFINITY;
+    st.l = 0.f;
+#pragma unroll
+    for (int t = 0; t < DH / 32; ++t)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) st.o[t][i] = 0.f;
     const int *bt = block_table + (size_t)r * max_pages;
     const size_t page_elems = kv_page_elems(nkvh, DH, page);
     const int blk0 = wg_lo_min / 32, blk_end = wg_p_max / 32 + 1;
-    // Double steps of 64 keys; double step d is read from buffer d % PRE_RING while the loads of the
-    // next two are on their way.  Before one, every wave waits for its own part of its copy, then
-    // the barrier makes the whole copy visible and says that the buffer of the double step before
-    // is free for the one two ahead.
     const int n_dsteps = (blk_end - blk0 + 1) / 2;
 #pragma unroll
     for (int d = 0; d < PRE_RING - 1; ++d)
         stage_issue<DH>(lds_ring + d * 16 * DH, cache, bt, max_pages, page, tile_magic, page_elems, nkvh, kvh, (blk0 + 2 * d) * 32,
-                        wave_id);
+                          wave_id);
     int slot = 0, fill = PRE_RING - 1;
     for (int d = 0; d < n_dsteps; ++d) {
         wait_loads<(PRE_RING - 2) * (DH / 32)>();
         lds_barrier();
-        ring_step<DH, QB>(lds_ring + slot * 16 * DH + half * 8 * DH, lds_ring + fill * 16 * DH, cache, bt, max_pages, page,
-                          tile_magic, page_elems, nkvh, kvh, (blk0 + 2 * (d + PRE_RING - 1)) * 32, wave_id, blk0 + 2 * d + half,
-                          blk_end, wave_has,
-                          p_max, p_min, lo_min, lo_max, tok_row, pos_of_tok, window, qv, st, scale_log2);
+        // the copy of a later double step goes into the buffer that the barrier has freed; the two buffers
+        // are different ones of the ring, which the qualifiers of the pointers say: a read from LDS otherwise
+        // waits for every copy in flight, the one into `dst` included, as if it read what that copy writes
+        const u32x4 *__restrict__ src = lds_ring + slot * 16 * DH + half * 8 * DH;
+        u32x4 *__restrict__ dst = lds_ring + fill * 16 * DH;
+        stage_issue<DH>(dst, cache, bt, max_pages, page, tile_magic, page_elems, nkvh, kvh, (blk0 + 2 * (d + PRE_RING - 1)) * 32,
+                          wave_id);
+        const int blk = blk0 + 2 * d + half, k0 = blk * 32;
+        if (wave_has && blk < blk_end && k0 <= p_max && k0 + 31 >= lo_min) {
+            if (k0 + 31 > p_min || k0 < lo_max) {
+                const int p_row = tok_row < 0 ? -1 : tok_row + pos_of_tok;
+                const int lo_row = tok_row >= 0 && window > 0 && p_row - window + 1 > 0 ? p_row - window + 1 : 0;
+                attn_compute_lds<DH, true>(src, k0, qv, st, p_row, lo_row, p_max, lo_min, scale_log2, n, hi);
+            } else {
+                attn_compute_lds<DH, false>(src, k0, qv, st, 0, 0, p_max, lo_min, scale_log2, n, hi);
+            }
+        }
         slot = slot + 1 == PRE_RING ? 0 : slot + 1;
         fill = fill + 1 == PRE_RING ? 0 : fill + 1;
     }
     // ---- the second half hands its state to the first, which merges and writes
-    // The last copies into the ring (two double steps that nobody reads) may still be on their way: a
-    // barrier does not wait for a wave's copies from memory into LDS, and the states below overlay the
-    // ring.  So every wave waits for its own copies first; after the barrier none is in flight.
-    wait_loads<0>();
+    wait_loads<0>();                               // the last copies into the ring, which nobody reads, have landed
     __syncthreads();                               // every wave is done with the buffers
     float *xch = (float *)lds_ring;                // [value][query wave][lane]
-    constexpr int NV = QB * (2 + (DH / 16) * 4);
+    constexpr int NV = 2 + (DH / 32) * 16;
+    static_assert(NV * PRE_QWAVES * WAVE * 4 <= PRE_RING * 16 * DH * 16, "the halves' states fit the ring");
     if (half == 1) {
         int v = 0;
+        xch[((v++) * PRE_QWAVES + wave) * WAVE + lane] = st.m;
+        xch[((v++) * PRE_QWAVES + wave) * WAVE + lane] = st.l;
 #pragma unroll
-        for (int b = 0; b < QB; ++b) {
-            xch[((v++) * PRE_QWAVES + wave) * WAVE + lane] = st.m[b];
-            xch[((v++) * PRE_QWAVES + wave) * WAVE + lane] = st.l[b];
+        for (int t = 0; t < DH / 32; ++t)
 #pragma unroll
-            for (int dt = 0; dt < DH / 16; ++dt)
-#pragma unroll
-                for (int e = 0; e < 4; ++e) xch[((v++) * PRE_QWAVES + wave) * WAVE + lane] = st.o[b][dt][e];
-        }
+            for (int i = 0; i < 16; ++i) xch[((v++) * PRE_QWAVES + wave) * WAVE + lane] = st.o[t][i];
     }
     __syncthreads();
     if (half == 0) {
         int v = 0;
+        const float m1 = xch[((v++) * PRE_QWAVES + wave) * WAVE + lane];
+        const float l1 = xch[((v++) * PRE_QWAVES + wave) * WAVE + lane];
+        const float m = fmaxf(st.m, m1);
+        const float m_safe = m == -INFINITY ? 0.f : m;
+        const float a0 = fast_exp2(st.m - m_safe), a1 = fast_exp2(m1 - m_safe);
+        float l_all = st.l * a0 + l1 * a1;
+        l_all += __shfl_xor(l_all, 32, WAVE);
+        const float inv = 1.0f / l_all;
+        bf16_t *o = tok_row < 0 ? nullptr : out + (size_t)tok_row * out_stride + (size_t)(head0 + n % hc) * DH;
 #pragma unroll
-        for (int b = 0; b < QB; ++b) {
-            const float m1 = xch[((v++) * PRE_QWAVES + wave) * WAVE + lane];
-            const float l1 = xch[((v++) * PRE_QWAVES + wave) * WAVE + lane];
-            const float m = fmaxf(st.m[b], m1);
-            const float m_safe = m == -INFINITY ? 0.f : m;
-            const float a0 = fast_exp2(st.m[b] - m_safe), a1 = fast_exp2(m1 - m_safe);
-            float l_all = st.l[b] * a0 + l1 * a1;
-            l_all += __shfl_xor(l_all, 16, WAVE);
-            l_all += __shfl_xor(l_all, 32, WAVE);
-            const float inv = 1.0f / l_all;
-            bf16_t *o = tok_row[b] < 0 ? nullptr : out + (size_t)tok_row[b] * out_stride + (size_t)(head0 + l16 % hc) * DH;
+        for (int t = 0; t < DH / 32; ++t)
 #pragma unroll
-            for (int dt = 0; dt < DH / 16; ++dt) {
+            for (int b = 0; b < 4; ++b) {
                 float e4[4];
 #pragma unroll
                 for (int e = 0; e < 4; ++e)
-                    e4[e] = (st.o[b][dt][e] * a0 + xch[((v++) * PRE_QWAVES + wave) * WAVE + lane] * a1) * inv;
+                    e4[e] = (st.o[t][4 * b + e] * a0 + xch[((v++) * PRE_QWAVES + wave) * WAVE + lane] * a1) * inv;
                 if (o) {
                     u32x2 w;
                     w.x = pack_bf16(e4[0], e4[1]);
                     w.y = pack_bf16(e4[2], e4[3]);
-                    *(u32x2 *)(o + 16 * dt + 4 * grp) = w;
+                    *(u32x2 *)(o + 32 * t + 8 * b + 4 * hi) = w;
                 }
             }
-        }
-        static_assert(NV * PRE_QWAVES * WAVE * 4 <= PRE_RING * 16 * DH * 16, "the halves' states fit the ring");
     }
     }
 }
 
-template <int DH, int QB>
+template <int DH>
 static int launch_prefill(const void *q, int q_stride, void *out, int out_stride, const void *cache,
-                          const int *block_table, int max_pages, const int *q_start, const int *ctx_len,
-                          const int *task_req, const int *task_tok0, int n_tasks, int tasks_per_wg, int nh, int nkvh,
-                          int page, float scale, int window, hipStream_t stream) {
+                            const int *block_table, int max_pages, const int *q_start, const int *ctx_len,
+                            const int *task_req, const int *task_tok0, int n_tasks, int tasks_per_wg, int nh, int nkvh,
+                            int page, float scale, int window, hipStream_t stream) {
     const int g = nh / nkvh, chunks = (g + 15) / 16;
-    dim3 grid((n_tasks + tasks_per_wg - 1) / tasks_per_wg, nkvh * chunks), block(PRE_WAVES * WAVE);
+    const long long n_wg = (long long)((n_tasks + tasks_per_wg - 1) / tasks_per_wg) * nkvh * chunks;
+    if (n_wg > 0x7fffffffll) return LCU_BAD_ARGUMENT;
+    dim3 grid((unsigned)n_wg), block(PRE_WAVES * WAVE);
     constexpr size_t lds_bytes = (size_t)PRE_RING * 16 * DH * sizeof(u32x4);
     static bool allowed = false;                   // more than 64 KB of LDS must be asked for once
     if (!allowed) {
-        const hipError_t e = hipFuncSetAttribute((const void *)attention_prefill_kernel<DH, QB>,
+        const hipError_t e = hipFuncSetAttribute((const void *)attention_prefill_kernel<DH>,
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
         if (e != hipSuccess) return (int)e;
         allowed = true;
     }
-    attention_prefill_kernel<DH, QB><<<grid, block, lds_bytes, stream>>>(
+    attention_prefill_kernel<DH><<<grid, block, lds_bytes, stream>>>(
         (const bf16_t *)q, q_stride, (bf16_t *)out, out_stride, (const bf16_t *)cache, block_table, max_pages, q_start,
         ctx_len, task_req, task_tok0, n_tasks, tasks_per_wg, nh, nkvh, page,
         page == 16 ? 0u : (uint32_t)(0x100000000ull / (unsigned)(page / 16)) + 1u, scale * 1.4426950408889634f, window);
@@ -886,7 +919,7 @@ LCU_API int lcu_attention_prefill_tokens_per_task(int nh, int nkvh) {
     const int g = nh / nkvh;
     if (g > 16 && g % 16) return 0;       // chunks of a group must be equal for one task size
     const int hc = g < 16 ? g : 16;
-    return PRE_QWAVES * PRE_QB * (16 / hc);
+    return PRE_QWAVES * (32 / hc);
 }
 
 // task_req / task_tok0: [n_tasks], tasks cut from the batch with the size above; a
@@ -902,7 +935,7 @@ LCU_API int lcu_attention_prefill_bf16(const void *q, int q_stride, void *out, i
     if (tasks_per_wg < 1 || lcu_attention_prefill_tokens_per_task(nh, nkvh) == 0 || page <= 0 || page % 16 || max_pages <= 0 ||
         window < 0 || q_stride % 8 || out_stride % 4 || nkvh * ((nh / nkvh + 15) / 16) > 65535)
         return LCU_BAD_ARGUMENT;
-#define GO(D) return launch_prefill<D, PRE_QB>(q, q_stride, out, out_stride, cache, block_table, max_pages, q_start, ctx_len, task_req, task_tok0, n_tasks, tasks_per_wg, nh, nkvh, page, scale, window, stream)
+#define GO(D) return launch_prefill<D>(q, q_stride, out, out_stride, cache, block_table, max_pages, q_start, ctx_len, task_req, task_tok0, n_tasks, tasks_per_wg, nh, nkvh, page, scale, window, stream)
     if (dh == 128) GO(128);
     if (dh == 64) GO(64);
     if (dh == 96) GO(96);

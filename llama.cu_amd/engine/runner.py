@@ -68,18 +68,24 @@ class ModelRunner:
             if need is not None and not isinstance(need, CacheNeed):
                 raise ValueError(f"run order entry {i}: {need!r} is no cache need (parts.base.CacheNeed)")
         pools = sorted({n.pool() for n in needs if n is not None and n.pool() is not None})
+        page_of = [p[1] or self.page_size for p in pools]            # a pool's own page size, or the engine's
+        for ps in page_of:
+            if ps % 8:
+                raise ValueError(f"page_size {ps} must be a multiple of 8")
         elem = torch.empty(0, dtype=self.dtype).element_size()
-        if num_pages is None and max_tokens is not None:
-            num_pages = (int(max_tokens) + self.page_size - 1) // self.page_size
-        if num_pages is None:
+        tokens = int(max_tokens) if max_tokens is not None else None
+        if num_pages is not None:
+            tokens = int(num_pages) * self.page_size                  # the pool's size was given in the engine's pages
+        if tokens is None:
             # what the free memory holds, and no more than every slot filled to the limit
-            page_bytes = sum(n.page_bytes(self.page_size, elem) for n in needs if n is not None)
+            token_bytes = sum(n.page_bytes(1, elem) for n in needs if n is not None)
             free, _ = torch.cuda.mem_get_info(self.device)
-            by_memory = int(free * kv_fraction) // max(page_bytes, 1)
-            by_need = self.max_seqs * ((self.max_model_len + self.page_size - 1) // self.page_size)
-            num_pages = max(1, min(by_memory, by_need))
-        self.num_pages = int(num_pages)
-        self.groups = [CacheGroup(self.num_pages, self.page_size, p[0]) for p in pools]
+            by_memory = int(free * kv_fraction) // max(token_bytes, 1)
+            by_need = self.max_seqs * ((self.max_model_len + max(page_of + [self.page_size]) - 1) // self.page_size * self.page_size)
+            tokens = max(self.page_size, min(by_memory, by_need))
+        # every pool holds the same number of tokens, in pages of its own size
+        self.num_pages = (tokens + self.page_size - 1) // self.page_size
+        self.groups = [CacheGroup((tokens + ps - 1) // ps, ps, p[0]) for p, ps in zip(pools, page_of)]
         # a request's cache can be cut back to a shorter length only if every need's can
         self.can_truncate = all(n.can_truncate for n in needs if n is not None)
         self.cache = CacheManager(self.groups, self.max_seqs, can_truncate=self.can_truncate)
@@ -92,8 +98,9 @@ class ModelRunner:
                 self.caches.append(LayerCache())
             else:
                 group = pools.index(need.pool()) if need.pool() is not None else -1
-                self.caches.append(need.allocate(group, self.num_pages, self.page_size, self.max_seqs, self.dtype, self.device))
-        max_pages = [(self.max_model_len + self.page_size - 1) // self.page_size for _ in self.groups]
+                pages, ps = (self.groups[group].num_pages, page_of[group]) if group >= 0 else (self.num_pages, self.page_size)
+                self.caches.append(need.allocate(group, pages, ps, self.max_seqs, self.dtype, self.device))
+        max_pages = [(self.max_model_len + g.page_size - 1) // g.page_size for g in self.groups]
         self.builder = BatchBuilder(self.cache, self.max_batch_tokens, self.max_seqs, max_pages, self.device)
         # a debugging aid: pages that were given back, or went to another request, since the last step are
         # filled with NaN before the step runs, so that a read of memory that its request does not own shows
@@ -221,9 +228,7 @@ class ModelRunner:
         them asks for; a mixer without keys asks for nothing)."""
         best = 1
         for layer in self.model.layers:
-            ask = getattr(layer, "decode_splits", None)
-            if callable(ask):
-                best = max(best, int(ask(batch, max_ctx_len)))
+            best = max(best, int(layer.decode_splits(batch, max_ctx_len)))
         return best
 
     def step(self, req_ids: Sequence[int], tokens: Sequence[Sequence[int]],

@@ -13,6 +13,7 @@ from typing import Optional
 import torch
 
 from . import build
+from .tuning import TUNING, Tuning  # noqa: F401  (ops.TUNING may be replaced to try other numbers)
 
 F32, BF16 = 0, 1
 _TYPE = {torch.float32: F32, torch.bfloat16: BF16}
@@ -410,26 +411,28 @@ def attention_prefill(q, out, cache, block_table, q_start, ctx_len, task_req, ta
 
 
 def decode_splits(n_req: int, n_heads: int, n_kv_heads: int, max_ctx_len: int) -> int:
-    """Into how many parts the decode kernel cuts each request's keys.  Few requests: about one
-    workgroup for each of the 256 compute units, no part shorter than 512 keys, at most 32 parts
-    (measured on the Llama-3-8B shape from 2k to 128k keys: more parts cost more in the merge
-    than they gain; a single request with 128k keys wants 32).  Between half the chip's worth of
-    workgroups and all of it (17 to 31 requests of 8 key/value heads), where one part leaves
-    compute units idle and two parts are a wave and a bit: one part up to 4k keys (whole decode
-    steps with 2k keys gained nothing from more), beyond that up to 4 parts of at least 2048
-    keys, the fewest with which the workgroups fill whole waves of 256 about as well as any (20
-    requests are 160 workgroups: over 8k keys 161 us in one part, 118 in three, the whole step
-    8.7 against 7.9 ms).  From 256 workgroups on one part: the chip is full, and more parts
-    gained nothing (48 requests over 8k keys: 13.1 ms a step in one part, 13.2 in two).  The
-    length counts rounded up to a power of two, so that a growing context changes the choice, and
-    with it the rounding of the result and the captured graph that fits, only rarely."""
+    """Into how many parts the decode kernel cuts each request's keys (the numbers are ``TUNING``'s).
+    Few requests: about one workgroup for each compute unit, no part shorter than 512 keys, at most
+    32 parts (measured from 2k to 128k keys: more parts cost more in the merge than they gain; a
+    single request with 128k keys wants 32).  Between half the chip's worth of workgroups and all of
+    it (17 to 31 requests of 8 key/value heads), where one part leaves compute units idle and two
+    parts are a wave and a bit: one part up to 4k keys (whole decode steps with 2k keys gained
+    nothing from more), beyond that up to 4 parts of at least 2048 keys, the fewest with which the
+    workgroups fill whole waves of 256 about as well as any (20 requests are 160 workgroups: over 8k
+    keys 161 us in one part, 118 in three, the whole step 8.7 against 7.9 ms).  From 256 workgroups on
+    one part: the chip is full, and more parts gained nothing (48 requests over 8k keys: 13.1 ms a
+    step in one part, 13.2 in two).  The length counts rounded up to a power of two, so that a
+    growing context changes the choice, and with it the rounding of the result and the captured
+    graph that fits, only rarely."""
+    t = TUNING
     base = max(1, n_req * n_kv_heads * ((n_heads // n_kv_heads + 15) // 16))
     rounded = 1 << max(int(max_ctx_len) - 1, 0).bit_length()     # up to a power of two: the choice changes rarely
-    if base <= 128:
-        return max(1, min(32, 256 // base, rounded // 512))
-    most = min(4, rounded // 2048) if (rounded >= 8192 and base < 256) else 1
-    fill = [(base * s / 256) / -(-base * s // 256) for s in range(1, most + 1)]
-    return 1 + next(i for i, f in enumerate(fill) if f >= max(fill) - 0.07)
+    if base <= t.decode_few_workgroups:
+        return max(1, min(t.decode_max_parts, t.compute_units // base, rounded // t.decode_min_part_keys))
+    most = min(t.decode_long_max_parts, rounded // t.decode_long_part_keys) \
+        if (rounded >= t.decode_long_context and base < t.compute_units) else 1
+    fill = [(base * s / t.compute_units) / -(-base * s // t.compute_units) for s in range(1, most + 1)]
+    return 1 + next(i for i, f in enumerate(fill) if f >= max(fill) - t.decode_fill_slack)
 
 
 def paged_attention(q: torch.Tensor, out: torch.Tensor, cache: torch.Tensor, step, group: int, n_heads: int,
@@ -470,16 +473,11 @@ def paged_attention(q: torch.Tensor, out: torch.Tensor, cache: torch.Tensor, ste
 
 
 SKINNY_MAX_ROWS = 32      # what the kernel takes
-SKINNY_ROWS = 16          # up to here it beats the library's product (measured on the Llama-3-8B shapes) ...
-SKINNY_ROWS_PACKED = 24   # ... and up to here when it reads a packed weight and its epilogues save the kernels around it
-                          # (whole decode steps of the Llama-3-8B shape: +9 % at 17 rows, +4 % at 24)
-SKINNY_ROWS_SHORT_K = 32  # ... and up to here for packed weights with K <= 8192 (q/k/v, output, gate/up: +4.5 % at 28
-                          # rows, +2 % at 32; with the down projection as well the step at 32 rows was 2 % slower)
 
 
 def skinny_max_rows(packed: bool) -> int:
     """The most rows for which the weight-streaming kernel is ever chosen over the library."""
-    return SKINNY_ROWS_SHORT_K if packed else SKINNY_ROWS
+    return TUNING.skinny_rows_short_k if packed else TUNING.skinny_rows
 
 
 _EPILOGUES = {"bf16": 0, "f32": 1, "add_f32": 2, "swiglu": 3}
@@ -519,28 +517,31 @@ def skinny_weight_ok(w: torch.Tensor) -> bool:
 
 def skinny_preferred(m: int, n: int, k: int, out_dtype: torch.dtype, packed: bool = False) -> bool:
     """Whether the weight-streaming kernel is the faster choice for a plain bfloat16 product
-    of ``m`` rows with an ``[n, k]`` weight (measured against the library on the Llama-3-8B
-    shapes): always for very few rows and for float32 output; with a packed weight up to 24
-    rows, and up to 32 where K is at most 8192 (there it is within a tenth of the library on the large weights, and its epilogues save
-    the kernels around the product); without one, beyond 4 and up to 16 rows, only for small
-    weights (the library's split over K wins on the large ones)."""
+    of ``m`` rows with an ``[n, k]`` weight (``TUNING``'s numbers): always for very few rows and for
+    float32 output; with a packed weight up to 24 rows, and up to 32 where K is at most 8192 (there
+    it is within a tenth of the library on the large weights, and its epilogues save the kernels
+    around the product); without one, beyond 4 and up to 16 rows, only for small weights (the
+    library's split over K wins on the large ones)."""
+    t = TUNING
     if m > skinny_max_rows(packed):
         return False
-    if packed and m > SKINNY_ROWS_PACKED:
-        return k <= 8192                  # up to 32 rows, but not the products with a long K (the down projection)
-    return m <= (SKINNY_ROWS_PACKED if packed else 4) or out_dtype == torch.float32 or n * k <= (1 << 24)
+    if packed and m > t.skinny_rows_packed:
+        return k <= t.skinny_short_k       # up to 32 rows, but not the products with a long K (the down projection)
+    return m <= (t.skinny_rows_packed if packed else t.skinny_rows_any_weight) or out_dtype == torch.float32 \
+        or n * k <= t.skinny_small_weight
 
 
 def _skinny_tiles(n_features: int, m: int, packed: bool = False) -> int:
-    """Output tiles of 16 features per workgroup (measured on the Llama-3-8B shapes).  Plain
-    weights: as many as still leave about four workgroups for each of the 256 compute units.
-    Packed weights: two from 6144 features on, four for the widest with more than 8 rows."""
+    """Output tiles of 16 features per workgroup.  Plain weights: as many as still leave about four
+    workgroups for each compute unit.  Packed weights: two from 6144 features on, four for the
+    widest with more than 8 rows."""
+    t = TUNING
     if packed:
-        if n_features >= 65536 and m > 8:
+        if n_features >= t.skinny_four_tiles_from and m > 8:
             return 4
-        return 2 if n_features >= 6144 else 1
+        return 2 if n_features >= t.skinny_two_tiles_from else 1
     for tiles in (4, 2):
-        if n_features // (16 * tiles) >= 1024 and (tiles < 4 or m <= 32):
+        if n_features // (16 * tiles) >= t.skinny_workgroups_per_cu * t.compute_units and (tiles < 4 or m <= 32):
             return tiles
     return 1
 
@@ -581,7 +582,7 @@ def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = 
     if out.shape != (m, width):
         raise KernelError(f"gemm_skinny out: shape {tuple(out.shape)}, expected {(m, width)}")
     tiles = tiles or ((4 if (m > 8 or packed) else 2) if swiglu else _skinny_tiles(width, m, packed))
-    waves = waves or (8 if width <= 8192 else 4)
+    waves = waves or (8 if width <= TUNING.skinny_eight_waves_to else 4)
     lib = build.load("gemm_skinny")
     if row_sumsq is not None:
         if row_sumsq.dtype != torch.float32 or row_sumsq.dim() != 2 or row_sumsq.shape[0] != m or not row_sumsq.is_contiguous() \
@@ -688,8 +689,8 @@ def gemm_skinny_add_norm(x: torch.Tensor, w: torch.Tensor, residual: torch.Tenso
         raise KernelError(f"gemm_skinny_add_norm: the residual must be float32 {(m, n)}")
     if norm_weight.shape != (n,) or not norm_weight.is_contiguous():
         raise KernelError(f"gemm_skinny_add_norm: the norm's weight must be a contiguous [{n}] tensor")
-    tiles = tiles or (1 if n <= 8192 else 2)
-    waves = waves or (8 if n <= 8192 else 4)
+    tiles = tiles or (1 if n <= TUNING.skinny_eight_waves_to else 2)
+    waves = waves or (8 if n <= TUNING.skinny_eight_waves_to else 4)
     parts = (n + 16 * tiles - 1) // (16 * tiles)
     h = torch.empty((m, n), dtype=torch.bfloat16, device=x.device)
     sumsq = torch.empty((m, parts), dtype=torch.float32, device=x.device)

@@ -1,0 +1,47 @@
+"""The numbers by which the dispatcher chooses between kernels that compute the same thing.
+
+They were measured on one MI355X with the layer sizes of the Llama-3-8B shape (and checked on
+the Llama-2-7B and Llama-3-70B shapes): they change which kernel runs and how it is launched,
+never what comes out, so another shape or another card may want other numbers and nothing
+else.  All of them are here, as data; ``ops`` and ``parts.linear`` read ``TUNING`` and hold
+no such number of their own.  Replace fields (``dataclasses.replace``) or assign ``ops.TUNING``
+to try others.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+
+@dataclass(frozen=True)
+class Tuning:
+    # ---- the weight-streaming product for few rows (gemm_skinny.hip)
+    skinny_rows: int = 16               # up to here it beats the library's product with a plain weight ...
+    skinny_rows_packed: int = 24        # ... up to here with a packed weight, whose epilogues save the kernels around it
+                                        # (whole decode steps: +9 % at 17 rows, +4 % at 24)
+    skinny_rows_short_k: int = 32       # ... and up to here for packed weights with K <= skinny_short_k (q/k/v, output,
+                                        # gate/up: +4.5 % at 28 rows, +2 % at 32; with the down projection too, 2 % slower)
+    skinny_short_k: int = 8192
+    skinny_rows_any_weight: int = 4     # so few rows always go to it
+    skinny_small_weight: int = 1 << 24  # without a packed copy, beyond 4 rows only weights up to this many elements
+    skinny_two_tiles_from: int = 6144   # packed: two tiles of 16 features a workgroup from this many features on ...
+    skinny_four_tiles_from: int = 65536  # ... four for the widest, with more than 8 rows
+    skinny_workgroups_per_cu: int = 4   # plain: as many tiles as still leave this many workgroups for each compute unit
+    skinny_eight_waves_to: int = 8192   # eight waves share a workgroup's K up to this many output features, four beyond
+    compute_units: int = 256
+    # ---- the product that shares the rows through LDS (gemm_mid.hip, 17 to 128 rows)
+    mid_long_k: int = 8192              # a weight with a longer K (the down projection) goes to it from 17 rows on,
+                                        # and with a plain (not packed) weight only such weights go to it at all
+    mid_swiglu_features: int = 8192     # gate/up with SwiGLU goes to it from this many rows of the weight on
+    mid_min_slice_steps: int = 4        # a slice of K keeps at least this many macro-steps of 128
+    mid_max_slices: int = 8
+    # ---- the decode attention's cut of a request's keys into parts (attention_mfma.hip)
+    decode_min_part_keys: int = 512     # no part shorter than this
+    decode_max_parts: int = 32
+    decode_few_workgroups: int = 128    # up to this many workgroups without parts: about one workgroup per compute unit
+    decode_long_context: int = 8192     # between half the chip's worth of workgroups and all of it: parts only from here on,
+    decode_long_part_keys: int = 2048   # of at least this many keys,
+    decode_long_max_parts: int = 4      # at most this many,
+    decode_fill_slack: float = 0.07     # the fewest that fill whole waves of workgroups within this of the best
+
+
+TUNING = Tuning()

@@ -24,7 +24,7 @@ from ..weights.loader import fused_rows
 class Attention(Part):
 
     def __init__(self, hidden_size: int, heads: int, kv_heads: int, head_dim: int, scale: Optional[float] = None,
-                 window: int = 0, position: Optional[PartSpec] = None, shares_kv: bool = False):
+                 window: int = 0, position: Optional[PartSpec] = None, shares_kv: bool = False, page_size: int = 0):
         if heads % kv_heads:
             raise ValueError(f"attention: {heads} heads are no multiple of {kv_heads} key/value heads")
         if head_dim % 16 or head_dim > 256:
@@ -33,6 +33,7 @@ class Attention(Part):
         self.hidden_size, self.heads, self.kv_heads, self.head_dim = int(hidden_size), int(heads), int(kv_heads), int(head_dim)
         self.scale = float(scale) if scale is not None else float(head_dim) ** -0.5
         self.window = int(window or 0)
+        self.own_page_size = int(page_size or 0)  # tokens per page of this layer's cache; 0: the engine's default
         self.shares_kv = bool(shares_kv)          # reads another layer's keys and values: has q and o only
         self.position = make_part("position", position or PartSpec("none"))
         self.graph_safe = self.position.graph_safe
@@ -51,7 +52,7 @@ class Attention(Part):
         return [] if self.shares_kv else [(("q_proj.weight", "k_proj.weight", "v_proj.weight"), 0)]
 
     def cache_need(self):
-        return PagedKV(self.kv_heads, self.head_dim, self.window)
+        return PagedKV(self.kv_heads, self.head_dim, self.window, self.own_page_size)
 
     def decode_splits(self, batch: int, max_ctx_len: int) -> int:
         """Into how many parts the decode kernel should cut each request's keys when ``batch``
@@ -88,6 +89,7 @@ class Attention(Part):
         if self.shares_kv == cache.writes:
             raise ops.KernelError("attention: a layer that shares another's keys and values must be given that "
                                   "layer's cache in the run order (and only such a layer)")
+        page_size = cache.page_size or self.page_size          # the cache's own page size (the engine's default)
         rot = self.position.rotary_tables()
         cos, sin, rot_dim, pairing = rot if rot is not None else (None, None, 0, 0)
         store = cache.writes and not self.shares_kv
@@ -97,7 +99,7 @@ class Attention(Part):
                 and self.dtype == torch.bfloat16 and skinny_takes(n_rows, self.w_qkv, preferred=True):
             # few rows: the product rotates q and k and writes k and v into the pages itself
             qkv = linear_qkv_rope(h, self.w_qkv, step.positions, step.slots(cache.group), cos, sin, cache.pages,
-                                  nh, nkv, dh, self.page_size)
+                                  nh, nkv, dh, page_size)
         if qkv is None:
             if isinstance(h, ScaledRows):
                 qkv = linear_scaled(h, self.w_qkv)
@@ -106,9 +108,9 @@ class Attention(Part):
             self.position.apply(qkv, step.positions, nh, 0 if self.shares_kv else nkv, dh)
             ops.rope_kv_store(qkv, step.positions, nh, nkv, dh, cos, sin, rot_dim, pairing,
                               cache.pages if store else None, step.slots(cache.group) if store else None,
-                              self.page_size)
+                              page_size)
         out = torch.empty((n_rows, nh * dh), dtype=self.dtype, device=qkv.device)
-        ops.paged_attention(qkv, out, cache.pages, step, cache.group, nh, nkv, dh, self.page_size, self.scale,
+        ops.paged_attention(qkv, out, cache.pages, step, cache.group, nh, nkv, dh, page_size, self.scale,
                             self.window)
         if into is not None:
             residual, norm = into

@@ -82,16 +82,17 @@ class LayerCache:
     pages: Optional[torch.Tensor] = None
     writes: bool = True
     state: Optional[torch.Tensor] = None
+    page_size: int = 0          # tokens per page of ``pages`` (0: no pages)
 
 
 class CacheNeed:
     """What a mixer asks of the cache manager.  The engine knows no kind of need by name: it asks
     every need these questions.
 
-    ``pool()``        None, or ``(window,)``: the need is pages of keys and values, and needs with
-                      an equal answer share one pool of page ids and one block table per request
+    ``pool()``        None, or ``(window, page_size)``: the need is pages of keys and values, and needs
+                      with an equal answer share one pool of page ids and one block table per request
                       (``window`` 0: every token is kept; w: pages that a window of w tokens has
-                      passed are given back);
+                      passed are given back; ``page_size`` 0: the engine's default);
     ``page_bytes(page_size, elem_size)``   bytes of one page of this need (0 if it has no pages);
     ``allocate(group, num_pages, page_size, slots, dtype, device)``   the memory, as a LayerCache;
     ``can_truncate``  whether what the need holds for a request can be cut back to a shorter
@@ -118,16 +119,17 @@ class PagedKV(CacheNeed):
     kv_heads: int
     head_dim: int
     window: int = 0          # 0: all tokens
+    page_size: int = 0       # tokens per page; 0: the engine's default
 
     def pool(self):
-        return (self.window,)
+        return (self.window, self.page_size)
 
     def page_bytes(self, page_size: int, elem_size: int) -> int:
         return 2 * self.kv_heads * self.head_dim * page_size * elem_size
 
     def allocate(self, group, num_pages, page_size, slots, dtype, device) -> LayerCache:
         pages = torch.zeros((num_pages, 2, self.kv_heads * self.head_dim * page_size), dtype=dtype, device=device)
-        return LayerCache(group=group, pages=pages)
+        return LayerCache(group=group, pages=pages, page_size=page_size)
 
 
 @dataclass(frozen=True)
@@ -175,6 +177,38 @@ class Part:
     # if all it does is launch work on the current stream whose shape depends on the batch's
     # sizes alone, never on values it reads on the host (lengths, positions, slots).
     graph_safe = False
+
+    # ---- what a part may offer so that kernels between it and its neighbours are saved.  All of it is
+    # optional: a part that leaves these as they are is never given anything but plain rows, and
+    # everything it returns is plain rows; blocks and the model ask through these names only.
+    #
+    # norm:  ``deferrable``: the norm is a factor per row times a weight per column (``weight``, ``size``,
+    #        ``eps``), so the factor may be applied after the next matrix product (ScaledRows);
+    #        ``takes_planes``: ``forward(x, delta)`` also takes float32 planes ``[planes, rows, width]``
+    #        of partial sums as ``delta``.
+    # mixer, feed-forward:  ``ends_in_norm``: ``forward(..., into=(residual, norm))`` may add its output to
+    #        the residual stream itself and return ScaledRows made with ``norm``;
+    #        ``ends_in_planes``: ``forward(..., planes_ok=True)`` may return float32 planes;
+    #        ``takes_scaled_rows(n_rows)``: whether ``forward`` takes ScaledRows of that many rows.
+    # block: ``ends_in_next_norm``: ``forward(..., next_norm=)`` may end in the norm that follows the block;
+    #        ``ends_in_planes`` / ``takes_planes`` / ``takes_scaled_rows`` as above, for its last branch
+    #        and its first norm.
+    deferrable = False
+    takes_planes = False
+    ends_in_norm = False
+    ends_in_planes = False
+    ends_in_next_norm = False
+
+    def takes_scaled_rows(self, n_rows: int) -> bool:
+        return False
+
+    # block: the norm that a block starts with, if whoever runs before it may end in it (else None)
+    first_norm = None
+
+    def decode_splits(self, batch: int, max_ctx_len: int) -> int:
+        """Into how many parts a mixer (or a block, for its mixer) wants a decoding request's keys cut when
+        ``batch`` requests decode over at most ``max_ctx_len`` keys; a captured graph fixes the number."""
+        return 1
 
     def tensors(self) -> Dict[str, TensorSpec]:
         return {}

@@ -25,8 +25,7 @@ class PreNormBlock(Part):
         self.ffn = make_part("ffn", ffn)
         self.graph_safe = all(p.graph_safe for p in (self.norm1, self.mixer, self.norm2, self.ffn))
         # parts that say so may pass rows between them whose normalisation is still to be applied
-        self._fuse = (getattr(self.mixer, "ends_in_norm", False) and getattr(self.norm2, "deferrable", False)
-                      and callable(getattr(self.ffn, "takes_scaled_rows", None)))
+        self._fuse = self.mixer.ends_in_norm and self.norm2.deferrable
 
     def _children(self):
         return [(self.specs[k].name, getattr(self, k)) for k in ("norm1", "mixer", "norm2", "ffn")]
@@ -53,8 +52,11 @@ class PreNormBlock(Part):
         return self.mixer.cache_need()
 
     def decode_splits(self, batch: int, max_ctx_len: int) -> int:
-        ask = getattr(self.mixer, "decode_splits", None)
-        return int(ask(batch, max_ctx_len)) if callable(ask) else 1
+        return int(self.mixer.decode_splits(batch, max_ctx_len))
+
+    @property
+    def first_norm(self):
+        return self.norm1
 
     ends_in_next_norm = True     # forward takes ``next_norm``
     ends_in_planes = True        # forward takes ``planes_ok``
@@ -62,13 +64,12 @@ class PreNormBlock(Part):
     @property
     def takes_planes(self) -> bool:
         """Whether ``pending`` may be float32 planes of partial sums: the first norm adds them."""
-        return bool(getattr(self.norm1, "takes_planes", False))
+        return bool(self.norm1.takes_planes)
 
     def takes_scaled_rows(self, n_rows: int) -> bool:
         """Whether ``forward`` could be given, as ``pending``, ScaledRows of ``n_rows`` rows made
         with this block's first norm in the place of the last branch's output."""
-        fn = getattr(self.mixer, "takes_scaled_rows", None)
-        return getattr(self.norm1, "deferrable", False) and callable(fn) and fn(n_rows)
+        return bool(self.norm1.deferrable and self.mixer.takes_scaled_rows(n_rows))
 
     def forward(self, x: torch.Tensor, pending, step, cache, next_norm=None, planes_ok=False):
         """``pending``: the last branch's output, not yet added to ``x`` (or None, or ScaledRows
@@ -79,12 +80,12 @@ class PreNormBlock(Part):
         ``pending``."""
         h = pending if isinstance(pending, ScaledRows) else self.norm1.forward(x, pending)
         n_rows = x.shape[0]
-        ffn_into = (x, next_norm) if next_norm is not None and getattr(self.ffn, "ends_in_norm", False) else None
+        ffn_into = (x, next_norm) if next_norm is not None and self.ffn.ends_in_norm else None
         ffn_kw = {"into": ffn_into} if ffn_into else {}
-        if planes_ok and getattr(self.ffn, "ends_in_planes", False):
+        if planes_ok and self.ffn.ends_in_planes:
             ffn_kw["planes_ok"] = True
         mixer_kw = {}
-        if getattr(self.norm2, "takes_planes", False) and getattr(self.mixer, "ends_in_planes", False):
+        if self.norm2.takes_planes and self.mixer.ends_in_planes:
             mixer_kw["planes_ok"] = True
         if self._fuse and self.ffn.takes_scaled_rows(n_rows):
             # the mixer may end with the residual sum and the second norm's weight in its last

@@ -141,10 +141,11 @@ def library_friendly_rows(di: int, d: int, device) -> int:
 
 def _mid_slices(n_features: int, k: int) -> int:
     """Into how many slices of K the kernel for 17 to 128 rows cuts a product, so that about one
-    workgroup (64 features and a slice) stands on each of the 256 compute units; a slice keeps at
-    least four macro-steps of 128."""
+    workgroup (64 features and a slice) stands on each compute unit; a slice keeps at least four
+    macro-steps of 128."""
+    t = ops.TUNING
     groups = -(-n_features // 64)
-    return max(1, min(round(256 / groups), 8, k // 512))
+    return max(1, min(round(t.compute_units / groups), t.mid_max_slices, k // (128 * t.mid_min_slice_steps)))
 
 
 def mid_takes(n_rows: int, weight: Union[torch.Tensor, Weight]) -> bool:
@@ -154,14 +155,16 @@ def mid_takes(n_rows: int, weight: Union[torch.Tensor, Weight]) -> bool:
     more beyond, the down projection with a plain one too).  A packed weight with a long K (the
     down projection) it takes from 17 rows on: 24 us and 5 for the norm kernel against 33 to 40 of
     the weight-streaming kernel."""
+    t = ops.TUNING
     w, packed = _split(weight)
-    fewest = ops.SKINNY_ROWS if (packed is not None and w.dim() == 2 and w.shape[1] > 8192) else ops.SKINNY_ROWS_SHORT_K
+    long_k = w.dim() == 2 and w.shape[1] > t.mid_long_k
+    fewest = t.skinny_rows if (packed is not None and long_k) else t.skinny_rows_short_k
     if not (fewest < n_rows <= ops.MID_MAX_ROWS and w.dtype == torch.bfloat16 and w.is_cuda and w.dim() == 2
             and w.shape[1] % 128 == 0 and w.shape[0] % 16 == 0):
         return False
     # products that are not cut over K stay with the library; a plain weight only with a long K (measured: the
     # output projections of the 8B and 70B shapes with plain weights are no faster than the library's)
-    return _mid_slices(w.shape[0], w.shape[1]) >= 2 and (packed is not None or w.shape[1] > 8192)
+    return _mid_slices(w.shape[0], w.shape[1]) >= 2 and (packed is not None or long_k)
 
 
 def linear_planes(a: torch.Tensor, weight: Union[torch.Tensor, Weight]) -> torch.Tensor:
@@ -180,8 +183,8 @@ def mid_swiglu_takes(n_rows: int, weight: Union[torch.Tensor, Weight]) -> bool:
     activation kernel after it, and from 17 rows on than the weight-streaming kernel: 46 against
     52 to 55 us on the Llama-3-8B shape)."""
     w, packed = _split(weight)
-    return (16 < n_rows <= ops.MID_MAX_ROWS and packed is not None and w.shape[0] % 32 == 0 and w.shape[1] % 128 == 0
-            and w.shape[0] >= 8192)
+    return (ops.TUNING.skinny_rows < n_rows <= ops.MID_MAX_ROWS and packed is not None and w.shape[0] % 32 == 0
+            and w.shape[1] % 128 == 0 and w.shape[0] >= ops.TUNING.mid_swiglu_features)
 
 
 def linear_swiglu_mid(h, weight: Union[torch.Tensor, Weight]) -> torch.Tensor:

@@ -145,25 +145,22 @@ class DecoderModel:
                 # matrix with the final norm
                 if i + 1 < len(order):
                     follower = self.layers[order[i + 1].layer]
-                    norm = getattr(follower, "norm1", None)
+                    norm = follower.first_norm
                 else:
-                    follower = self.head if step.logits_all and getattr(self.final_norm, "deferrable", False) else None
+                    follower = self.head if step.logits_all and self.final_norm.deferrable else None
                     norm = self.final_norm
-                takes = getattr(follower, "takes_scaled_rows", None)
                 layer = self.layers[e.layer]
                 kw = {}
-                if callable(takes) and getattr(layer, "ends_in_next_norm", False) and takes(x.shape[0]):
+                if follower is not None and norm is not None and layer.ends_in_next_norm and follower.takes_scaled_rows(x.shape[0]):
                     kw["next_norm"] = norm
                 # a block may leave its last product's partial sums to the norm that adds its output,
                 # if that norm takes them: the next block's first, or the final norm when no rows are
                 # gathered before it
-                if getattr(layer, "ends_in_planes", False):
-                    if i + 1 < len(order):
-                        kw["planes_ok"] = bool(getattr(self.layers[order[i + 1].layer], "takes_planes", False))
-                    else:
-                        kw["planes_ok"] = bool(step.logits_all and getattr(self.final_norm, "takes_planes", False))
-                if not kw.get("planes_ok"):
-                    kw.pop("planes_ok", None)
+                if layer.ends_in_planes:
+                    takes = self.layers[order[i + 1].layer].takes_planes if i + 1 < len(order) \
+                        else (step.logits_all and self.final_norm.takes_planes)
+                    if takes:
+                        kw["planes_ok"] = True
                 pending = layer.forward(x, pending, step, caches[i], **kw)
             if step.n_logits == 0:
                 return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=x.device)

@@ -11,7 +11,7 @@ from typing import List, Sequence, Tuple
 
 import torch
 
-from ..kernels import build
+from ..kernels import build, ops
 from ..kernels.ops import KernelError, _check, _gpu, _ptr, _stream, to_device as _to_device
 from .params import SamplingParams
 
@@ -87,12 +87,13 @@ class Sampler:
                                [uniform(p.seed, k[0], k[1]) for p, k in zip(params, keys)])
         out = argmax(logits)
         if random_rows:
-            idx = _to_device(random_rows, torch.long, logits.device)
-            sub = logits if len(random_rows) == logits.shape[0] else logits[idx]
+            # the rows that draw are gathered, drawn from and put back by the engine's own small kernels
+            both = _to_device([random_rows, list(range(len(random_rows)))], torch.int32, logits.device)
+            sub = ops.gather_rows(logits, both[0])
             drawn = sample_rows(sub, [params[i].temperature for i in random_rows], [params[i].top_p for i in random_rows],
                                 [params[i].top_k for i in random_rows],
                                 [uniform(params[i].seed, keys[i][0], keys[i][1]) for i in random_rows])
-            out[idx] = drawn
+            ops.feed_tokens(out, drawn, both[1], both[0])               # out[random_rows[i]] = drawn[i]
         return out
 
     def sample(self, logits: torch.Tensor, params: Sequence[SamplingParams],
@@ -105,7 +106,7 @@ class Sampler:
         random_rows = [i for i, p in enumerate(params) if not p.is_argmax]
         if not random_rows:
             return greedy.tolist()
-        sub = logits if len(random_rows) == rows else logits[torch.tensor(random_rows, device=logits.device)]
+        sub = logits if len(random_rows) == rows else ops.gather_rows(logits, _to_device(random_rows, torch.int32, logits.device))
         drawn = sample_rows(sub, [params[i].temperature for i in random_rows], [params[i].top_p for i in random_rows],
                             [params[i].top_k for i in random_rows],
                             [uniform(params[i].seed, keys[i][0], keys[i][1]) for i in random_rows]).tolist()

@@ -227,6 +227,36 @@ def test_window_with_pages_of_its_own(dtype):
     runner.cache.check()
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_layer_with_pages_of_its_own_size(dtype):
+    """Layer 1 asks for pages of 32 tokens while the engine's are 16: its keys and values get a pool of
+    their own, with its own block table, and the logits are those of the plain implementation; a mixed
+    replay gives all pages of both pools back."""
+    from llama_cu_amd.config import LlamaConfig
+    from llama_cu_amd.engine.trace import TraceReplayer
+    from llama_cu_amd.models.llama import llama_spec
+    cfg_d = dict(common.TINY_B, num_hidden_layers=2, head_dim=64, num_attention_heads=2, num_key_value_heads=1)
+    spec = llama_spec(LlamaConfig.from_dict(cfg_d))
+    spec.layers[1].params["mixer"].params["page_size"] = 32
+    std = 0.15 if dtype == "float32" else common.BF16_STD
+    reqs = common.random_requests(384, [70, 33, 120, 9], 4)
+    steps, max_tokens = common.trace_mixed(reqs, seed=1, max_live=3)
+    runner, w = runner_for(spec, 6, dtype, std=std, max_tokens=max_tokens, max_seqs=4, max_batch_tokens=max_tokens, page_size=16)
+    assert [(g.page_size, g.num_pages) for g in runner.groups] == [(16, max_tokens // 16), (32, max_tokens // 32)]
+    assert runner.caches[0].pages.shape[2] == 64 * 16 and runner.caches[1].pages.shape[2] == 64 * 32
+    pcfg = plain.PlainConfig.from_dict(cfg_d)
+    want = {name: plain.forward(pcfg, w, toks) for name, toks in reqs.items()}
+    rep = TraceReplayer(runner)
+    outputs = {}
+    for st in steps:
+        out = rep.step(st)
+        if out is not None:
+            outputs[st["step"]] = out
+    common.assert_matches_plain(common.collect(steps, outputs, 384), want, dtype, "pages of 16 and 32")
+    runner.cache.check()
+    assert [runner.cache.free_pages(g) for g in range(2)] == [max_tokens // 16, max_tokens // 32]
+
+
 # ----------------------------------------------------------------------------- a toy mixer with state of its own
 def test_a_toy_mixer_with_state_is_registered_built_and_stepped():
     """The mixer ``running_mean`` is defined here: its output at a token is a matrix times
