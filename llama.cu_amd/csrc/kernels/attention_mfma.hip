@@ -612,49 +612,102 @@ __device__ __forceinline__ float max_over_halves(float x) {
 // tile).  Steps beyond the end of the keys are copied all the same, from the pages that the clamped block
 // table names (valid memory), into a buffer that nobody reads: no branch around a load.  A page holds
 // less than 2 GiB (the host checks).
+// What a lane adds to the scalar part of its chunks' addresses: the same in every step, so it is made
+// once per task and kept (one register for the keys, one per load for the values).
 template <int DH>
-__device__ __forceinline__ void stage_issue(u32x4 *__restrict__ buf, const bf16_t *__restrict__ cache,
-                                              const int *__restrict__ bt, int max_pages, int page, uint32_t tile_magic,
-                                              size_t page_elems, int nkvh, int kvh, int k0, int wave_id) {
+struct StageLane {
+    uint32_t k;               // keys: a wave holds 4 dim chunks x 16 slots
+    uint32_t v[DH / 32];      // values: the lane's chunk is number w0 + lane of [half][dim] (a wave may hold the end of
+                              // one half and the start of the other where head_dim is no multiple of 64)
+};
+
+template <int DH>
+__device__ __forceinline__ void stage_lane(StageLane<DH> &sl, int page, int wave_id, int lane) {
     constexpr uint32_t E = sizeof(bf16_t);
-    const int tiles_per_page = page / 16;
-    int tid = threadIdx.x;
-    asm volatile("" : "+v"(tid));                  // made anew in every step, not kept in registers across the loop
-    const int lane = tid & (WAVE - 1);
     const uint32_t k_tok = (lane & 3) | ((lane & 4) << 1) | ((lane & 8) >> 1);
-    const uint32_t k_lane = ((uint32_t)(lane >> 4) * page + k_tok) * 8 * E;      // a wave: 4 dim chunks x 16 slots
+    sl.k = ((uint32_t)(lane >> 4) * page + k_tok) * 8 * E;
+#pragma unroll
+    for (int i = 0; i < DH / 32; ++i) {
+        const int w0 = (wave_id * WAVE + 512 * i) % (2 * DH);
+        const uint32_t v_at = (uint32_t)(w0 + lane), v_half = v_at / DH, v_dim = v_at - v_half * DH;
+        sl.v[i] = (v_dim * page + 8 * v_half) * E;
+    }
+}
+
+// The pages of the wave's chunks of the double step at k0 (through the scalar unit), and each chunk's
+// first token in its page.  Read one double step before the copy that uses them, so that the copy does not
+// wait for the table.
+template <int DH, bool PAGE16>
+__device__ __forceinline__ void stage_pages(int *page_id, uint32_t *tok0, const int *__restrict__ bt,
+                                            int max_pages, int page, uint32_t tile_magic, int k0, int wave_id) {
+    const int tiles_per_page = page / 16;
 #pragma unroll
     for (int i = 0; i < DH / 32; ++i) {
         const int cw = wave_id * WAVE + 512 * i;                  // the wave's first chunk
-        const int sub = cw / (8 * DH), c = cw % (8 * DH);
-        const int region = c / (2 * DH), w0 = c % (2 * DH), t = region & 1;
-        // values: the lane's chunk is number w0 + lane of [half][dim] (a wave may hold the end of one half
-        // and the start of the other where head_dim is no multiple of 64)
-        const uint32_t v_at = (uint32_t)(w0 + lane), v_half = v_at / DH, v_dim = v_at - v_half * DH;
-        const uint32_t v_lane = (v_dim * page + 8 * v_half) * E;
+        const int sub = cw / (8 * DH), region = (cw % (8 * DH)) / (2 * DH), t = region & 1;
         const uint32_t tile = (uint32_t)(k0 >> 4) + 2 * sub + t;
-        int pi = tile_magic ? (int)__umulhi(tile, tile_magic) : (int)tile;
-        const uint32_t tok0 = (tile - (uint32_t)pi * tiles_per_page) * 16;
+        int pi = (int)tile;                                       // pages of 16 keys: the page is the tile
+        tok0[i] = 0;
+        if (!PAGE16) {
+            pi = (int)__umulhi(tile, tile_magic);
+            tok0[i] = (tile - (uint32_t)pi * tiles_per_page) * 16;
+        }
         pi = pi < max_pages ? pi : max_pages - 1;
-        const int page_id = bt[pi];
-        // keys: dim chunks w0 / 16 .. + 3
-        const uint32_t s_off = region < 2 ? ((uint32_t)(kvh * (DH / 8) + w0 / 16) * page + tok0) * 8 * E
-                                          : ((uint32_t)((nkvh + kvh) * DH) * page + tok0) * E;
-        const __amdgpu_buffer_rsrc_t pg = __builtin_amdgcn_make_buffer_rsrc(
-            const_cast<bf16_t *>(cache + (size_t)page_id * page_elems), 0, (uint32_t)(page_elems * E), 0x00020000);
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(pg, (__attribute__((address_space(3))) void *)(buf + 512 * i + WAVE * wave_id), 16,
-                                                 region < 2 ? k_lane : v_lane, s_off, 0, 0);
+        page_id[i] = bt[pi];
+    }
+}
+
+// FLAT: the whole cache of the layer is one buffer of less than 4 GiB (the host says), and a page is an
+// offset in it: two scalar instructions per chunk.  Else the buffer of a load is its page, whose 64-bit
+// address is made per chunk (a dozen scalar instructions: with four chunks a double step they were a third
+// of all the instructions a wave issued).
+template <int DH>
+__device__ __forceinline__ void stage_issue(u32x4 *__restrict__ buf, const bf16_t *__restrict__ cache, bool FLAT,
+                                            uint32_t cache_bytes, const int *page_id,
+                                            const uint32_t *tok0, const StageLane<DH> &sl, int page, size_t page_elems,
+                                            int nkvh, int kvh, int wave_id) {
+    constexpr uint32_t E = sizeof(bf16_t);
+#pragma unroll
+    for (int i = 0; i < DH / 32; ++i) {
+        const int cw = wave_id * WAVE + 512 * i;                  // the wave's first chunk
+        const int c = cw % (8 * DH);
+        const int region = c / (2 * DH), w0 = c % (2 * DH);
+        // keys: dim chunks w0 / 16 .. + 3 of the tile
+        const uint32_t s_off = region < 2 ? ((uint32_t)(kvh * (DH / 8) + w0 / 16) * page + tok0[i]) * 8 * E
+                                          : ((uint32_t)((nkvh + kvh) * DH) * page + tok0[i]) * E;
+        // (a plain variable: the compiler's pass for the host refuses the load builtin with an argument whose
+        // type depends on a template parameter)
+        const uint32_t lane_off = region < 2 ? sl.k : sl.v[i];
+        if (FLAT) {
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(
+                __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t *>(cache), 0, cache_bytes, 0x00020000),
+                (__attribute__((address_space(3))) void *)(buf + 512 * i + WAVE * wave_id), 16, lane_off,
+                (uint32_t)page_id[i] * (uint32_t)(page_elems * E) + s_off, 0, 0);
+        } else {
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(
+                __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t *>(cache + (size_t)page_id[i] * page_elems), 0,
+                                                  (uint32_t)(page_elems * E), 0x00020000),
+                (__attribute__((address_space(3))) void *)(buf + 512 * i + WAVE * wave_id), 16, lane_off,
+                s_off, 0, 0);
+        }
     }
 }
 
 // One step of 32 keys for the wave's 32 rows, operands from the copy in LDS (`buf`: the step's 8 * DH
-// chunks).  p_row / lo_row: the last and first key that the lane's row may see; MASK: some row of
-// the wave does not see all 32 keys; p_max / lo_min bound what any row of the wave sees (values of
-// keys outside are not used at all, whatever the memory holds).
-template <int DH, bool MASK>
-__device__ __forceinline__ void attn_compute_lds(const u32x4 *__restrict__ buf, int k0, const u32x4 (&q)[DH / 16],
-                                               PrefillState<DH> &st, int p_row, int lo_row, int p_max, int lo_min,
-                                               float scale_log2, int n, int hi) {
+// chunks).  p_row / lo_row: the last and first key that the lane's row may see; mask (the same in the
+// whole wave): some row of the wave does not see all 32 keys; p_max / lo_min bound what any row of the
+// wave sees (values of keys outside are not used at all, whatever the memory holds).
+//
+// There is one body for masked and unmasked steps, and everything that changes the output in it works
+// in place (the matrix instructions add to their own operand, the rescaling and the clearing of unseen
+// values are written as instructions on their own registers).  With a body for each case, or with the
+// rescaling as plain arithmetic under its branch, the compiler kept the 64 registers of the output in
+// one place across the loop and in another inside it, and copied them both ways in every step: more
+// instructions than the softmax itself.
+template <int DH>
+__device__ __forceinline__ void attn_compute_lds(const u32x4 *__restrict__ buf, int k0, bool mask, const u32x4 (&q)[DH / 16],
+                                                 PrefillState<DH> &st, int p_row, int lo_row, int p_max, int lo_min,
+                                                 float scale_log2, int n, int hi) {
     f32x16 s;
 #pragma unroll
     for (int i = 0; i < 16; ++i) s[i] = 0.f;
@@ -678,7 +731,7 @@ __device__ __forceinline__ void attn_compute_lds(const u32x4 *__restrict__ buf, 
     float x[16];
 #pragma unroll
     for (int i = 0; i < 16; ++i) x[i] = s[i];
-    if (MASK) {
+    if (mask) {
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
             const int j = key_of_score(k0, i, hi);
@@ -691,7 +744,7 @@ __device__ __forceinline__ void attn_compute_lds(const u32x4 *__restrict__ buf, 
     mx = fmaxf(mx, x[15]);
     mx = max_over_halves(mx);
     // the reference point of the exponentials moves only when the maximum has grown by more than
-    // 2^RESCALE_SLACK (see attn_softmax)
+    // 2^RESCALE_SLACK: the weights stay below that, and the output is rarely rescaled
     const float m_true = fmaxf(st.m, mx * scale_log2);
     const float m_new = m_true - st.m <= RESCALE_SLACK ? st.m : m_true;       // false for the first keys (-inf)
     const float m_safe = m_new == -INFINITY ? 0.f : m_new;
@@ -706,35 +759,38 @@ __device__ __forceinline__ void attn_compute_lds(const u32x4 *__restrict__ buf, 
     st.m = m_new;
     if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
 #pragma unroll
-        for (int t = 0; t < DH / 32; ++t) st.o[t] *= alpha;
+        for (int t = 0; t < DH / 32; ++t)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) asm volatile("v_mul_f32 %0, %0, %1" : "+v"(st.o[t][i]) : "v"(alpha));
     }
     u32x4 pb[2];
 #pragma unroll
     for (int kk = 0; kk < 2; ++kk)
         pb[kk] = u32x4{pack_bf16(p[8 * kk], p[8 * kk + 1]), pack_bf16(p[8 * kk + 2], p[8 * kk + 3]),
                        pack_bf16(p[8 * kk + 4], p[8 * kk + 5]), pack_bf16(p[8 * kk + 6], p[8 * kk + 7])};
-    uint32_t keep[2][4];
-    if (MASK) {
+    if (mask) {
         // values of keys that no row sees are taken as zero: their memory may hold anything
 #pragma unroll
         for (int kk = 0; kk < 2; ++kk) {
-#pragma unroll
-            for (int w = 0; w < 4; ++w) keep[kk][w] = 0xffffffffu;
+            uint32_t keep[4] = {0xffffffffu, 0xffffffffu, 0xffffffffu, 0xffffffffu};
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
                 const int j = k0 + 16 * kk + 8 * hi + e;
-                if (j > p_max || j < lo_min) keep[kk][e / 2] &= (e & 1) ? 0x0000ffffu : 0xffff0000u;
+                if (j > p_max || j < lo_min) keep[e / 2] &= (e & 1) ? 0x0000ffffu : 0xffff0000u;
+            }
+#pragma unroll
+            for (int t = 0; t < DH / 32; ++t) {
+                asm volatile("v_and_b32 %0, %0, %1" : "+v"(v[t][kk].x) : "v"(keep[0]));
+                asm volatile("v_and_b32 %0, %0, %1" : "+v"(v[t][kk].y) : "v"(keep[1]));
+                asm volatile("v_and_b32 %0, %0, %1" : "+v"(v[t][kk].z) : "v"(keep[2]));
+                asm volatile("v_and_b32 %0, %0, %1" : "+v"(v[t][kk].w) : "v"(keep[3]));
             }
         }
     }
 #pragma unroll
     for (int kk = 0; kk < 2; ++kk)
 #pragma unroll
-        for (int t = 0; t < DH / 32; ++t) {
-            u32x4 a = v[t][kk];
-            if (MASK) { a.x &= keep[kk][0]; a.y &= keep[kk][1]; a.z &= keep[kk][2]; a.w &= keep[kk][3]; }
-            st.o[t] = mfma32(a, pb[kk], st.o[t]);
-        }
+        for (int t = 0; t < DH / 32; ++t) st.o[t] = mfma32(v[t][kk], pb[kk], st.o[t]);
 }
 
 // A task is a block of consecutive tokens of one request: a workgroup has PRE_QWAVES x 2 waves; wave q of
@@ -747,10 +803,10 @@ __device__ __forceinline__ void attn_compute_lds(const u32x4 *__restrict__ buf, 
 // copied to LDS once per workgroup, two buffers ahead of the one that is read: before a double step every
 // wave waits for its own part of its copy, then a barrier (which waits for LDS only) makes the whole copy
 // visible and says that the buffer of the double step before is free for the one two ahead.
-template <int DH>
+template <int DH, bool PAGE16, bool FLAT>
 __global__ void __launch_bounds__(PRE_WAVES *WAVE, LCU_PRE_MIN_WAVES)
 attention_prefill_kernel(const bf16_t *__restrict__ q, int q_stride, bf16_t *__restrict__ out, int out_stride,
-                           const bf16_t *__restrict__ cache, const int *__restrict__ block_table, int max_pages,
+                           const bf16_t *__restrict__ cache, uint32_t cache_bytes, const int *__restrict__ block_table, int max_pages,
                            const int *__restrict__ q_start, const int *__restrict__ ctx_len,
                            const int *__restrict__ task_req, const int *__restrict__ task_tok0, int n_tasks,
                            int tasks_per_wg, int nh, int nkvh, int page, uint32_t tile_magic, float scale_log2, int window) {
@@ -813,10 +869,16 @@ attention_prefill_kernel(const bf16_t *__restrict__ q, int q_stride, bf16_t *__r
     const size_t page_elems = kv_page_elems(nkvh, DH, page);
     const int blk0 = wg_lo_min / 32, blk_end = wg_p_max / 32 + 1;
     const int n_dsteps = (blk_end - blk0 + 1) / 2;
+    StageLane<DH> sl;
+    stage_lane<DH>(sl, page, wave_id, lane);
+    int page_id[DH / 32];
+    uint32_t tok_in_page[DH / 32];
 #pragma unroll
-    for (int d = 0; d < PRE_RING - 1; ++d)
-        stage_issue<DH>(lds_ring + d * 16 * DH, cache, bt, max_pages, page, tile_magic, page_elems, nkvh, kvh, (blk0 + 2 * d) * 32,
-                          wave_id);
+    for (int d = 0; d < PRE_RING - 1; ++d) {
+        stage_pages<DH, PAGE16>(page_id, tok_in_page, bt, max_pages, page, tile_magic, (blk0 + 2 * d) * 32, wave_id);
+        stage_issue<DH>(lds_ring + d * 16 * DH, cache, FLAT, cache_bytes, page_id, tok_in_page, sl, page, page_elems, nkvh, kvh, wave_id);
+    }
+    stage_pages<DH, PAGE16>(page_id, tok_in_page, bt, max_pages, page, tile_magic, (blk0 + 2 * (PRE_RING - 1)) * 32, wave_id);
     int slot = 0, fill = PRE_RING - 1;
     for (int d = 0; d < n_dsteps; ++d) {
         wait_loads<(PRE_RING - 2) * (DH / 32)>();
@@ -826,17 +888,15 @@ attention_prefill_kernel(const bf16_t *__restrict__ q, int q_stride, bf16_t *__r
         // waits for every copy in flight, the one into `dst` included, as if it read what that copy writes
         const u32x4 *__restrict__ src = lds_ring + slot * 16 * DH + half * 8 * DH;
         u32x4 *__restrict__ dst = lds_ring + fill * 16 * DH;
-        stage_issue<DH>(dst, cache, bt, max_pages, page, tile_magic, page_elems, nkvh, kvh, (blk0 + 2 * (d + PRE_RING - 1)) * 32,
-                          wave_id);
+        stage_issue<DH>(dst, cache, FLAT, cache_bytes, page_id, tok_in_page, sl, page, page_elems, nkvh, kvh, wave_id);
+        // the pages of the copy after that one: asked for now, there when the next turn needs them
+        stage_pages<DH, PAGE16>(page_id, tok_in_page, bt, max_pages, page, tile_magic, (blk0 + 2 * (d + PRE_RING)) * 32, wave_id);
         const int blk = blk0 + 2 * d + half, k0 = blk * 32;
         if (wave_has && blk < blk_end && k0 <= p_max && k0 + 31 >= lo_min) {
-            if (k0 + 31 > p_min || k0 < lo_max) {
-                const int p_row = tok_row < 0 ? -1 : tok_row + pos_of_tok;
-                const int lo_row = tok_row >= 0 && window > 0 && p_row - window + 1 > 0 ? p_row - window + 1 : 0;
-                attn_compute_lds<DH, true>(src, k0, qv, st, p_row, lo_row, p_max, lo_min, scale_log2, n, hi);
-            } else {
-                attn_compute_lds<DH, false>(src, k0, qv, st, 0, 0, p_max, lo_min, scale_log2, n, hi);
-            }
+            const bool mask = k0 + 31 > p_min || k0 < lo_max;          // some row does not see all 32 keys
+            const int p_row = tok_row < 0 ? -1 : tok_row + pos_of_tok;
+            const int lo_row = tok_row >= 0 && window > 0 && p_row - window + 1 > 0 ? p_row - window + 1 : 0;
+            attn_compute_lds<DH>(src, k0, mask, qv, st, p_row, lo_row, p_max, lo_min, scale_log2, n, hi);
         }
         slot = slot + 1 == PRE_RING ? 0 : slot + 1;
         fill = fill + 1 == PRE_RING ? 0 : fill + 1;
@@ -887,11 +947,11 @@ attention_prefill_kernel(const bf16_t *__restrict__ q, int q_stride, bf16_t *__r
     }
 }
 
-template <int DH>
-static int launch_prefill(const void *q, int q_stride, void *out, int out_stride, const void *cache,
-                            const int *block_table, int max_pages, const int *q_start, const int *ctx_len,
-                            const int *task_req, const int *task_tok0, int n_tasks, int tasks_per_wg, int nh, int nkvh,
-                            int page, float scale, int window, hipStream_t stream) {
+template <int DH, bool PAGE16, bool FLAT>
+static int launch_prefill_as(const void *q, int q_stride, void *out, int out_stride, const void *cache, uint32_t cache_bytes,
+                             const int *block_table, int max_pages, const int *q_start, const int *ctx_len,
+                             const int *task_req, const int *task_tok0, int n_tasks, int tasks_per_wg, int nh, int nkvh,
+                             int page, float scale, int window, hipStream_t stream) {
     const int g = nh / nkvh, chunks = (g + 15) / 16;
     const long long n_wg = (long long)((n_tasks + tasks_per_wg - 1) / tasks_per_wg) * nkvh * chunks;
     if (n_wg > 0x7fffffffll) return LCU_BAD_ARGUMENT;
@@ -899,17 +959,35 @@ static int launch_prefill(const void *q, int q_stride, void *out, int out_stride
     constexpr size_t lds_bytes = (size_t)PRE_RING * 16 * DH * sizeof(u32x4);
     static bool allowed = false;                   // more than 64 KB of LDS must be asked for once
     if (!allowed) {
-        const hipError_t e = hipFuncSetAttribute((const void *)attention_prefill_kernel<DH>,
+        const hipError_t e = hipFuncSetAttribute((const void *)attention_prefill_kernel<DH, PAGE16, FLAT>,
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
         if (e != hipSuccess) return (int)e;
         allowed = true;
     }
-    attention_prefill_kernel<DH><<<grid, block, lds_bytes, stream>>>(
-        (const bf16_t *)q, q_stride, (bf16_t *)out, out_stride, (const bf16_t *)cache, block_table, max_pages, q_start,
+    attention_prefill_kernel<DH, PAGE16, FLAT><<<grid, block, lds_bytes, stream>>>(
+        (const bf16_t *)q, q_stride, (bf16_t *)out, out_stride, (const bf16_t *)cache, cache_bytes, block_table, max_pages, q_start,
         ctx_len, task_req, task_tok0, n_tasks, tasks_per_wg, nh, nkvh, page,
         page == 16 ? 0u : (uint32_t)(0x100000000ull / (unsigned)(page / 16)) + 1u, scale * 1.4426950408889634f, window);
     LCU_LAUNCH_CHECK();
     return LCU_OK;
+}
+
+// cache_pages: the number of pages of the layer's cache (its size decides how pages are addressed).
+template <int DH>
+static int launch_prefill(const void *q, int q_stride, void *out, int out_stride, const void *cache, long long cache_pages,
+                          const int *block_table, int max_pages, const int *q_start, const int *ctx_len,
+                          const int *task_req, const int *task_tok0, int n_tasks, int tasks_per_wg, int nh, int nkvh,
+                          int page, float scale, int window, hipStream_t stream) {
+    const unsigned long long bytes = (unsigned long long)cache_pages * kv_page_elems(nkvh, DH, page) * sizeof(bf16_t);
+    const bool flat = bytes < (1ull << 32);
+#define AS(P, F) return launch_prefill_as<DH, P, F>(q, q_stride, out, out_stride, cache, (uint32_t)(F ? bytes : 0), block_table, max_pages, q_start, ctx_len, task_req, task_tok0, n_tasks, tasks_per_wg, nh, nkvh, page, scale, window, stream)
+    if (page == 16) {
+        if (flat) AS(true, true);
+        AS(true, false);
+    }
+    if (flat) AS(false, true);
+    AS(false, false);
+#undef AS
 }
 
 // How many consecutive tokens of one request a task of the prefill kernel covers, for a
@@ -926,16 +1004,16 @@ LCU_API int lcu_attention_prefill_tokens_per_task(int nh, int nkvh) {
 // request's last task may be shorter.  Workgroup i takes tasks i*tasks_per_wg .. + tasks_per_wg-1.
 // bfloat16 only; head_dim 32, 64, 96 or 128; page_size a multiple of 16.
 LCU_API int lcu_attention_prefill_bf16(const void *q, int q_stride, void *out, int out_stride, const void *cache,
-                                       const int *block_table, int max_pages, const int *q_start, const int *ctx_len,
+                                       long long cache_pages, const int *block_table, int max_pages, const int *q_start, const int *ctx_len,
                                        const int *task_req, const int *task_tok0, int n_tasks, int tasks_per_wg,
                                        int nh, int nkvh, int dh, int page, float scale, int window,
                                        hipStream_t stream) {
     if (n_tasks <= 0) return LCU_OK;
     if ((unsigned long long)kv_page_elems(nkvh, dh, page) * 2ull >= (1ull << 31)) return LCU_UNSUPPORTED;
-    if (tasks_per_wg < 1 || lcu_attention_prefill_tokens_per_task(nh, nkvh) == 0 || page <= 0 || page % 16 || max_pages <= 0 ||
+    if (cache_pages <= 0 || tasks_per_wg < 1 || lcu_attention_prefill_tokens_per_task(nh, nkvh) == 0 || page <= 0 || page % 16 || max_pages <= 0 ||
         window < 0 || q_stride % 8 || out_stride % 4 || nkvh * ((nh / nkvh + 15) / 16) > 65535)
         return LCU_BAD_ARGUMENT;
-#define GO(D) return launch_prefill<D>(q, q_stride, out, out_stride, cache, block_table, max_pages, q_start, ctx_len, task_req, task_tok0, n_tasks, tasks_per_wg, nh, nkvh, page, scale, window, stream)
+#define GO(D) return launch_prefill<D>(q, q_stride, out, out_stride, cache, cache_pages, block_table, max_pages, q_start, ctx_len, task_req, task_tok0, n_tasks, tasks_per_wg, nh, nkvh, page, scale, window, stream)
     if (dh == 128) GO(128);
     if (dh == 64) GO(64);
     if (dh == 96) GO(96);

@@ -403,7 +403,8 @@ def attention_prefill(q, out, cache, block_table, q_start, ctx_len, task_req, ta
     """Matrix-core attention for any mix of portions and single tokens."""
     _i32(task_req, "task_req", n_tasks); _i32(task_tok0, "task_tok0", n_tasks)
     lib = build.load("attention_mfma")
-    _check(lib.lcu_attention_prefill_bf16(_ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(cache), _ptr(block_table),
+    _check(lib.lcu_attention_prefill_bf16(_ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(cache),
+                                          ctypes.c_longlong(cache.shape[0]), _ptr(block_table),
                                           block_table.shape[1], _ptr(q_start), _ptr(ctx_len), _ptr(task_req),
                                           _ptr(task_tok0), n_tasks, tasks_per_wg, n_heads, n_kv_heads, head_dim, page_size,
                                           ctypes.c_float(scale), int(window), _stream()), "attention_prefill")

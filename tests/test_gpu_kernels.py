@@ -389,6 +389,29 @@ def test_attention_prefill_kernel_long(nh, nkv, dh, page):
     close(out, want, "bfloat16")
 
 
+@pytest.mark.parametrize("page", [16, 32])
+def test_attention_in_a_cache_of_more_than_4_gib(page):
+    """A layer's cache beyond 4 GiB: a page's place no longer fits a 32-bit offset from the cache's start,
+    and the kernels must address it by its own 64-bit address.  The requests' pages lie spread over the
+    whole cache, its last page among them."""
+    from llama_cu_amd.kernels import ops
+    nh, nkv, dh = 8, 4, 128
+    q_lens, ctx_lens = [150, 1, 40], [150, 333, 600]
+    q, cache, step, want = paged_case("bfloat16", nh, nkv, dh, page, q_lens, ctx_lens, 0, seed=page)
+    page_bytes = 2 * nkv * dh * page * 2
+    n_big = (4 << 30) // page_bytes + 1000
+    big = torch.empty(n_big, 2, nkv * dh * page, dtype=torch.bfloat16, device="cuda")
+    n_small = cache.shape[0]
+    place = torch.linspace(0, n_big - 1, n_small).round().long()       # small page i lies in big page place[i]
+    assert place[-1] == n_big - 1 and len(set(place.tolist())) == n_small
+    big[place.cuda()] = cache.cuda()
+    step.block_tables[0] = place.cuda()[step.block_tables[0].long()].int()
+    assert int(step.block_tables[0].max()) * page_bytes >= 1 << 32
+    out = torch.empty(q.shape[0], nh * dh, dtype=torch.bfloat16, device="cuda")
+    ops.paged_attention(q.cuda(), out, big, step, 0, nh, nkv, dh, page, dh ** -0.5, 0)
+    close(out, want, "bfloat16")
+
+
 def test_attention_float32_result_does_not_depend_on_the_batch():
     from llama_cu_amd.kernels import ops
     nh, nkv, dh, page = 4, 2, 32, 16
