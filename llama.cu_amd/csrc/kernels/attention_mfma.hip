@@ -27,6 +27,8 @@
 //                   step are copied to LDS once and shared by the waves.
 #include <mutex>
 
+#include <utility>
+
 #include "attention_static.h"
 #include "common.h"
 #include "kv_layout.h"
@@ -634,18 +636,19 @@ __device__ __forceinline__ void stage_lane(StageLane<DH> &sl, int page, int wave
     }
 }
 
-// The pages of the wave's chunks of the double step at k0 (through the scalar unit), and each chunk's
-// first token in its page.  Read one double step before the copy that uses them, so that the copy does not
-// wait for the table.
+// The pages of the wave's chunks of a copy (through the scalar unit), and each chunk's first token in its
+// page: the keys of the double step at kk0 and the values of the double step at vk0 (the keys run a double
+// step ahead of the values, see the kernel).  Read one turn before the copy that uses them, so that the
+// copy does not wait for the table.
 template <int DH, bool PAGE16>
 __device__ __forceinline__ void stage_pages(int *page_id, uint32_t *tok0, const int *__restrict__ bt,
-                                            int max_pages, int page, uint32_t tile_magic, int k0, int wave_id) {
+                                            int max_pages, int page, uint32_t tile_magic, int kk0, int vk0, int wave_id) {
     const int tiles_per_page = page / 16;
 #pragma unroll
     for (int i = 0; i < DH / 32; ++i) {
         const int cw = wave_id * WAVE + 512 * i;                  // the wave's first chunk
         const int sub = cw / (8 * DH), region = (cw % (8 * DH)) / (2 * DH), t = region & 1;
-        const uint32_t tile = (uint32_t)(k0 >> 4) + 2 * sub + t;
+        const uint32_t tile = (uint32_t)((region < 2 ? kk0 : vk0) >> 4) + 2 * sub + t;
         int pi = (int)tile;                                       // pages of 16 keys: the page is the tile
         tok0[i] = 0;
         if (!PAGE16) {
@@ -693,10 +696,68 @@ __device__ __forceinline__ void stage_issue(u32x4 *__restrict__ buf, const bf16_
     }
 }
 
-// One step of 32 keys for the wave's 32 rows, operands from the copy in LDS (`buf`: the step's 8 * DH
-// chunks).  p_row / lo_row: the last and first key that the lane's row may see; mask (the same in the
-// whole wave): some row of the wave does not see all 32 keys; p_max / lo_min bound what any row of the
-// wave sees (values of keys outside are not used at all, whatever the memory holds).
+// Where a lane's keys (for the scores) and values (for the output) of a step's copy stand in LDS.
+// values: dim 32 t + n, keys 16 kk + 8 hi .. + 7: V tile kk, half hi; chunk kk * 2 DH + 32 t from there
+// keys: row m = n of the instruction: key tile n / 16, slot n % 16; dims 16 sidx + 8 hi ..: dim chunk 2 sidx + hi;
+// chunk 32 sidx from there
+template <int DH>
+__device__ __forceinline__ const u32x4 *lane_values(const u32x4 *buf, int n, int hi) { return buf + 4 * DH + hi * DH + n; }
+template <int DH>
+__device__ __forceinline__ const u32x4 *lane_keys(const u32x4 *buf, int n, int hi) { return buf + (n >> 4) * 2 * DH + hi * 16 + (n & 15); }
+
+__device__ __forceinline__ uint32_t lds_address(const void *p) {
+    return (uint32_t)(__SIZE_TYPE__)(__attribute__((address_space(3))) const void *)p;
+}
+
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>): a loop whose index is a constant in its body.
+template <int... I, class F>
+__device__ __forceinline__ void static_for_impl(std::integer_sequence<int, I...>, F &&f) { (f(std::integral_constant<int, I>{}), ...); }
+template <int N, class F>
+__device__ __forceinline__ void static_for(F &&f) { static_for_impl(std::make_integer_sequence<int, N>{}, f); }
+
+// The 16 bytes at LDS address `addr` + OFF into the registers of `r`, as an instruction of its own: `r` is
+// read and written ("+v"), so the read stands behind every instruction that uses the old contents and takes
+// no registers of its own (as a plain load the compiler read into new registers, all at once and early, and
+// copied them over at the end of every turn).  The compiler does not know that the data is still on its way:
+// NOTHING may touch `r` before operands_arrived().
+template <int OFF>
+__device__ __forceinline__ void lds_read_in_place(u32x4 &r, uint32_t addr) {
+    static_assert(OFF >= 0 && OFF < 65536 && OFF % 16 == 0, "the instruction's offset has 16 bits");
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "+v"(r) : "v"(addr), "n"(OFF));
+}
+
+// Waits for the reads above and says that the operands are defined here: nothing that uses them moves above.
+template <int DH>
+__device__ __forceinline__ void operands_arrived(u32x4 (&k)[DH / 16], u32x4 (&v)[DH / 32][2]) {
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+    for (int sidx = 0; sidx < DH / 16; ++sidx) asm volatile("" : "+v"(k[sidx]));
+#pragma unroll
+    for (int t = 0; t < DH / 32; ++t)
+#pragma unroll
+        for (int kk = 0; kk < 2; ++kk) asm volatile("" : "+v"(v[t][kk]));
+}
+
+// One turn of a wave: the output of step e - 1 and the scores and the softmax of step e, 32 keys each, for
+// the wave's 32 rows.
+//   output   O += V(e - 1)^T P(e - 1)     `v` and `pb` as the turn before has left them
+//   scores   S(e) = K(e) Q^T              `k` as the turn before has left it
+//   softmax  P(e) from S(e)               into `pb`; then O goes over to the new reference point
+// The operands are in registers when the turn begins; it reads the next turn's (V(e) and K(e + 1), from
+// `next`: 8 * DH chunks) into the same registers, each as soon as the matrix instruction that uses the old
+// contents is issued.  With the output a turn behind, all these reads are issued before the softmax, whose
+// arithmetic they have to arrive: no wave waits for LDS after the turn's barrier.
+//
+// It also issues a copy into `dst`, a buffer of the ring other than `next`, which the qualifiers of the two
+// pointers say: both must be parameters of ONE function for that (the compiler knows nothing about two
+// pointers that are parameters of different functions, or local variables, and then makes every read from
+// LDS wait for every copy in flight, which empties the ring of copies in every turn).
+//
+// k0: the first key of step e; p_row / lo_row: the last and first key that the lane's row may see; mask (the
+// same in the whole wave): some row does not see all 32 keys of step e.  A step that is none of the wave's
+// comes with mask and p_row = -1: all its weights are zero and nothing changes.  maskv, p_max / lo_min: the
+// same for the values of step e - 1: values of keys that no row of the wave sees are taken as zero,
+// whatever the memory holds (all of them with p_max = -1).
 //
 // There is one body for masked and unmasked steps, and everything that changes the output in it works
 // in place (the matrix instructions add to their own operand, the rescaling and the clearing of unseen
@@ -704,38 +765,63 @@ __device__ __forceinline__ void stage_issue(u32x4 *__restrict__ buf, const bf16_
 // rescaling as plain arithmetic under its branch, the compiler kept the 64 registers of the output in
 // one place across the loop and in another inside it, and copied them both ways in every step: more
 // instructions than the softmax itself.
-template <int DH>
-__device__ __forceinline__ void attn_compute_lds(const u32x4 *__restrict__ buf, int k0, bool mask, const u32x4 (&q)[DH / 16],
-                                                 PrefillState<DH> &st, int p_row, int lo_row, int p_max, int lo_min,
-                                                 float scale_log2, int n, int hi) {
+template <int DH, class Issue>
+__device__ __forceinline__ void attn_turn(const u32x4 *__restrict__ next, u32x4 *__restrict__ dst, Issue &&issue_copy,
+                                          u32x4 (&k)[DH / 16], u32x4 (&v)[DH / 32][2], u32x4 (&pb)[2], const u32x4 (&q)[DH / 16],
+                                          PrefillState<DH> &st, float &alpha, int k0, bool mask, int p_row, int lo_row, bool maskv,
+                                          int p_max, int lo_min, float scale_log2, int n, int hi) {
+    issue_copy(dst);
+    // the output so far goes over to the reference point that the turn before has chosen (here, and not where
+    // that turn made the factor: a branch behind the softmax would cut it off the block of the matrix
+    // instructions, and the wait for the operands would stand before the exponentials instead of behind them)
+    if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+#pragma unroll
+        for (int t = 0; t < DH / 32; ++t)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) asm volatile("v_mul_f32 %0, %0, %1" : "+v"(st.o[t][i]) : "v"(alpha));
+    }
+    if (maskv) {
+#pragma unroll
+        for (int kk = 0; kk < 2; ++kk) {
+            uint32_t keep[4] = {0xffffffffu, 0xffffffffu, 0xffffffffu, 0xffffffffu};
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const int j = k0 - 64 + 16 * kk + 8 * hi + e;
+                if (j > p_max || j < lo_min) keep[e / 2] &= (e & 1) ? 0x0000ffffu : 0xffff0000u;
+            }
+#pragma unroll
+            for (int t = 0; t < DH / 32; ++t) {
+                asm volatile("v_and_b32 %0, %0, %1" : "+v"(v[t][kk].x) : "v"(keep[0]));
+                asm volatile("v_and_b32 %0, %0, %1" : "+v"(v[t][kk].y) : "v"(keep[1]));
+                asm volatile("v_and_b32 %0, %0, %1" : "+v"(v[t][kk].z) : "v"(keep[2]));
+                asm volatile("v_and_b32 %0, %0, %1" : "+v"(v[t][kk].w) : "v"(keep[3]));
+            }
+        }
+    }
+    const uint32_t ka = lds_address(lane_keys<DH>(next, n, hi)), va = lds_address(lane_values<DH>(next, n, hi));
+    static_for<2 * (DH / 32)>([&](auto i) {
+        constexpr int kk = decltype(i)::value / (DH / 32), t = decltype(i)::value % (DH / 32);
+        st.o[t] = mfma32(v[t][kk], pb[kk], st.o[t]);
+        lds_read_in_place<(kk * 2 * DH + 32 * t) * 16>(v[t][kk], va);
+    });
     f32x16 s;
 #pragma unroll
     for (int i = 0; i < 16; ++i) s[i] = 0.f;
-    {
-        // row m = n of the instruction: key tile n / 16, slot n % 16; dims 16 sidx + 8 hi ..: dim chunk 2 sidx + hi
-        const u32x4 *kb = buf + (n >> 4) * 2 * DH + hi * 16 + (n & 15);
-        u32x4 k[DH / 16];
-#pragma unroll
-        for (int sidx = 0; sidx < DH / 16; ++sidx) k[sidx] = kb[32 * sidx];
-#pragma unroll
-        for (int sidx = 0; sidx < DH / 16; ++sidx) s = mfma32(k[sidx], q[sidx], s);
-    }
-    __builtin_amdgcn_sched_barrier(0);             // the values' reads stay below the scores
-    // dim 32 t + n, keys 16 kk + 8 hi .. + 7: V tile kk, half hi
-    u32x4 v[DH / 32][2];
-    const u32x4 *vb = buf + 4 * DH + hi * DH + n;
-#pragma unroll
-    for (int t = 0; t < DH / 32; ++t)
-#pragma unroll
-        for (int kk = 0; kk < 2; ++kk) v[t][kk] = vb[kk * 2 * DH + 32 * t];
+    static_for<DH / 16>([&](auto i) {
+        constexpr int sidx = decltype(i)::value;
+        s = mfma32(k[sidx], q[sidx], s);
+        lds_read_in_place<32 * 16 * sidx>(k[sidx], ka);
+    });
     float x[16];
 #pragma unroll
     for (int i = 0; i < 16; ++i) x[i] = s[i];
     if (mask) {
+        // score i is key k0 + 8 hi + c with c = 16 (i / 8) + i % 8 (key_of_score): compared as c against the bounds less k0 + 8 hi
+        const int last = p_row - k0 - 8 * hi, first = lo_row - k0 - 8 * hi;
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
-            const int j = key_of_score(k0, i, hi);
-            if (j > p_row || j < lo_row) x[i] = -INFINITY;
+            const int c = 16 * (i / 8) + i % 8;
+            if (c > last || c < first) x[i] = -INFINITY;
         }
     }
     float mx = fmaxf(fmaxf(x[0], x[1]), x[2]);
@@ -748,7 +834,7 @@ __device__ __forceinline__ void attn_compute_lds(const u32x4 *__restrict__ buf, 
     const float m_true = fmaxf(st.m, mx * scale_log2);
     const float m_new = m_true - st.m <= RESCALE_SLACK ? st.m : m_true;       // false for the first keys (-inf)
     const float m_safe = m_new == -INFINITY ? 0.f : m_new;
-    const float alpha = fast_exp2(st.m - m_safe);
+    alpha = fast_exp2(st.m - m_safe);              // for the output, the values of step e included: in the next turn
     float p[16], sum = 0.f;
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
@@ -757,40 +843,11 @@ __device__ __forceinline__ void attn_compute_lds(const u32x4 *__restrict__ buf, 
     }
     st.l = st.l * alpha + sum;
     st.m = m_new;
-    if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
-#pragma unroll
-        for (int t = 0; t < DH / 32; ++t)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) asm volatile("v_mul_f32 %0, %0, %1" : "+v"(st.o[t][i]) : "v"(alpha));
-    }
-    u32x4 pb[2];
 #pragma unroll
     for (int kk = 0; kk < 2; ++kk)
         pb[kk] = u32x4{pack_bf16(p[8 * kk], p[8 * kk + 1]), pack_bf16(p[8 * kk + 2], p[8 * kk + 3]),
                        pack_bf16(p[8 * kk + 4], p[8 * kk + 5]), pack_bf16(p[8 * kk + 6], p[8 * kk + 7])};
-    if (mask) {
-        // values of keys that no row sees are taken as zero: their memory may hold anything
-#pragma unroll
-        for (int kk = 0; kk < 2; ++kk) {
-            uint32_t keep[4] = {0xffffffffu, 0xffffffffu, 0xffffffffu, 0xffffffffu};
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                const int j = k0 + 16 * kk + 8 * hi + e;
-                if (j > p_max || j < lo_min) keep[e / 2] &= (e & 1) ? 0x0000ffffu : 0xffff0000u;
-            }
-#pragma unroll
-            for (int t = 0; t < DH / 32; ++t) {
-                asm volatile("v_and_b32 %0, %0, %1" : "+v"(v[t][kk].x) : "v"(keep[0]));
-                asm volatile("v_and_b32 %0, %0, %1" : "+v"(v[t][kk].y) : "v"(keep[1]));
-                asm volatile("v_and_b32 %0, %0, %1" : "+v"(v[t][kk].z) : "v"(keep[2]));
-                asm volatile("v_and_b32 %0, %0, %1" : "+v"(v[t][kk].w) : "v"(keep[3]));
-            }
-        }
-    }
-#pragma unroll
-    for (int kk = 0; kk < 2; ++kk)
-#pragma unroll
-        for (int t = 0; t < DH / 32; ++t) st.o[t] = mfma32(v[t][kk], pb[kk], st.o[t]);
+    operands_arrived<DH>(k, v);
 }
 
 // A task is a block of consecutive tokens of one request: a workgroup has PRE_QWAVES x 2 waves; wave q of
@@ -873,31 +930,58 @@ attention_prefill_kernel(const bf16_t *__restrict__ q, int q_stride, bf16_t *__r
     stage_lane<DH>(sl, page, wave_id, lane);
     int page_id[DH / 32];
     uint32_t tok_in_page[DH / 32];
+    // Copy c holds the keys of double step c and the values of double step c - 1 (of double step 0 where
+    // there is none: nobody uses them): what turn c of a wave needs in its registers.  Turn e reads copy e + 1
+    // from LDS into the registers, and copy e + 3 is issued in it, into the buffer of copy e.
+    auto values_from = [&](int c) { return (blk0 + 2 * (c > 0 ? c - 1 : 0)) * 32; };
 #pragma unroll
-    for (int d = 0; d < PRE_RING - 1; ++d) {
-        stage_pages<DH, PAGE16>(page_id, tok_in_page, bt, max_pages, page, tile_magic, (blk0 + 2 * d) * 32, wave_id);
-        stage_issue<DH>(lds_ring + d * 16 * DH, cache, FLAT, cache_bytes, page_id, tok_in_page, sl, page, page_elems, nkvh, kvh, wave_id);
+    for (int c = 0; c < PRE_RING; ++c) {
+        stage_pages<DH, PAGE16>(page_id, tok_in_page, bt, max_pages, page, tile_magic, (blk0 + 2 * c) * 32, values_from(c), wave_id);
+        stage_issue<DH>(lds_ring + c * 16 * DH, cache, FLAT, cache_bytes, page_id, tok_in_page, sl, page, page_elems, nkvh, kvh, wave_id);
     }
-    stage_pages<DH, PAGE16>(page_id, tok_in_page, bt, max_pages, page, tile_magic, (blk0 + 2 * (PRE_RING - 1)) * 32, wave_id);
-    int slot = 0, fill = PRE_RING - 1;
-    for (int d = 0; d < n_dsteps; ++d) {
+    stage_pages<DH, PAGE16>(page_id, tok_in_page, bt, max_pages, page, tile_magic, (blk0 + 2 * PRE_RING) * 32, values_from(PRE_RING), wave_id);
+    const int p_row = tok_row < 0 ? -1 : tok_row + pos_of_tok;
+    const int lo_row = tok_row >= 0 && window > 0 && p_row - window + 1 > 0 ? p_row - window + 1 : 0;
+    u32x4 kreg[DH / 16], vreg[DH / 32][2];
+    u32x4 pb[2] = {u32x4{0u, 0u, 0u, 0u}, u32x4{0u, 0u, 0u, 0u}};
+    wait_loads<(PRE_RING - 1) * (DH / 32)>();
+    lds_barrier();
+    {
+        const u32x4 *kb = lane_keys<DH>(lds_ring + half * 8 * DH, n, hi), *vb = lane_values<DH>(lds_ring + half * 8 * DH, n, hi);
+#pragma unroll
+        for (int sidx = 0; sidx < DH / 16; ++sidx) kreg[sidx] = kb[32 * sidx];
+#pragma unroll
+        for (int t = 0; t < DH / 32; ++t)
+#pragma unroll
+            for (int kk = 0; kk < 2; ++kk) vreg[t][kk] = vb[kk * 2 * DH + 32 * t];
+    }
+    int slot = 1, fill = 0;                       // the buffers of copy e + 1 and of copy e
+    bool own_before = false, mask_before = true;      // the first turn's values are nobody's: all taken as zero
+    float alpha = 1.0f;
+    for (int e = 0; e < n_dsteps + 1; ++e) {
+        // copy e + 1 has landed (this wave's part of it; the barrier says so for the others'), and every wave
+        // has read copy e (a turn ends with its reads from LDS over)
         wait_loads<(PRE_RING - 2) * (DH / 32)>();
         lds_barrier();
-        // the copy of a later double step goes into the buffer that the barrier has freed; the two buffers
-        // are different ones of the ring, which the qualifiers of the pointers say: a read from LDS otherwise
-        // waits for every copy in flight, the one into `dst` included, as if it read what that copy writes
-        const u32x4 *__restrict__ src = lds_ring + slot * 16 * DH + half * 8 * DH;
-        u32x4 *__restrict__ dst = lds_ring + fill * 16 * DH;
-        stage_issue<DH>(dst, cache, FLAT, cache_bytes, page_id, tok_in_page, sl, page, page_elems, nkvh, kvh, wave_id);
-        // the pages of the copy after that one: asked for now, there when the next turn needs them
-        stage_pages<DH, PAGE16>(page_id, tok_in_page, bt, max_pages, page, tile_magic, (blk0 + 2 * (d + PRE_RING)) * 32, wave_id);
-        const int blk = blk0 + 2 * d + half, k0 = blk * 32;
-        if (wave_has && blk < blk_end && k0 <= p_max && k0 + 31 >= lo_min) {
-            const bool mask = k0 + 31 > p_min || k0 < lo_max;          // some row does not see all 32 keys
-            const int p_row = tok_row < 0 ? -1 : tok_row + pos_of_tok;
-            const int lo_row = tok_row >= 0 && window > 0 && p_row - window + 1 > 0 ? p_row - window + 1 : 0;
-            attn_compute_lds<DH>(src, k0, mask, qv, st, p_row, lo_row, p_max, lo_min, scale_log2, n, hi);
-        }
+        // the copy into the freed buffer uses the pages read a turn ago; then the pages of the copy after that
+        // one are asked for, there when the next turn needs them
+        int page_now[DH / 32];
+        uint32_t tok_now[DH / 32];
+#pragma unroll
+        for (int i = 0; i < DH / 32; ++i) page_now[i] = page_id[i], tok_now[i] = tok_in_page[i];
+        auto issue_copy = [&](u32x4 *__restrict__ to) {
+            stage_issue<DH>(to, cache, FLAT, cache_bytes, page_now, tok_now, sl, page, page_elems, nkvh, kvh, wave_id);
+        };
+        stage_pages<DH, PAGE16>(page_id, tok_in_page, bt, max_pages, page, tile_magic, (blk0 + 2 * (e + PRE_RING + 1)) * 32, values_from(e + PRE_RING + 1), wave_id);
+        // is step e one of the wave's, and does some row not see all its keys?  (the same of step e - 1, for
+        // its values, from the turn before)
+        const int blk = blk0 + 2 * e + half, k0 = blk * 32;
+        const bool own = e < n_dsteps && wave_has && blk < blk_end && k0 <= p_max && k0 + 31 >= lo_min;
+        const bool mask = !own || k0 + 31 > p_min || k0 < lo_max;
+        attn_turn<DH>(lds_ring + slot * 16 * DH + half * 8 * DH, lds_ring + fill * 16 * DH, issue_copy, kreg, vreg, pb, qv, st,
+                      alpha, k0, mask, own ? p_row : -1, lo_row, mask_before, own_before ? p_max : -1, lo_min, scale_log2, n, hi);
+        own_before = own;
+        mask_before = mask;
         slot = slot + 1 == PRE_RING ? 0 : slot + 1;
         fill = fill + 1 == PRE_RING ? 0 : fill + 1;
     }
