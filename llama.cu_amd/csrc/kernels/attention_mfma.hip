@@ -726,16 +726,15 @@ __device__ __forceinline__ void lds_read_in_place(u32x4 &r, uint32_t addr) {
     asm volatile("ds_read_b128 %0, %1 offset:%2" : "+v"(r) : "v"(addr), "n"(OFF));
 }
 
-// Waits for the reads above and says that the operands are defined here: nothing that uses them moves above.
-template <int DH>
-__device__ __forceinline__ void operands_arrived(u32x4 (&k)[DH / 16], u32x4 (&v)[DH / 32][2]) {
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+// Waits until at most LEFT of the wave's reads from LDS are on their way (they arrive in the order in which
+// they were issued; scalar loads in flight count with them, which makes the wait longer, never shorter),
+// and says that the operands are defined here: nothing that uses them moves above.
+template <int LEFT, int N>
+__device__ __forceinline__ void operands_arrived(u32x4 (&r)[N]) {
+    static_assert(LEFT >= 0 && LEFT < 16, "lgkmcnt has four bits");
+    __builtin_amdgcn_s_waitcnt(0xc07f | (LEFT << 8));          // vmcnt and expcnt: no wait
 #pragma unroll
-    for (int sidx = 0; sidx < DH / 16; ++sidx) asm volatile("" : "+v"(k[sidx]));
-#pragma unroll
-    for (int t = 0; t < DH / 32; ++t)
-#pragma unroll
-        for (int kk = 0; kk < 2; ++kk) asm volatile("" : "+v"(v[t][kk]));
+    for (int i = 0; i < N; ++i) asm volatile("" : "+v"(r[i]));
 }
 
 // One turn of a wave: the output of step e - 1 and the scores and the softmax of step e, 32 keys each, for
@@ -743,10 +742,13 @@ __device__ __forceinline__ void operands_arrived(u32x4 (&k)[DH / 16], u32x4 (&v)
 //   output   O += V(e - 1)^T P(e - 1)     `v` and `pb` as the turn before has left them
 //   scores   S(e) = K(e) Q^T              `k` as the turn before has left it
 //   softmax  P(e) from S(e)               into `pb`; then O goes over to the new reference point
-// The operands are in registers when the turn begins; it reads the next turn's (V(e) and K(e + 1), from
-// `next`: 8 * DH chunks) into the same registers, each as soon as the matrix instruction that uses the old
-// contents is issued.  With the output a turn behind, all these reads are issued before the softmax, whose
-// arithmetic they have to arrive: no wave waits for LDS after the turn's barrier.
+// The keys are in registers when the turn begins (the turn before has read them from LDS).  The turn reads
+// the values V(e - 1) into the registers that the turn before has used up, first of all, so that they arrive
+// during the scores' matrix instructions, and the keys of the next turn, K(e + 1), each into the registers of
+// the keys that a matrix instruction has just used, so that they arrive during the softmax (both from `next`:
+// 8 * DH chunks).  The output's matrix instructions and the softmax need nothing of each other and stand in
+// one block: the vector unit works while the matrix cores do (a matrix instruction takes 8 passes; about 7
+// vector instructions fit beside it; with the stages one after the other the two units took turns).
 //
 // It also issues a copy into `dst`, a buffer of the ring other than `next`, which the qualifiers of the two
 // pointers say: both must be parameters of ONE function for that (the compiler knows nothing about two
@@ -765,21 +767,37 @@ __device__ __forceinline__ void operands_arrived(u32x4 (&k)[DH / 16], u32x4 (&v)
 // rescaling as plain arithmetic under its branch, the compiler kept the 64 registers of the output in
 // one place across the loop and in another inside it, and copied them both ways in every step: more
 // instructions than the softmax itself.
-template <int DH, class Issue>
-__device__ __forceinline__ void attn_turn(const u32x4 *__restrict__ next, u32x4 *__restrict__ dst, Issue &&issue_copy,
-                                          u32x4 (&k)[DH / 16], u32x4 (&v)[DH / 32][2], u32x4 (&pb)[2], const u32x4 (&q)[DH / 16],
+template <int DH, class Issue, class Pages>
+__device__ __forceinline__ void attn_turn(const u32x4 *__restrict__ next, u32x4 *__restrict__ dst, Issue &&issue_copy, Pages &&ask_pages,
+                                          u32x4 (&k)[DH / 16], u32x4 (&v)[2 * (DH / 32)], u32x4 (&pb)[2], const u32x4 (&q)[DH / 16],
                                           PrefillState<DH> &st, float &alpha, int k0, bool mask, int p_row, int lo_row, bool maskv,
                                           int p_max, int lo_min, float scale_log2, int n, int hi) {
     issue_copy(dst);
+    // the values of step e - 1: on their way during the scores' matrix instructions
+    const uint32_t ka = lds_address(lane_keys<DH>(next, n, hi)), va = lds_address(lane_values<DH>(next, n, hi));
+    static_for<2 * (DH / 32)>([&](auto i) {
+        constexpr int kk = decltype(i)::value / (DH / 32), t = decltype(i)::value % (DH / 32);
+        lds_read_in_place<(kk * 2 * DH + 32 * t) * 16>(v[decltype(i)::value], va);
+    });
     // the output so far goes over to the reference point that the turn before has chosen (here, and not where
     // that turn made the factor: a branch behind the softmax would cut it off the block of the matrix
-    // instructions, and the wait for the operands would stand before the exponentials instead of behind them)
+    // instructions)
     if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
 #pragma unroll
         for (int t = 0; t < DH / 32; ++t)
 #pragma unroll
             for (int i = 0; i < 16; ++i) asm volatile("v_mul_f32 %0, %0, %1" : "+v"(st.o[t][i]) : "v"(alpha));
     }
+    f32x16 s;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) s[i] = 0.f;
+    static_for<DH / 16>([&](auto i) {
+        constexpr int sidx = decltype(i)::value;
+        s = mfma32(k[sidx], q[sidx], s);
+        lds_read_in_place<32 * 16 * sidx>(k[sidx], ka);            // the keys of step e + 1
+    });
+    operands_arrived<DH / 16>(v);                  // all but the reads of the keys, which came later
+    ask_pages();                                   // (scalar loads: behind the wait, which they would make longer)
     if (maskv) {
 #pragma unroll
         for (int kk = 0; kk < 2; ++kk) {
@@ -791,27 +809,13 @@ __device__ __forceinline__ void attn_turn(const u32x4 *__restrict__ next, u32x4 
             }
 #pragma unroll
             for (int t = 0; t < DH / 32; ++t) {
-                asm volatile("v_and_b32 %0, %0, %1" : "+v"(v[t][kk].x) : "v"(keep[0]));
-                asm volatile("v_and_b32 %0, %0, %1" : "+v"(v[t][kk].y) : "v"(keep[1]));
-                asm volatile("v_and_b32 %0, %0, %1" : "+v"(v[t][kk].z) : "v"(keep[2]));
-                asm volatile("v_and_b32 %0, %0, %1" : "+v"(v[t][kk].w) : "v"(keep[3]));
+                asm volatile("v_and_b32 %0, %0, %1" : "+v"(v[kk * (DH / 32) + t].x) : "v"(keep[0]));
+                asm volatile("v_and_b32 %0, %0, %1" : "+v"(v[kk * (DH / 32) + t].y) : "v"(keep[1]));
+                asm volatile("v_and_b32 %0, %0, %1" : "+v"(v[kk * (DH / 32) + t].z) : "v"(keep[2]));
+                asm volatile("v_and_b32 %0, %0, %1" : "+v"(v[kk * (DH / 32) + t].w) : "v"(keep[3]));
             }
         }
     }
-    const uint32_t ka = lds_address(lane_keys<DH>(next, n, hi)), va = lds_address(lane_values<DH>(next, n, hi));
-    static_for<2 * (DH / 32)>([&](auto i) {
-        constexpr int kk = decltype(i)::value / (DH / 32), t = decltype(i)::value % (DH / 32);
-        st.o[t] = mfma32(v[t][kk], pb[kk], st.o[t]);
-        lds_read_in_place<(kk * 2 * DH + 32 * t) * 16>(v[t][kk], va);
-    });
-    f32x16 s;
-#pragma unroll
-    for (int i = 0; i < 16; ++i) s[i] = 0.f;
-    static_for<DH / 16>([&](auto i) {
-        constexpr int sidx = decltype(i)::value;
-        s = mfma32(k[sidx], q[sidx], s);
-        lds_read_in_place<32 * 16 * sidx>(k[sidx], ka);
-    });
     float x[16];
 #pragma unroll
     for (int i = 0; i < 16; ++i) x[i] = s[i];
@@ -824,6 +828,14 @@ __device__ __forceinline__ void attn_turn(const u32x4 *__restrict__ next, u32x4 
             if (c > last || c < first) x[i] = -INFINITY;
         }
     }
+    // the output's matrix instructions stand here, beside the softmax that does not need them: the
+    // compiler's scheduler puts vector instructions between them (its own mix was the fastest: with ten
+    // vector instructions forced behind each matrix instruction the kernel was 11 % slower, with all the
+    // matrix instructions first 4 %)
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+        for (int t = 0; t < DH / 32; ++t) st.o[t] = mfma32(v[kk * (DH / 32) + t], pb[kk], st.o[t]);
     float mx = fmaxf(fmaxf(x[0], x[1]), x[2]);
 #pragma unroll
     for (int i = 3; i < 15; i += 2) mx = fmaxf(fmaxf(mx, x[i]), x[i + 1]);
@@ -834,7 +846,7 @@ __device__ __forceinline__ void attn_turn(const u32x4 *__restrict__ next, u32x4 
     const float m_true = fmaxf(st.m, mx * scale_log2);
     const float m_new = m_true - st.m <= RESCALE_SLACK ? st.m : m_true;       // false for the first keys (-inf)
     const float m_safe = m_new == -INFINITY ? 0.f : m_new;
-    alpha = fast_exp2(st.m - m_safe);              // for the output, the values of step e included: in the next turn
+    alpha = fast_exp2(st.m - m_safe);              // for the output, the values of step e - 1 included: in the next turn
     float p[16], sum = 0.f;
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
@@ -843,11 +855,14 @@ __device__ __forceinline__ void attn_turn(const u32x4 *__restrict__ next, u32x4 
     }
     st.l = st.l * alpha + sum;
     st.m = m_new;
+    u32x4 pb_new[2];
 #pragma unroll
     for (int kk = 0; kk < 2; ++kk)
-        pb[kk] = u32x4{pack_bf16(p[8 * kk], p[8 * kk + 1]), pack_bf16(p[8 * kk + 2], p[8 * kk + 3]),
-                       pack_bf16(p[8 * kk + 4], p[8 * kk + 5]), pack_bf16(p[8 * kk + 6], p[8 * kk + 7])};
-    operands_arrived<DH>(k, v);
+        pb_new[kk] = u32x4{pack_bf16(p[8 * kk], p[8 * kk + 1]), pack_bf16(p[8 * kk + 2], p[8 * kk + 3]),
+                           pack_bf16(p[8 * kk + 4], p[8 * kk + 5]), pack_bf16(p[8 * kk + 6], p[8 * kk + 7])};
+    pb[0] = pb_new[0];
+    pb[1] = pb_new[1];
+    operands_arrived<0>(k);
 }
 
 // A task is a block of consecutive tokens of one request: a workgroup has PRE_QWAVES x 2 waves; wave q of
@@ -930,10 +945,10 @@ attention_prefill_kernel(const bf16_t *__restrict__ q, int q_stride, bf16_t *__r
     stage_lane<DH>(sl, page, wave_id, lane);
     int page_id[DH / 32];
     uint32_t tok_in_page[DH / 32];
-    // Copy c holds the keys of double step c and the values of double step c - 1 (of double step 0 where
-    // there is none: nobody uses them): what turn c of a wave needs in its registers.  Turn e reads copy e + 1
-    // from LDS into the registers, and copy e + 3 is issued in it, into the buffer of copy e.
-    auto values_from = [&](int c) { return (blk0 + 2 * (c > 0 ? c - 1 : 0)) * 32; };
+    // Copy c holds the keys of double step c and the values of double step c - 2 (of double step 0 where
+    // there is none: nobody uses them): what turn c - 1 of a wave reads into its registers.  Copy e + 3 is
+    // issued in turn e, into the buffer of copy e.
+    auto values_from = [&](int c) { return (blk0 + 2 * (c > 1 ? c - 2 : 0)) * 32; };
 #pragma unroll
     for (int c = 0; c < PRE_RING; ++c) {
         stage_pages<DH, PAGE16>(page_id, tok_in_page, bt, max_pages, page, tile_magic, (blk0 + 2 * c) * 32, values_from(c), wave_id);
@@ -942,18 +957,16 @@ attention_prefill_kernel(const bf16_t *__restrict__ q, int q_stride, bf16_t *__r
     stage_pages<DH, PAGE16>(page_id, tok_in_page, bt, max_pages, page, tile_magic, (blk0 + 2 * PRE_RING) * 32, values_from(PRE_RING), wave_id);
     const int p_row = tok_row < 0 ? -1 : tok_row + pos_of_tok;
     const int lo_row = tok_row >= 0 && window > 0 && p_row - window + 1 > 0 ? p_row - window + 1 : 0;
-    u32x4 kreg[DH / 16], vreg[DH / 32][2];
+    u32x4 kreg[DH / 16], vreg[2 * (DH / 32)];
     u32x4 pb[2] = {u32x4{0u, 0u, 0u, 0u}, u32x4{0u, 0u, 0u, 0u}};
     wait_loads<(PRE_RING - 1) * (DH / 32)>();
     lds_barrier();
     {
-        const u32x4 *kb = lane_keys<DH>(lds_ring + half * 8 * DH, n, hi), *vb = lane_values<DH>(lds_ring + half * 8 * DH, n, hi);
+        const u32x4 *kb = lane_keys<DH>(lds_ring + half * 8 * DH, n, hi);
 #pragma unroll
         for (int sidx = 0; sidx < DH / 16; ++sidx) kreg[sidx] = kb[32 * sidx];
 #pragma unroll
-        for (int t = 0; t < DH / 32; ++t)
-#pragma unroll
-            for (int kk = 0; kk < 2; ++kk) vreg[t][kk] = vb[kk * 2 * DH + 32 * t];
+        for (int i = 0; i < 2 * (DH / 32); ++i) vreg[i] = u32x4{0u, 0u, 0u, 0u};
     }
     int slot = 1, fill = 0;                       // the buffers of copy e + 1 and of copy e
     bool own_before = false, mask_before = true;      // the first turn's values are nobody's: all taken as zero
@@ -972,13 +985,15 @@ attention_prefill_kernel(const bf16_t *__restrict__ q, int q_stride, bf16_t *__r
         auto issue_copy = [&](u32x4 *__restrict__ to) {
             stage_issue<DH>(to, cache, FLAT, cache_bytes, page_now, tok_now, sl, page, page_elems, nkvh, kvh, wave_id);
         };
-        stage_pages<DH, PAGE16>(page_id, tok_in_page, bt, max_pages, page, tile_magic, (blk0 + 2 * (e + PRE_RING + 1)) * 32, values_from(e + PRE_RING + 1), wave_id);
+        auto ask_pages = [&]() {
+            stage_pages<DH, PAGE16>(page_id, tok_in_page, bt, max_pages, page, tile_magic, (blk0 + 2 * (e + PRE_RING + 1)) * 32, values_from(e + PRE_RING + 1), wave_id);
+        };
         // is step e one of the wave's, and does some row not see all its keys?  (the same of step e - 1, for
         // its values, from the turn before)
         const int blk = blk0 + 2 * e + half, k0 = blk * 32;
         const bool own = e < n_dsteps && wave_has && blk < blk_end && k0 <= p_max && k0 + 31 >= lo_min;
         const bool mask = !own || k0 + 31 > p_min || k0 < lo_max;
-        attn_turn<DH>(lds_ring + slot * 16 * DH + half * 8 * DH, lds_ring + fill * 16 * DH, issue_copy, kreg, vreg, pb, qv, st,
+        attn_turn<DH>(lds_ring + slot * 16 * DH + half * 8 * DH, lds_ring + fill * 16 * DH, issue_copy, ask_pages, kreg, vreg, pb, qv, st,
                       alpha, k0, mask, own ? p_row : -1, lo_row, mask_before, own_before ? p_max : -1, lo_min, scale_log2, n, hi);
         own_before = own;
         mask_before = mask;
