@@ -290,17 +290,22 @@ def _attention_args(q, out, cache, block_table, q_start, ctx_len, req_of_token, 
 def paged_attention_generic(q: torch.Tensor, out: torch.Tensor, cache: torch.Tensor, block_table: torch.Tensor,
                             q_start: torch.Tensor, ctx_len: torch.Tensor, req_of_token: torch.Tensor,
                             n_heads: int, n_kv_heads: int, head_dim: int, page_size: int, scale: float,
-                            window: int = 0) -> torch.Tensor:
-    """Causal attention of the step's queries over the paged cache (every shape)."""
+                            window: int = 0, head_slopes: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Causal attention of the step's queries over the paged cache (every shape).  ``head_slopes``
+    (float32 [n_heads]) adds ``slope[h] * (key position - query position)`` to the scaled scores."""
     n = _attention_args(q, out, cache, block_table, q_start, ctx_len, req_of_token, n_heads, n_kv_heads, head_dim,
                         page_size)
     if head_dim % 8 or head_dim > 256:
         raise KernelError(f"attention: head_dim {head_dim} must be a multiple of 8, at most 256")
+    if head_slopes is not None:
+        _gpu(head_slopes)
+        if head_slopes.dtype != torch.float32 or head_slopes.shape != (n_heads,) or not head_slopes.is_contiguous():
+            raise KernelError(f"attention: head_slopes must be contiguous float32 [{n_heads}], got {head_slopes.dtype} {tuple(head_slopes.shape)}")
     lib = build.load("attention_generic")
     _check(lib.lcu_paged_attention_generic(_ptr(q), q.stride(0), _ptr(out), out.stride(0), _type(q, "q"), _ptr(cache),
                                            _ptr(block_table), block_table.shape[1], _ptr(q_start), _ptr(ctx_len),
                                            _ptr(req_of_token), n, n_heads, n_kv_heads, head_dim, page_size,
-                                           ctypes.c_float(scale), int(window), _stream()), "paged_attention_generic")
+                                           ctypes.c_float(scale), int(window), _ptr(head_slopes), _stream()), "paged_attention_generic")
     return out
 
 
@@ -438,13 +443,14 @@ def decode_splits(n_req: int, n_heads: int, n_kv_heads: int, max_ctx_len: int) -
 
 def paged_attention(q: torch.Tensor, out: torch.Tensor, cache: torch.Tensor, step, group: int, n_heads: int,
                     n_kv_heads: int, head_dim: int, page_size: int, scale: float, window: int = 0,
-                    force_generic: bool = False) -> torch.Tensor:
+                    force_generic: bool = False, head_slopes: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Attention for the batch ``step`` (an engine.batch.StepContext) over cache group
-    ``group``: picks the kernel for the batch's shape and type."""
+    ``group``: picks the kernel for the batch's shape and type.  A bias inside the scores
+    (``head_slopes``) is the generic kernel's: the matrix-core kernels take none."""
     bt = step.block_table(group)
-    if force_generic or not mfma_attention_supported(q, n_heads, n_kv_heads, head_dim, page_size):
+    if force_generic or head_slopes is not None or not mfma_attention_supported(q, n_heads, n_kv_heads, head_dim, page_size):
         return paged_attention_generic(q, out, cache, bt, step.q_start, step.ctx_len, step.req_of_token, n_heads,
-                                       n_kv_heads, head_dim, page_size, scale, window)
+                                       n_kv_heads, head_dim, page_size, scale, window, head_slopes)
     n = _attention_args(q, out, cache, bt, step.q_start, step.ctx_len, step.req_of_token, n_heads, n_kv_heads, head_dim,
                         page_size)
     if step.decode_only:

@@ -17,7 +17,6 @@ from ..kernels import ops
 from .base import BuildContext, PagedKV, Part, PartSpec, ScaledRows, TensorSpec, make_part, register_part
 from .linear import (Weight, linear, linear_into_norm, linear_planes, linear_qkv_rope, linear_scaled, mid_takes,
                      skinny_takes)
-from .position import NoPosition
 from ..weights.loader import fused_rows
 
 
@@ -68,7 +67,7 @@ class Attention(Part):
         self.w_o = Weight(tensors["o_proj.weight"], build)
         self.position.load({}, build)
         # a position encoding that is its rotation tables alone (apply() does nothing of its own)
-        self._rotation_only = getattr(type(self.position), "apply", None) is NoPosition.apply
+        self._rotation_only = type(self.position).apply is Part.apply
         self.page_size = build.page_size
         self.dtype = build.dtype
 
@@ -111,7 +110,7 @@ class Attention(Part):
                               page_size)
         out = torch.empty((n_rows, nh * dh), dtype=self.dtype, device=qkv.device)
         ops.paged_attention(qkv, out, cache.pages, step, cache.group, nh, nkv, dh, page_size, self.scale,
-                            self.window)
+                            self.window, head_slopes=self.position.score_slopes())
         if into is not None:
             residual, norm = into
             fused = linear_into_norm(out, self.w_o, residual, norm.weight)

@@ -210,6 +210,17 @@ class Part:
         ``batch`` requests decode over at most ``max_ctx_len`` keys; a captured graph fixes the number."""
         return 1
 
+    # position: what a position encoding may be, each optional (``parts/position.py`` describes them): tables of
+    # a rotation, any other change of queries and keys in place, a bias inside the scores.
+    def rotary_tables(self):
+        return None
+
+    def apply(self, qkv, positions, heads, kv_heads, head_dim) -> None:
+        pass
+
+    def score_slopes(self):
+        return None
+
     def tensors(self) -> Dict[str, TensorSpec]:
         return {}
 

@@ -9,7 +9,10 @@ token's place.  The interface:
         keys and values to the cache;
   ``apply(qkv, positions, heads, kv_heads, head_dim)``
         any other change of queries and keys, in place, before the cache write
-        (the default does nothing).
+        (the default does nothing);
+  ``score_slopes() -> float32 [heads] or None``
+        a bias inside the scores that grows with the distance between key and query
+        (the default: none).
 """
 from __future__ import annotations
 
@@ -27,11 +30,11 @@ class NoPosition(Part):
     def load(self, tensors, build: BuildContext) -> None:
         pass
 
-    def rotary_tables(self):
+    def score_slopes(self):
+        """None, or float32 [heads] on the device: the encoding is (also) a bias inside the scores,
+        ``slope[h] * (key position - query position)`` added to the scaled score.  The mixer hands it to
+        the attention kernel (the generic one: the matrix-core kernels take no bias)."""
         return None
-
-    def apply(self, qkv, positions, heads, kv_heads, head_dim) -> None:
-        pass
 
 
 class Rotary(NoPosition):

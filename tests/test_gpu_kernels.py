@@ -412,6 +412,52 @@ def test_attention_in_a_cache_of_more_than_4_gib(page):
     close(out, want, "bfloat16")
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("window", [0, 20])
+def test_attention_with_a_bias_that_grows_with_the_distance(dtype, window):
+    """``head_slopes``: slope[h] * (key position - query position) inside the scores, for portions and
+    single tokens from the cache.  The expectation is written out here (the plain implementation has no
+    such bias); slopes so steep that leaving the bias out, or its sign, would be far off."""
+    from llama_cu_amd.kernels import ops
+    nh, nkv, dh, page = 6, 2, 32, 16
+    q_lens, ctx_lens = [30, 1, 7], [30, 65, 50]
+    q, cache, step, _ = paged_case(dtype, nh, nkv, dh, page, q_lens, ctx_lens, window, seed=9, standout=False, poison=False)
+    slopes = torch.tensor([0.5, 0.25, 0.125, 0.3, 0.0, 1.0])
+    # the keys and values back from the pages, then the formula
+    want, row = [], 0
+    cf = cache.float().view(cache.shape[0], -1)
+    for r, (ql, cl) in enumerate(zip(q_lens, ctx_lens)):
+        table = step.block_tables[0][r].tolist()
+        k = torch.zeros(cl, nkv, dh, dtype=torch.float64); v = torch.zeros(cl, nkv, dh, dtype=torch.float64)
+        lo_all = max(cl - ql - window + 1, 0) if window else 0
+        for j in range(lo_all, cl):
+            pg, tok = table[j // page], j % page
+            for h in range(nkv):
+                for c8 in range(dh // 8):
+                    base = key_offset(h, tok, c8 * 8, dh, page)
+                    k[j, h, c8 * 8:c8 * 8 + 8] = cf[pg, base:base + 8]
+                vo = value_offset(nkv, h, tok, 0, dh, page)
+                v[j, h] = cf[pg, vo:vo + dh * page:page]
+        qq = q[row:row + ql].double().view(ql, nh, dh)
+        for i in range(ql):
+            p = cl - ql + i
+            lo = max(p - window + 1, 0) if window else 0
+            js = torch.arange(lo, p + 1)
+            for h in range(nh):
+                sc = (k[lo:p + 1, h // (nh // nkv)] @ qq[i, h]) * dh ** -0.5 + float(slopes[h]) * (js - p).double()
+                want.append(torch.softmax(sc, dim=0) @ v[lo:p + 1, h // (nh // nkv)])
+        row += ql
+    want = torch.stack(want).view(sum(q_lens), nh * dh)
+    out = torch.empty(q.shape[0], nh * dh, dtype=DT[dtype], device="cuda")
+    ops.paged_attention(q.cuda(), out, cache.cuda(), step, 0, nh, nkv, dh, page, dh ** -0.5, window, head_slopes=slopes.cuda())
+    close(out, want, dtype)
+    flat = torch.empty_like(out)
+    ops.paged_attention(q.cuda(), flat, cache.cuda(), step, 0, nh, nkv, dh, page, dh ** -0.5, window)
+    assert float((flat.double().cpu() - want).abs().max()) > 20 * TOL[dtype] * float(want.abs().max()), "the bias must matter here"
+    with pytest.raises(ops.KernelError):
+        ops.paged_attention(q.cuda(), out, cache.cuda(), step, 0, nh, nkv, dh, page, dh ** -0.5, window, head_slopes=slopes[:3].cuda())
+
+
 def test_attention_float32_result_does_not_depend_on_the_batch():
     from llama_cu_amd.kernels import ops
     nh, nkv, dh, page = 4, 2, 32, 16

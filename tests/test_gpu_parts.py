@@ -458,6 +458,86 @@ def test_a_toy_routed_feed_forward_and_a_toy_position_encoding_are_registered_an
     runner.cache.check()
 
 
+def test_a_toy_position_encoding_that_is_a_bias_inside_the_scores():
+    """A third kind of position encoding, defined here and not in the package: nothing is done to
+    queries and keys; instead every head adds ``slope[h] * (key position - query position)`` to its
+    scaled scores (the part hands the slopes to the mixer through ``score_slopes()``).  Layer 0 gets
+    it, layer 1 keeps the rotation; whole, in portions, token by token and mixed against a direct
+    computation.  With slopes this steep the far keys hardly count: a kernel that left the bias out
+    would be far off."""
+    from llama_cu_amd.config import LlamaConfig
+    from llama_cu_amd.models.llama import llama_spec
+    from llama_cu_amd.parts import Part, PartSpec, register_part
+
+    class DistanceBias(Part):
+        graph_safe = True
+
+        def __init__(self, heads):
+            self.heads = heads
+
+        def tensors(self):
+            return {}
+
+        def load(self, tensors, build):
+            self.slopes = torch.tensor([2.0 ** -(h + 1) for h in range(self.heads)], dtype=torch.float32, device=build.device)
+
+        def rotary_tables(self):
+            return None
+
+        def apply(self, qkv, positions, heads, kv_heads, head_dim):
+            pass
+
+        def score_slopes(self):
+            return self.slopes
+
+    register_part("position", "distance_bias", DistanceBias, replace=True)
+    cfg_d = dict(common.TINY_A)
+    cfg = LlamaConfig.from_dict(cfg_d)
+    spec = llama_spec(cfg)
+    spec.layers[0].params["mixer"].params["position"] = PartSpec("distance_bias", {"heads": cfg.num_attention_heads})
+    runner, w = runner_for(spec, 17, "float32", max_tokens=512, max_seqs=3)
+    nh, nkv, dh = cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim
+
+    def direct(toks):
+        pcfg = plain.PlainConfig.from_dict(cfg_d)
+        n = len(toks)
+        pos = list(range(n))
+        sin, cos = plain.rope_tables(n, dh, pcfg.rope_theta)
+        x = plain.embedding(w["model.embed_tokens.weight"], toks)
+        p = "model.layers.0."
+        h = plain.rms_norm(x, w[p + "input_layernorm.weight"], cfg.rms_norm_eps)
+        q = plain.linear(h, w[p + "self_attn.q_proj.weight"]).view(n, nh, dh).double()
+        k = plain.linear(h, w[p + "self_attn.k_proj.weight"]).view(n, nkv, dh).double()
+        v = plain.linear(h, w[p + "self_attn.v_proj.weight"]).view(n, nkv, dh).double()
+        dist = (torch.arange(n)[None, :] - torch.arange(n)[:, None]).double()          # key position - query position
+        o = torch.empty(n, nh, dh, dtype=torch.float64)
+        for hd in range(nh):
+            sc = q[:, hd] @ k[:, hd // (nh // nkv)].T * dh ** -0.5 + 2.0 ** -(hd + 1) * dist
+            sc = sc.masked_fill(dist > 0, float("-inf"))
+            o[:, hd] = torch.softmax(sc, dim=-1) @ v[:, hd // (nh // nkv)]
+        x = x + plain.linear(o.reshape(n, nh * dh), w[p + "self_attn.o_proj.weight"])
+        x = x + plain.feed_forward(w, p, plain.rms_norm(x, w[p + "post_attention_layernorm.weight"], cfg.rms_norm_eps))
+        p = "model.layers.1."
+        x = x + plain.attention_block(pcfg, w, p, plain.rms_norm(x, w[p + "input_layernorm.weight"], cfg.rms_norm_eps), pos, sin, cos)
+        x = x + plain.feed_forward(w, p, plain.rms_norm(x, w[p + "post_attention_layernorm.weight"], cfg.rms_norm_eps))
+        return plain.linear(plain.rms_norm(x, w["model.norm.weight"], cfg.rms_norm_eps), w["lm_head.weight"])
+
+    reqs = common.random_requests(256, [40, 9, 77, 30], 15)
+    want = {name: direct(toks) for name, toks in reqs.items()}
+    for mode in (common.trace_whole, common.trace_portions, common.trace_tail_decode, lambda r: common.trace_mixed(r, max_live=3)):
+        steps, _ = mode(reqs)
+        ids, outputs = {}, {}
+        for st in steps:
+            es = st["entries"]
+            logits = runner.step([ids.setdefault(e["id"], len(ids)) for e in es], [e["tokens"] for e in es], [e["want"] for e in es])
+            outputs[st["step"]] = logits.cpu().numpy()
+            for name in st["end"]:
+                runner.end(ids[name])
+        got = common.collect(steps, outputs, 256)
+        common.assert_matches_plain(got, want, "float32", "distance bias")
+    runner.cache.check()
+
+
 def _engine_turns(engine, prompt, eos, more, steps):
     """A kept request: one turn until the end-of-sequence token, then a turn with ``more``."""
     from llama_cu_amd.sampling import GREEDY
