@@ -548,10 +548,10 @@ LCU_API int lcu_attention_decode_bf16_static(const void *q, int q_stride, void *
 #ifndef LCU_PRE_MIN_WAVES
 #define LCU_PRE_MIN_WAVES 2
 #endif
-constexpr int PRE_QWAVES = 4;             // waves of a workgroup that hold different rows
-constexpr int PRE_HALVES = 2;             // wave groups that share the rows and take every second step of 32 keys
-constexpr int PRE_WAVES = PRE_QWAVES * PRE_HALVES;
-constexpr int PRE_RING = 3;               // buffers of 64 keys in LDS: one is read, two are on their way
+constexpr int PRE_WAVES = 4;              // waves of a workgroup, each with 32 rows of its own: one wave per SIMD, so that a
+                                          // compute unit holds two workgroups (two tasks) whose turns are not in step
+constexpr int PRE_THREADS = PRE_WAVES * WAVE;
+constexpr int PRE_RING = 3;               // buffers of 32 keys in LDS: one is read, two are on their way
 
 // Wait until at most `left` of this wave's vector memory operations are outstanding.
 template <int LEFT>
@@ -595,13 +595,12 @@ __device__ __forceinline__ float max_over_halves(float x) {
     return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
 }
 
-// The keys and values of two steps of 32 keys, copied into LDS in chunks of 16 bytes.  Per step 8 * DH
-// chunks: [K tile 0 | K tile 1 | V tile 0 | V tile 1], 2 * DH chunks per tile of 16 keys; a buffer holds two
-// steps.  Keys as the page holds them, [dim / 8][slot 16], the token in slot p being p with bits 2 and 3
+// The keys and values of a step of 32 keys, copied into LDS in chunks of 16 bytes: 8 * DH
+// chunks, [K tile 0 | K tile 1 | V tile 0 | V tile 1], 2 * DH chunks per tile of 16 keys.  Keys as the page holds them, [dim / 8][slot 16], the token in slot p being p with bits 2 and 3
 // swapped.  Values: [half][dim], the chunk of tokens 8 half .. + 7 of the tile for every dim (the page holds
 // [dim][token]).  With these orders the lanes of every read of an operand take neighbouring bytes: no bank
 // conflicts (with the values as their page has them four lanes of a read fell into one bank, and the
-// conflicts took a quarter of the kernel's time).  A thread of the workgroup copies chunks tid, tid + 512, ...
+// conflicts took a quarter of the kernel's time).  A thread of the workgroup copies chunks tid, tid + 256, ...
 //
 // The copy goes from memory straight into LDS (buffer_load ... lds: no registers hold the data on its way,
 // lane l of a wave writes the 16 bytes l of the wave's 1 KB), so the loads of two buffers can be in flight
@@ -630,15 +629,15 @@ __device__ __forceinline__ void stage_lane(StageLane<DH> &sl, int page, int wave
     sl.k = ((uint32_t)(lane >> 4) * page + k_tok) * 8 * E;
 #pragma unroll
     for (int i = 0; i < DH / 32; ++i) {
-        const int w0 = (wave_id * WAVE + 512 * i) % (2 * DH);
+        const int w0 = (wave_id * WAVE + PRE_THREADS * i) % (2 * DH);
         const uint32_t v_at = (uint32_t)(w0 + lane), v_half = v_at / DH, v_dim = v_at - v_half * DH;
         sl.v[i] = (v_dim * page + 8 * v_half) * E;
     }
 }
 
 // The pages of the wave's chunks of a copy (through the scalar unit), and each chunk's first token in its
-// page: the keys of the double step at kk0 and the values of the double step at vk0 (the keys run a double
-// step ahead of the values, see the kernel).  Read one turn before the copy that uses them, so that the
+// page: the keys of the step at kk0 and the values of the step at vk0 (the keys run two steps ahead of the
+// values, see the kernel).  Read one turn before the copy that uses them, so that the
 // copy does not wait for the table.
 template <int DH, bool PAGE16>
 __device__ __forceinline__ void stage_pages(int *page_id, uint32_t *tok0, const int *__restrict__ bt,
@@ -646,9 +645,9 @@ __device__ __forceinline__ void stage_pages(int *page_id, uint32_t *tok0, const 
     const int tiles_per_page = page / 16;
 #pragma unroll
     for (int i = 0; i < DH / 32; ++i) {
-        const int cw = wave_id * WAVE + 512 * i;                  // the wave's first chunk
-        const int sub = cw / (8 * DH), region = (cw % (8 * DH)) / (2 * DH), t = region & 1;
-        const uint32_t tile = (uint32_t)((region < 2 ? kk0 : vk0) >> 4) + 2 * sub + t;
+        const int cw = wave_id * WAVE + PRE_THREADS * i;          // the wave's first chunk
+        const int region = cw / (2 * DH), t = region & 1;
+        const uint32_t tile = (uint32_t)((region < 2 ? kk0 : vk0) >> 4) + t;
         int pi = (int)tile;                                       // pages of 16 keys: the page is the tile
         tok0[i] = 0;
         if (!PAGE16) {
@@ -662,7 +661,7 @@ __device__ __forceinline__ void stage_pages(int *page_id, uint32_t *tok0, const 
 
 // FLAT: the whole cache of the layer is one buffer of less than 4 GiB (the host says), and a page is an
 // offset in it: two scalar instructions per chunk.  Else the buffer of a load is its page, whose 64-bit
-// address is made per chunk (a dozen scalar instructions: with four chunks a double step they were a third
+// address is made per chunk (a dozen scalar instructions: with four chunks a step they were a third
 // of all the instructions a wave issued).
 template <int DH>
 __device__ __forceinline__ void stage_issue(u32x4 *__restrict__ buf, const bf16_t *__restrict__ cache, bool FLAT,
@@ -672,9 +671,8 @@ __device__ __forceinline__ void stage_issue(u32x4 *__restrict__ buf, const bf16_
     constexpr uint32_t E = sizeof(bf16_t);
 #pragma unroll
     for (int i = 0; i < DH / 32; ++i) {
-        const int cw = wave_id * WAVE + 512 * i;                  // the wave's first chunk
-        const int c = cw % (8 * DH);
-        const int region = c / (2 * DH), w0 = c % (2 * DH);
+        const int cw = wave_id * WAVE + PRE_THREADS * i;          // the wave's first chunk
+        const int region = cw / (2 * DH), w0 = cw % (2 * DH);
         // keys: dim chunks w0 / 16 .. + 3 of the tile
         const uint32_t s_off = region < 2 ? ((uint32_t)(kvh * (DH / 8) + w0 / 16) * page + tok0[i]) * 8 * E
                                           : ((uint32_t)((nkvh + kvh) * DH) * page + tok0[i]) * E;
@@ -684,13 +682,13 @@ __device__ __forceinline__ void stage_issue(u32x4 *__restrict__ buf, const bf16_
         if (FLAT) {
             __builtin_amdgcn_raw_ptr_buffer_load_lds(
                 __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t *>(cache), 0, cache_bytes, 0x00020000),
-                (__attribute__((address_space(3))) void *)(buf + 512 * i + WAVE * wave_id), 16, lane_off,
+                (__attribute__((address_space(3))) void *)(buf + cw), 16, lane_off,
                 (uint32_t)page_id[i] * (uint32_t)(page_elems * E) + s_off, 0, 0);
         } else {
             __builtin_amdgcn_raw_ptr_buffer_load_lds(
                 __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t *>(cache + (size_t)page_id[i] * page_elems), 0,
                                                   (uint32_t)(page_elems * E), 0x00020000),
-                (__attribute__((address_space(3))) void *)(buf + 512 * i + WAVE * wave_id), 16, lane_off,
+                (__attribute__((address_space(3))) void *)(buf + cw), 16, lane_off,
                 s_off, 0, 0);
         }
     }
@@ -804,7 +802,7 @@ __device__ __forceinline__ void attn_turn(const u32x4 *__restrict__ next, u32x4 
             uint32_t keep[4] = {0xffffffffu, 0xffffffffu, 0xffffffffu, 0xffffffffu};
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-                const int j = k0 - 64 + 16 * kk + 8 * hi + e;
+                const int j = k0 - 32 + 16 * kk + 8 * hi + e;
                 if (j > p_max || j < lo_min) keep[e / 2] &= (e & 1) ? 0x0000ffffu : 0xffff0000u;
             }
 #pragma unroll
@@ -865,26 +863,29 @@ __device__ __forceinline__ void attn_turn(const u32x4 *__restrict__ next, u32x4 
     operands_arrived<0>(k);
 }
 
-// A task is a block of consecutive tokens of one request: a workgroup has PRE_QWAVES x 2 waves; wave q of
-// either half takes 32 rows (tokens x the heads of one chunk of a group), so a task covers
-// 4 * (32 / heads per chunk) tokens, starting at batch index task_tok0[t].  The workgroup walks the keys
-// that any of its rows sees, 64 at a time: the first half of the waves takes the first 32 of them, the
-// second half the other 32, each with an online softmax of its own, and the two are merged at the end.
-// So a compute unit holds two waves per SIMD that work on one task (while one waits for the softmax's
-// arithmetic the other feeds the matrix cores), however few tasks there are.  The keys and values are
-// copied to LDS once per workgroup, two buffers ahead of the one that is read: before a double step every
-// wave waits for its own part of its copy, then a barrier (which waits for LDS only) makes the whole copy
-// visible and says that the buffer of the double step before is free for the one two ahead.
+// A task is a block of consecutive tokens of one request: a workgroup has 4 waves, one per SIMD; each takes
+// 32 rows (tokens x the heads of one chunk of a group), so a task covers 4 * (32 / heads per chunk) tokens,
+// starting at batch index task_tok0[t].  The workgroup walks the keys that any of its rows sees, 32 at a
+// time; the keys and values are copied to LDS once per workgroup, two buffers ahead of the one that is
+// read: before a turn every wave waits for its own part of a copy, then a barrier (which waits for LDS
+// only) makes the whole copy visible and says that the buffer of the turn before is free for the copy two
+// ahead.  A compute unit holds two workgroups (48 KB of LDS and half the registers each), so every SIMD has
+// two waves of two different tasks: their turns are not in step (while one wave's softmax keeps the vector
+// unit busy the other's matrix instructions run), and what a task costs before its first and after its last
+// turn (its tables, its queries, the first copy: some microseconds of waiting for memory) the other task
+// fills.  (Eight waves that worked on one task, in two halves that split the keys and met at a barrier every
+// turn, were as fast over long contexts and a tenth slower where tasks are short: portions of 256 tokens over
+// 2k keys 83 against 75 us, a single task of 32 tokens 11.9 against 8.8 us.)
 template <int DH, bool PAGE16, bool FLAT>
-__global__ void __launch_bounds__(PRE_WAVES *WAVE, LCU_PRE_MIN_WAVES)
+__global__ void __launch_bounds__(PRE_THREADS, LCU_PRE_MIN_WAVES)
 attention_prefill_kernel(const bf16_t *__restrict__ q, int q_stride, bf16_t *__restrict__ out, int out_stride,
                            const bf16_t *__restrict__ cache, uint32_t cache_bytes, const int *__restrict__ block_table, int max_pages,
                            const int *__restrict__ q_start, const int *__restrict__ ctx_len,
                            const int *__restrict__ task_req, const int *__restrict__ task_tok0, int n_tasks,
                            int tasks_per_wg, int nh, int nkvh, int page, uint32_t tile_magic, float scale_log2, int window) {
-    extern __shared__ u32x4 lds_ring[];            // [PRE_RING][16 * DH]; at the end the halves' states
-    const int wave_id = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
-    const int lane = threadIdx.x & (WAVE - 1), wave = wave_id % PRE_QWAVES, half = wave_id / PRE_QWAVES;
+    extern __shared__ u32x4 lds_ring[];            // [PRE_RING][8 * DH]
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
+    const int lane = threadIdx.x & (WAVE - 1);
     // Workgroups go to the chip's eight dies in turn (workgroup i to die i % 8), and each die has an L2 of
     // its own.  The key/value head is the fastest index of the grid, so that the workgroups of one head
     // (with 8 heads, or a multiple or a divisor of 8) all run on one die, whose L2 then holds that head's keys and
@@ -893,7 +894,7 @@ attention_prefill_kernel(const bf16_t *__restrict__ q, int q_stride, bf16_t *__r
     const int chunks = (g + 15) / 16;
     const int head_chunk = blockIdx.x % (nkvh * chunks), wg = blockIdx.x / (nkvh * chunks);
     for (int task = wg * tasks_per_wg; task < (wg + 1) * tasks_per_wg && task < n_tasks; ++task) {
-    __syncthreads();                               // the last task's use of LDS is over (its copies landed before its merge)
+    __syncthreads();                               // the last task's use of LDS is over (it waited for its copies)
     const int n = lane & 31, hi = lane >> 5;
     const int kvh = head_chunk / chunks, chunk = head_chunk % chunks;
     const int hc = (g - 16 * chunk) < 16 ? (g - 16 * chunk) : 16;      // heads of this chunk
@@ -925,7 +926,7 @@ attention_prefill_kernel(const bf16_t *__restrict__ q, int q_stride, bf16_t *__r
         lo_min = window > 0 && p_min - window + 1 > 0 ? p_min - window + 1 : 0;
         lo_max = window > 0 && p_max - window + 1 > 0 ? p_max - window + 1 : 0;
     }
-    const int wg_last_tok = (task_tok + PRE_QWAVES * tokens_per_wave < q_end ? task_tok + PRE_QWAVES * tokens_per_wave : q_end) - 1;
+    const int wg_last_tok = (task_tok + PRE_WAVES * tokens_per_wave < q_end ? task_tok + PRE_WAVES * tokens_per_wave : q_end) - 1;
     const int wg_p_max = ctx - (q_end - wg_last_tok);
     const int wg_p_min = ctx - (q_end - task_tok);
     const int wg_lo_min = window > 0 && wg_p_min - window + 1 > 0 ? wg_p_min - window + 1 : 0;
@@ -939,22 +940,22 @@ attention_prefill_kernel(const bf16_t *__restrict__ q, int q_stride, bf16_t *__r
         for (int i = 0; i < 16; ++i) st.o[t][i] = 0.f;
     const int *bt = block_table + (size_t)r * max_pages;
     const size_t page_elems = kv_page_elems(nkvh, DH, page);
-    const int blk0 = wg_lo_min / 32, blk_end = wg_p_max / 32 + 1;
-    const int n_dsteps = (blk_end - blk0 + 1) / 2;
+    const int blk0 = wg_lo_min / 32, n_steps = wg_p_max / 32 + 1 - blk0;
     StageLane<DH> sl;
-    stage_lane<DH>(sl, page, wave_id, lane);
+    stage_lane<DH>(sl, page, wave, lane);
     int page_id[DH / 32];
     uint32_t tok_in_page[DH / 32];
-    // Copy c holds the keys of double step c and the values of double step c - 2 (of double step 0 where
-    // there is none: nobody uses them): what turn c - 1 of a wave reads into its registers.  Copy e + 3 is
-    // issued in turn e, into the buffer of copy e.
-    auto values_from = [&](int c) { return (blk0 + 2 * (c > 1 ? c - 2 : 0)) * 32; };
+    // Copy c holds the keys of step c and the values of step c - 2 (of step 0 where there is none: nobody
+    // uses them): what turn c - 1 of a wave reads into its registers.  Copy e + 3 is issued in turn e, into
+    // the buffer of copy e.
+    auto keys_from = [&](int c) { return (blk0 + c) * 32; };
+    auto values_from = [&](int c) { return (blk0 + (c > 1 ? c - 2 : 0)) * 32; };
 #pragma unroll
     for (int c = 0; c < PRE_RING; ++c) {
-        stage_pages<DH, PAGE16>(page_id, tok_in_page, bt, max_pages, page, tile_magic, (blk0 + 2 * c) * 32, values_from(c), wave_id);
-        stage_issue<DH>(lds_ring + c * 16 * DH, cache, FLAT, cache_bytes, page_id, tok_in_page, sl, page, page_elems, nkvh, kvh, wave_id);
+        stage_pages<DH, PAGE16>(page_id, tok_in_page, bt, max_pages, page, tile_magic, keys_from(c), values_from(c), wave);
+        stage_issue<DH>(lds_ring + c * 8 * DH, cache, FLAT, cache_bytes, page_id, tok_in_page, sl, page, page_elems, nkvh, kvh, wave);
     }
-    stage_pages<DH, PAGE16>(page_id, tok_in_page, bt, max_pages, page, tile_magic, (blk0 + 2 * PRE_RING) * 32, values_from(PRE_RING), wave_id);
+    stage_pages<DH, PAGE16>(page_id, tok_in_page, bt, max_pages, page, tile_magic, keys_from(PRE_RING), values_from(PRE_RING), wave);
     const int p_row = tok_row < 0 ? -1 : tok_row + pos_of_tok;
     const int lo_row = tok_row >= 0 && window > 0 && p_row - window + 1 > 0 ? p_row - window + 1 : 0;
     u32x4 kreg[DH / 16], vreg[2 * (DH / 32)];
@@ -962,7 +963,7 @@ attention_prefill_kernel(const bf16_t *__restrict__ q, int q_stride, bf16_t *__r
     wait_loads<(PRE_RING - 1) * (DH / 32)>();
     lds_barrier();
     {
-        const u32x4 *kb = lane_keys<DH>(lds_ring + half * 8 * DH, n, hi);
+        const u32x4 *kb = lane_keys<DH>(lds_ring, n, hi);
 #pragma unroll
         for (int sidx = 0; sidx < DH / 16; ++sidx) kreg[sidx] = kb[32 * sidx];
 #pragma unroll
@@ -971,7 +972,7 @@ attention_prefill_kernel(const bf16_t *__restrict__ q, int q_stride, bf16_t *__r
     int slot = 1, fill = 0;                       // the buffers of copy e + 1 and of copy e
     bool own_before = false, mask_before = true;      // the first turn's values are nobody's: all taken as zero
     float alpha = 1.0f;
-    for (int e = 0; e < n_dsteps + 1; ++e) {
+    for (int e = 0; e < n_steps + 1; ++e) {
         // copy e + 1 has landed (this wave's part of it; the barrier says so for the others'), and every wave
         // has read copy e (a turn ends with its reads from LDS over)
         wait_loads<(PRE_RING - 2) * (DH / 32)>();
@@ -983,64 +984,38 @@ attention_prefill_kernel(const bf16_t *__restrict__ q, int q_stride, bf16_t *__r
 #pragma unroll
         for (int i = 0; i < DH / 32; ++i) page_now[i] = page_id[i], tok_now[i] = tok_in_page[i];
         auto issue_copy = [&](u32x4 *__restrict__ to) {
-            stage_issue<DH>(to, cache, FLAT, cache_bytes, page_now, tok_now, sl, page, page_elems, nkvh, kvh, wave_id);
+            stage_issue<DH>(to, cache, FLAT, cache_bytes, page_now, tok_now, sl, page, page_elems, nkvh, kvh, wave);
         };
         auto ask_pages = [&]() {
-            stage_pages<DH, PAGE16>(page_id, tok_in_page, bt, max_pages, page, tile_magic, (blk0 + 2 * (e + PRE_RING + 1)) * 32, values_from(e + PRE_RING + 1), wave_id);
+            stage_pages<DH, PAGE16>(page_id, tok_in_page, bt, max_pages, page, tile_magic, keys_from(e + PRE_RING + 1), values_from(e + PRE_RING + 1), wave);
         };
         // is step e one of the wave's, and does some row not see all its keys?  (the same of step e - 1, for
         // its values, from the turn before)
-        const int blk = blk0 + 2 * e + half, k0 = blk * 32;
-        const bool own = e < n_dsteps && wave_has && blk < blk_end && k0 <= p_max && k0 + 31 >= lo_min;
+        const int k0 = (blk0 + e) * 32;
+        const bool own = e < n_steps && wave_has && k0 <= p_max && k0 + 31 >= lo_min;
         const bool mask = !own || k0 + 31 > p_min || k0 < lo_max;
-        attn_turn<DH>(lds_ring + slot * 16 * DH + half * 8 * DH, lds_ring + fill * 16 * DH, issue_copy, ask_pages, kreg, vreg, pb, qv, st,
+        attn_turn<DH>(lds_ring + slot * 8 * DH, lds_ring + fill * 8 * DH, issue_copy, ask_pages, kreg, vreg, pb, qv, st,
                       alpha, k0, mask, own ? p_row : -1, lo_row, mask_before, own_before ? p_max : -1, lo_min, scale_log2, n, hi);
         own_before = own;
         mask_before = mask;
         slot = slot + 1 == PRE_RING ? 0 : slot + 1;
         fill = fill + 1 == PRE_RING ? 0 : fill + 1;
     }
-    // ---- the second half hands its state to the first, which merges and writes
     wait_loads<0>();                               // the last copies into the ring, which nobody reads, have landed
-    __syncthreads();                               // every wave is done with the buffers
-    float *xch = (float *)lds_ring;                // [value][query wave][lane]
-    constexpr int NV = 2 + (DH / 32) * 16;
-    static_assert(NV * PRE_QWAVES * WAVE * 4 <= PRE_RING * 16 * DH * 16, "the halves' states fit the ring");
-    if (half == 1) {
-        int v = 0;
-        xch[((v++) * PRE_QWAVES + wave) * WAVE + lane] = st.m;
-        xch[((v++) * PRE_QWAVES + wave) * WAVE + lane] = st.l;
-#pragma unroll
-        for (int t = 0; t < DH / 32; ++t)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) xch[((v++) * PRE_QWAVES + wave) * WAVE + lane] = st.o[t][i];
-    }
-    __syncthreads();
-    if (half == 0) {
-        int v = 0;
-        const float m1 = xch[((v++) * PRE_QWAVES + wave) * WAVE + lane];
-        const float l1 = xch[((v++) * PRE_QWAVES + wave) * WAVE + lane];
-        const float m = fmaxf(st.m, m1);
-        const float m_safe = m == -INFINITY ? 0.f : m;
-        const float a0 = fast_exp2(st.m - m_safe), a1 = fast_exp2(m1 - m_safe);
-        float l_all = st.l * a0 + l1 * a1;
-        l_all += __shfl_xor(l_all, 32, WAVE);
-        const float inv = 1.0f / l_all;
-        bf16_t *o = tok_row < 0 ? nullptr : out + (size_t)tok_row * out_stride + (size_t)(head0 + n % hc) * DH;
+    // ---- a row's sum lies in its two lanes (each added the keys it held); the output is written as it stands
+    float l_all = st.l;
+    l_all += __shfl_xor(l_all, 32, WAVE);
+    const float inv = 1.0f / l_all;
+    if (tok_row >= 0) {
+        bf16_t *o = out + (size_t)tok_row * out_stride + (size_t)(head0 + n % hc) * DH;
 #pragma unroll
         for (int t = 0; t < DH / 32; ++t)
 #pragma unroll
             for (int b = 0; b < 4; ++b) {
-                float e4[4];
-#pragma unroll
-                for (int e = 0; e < 4; ++e)
-                    e4[e] = (st.o[t][4 * b + e] * a0 + xch[((v++) * PRE_QWAVES + wave) * WAVE + lane] * a1) * inv;
-                if (o) {
-                    u32x2 w;
-                    w.x = pack_bf16(e4[0], e4[1]);
-                    w.y = pack_bf16(e4[2], e4[3]);
-                    *(u32x2 *)(o + 32 * t + 8 * b + 4 * hi) = w;
-                }
+                u32x2 w;
+                w.x = pack_bf16(st.o[t][4 * b] * inv, st.o[t][4 * b + 1] * inv);
+                w.y = pack_bf16(st.o[t][4 * b + 2] * inv, st.o[t][4 * b + 3] * inv);
+                *(u32x2 *)(o + 32 * t + 8 * b + 4 * hi) = w;
             }
     }
     }
@@ -1054,8 +1029,8 @@ static int launch_prefill_as(const void *q, int q_stride, void *out, int out_str
     const int g = nh / nkvh, chunks = (g + 15) / 16;
     const long long n_wg = (long long)((n_tasks + tasks_per_wg - 1) / tasks_per_wg) * nkvh * chunks;
     if (n_wg > 0x7fffffffll) return LCU_BAD_ARGUMENT;
-    dim3 grid((unsigned)n_wg), block(PRE_WAVES * WAVE);
-    constexpr size_t lds_bytes = (size_t)PRE_RING * 16 * DH * sizeof(u32x4);
+    dim3 grid((unsigned)n_wg), block(PRE_THREADS);
+    constexpr size_t lds_bytes = (size_t)PRE_RING * 8 * DH * sizeof(u32x4);
     static bool allowed = false;                   // more than 64 KB of LDS must be asked for once
     if (!allowed) {
         const hipError_t e = hipFuncSetAttribute((const void *)attention_prefill_kernel<DH, PAGE16, FLAT>,
@@ -1096,7 +1071,7 @@ LCU_API int lcu_attention_prefill_tokens_per_task(int nh, int nkvh) {
     const int g = nh / nkvh;
     if (g > 16 && g % 16) return 0;       // chunks of a group must be equal for one task size
     const int hc = g < 16 ? g : 16;
-    return PRE_QWAVES * (32 / hc);
+    return PRE_WAVES * (32 / hc);
 }
 
 // task_req / task_tok0: [n_tasks], tasks cut from the batch with the size above; a

@@ -364,10 +364,12 @@ def attention_decode(q, out, cache, block_table, q_start, ctx_len, n_req, n_head
     return out
 
 
-def prefill_tasks(q_lens, ctx_lens, tokens_per_task: int, device, pair: Optional[bool] = None, skip_single: bool = False):
+def prefill_tasks(q_lens, ctx_lens, tokens_per_task: int, device, skip_single: bool = False, per_wg: int = 1):
     """Cut the batch into the prefill kernel's tasks: (request index, first token) pairs, the
     tasks that walk the most keys first (workgroups start in this order, so the long ones
-    do not start last and leave the other compute units waiting for them)."""
+    do not start last and leave the other compute units waiting for them).  A compute unit
+    holds two workgroups, so the tasks of a whole prompt (the last block walks all keys, the
+    first none) even out by themselves; ``per_wg`` tasks go to one workgroup, one after the other."""
     tasks = []
     start = 0
     for r, n in enumerate(q_lens):
@@ -376,27 +378,6 @@ def prefill_tasks(q_lens, ctx_lens, tokens_per_task: int, device, pair: Optional
             tasks.append((-keys, r, start + t))
         start += n
     tasks.sort()
-    per_wg = 1
-    if pair is None:
-        # Tasks of very unequal length (a whole prompt: the last block walks all keys, the first
-        # none) leave compute units idle, since all workgroups are resident at once; then a
-        # workgroup takes a long and a short task.  Equal tasks run better one per workgroup
-        # (measured on the Llama-3-8B shape).
-        keys = [-t[0] for t in tasks]
-        pair = len(tasks) >= 2 and max(keys) >= 1.5 * (sum(keys) / len(keys))
-    if pair:
-        # the longest with the shortest, the second longest with the second shortest, ...
-        half = (len(tasks) + 1) // 2
-        paired = []
-        for i in range(half):
-            paired.append(tasks[i])
-            if len(tasks) - 1 - i > i:
-                paired.append(tasks[len(tasks) - 1 - i])
-            else:
-                paired.append(tasks[i])            # an odd one out: placeholder, removed below
-        if len(tasks) % 2:
-            paired.pop()
-        tasks, per_wg = paired, 2
     if not tasks:
         return None, None, 0, 1
     both = to_device([[t[1] for t in tasks], [t[2] for t in tasks]], torch.int32, device)

@@ -389,6 +389,23 @@ def test_attention_prefill_kernel_long(nh, nkv, dh, page):
     close(out, want, "bfloat16")
 
 
+@pytest.mark.parametrize("per_wg", [2, 3])
+def test_attention_prefill_kernel_with_several_tasks_a_workgroup(per_wg):
+    """A workgroup that takes several tasks one after the other (the ring in LDS and the registers are
+    used again): portions and single tokens, with a window."""
+    from llama_cu_amd.kernels import build, ops
+    nh, nkv, dh, page, window = 8, 2, 64, 16, 70
+    q_lens, ctx_lens = [100, 1, 37, 64], [100, 90, 300, 64]
+    q, cache, step, want = paged_case("bfloat16", nh, nkv, dh, page, q_lens, ctx_lens, window, seed=per_wg)
+    tpt = build.load("attention_mfma").lcu_attention_prefill_tokens_per_task(nh, nkv)
+    task_req, task_tok0, n_tasks, got_per_wg = ops.prefill_tasks(q_lens, ctx_lens, tpt, "cuda", per_wg=per_wg)
+    assert got_per_wg == per_wg and n_tasks == sum((n + tpt - 1) // tpt for n in q_lens)
+    out = torch.empty(q.shape[0], nh * dh, dtype=torch.bfloat16, device="cuda")
+    ops.attention_prefill(q.cuda(), out, cache.cuda(), step.block_tables[0], step.q_start, step.ctx_len, task_req, task_tok0,
+                          n_tasks, per_wg, nh, nkv, dh, page, dh ** -0.5, window)
+    close(out, want, "bfloat16")
+
+
 @pytest.mark.parametrize("page", [16, 32])
 def test_attention_in_a_cache_of_more_than_4_gib(page):
     """A layer's cache beyond 4 GiB: a page's place no longer fits a 32-bit offset from the cache's start,
