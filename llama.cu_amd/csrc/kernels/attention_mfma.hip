@@ -771,7 +771,9 @@ __device__ __forceinline__ void attn_turn(const u32x4 *__restrict__ next, u32x4 
                                           PrefillState<DH> &st, float &alpha, int k0, bool mask, int p_row, int lo_row, bool maskv,
                                           int p_max, int lo_min, float scale_log2, int n, int hi) {
     issue_copy(dst);
-    // the values of step e - 1: on their way during the scores' matrix instructions
+    // the values of step e - 1: on their way during the scores' matrix instructions (they stand before the
+    // branch below, in a block of their own: in one block with the matrix instructions the compiler's
+    // scheduler put them behind most of those, and the wait for them was 5 % of the kernel's time)
     const uint32_t ka = lds_address(lane_keys<DH>(next, n, hi)), va = lds_address(lane_values<DH>(next, n, hi));
     static_for<2 * (DH / 32)>([&](auto i) {
         constexpr int kk = decltype(i)::value / (DH / 32), t = decltype(i)::value % (DH / 32);
@@ -826,6 +828,10 @@ __device__ __forceinline__ void attn_turn(const u32x4 *__restrict__ next, u32x4 
             if (c > last || c < first) x[i] = -INFINITY;
         }
     }
+    // the keys of the next turn: here rather than at the turn's end (it costs nothing: the other workgroup's
+    // waves have work), so that the long block below, where registers are scarce, is outside the stretch
+    // in which the keys' registers may not be touched
+    operands_arrived<0>(k);
     // the output's matrix instructions stand here, beside the softmax that does not need them: the
     // compiler's scheduler puts vector instructions between them (its own mix was the fastest: with ten
     // vector instructions forced behind each matrix instruction the kernel was 11 % slower, with all the
@@ -860,7 +866,6 @@ __device__ __forceinline__ void attn_turn(const u32x4 *__restrict__ next, u32x4 
                            pack_bf16(p[8 * kk + 4], p[8 * kk + 5]), pack_bf16(p[8 * kk + 6], p[8 * kk + 7])};
     pb[0] = pb_new[0];
     pb[1] = pb_new[1];
-    operands_arrived<0>(k);
 }
 
 // A task is a block of consecutive tokens of one request: a workgroup has 4 waves, one per SIMD; each takes
