@@ -585,9 +585,6 @@ struct PrefillState {
     float l;                // running sum over the lane's own keys only
 };
 
-// The key of the step that a lane's score i belongs to (k0: the step's first key).
-__device__ __forceinline__ int key_of_score(int k0, int i, int hi) { return k0 + 16 * (i / 8) + 8 * hi + (i % 8); }
-
 // The larger of the values that lane l and lane l ^ 32 hold, in both.
 __device__ __forceinline__ float max_over_halves(float x) {
     const unsigned u = __float_as_uint(x);
@@ -820,7 +817,7 @@ __device__ __forceinline__ void attn_turn(const u32x4 *__restrict__ next, u32x4 
 #pragma unroll
     for (int i = 0; i < 16; ++i) x[i] = s[i];
     if (mask) {
-        // score i is key k0 + 8 hi + c with c = 16 (i / 8) + i % 8 (key_of_score): compared as c against the bounds less k0 + 8 hi
+        // a lane's score i is key k0 + 8 hi + c with c = 16 (i / 8) + i % 8: compared as c against the bounds less k0 + 8 hi
         const int last = p_row - k0 - 8 * hi, first = lo_row - k0 - 8 * hi;
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
