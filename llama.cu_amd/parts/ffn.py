@@ -50,9 +50,9 @@ class SwiGLU(Part):
             # the plain copy, which the library multiplies, has rows of zeros behind each half; the
             # copy that the decode kernels stream does not
             plain = fused_rows([g, u], pad_rows_to=rows)
-            self.w_gate_up = Weight(plain, build, packed_from=torch.cat([g, u], dim=0) if build.pack_weights else None)
+            self.w_gate_up = Weight(plain, build, packed_from=torch.cat([g, u], dim=0) if build.pack_weights else None, halves=True)
         else:
-            self.w_gate_up = Weight(fused_rows([g, u]), build)
+            self.w_gate_up = Weight(fused_rows([g, u]), build, halves=True)
         self.w_down = Weight(tensors["down_proj.weight"], build)
         self.dtype = build.dtype
 

@@ -31,13 +31,16 @@ class Weight:
     (measured on the Llama-3-8B shapes).  The copy doubles the memory of the matrices;
     ``BuildContext.pack_weights`` switches it off."""
 
-    def __init__(self, tensor: torch.Tensor, build=None, packed_from: Optional[torch.Tensor] = None):
+    def __init__(self, tensor: torch.Tensor, build=None, packed_from: Optional[torch.Tensor] = None, halves: bool = False):
         """``packed_from``: the matrix to pack if it is not ``tensor`` (a gate/up matrix whose plain copy
-        has rows of zeros for the library's sake, see ``library_friendly_rows``, is packed without them)."""
+        has rows of zeros for the library's sake, see ``library_friendly_rows``, is packed without them).
+        ``halves``: the matrix is two matrices one above the other (gate and up) whose rows a kernel pairs:
+        it is packed only if each half is whole blocks of 16 rows."""
         self.plain = tensor.contiguous()
         want = build is None or getattr(build, "pack_weights", True)
         src = self.plain if packed_from is None else packed_from.contiguous()
-        self.packed = ops.pack_weight(src) if (want and src.is_cuda and ops.packable(src)) else None
+        fits = ops.packable(src) and (not halves or src.shape[0] % 32 == 0)
+        self.packed = ops.pack_weight(src) if (want and src.is_cuda and fits) else None
 
     @property
     def shape(self):

@@ -55,6 +55,23 @@ def test_feed_forward_part(dtype):
         close(part.forward(h.cuda()), plain.feed_forward(w, "L.", h), dtype)
 
 
+@pytest.mark.parametrize("inner,packed", [(56, False), (24, False), (96, True), (352, True)])
+def test_feed_forward_whose_width_allows_a_packed_copy_but_whose_halves_may_not(inner, packed):
+    """A width of whole blocks of 128: the matrices may get a copy in the order the decode kernel streams.
+    Gate and up are one matrix of 2 x inner rows, which is whole blocks of 16 rows for inner = 56 too, but
+    its halves are not: such a matrix must stay unpacked (the kernel pairs row i of the one half with row i
+    of the other, block by block), and every number of rows must give the plain formula's result."""
+    from llama_cu_amd.parts import PartSpec, make_part
+    part = make_part("ffn", PartSpec("swiglu", {"hidden_size": 128, "intermediate_size": inner}))
+    t = random_part_tensors(part, 4, "bfloat16", std=0.05)
+    part.load(dict(t), build_ctx("bfloat16"))
+    assert (part.w_gate_up.packed is not None) == packed
+    w = {"L.mlp." + k: v.cpu() for k, v in t.items()}
+    for n in (1, 8, 20, 70, 200):
+        h = rnd(n, 128, seed=n).to(torch.bfloat16)
+        close(part.forward(h.cuda()), plain.feed_forward(w, "L.", h), "bfloat16", f"{n} rows")
+
+
 @pytest.mark.parametrize("pack", [True, False])
 def test_feed_forward_with_rows_of_zeros_for_the_library(monkeypatch, pack):
     """Where the library's product is faster with more output features, each half of the plain
