@@ -121,7 +121,7 @@ def test_float32_does_not_depend_on_cutting(models):
                 assert np.array_equal(results[0][name][pos], other[name][pos]), (name, pos)
 
 
-@pytest.mark.parametrize("seed", [1, 2, 3, 4, 5, 6])
+@pytest.mark.parametrize("seed", [1, 2, 3, 4, 5, 6, 101, 102, 103])
 def test_random_configurations_match_plain(seed):
     """Configurations drawn at random from what config.json allows: head sizes in steps of 16
     up to 256, any number of heads and groups, widths and vocabularies that are no power of
@@ -130,10 +130,13 @@ def test_random_configurations_match_plain(seed):
     import random
     rng = random.Random(seed)
     nkv = rng.choice([1, 2, 3, 5])
+    # seeds from 100 on: widths of whole blocks of 128, for which the matrices get the copy that the decode
+    # kernels stream, with intermediate sizes that are and are not whole blocks of 16
+    widths, inner = ([40, 72, 88, 104, 136, 200, 264], [56, 100, 172, 232, 352]) if seed < 100 else ([128, 256], [56, 104, 128, 172])
     cfg = dict(architectures=["LlamaForCausalLM"], num_hidden_layers=rng.choice([1, 2]),
-               hidden_size=rng.choice([40, 72, 88, 104, 136, 200, 264]), num_attention_heads=nkv * rng.choice([1, 2, 3, 4, 7, 8]),
+               hidden_size=rng.choice(widths), num_attention_heads=nkv * rng.choice([1, 2, 3, 4, 7, 8]),
                num_key_value_heads=nkv, head_dim=rng.choice([16, 32, 48, 64, 80, 96, 112, 128, 144, 192, 256]),
-               intermediate_size=rng.choice([56, 100, 172, 232, 352]), vocab_size=rng.choice([257, 301, 384, 1000, 1537]),
+               intermediate_size=rng.choice(inner), vocab_size=rng.choice([257, 301, 384, 1000, 1537]),
                max_position_embeddings=256, rope_theta=rng.choice([1e4, 5e5, 333.0]),
                rms_norm_eps=rng.choice([1e-5, 1e-6, 1e-3]), tie_word_embeddings=rng.random() < 0.5,
                rope_interleaved=rng.random() < 0.3)
