@@ -593,8 +593,8 @@ __device__ __forceinline__ float max_over_halves(float x) {
 }
 
 // The keys and values of a step of 32 keys, copied into LDS in chunks of 16 bytes: 8 * DH
-// chunks, [K tile 0 | K tile 1 | V tile 0 | V tile 1], 2 * DH chunks per tile of 16 keys.  Keys as the page holds them, [dim / 8][slot 16], the token in slot p being p with bits 2 and 3
-// swapped.  Values: [half][dim], the chunk of tokens 8 half .. + 7 of the tile for every dim (the page holds
+// chunks, [K tile 0 | K tile 1 | V tile 0 | V tile 1], 2 * DH chunks per tile of 16 keys.  Keys as the page
+// holds them, [dim / 8][slot 16], the token in slot p being p with bits 2 and 3 swapped.  Values: [half][dim], the chunk of tokens 8 half .. + 7 of the tile for every dim (the page holds
 // [dim][token]).  With these orders the lanes of every read of an operand take neighbouring bytes: no bank
 // conflicts (with the values as their page has them four lanes of a read fell into one bank, and the
 // conflicts took a quarter of the kernel's time).  A thread of the workgroup copies chunks tid, tid + 256, ...
