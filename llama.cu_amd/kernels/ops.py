@@ -609,7 +609,7 @@ def mid_planes(k: int, slices: int) -> int:
 def gemm_mid(x: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = None, swiglu: bool = False,
              slices: Optional[int] = None, packed: bool = False, row_sumsq: Optional[torch.Tensor] = None,
              norm_width: int = 0, eps: float = 0.0) -> torch.Tensor:
-    """``x @ w.T`` for 17 to 128 rows of bfloat16 ``x`` (it takes fewer too), streaming ``w`` once while
+    """``x @ w.T`` for up to 128 rows of bfloat16 ``x`` (chosen from 12 to 33 rows on, by the product), streaming ``w`` once while
     the waves of a workgroup share ``x`` through LDS.  ``slices=None``: ``out [m, n]`` bfloat16
     (``swiglu``: ``w`` holds gate rows, then up rows, ``out [m, n/2] = silu(gate) * up``).
     ``slices=s``: K is cut into (at most) ``s`` slices and ``out [planes, m, n]`` float32 holds

@@ -28,10 +28,13 @@ class Tuning:
     skinny_workgroups_per_cu: int = 4   # plain: as many tiles as still leave this many workgroups for each compute unit
     skinny_eight_waves_to: int = 8192   # eight waves share a workgroup's K up to this many output features, four beyond
     compute_units: int = 256
-    # ---- the product that shares the rows through LDS (gemm_mid.hip, 17 to 128 rows)
-    mid_long_k: int = 8192              # a weight with a longer K (the down projection) goes to it from 17 rows on,
-                                        # and with a plain (not packed) weight only such weights go to it at all
-    mid_swiglu_features: int = 8192     # gate/up with SwiGLU goes to it from this many rows of the weight on
+    # ---- the product that shares the rows through LDS (gemm_mid.hip, up to 128 rows)
+    mid_long_k: int = 8192              # with a plain (not packed) weight only weights with a longer K than this (the down
+                                        # projection) go to it at all; a packed weight with a longer K goes to it
+    mid_long_k_rows: int = 11           # ... above this many rows (whole decode steps: 0.9 % faster at 12 rows, 3 % at 16;
+                                        # 0.3 % slower at 11: below, the weight-streaming kernel with the norm in its epilogue)
+    mid_swiglu_features: int = 8192     # gate/up with SwiGLU goes to it from this many rows of the weight on,
+    mid_swiglu_rows: int = 14           # above this many rows of the batch (0.4 % at 16 rows, nothing below 15)
     mid_min_slice_steps: int = 4        # a slice of K keeps at least this many macro-steps of 128
     mid_max_slices: int = 8
     # ---- the decode attention's cut of a request's keys into parts (attention_mfma.hip)

@@ -76,7 +76,7 @@ class SwiGLU(Part):
                 raise ops.KernelError("feed-forward: rows that wait for their normalisation need the kernel for few rows")
             act = linear_swiglu(h.rows, self.w_gate_up, row_sumsq=h.sumsq, norm_width=h.width, eps=h.eps)
         elif self.dtype == torch.bfloat16 and mid_swiglu_takes(h.shape[0], self.w_gate_up) and ops.mid_supported(h, self.w_gate_up.plain):
-            # 17 to 128 rows: the rows shared through LDS, the activation in the product's epilogue
+            # 15 to 128 rows: the rows shared through LDS, the activation in the product's epilogue
             act = linear_swiglu_mid(h, self.w_gate_up)
         elif (self.dtype == torch.bfloat16 and h.shape[0] <= skinny_row_limit(self.w_gate_up)
               and ops.skinny_supported(h, self.w_gate_up.plain, self.dtype)):
@@ -88,7 +88,7 @@ class SwiGLU(Part):
         if act.shape[1] != self.intermediate_size:
             act = act[:, :self.intermediate_size]      # without what the rows of zeros gave
         if planes_ok and act.dtype == torch.bfloat16 and mid_takes(act.shape[0], self.w_down):
-            # from 17 rows on the product cut over K and the norm kernel that adds its planes are faster
+            # from 12 rows on the product cut over K and the norm kernel that adds its planes are faster
             # than the weight-streaming product with that norm in its epilogue (30 against 35 us)
             return linear_planes(act, self.w_down)
         if into is not None and act.dtype == torch.bfloat16 and skinny_takes(act.shape[0], self.w_down, preferred=True):
