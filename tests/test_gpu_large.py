@@ -216,3 +216,33 @@ def test_captured_steps_of_36_requests_equal_eager_ones(big):
     for i, (a, b) in enumerate(zip(eager, graphed)):
         assert torch.isfinite(a).all()
         assert torch.equal(a, b), f"decode step {i} differs between eager and captured"
+
+
+def test_the_engines_big_tensors_come_out_of_one_allocation():
+    """Weights, their packed copies and the cache are carved out of one allocation of the driver's
+    (engine.runner.reserve_in_one_piece): a fresh process builds an engine and asks torch's allocator
+    in which of its segments the tensors lie."""
+    import os
+    import subprocess
+    import sys
+    script = r'''
+import sys
+sys.path.insert(0, %r); sys.path.insert(0, %r)
+import torch
+import llama_cu_amd
+from test_gpu_large import runner_for
+runner = runner_for("bfloat16", max_tokens=4096, max_seqs=4)
+segments = [(s["address"], s["address"] + s["total_size"]) for s in torch.cuda.memory_snapshot()]
+def segment_of(t):
+    a = t.data_ptr()
+    return [i for i, (lo, hi) in enumerate(segments) if lo <= a < hi][0]
+layer = runner.model.layers[1]
+big = [layer.mixer.w_qkv.plain, layer.mixer.w_qkv.packed, layer.ffn.w_gate_up.plain, layer.ffn.w_gate_up.packed,
+       layer.ffn.w_down.packed, runner.model.head.weight.plain, runner.caches[0].pages, runner.caches[1].pages]
+assert all(t is not None for t in big)
+where = {segment_of(t) for t in big}
+print("segments", len(segments), "of the big tensors", sorted(where))
+assert len(where) == 1, where
+''' % (common.ROOT, os.path.join(common.ROOT, "tests"))
+    proc = subprocess.run([sys.executable, "-c", script], capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stdout[-500:] + proc.stderr[-1500:]
