@@ -162,17 +162,19 @@ class ModelRunner:
 
     # ------------------------------------------------------------ construction helpers
     @classmethod
-    def from_folder(cls, folder: str, dtype="bfloat16", device="cuda:0", **kw) -> "ModelRunner":
-        """The model of a folder (config.json picks the architecture; model.safetensors)."""
+    def from_folder(cls, folder: str, dtype="bfloat16", device="cuda:0", one_piece: bool = True, **kw) -> "ModelRunner":
+        """The model of a folder (config.json picks the architecture; model.safetensors).  ``one_piece``: the
+        engine's memory is asked of the driver in one allocation (reserve_in_one_piece)."""
         from .. import models  # noqa: F401  (registers the architectures)
         device = require_gpu(device)
         arch, cfg = load_config(folder)
         spec = arch.build_spec(cfg)
         files = open_safetensors(folder)
         model = DecoderModel(spec)
-        reserve_in_one_piece(device, engine_bytes(spec, model.tensors(), DTYPES[dtype], device, int(kw.get("page_size", 16)),
-                                                  kw.get("max_tokens"), kw.get("num_pages"), int(kw.get("max_seqs", 8)),
-                                                  int(kw.get("max_batch_tokens", 2048)), float(kw.get("kv_fraction", 0.85))))
+        if one_piece:
+            reserve_in_one_piece(device, engine_bytes(spec, model.tensors(), DTYPES[dtype], device, int(kw.get("page_size", 16)),
+                                                      kw.get("max_tokens"), kw.get("num_pages"), int(kw.get("max_seqs", 8)),
+                                                      int(kw.get("max_batch_tokens", 2048)), float(kw.get("kv_fraction", 0.85))))
         tensors = load_weights(files, model.tensors(), DTYPES[dtype], device, groups=model.fused_groups(DTYPES[dtype], device),
                                log=lambda line: print(f"[llama.cu_amd] {line}", file=sys.stderr, flush=True))
         runner = cls(spec, tensors, dtype, device, **kw)
@@ -181,7 +183,7 @@ class ModelRunner:
 
     @classmethod
     def from_config(cls, cfg, seed: int, dtype="bfloat16", device="cuda:0", std: float = 0.02, stored=None,
-                    **kw) -> "ModelRunner":
+                    one_piece: bool = True, **kw) -> "ModelRunner":
         """Random weights made on the device from ``seed`` (nothing is written or read): bit for
         bit the weights that ``write_random_model`` writes for the same seed.  ``stored``: the
         type that a file would hold them in, if not the compute type (``"bfloat16"`` with the
@@ -191,9 +193,10 @@ class ModelRunner:
         device = require_gpu(device)
         spec = architecture_of(cfg.to_dict()).build_spec(cfg)
         expected = DecoderModel(spec).tensors()
-        reserve_in_one_piece(device, engine_bytes(spec, expected, DTYPES[dtype], device, int(kw.get("page_size", 16)),
-                                                  kw.get("max_tokens"), kw.get("num_pages"), int(kw.get("max_seqs", 8)),
-                                                  int(kw.get("max_batch_tokens", 2048)), float(kw.get("kv_fraction", 0.85))))
+        if one_piece:
+            reserve_in_one_piece(device, engine_bytes(spec, expected, DTYPES[dtype], device, int(kw.get("page_size", 16)),
+                                                      kw.get("max_tokens"), kw.get("num_pages"), int(kw.get("max_seqs", 8)),
+                                                      int(kw.get("max_batch_tokens", 2048)), float(kw.get("kv_fraction", 0.85))))
         tensors = random_tensors(expected, seed, dtype=DTYPES[stored or dtype], std=std, device=device)
         tensors = {n: convert(t, expected[n], DTYPES[dtype]) for n, t in tensors.items()}
         runner = cls(spec, tensors, dtype, device, **kw)
