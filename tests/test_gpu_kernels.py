@@ -475,6 +475,54 @@ def test_attention_with_a_bias_that_grows_with_the_distance(dtype, window):
         ops.paged_attention(q.cuda(), out, cache.cuda(), step, 0, nh, nkv, dh, page, dh ** -0.5, window, head_slopes=slopes[:3].cuda())
 
 
+def _pages_of(k, v, page):
+    """Keys and values ``[tokens, kv_heads, dim]`` as whole pages in the cache's layout (kv_layout.h): keys
+    [kv_head][dim / 8][token][8], values [kv_head][dim][token]; the last page is filled up with NaN."""
+    n, nkv, dh = k.shape
+    n_pages = (n + page - 1) // page
+    pad = n_pages * page - n
+    if pad:
+        k = torch.cat([k, torch.full((pad, nkv, dh), float("nan"))])
+        v = torch.cat([v, torch.full((pad, nkv, dh), float("nan"))])
+    kp = k.view(n_pages, page, nkv, dh // 8, 8).permute(0, 2, 3, 1, 4).reshape(n_pages, -1)
+    vp = v.view(n_pages, page, nkv, dh).permute(0, 2, 3, 1).reshape(n_pages, -1)
+    return torch.stack([kp, vp], dim=1)                  # [pages, 2, kv_heads * dim * page]
+
+
+@pytest.mark.parametrize("top_of_a_cache_just_below_4_gib", [False, True])
+def test_attention_over_more_than_32k_keys(top_of_a_cache_just_below_4_gib):
+    """A portion and a single token over 33,000 and 40,000 keys (the counters of tiles and turns, the
+    offsets of pages); with the pages at the top of a cache of just under 4 GiB, where a page's offset
+    from the cache's start still fits 32 bits and nearly fills them."""
+    from llama_cu_amd.kernels import ops
+    nh, nkv, dh, page = 16, 8, 128, 16
+    q_lens, ctx_lens = [48, 1], [33000, 40000]
+    page_bytes = 2 * nkv * dh * page * 2
+    need = [(c + page - 1) // page for c in ctx_lens]
+    n_pages = ((1 << 32) - 1) // page_bytes if top_of_a_cache_just_below_4_gib else sum(need) + 5
+    assert n_pages * page_bytes < 1 << 32
+    cache = torch.empty(n_pages, 2, nkv * dh * page, dtype=torch.bfloat16, device="cuda")
+    rng = random.Random(5)
+    ids = list(range(n_pages - sum(need), n_pages))       # the last pages of the cache, in a random order
+    rng.shuffle(ids)
+    tables, qs, wants = [], [], []
+    for r, (ql, cl) in enumerate(zip(q_lens, ctx_lens)):
+        k = rnd(cl, nkv, dh, seed=70 + r).to(torch.bfloat16).float()
+        v = rnd(cl, nkv, dh, seed=80 + r).to(torch.bfloat16).float()
+        q = rnd(ql, nh, dh, seed=90 + r).to(torch.bfloat16).float()
+        k[7, :] = (q[-1, ::nh // nkv] * 1.5).to(torch.bfloat16).float()       # a key far back that the last query points at
+        table = [ids.pop() for _ in range(need[r])]
+        cache[torch.tensor(table, device="cuda")] = _pages_of(k, v, page).to(torch.bfloat16).cuda()
+        tables.append(table)
+        qs.append(q)
+        wants.append(plain.attention(q, k, v, dh ** -0.5, first_pos=cl - ql, window=None))
+    step = Batch(q_lens, ctx_lens, tables, max(need) + 1).step
+    q_all = torch.cat(qs).reshape(sum(q_lens), nh * dh).to(torch.bfloat16)
+    out = torch.empty(sum(q_lens), nh * dh, dtype=torch.bfloat16, device="cuda")
+    ops.paged_attention(q_all.cuda(), out, cache, step, 0, nh, nkv, dh, page, dh ** -0.5, 0)
+    close(out, torch.cat(wants).reshape(sum(q_lens), nh * dh), "bfloat16")
+
+
 def test_attention_float32_result_does_not_depend_on_the_batch():
     from llama_cu_amd.kernels import ops
     nh, nkv, dh, page = 4, 2, 32, 16
