@@ -168,6 +168,33 @@ def run_mixed(engine, cfg, n_requests, rng, sync, new_tokens=128, lo=16, hi=2048
             "decode_step_median_ms": decode_steps[len(decode_steps) // 2], "preemptions": engine.sched.preemptions}
 
 
+def library_product(cfg, sync, calls=400):
+    """Time of the library's gate/up product of a 2,048-token prefill (the largest of a layer's four), once with
+    random rows and once with rows of zeros: the same instructions on the same addresses, but zeros switch far fewer
+    wires, so the difference is what the chip's power limit takes off its clock while it multiplies random numbers."""
+    import torch
+    g = torch.Generator(device="cuda").manual_seed(0)
+    w = (torch.randn(2 * cfg.intermediate_size, cfg.hidden_size, device="cuda", generator=g) * 0.02).to(torch.bfloat16)
+    x = torch.randn(PREFILL_TOKENS, cfg.hidden_size, device="cuda", generator=g).to(torch.bfloat16)
+    flops = 2.0 * PREFILL_TOKENS * cfg.hidden_size * 2 * cfg.intermediate_size
+    out = {}
+    for name in ("random_rows", "zero_rows"):
+        if name == "zero_rows":
+            x.zero_()
+        best = None
+        for _ in range(4):                          # the first round warms up; the clock settles within it
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            for _ in range(calls):
+                torch.nn.functional.linear(x, w)
+            b.record()
+            sync()
+            t = a.elapsed_time(b) / calls * 1e-3
+            best = t if best is None else min(best, t)
+        out[name] = {"us": round(best * 1e6, 1), "pflops": round(flops / best / 1e15, 3)}
+    return out
+
+
 def kernel_summary(db: str, steps: int) -> int:
     """Per-step table of kernels from the database that ``rocprofv3 --kernel-trace`` wrote for a
     run of this program: the kernels between two embedding gathers are one step of the model;
@@ -220,6 +247,8 @@ def main() -> int:
     ap.add_argument("--only-prefill", action="store_true", help="time the 2048-token prefill alone (for profiles)")
     ap.add_argument("--prefill-history", type=int, default=0,
                     help="with --only-prefill: time the 2048 tokens that follow this many tokens of the same prompt")
+    ap.add_argument("--library-product", action="store_true",
+                    help="time the library's gate/up product of 2048 rows with random rows and with rows of zeros, and exit")
     ap.add_argument("--kernel-summary", metavar="DB", help="print the per-step kernel table of a rocprofv3 database and exit")
     ap.add_argument("--summary-steps", type=int, default=8)
     args = ap.parse_args()
@@ -249,6 +278,10 @@ def main() -> int:
     rng = random.Random(0)
     sync = torch.cuda.synchronize
     page = args.page_size
+    if args.library_product:
+        print(json.dumps({"library_product": library_product(cfg, sync), "rows": PREFILL_TOKENS,
+                          "in": cfg.hidden_size, "out": 2 * cfg.intermediate_size, "dtype": "bf16"}))
+        return 0
     biggest = max(args.batch, 1 if (args.no_points or args.only_prefill or args.workload == "mixed") else 64)
     # a request decodes while later ones still prefill: room for that too
     per_req = max(args.prompt_len, PROMPT_LEN) + grow
