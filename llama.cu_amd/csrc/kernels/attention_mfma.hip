@@ -23,7 +23,7 @@
 //                   merged by a second kernel.
 //   prefill kernel  any number of tokens per request (also one), v_mfma_f32_32x32x16_bf16 (blocks
 //                   of 32 rows; a lane owns row lane % 32 and 16 of each 32 keys).  A workgroup of
-//                   8 waves takes consecutive tokens of one request; the keys and values of a
+//                   4 waves takes consecutive tokens of one request; the keys and values of a
 //                   step are copied to LDS once and shared by the waves.
 #include <mutex>
 
