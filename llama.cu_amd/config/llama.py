@@ -7,7 +7,7 @@ rotation base to 1e4.  Here they come from config.json under its own key names.
 """
 from __future__ import annotations
 
-from dataclasses import dataclass, field
+from dataclasses import dataclass
 from typing import Any, Dict, Tuple
 
 from .base import ConfigError, KeyReader

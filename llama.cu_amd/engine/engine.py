@@ -13,16 +13,15 @@ beyond an end-of-sequence token that was learned late is cut away again.  With
 """
 from __future__ import annotations
 
-import time
-from dataclasses import dataclass, field
-from typing import Callable, Dict, List, Optional, Sequence, Tuple, Union
+from dataclasses import dataclass
+from typing import Callable, Dict, List, Optional, Sequence, Union
 
 import torch
 
 from ..kernels import ops
 from ..sampling import GREEDY, Sampler, SamplingParams
 from .runner import ModelRunner
-from .scheduler import PlanEntry, Scheduler
+from .scheduler import Scheduler
 
 
 @dataclass

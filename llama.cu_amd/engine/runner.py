@@ -11,7 +11,6 @@ sampled ids instead of logits.)
 from __future__ import annotations
 
 import sys
-from dataclasses import dataclass
 from typing import Any, Dict, List, Optional, Sequence
 
 import torch

@@ -9,7 +9,7 @@ branch's output as ``pending``, and whoever norms next adds it.
 """
 from __future__ import annotations
 
-from typing import Dict, Optional
+from typing import Dict
 
 import torch
 

@@ -15,7 +15,7 @@ from typing import Dict, List, Optional
 import torch
 
 from ..kernels import ops
-from .base import BuildContext, ModelSpec, Part, PartSpec, ScaledRows, TensorSpec, make_part, prefixed, register_part
+from .base import BuildContext, ModelSpec, Part, ScaledRows, TensorSpec, make_part, prefixed, register_part
 from .linear import Weight, linear, linear_scaled, skinny_takes
 
 

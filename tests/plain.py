@@ -10,10 +10,9 @@ Paths are relative to the reference's root.
 from __future__ import annotations
 
 import json
-import math
 import os
 import struct
-from dataclasses import dataclass, field
+from dataclasses import dataclass
 from typing import Dict, List, Optional, Sequence
 
 import numpy as np

@@ -1,6 +1,5 @@
 """The cache manager on the CPU: pages in groups, block tables, windows, state slots.
 No page is lost, held twice or freed twice, under random orders of requests."""
-import ctypes
 import random
 
 import pytest

@@ -1,7 +1,6 @@
 """Configuration and registry: every size and constant comes from config.json's keys,
 errors name the key, and the architecture's name picks the model."""
 import json
-import os
 
 import pytest
 

@@ -4,7 +4,6 @@ a window with pages of its own, and a toy mixer with per-request state that is d
 here, registered, built and stepped without a change to the framework."""
 import copy
 
-import numpy as np
 import pytest
 import torch
 
