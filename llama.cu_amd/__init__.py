@@ -41,3 +41,7 @@ def generate(model: str, prompts, sampling: SamplingParams = SamplingParams(), m
 
 __all__ = ["config", "parts", "models", "weights", "LlamaConfig", "register_architecture", "register_part",
            "SamplingParams", "Engine", "generate"]
+
+# modules of the user's that register further architectures or parts (LLAMA_CU_AMD_PLUGINS=module[,module]): imported
+# last, when everything they may import from here is there
+config.load_plugins_from_env()

@@ -27,12 +27,19 @@ def _base(p: argparse.ArgumentParser) -> None:
     p.add_argument("--num-pages", type=int, default=None, help="pages in the cache pool (default: from free memory)")
     p.add_argument("--max-tokens", type=int, default=None, help="size of the cache pool in tokens, instead of --num-pages")
     p.add_argument("--max-seqs", type=int, default=4, help="most requests that run at a time (default 4)")
+    _plugin_option(p)
 
 
 def model_folder(path: str) -> str:
     """The folder of MODEL: MODEL itself, or the folder of a config.json that was named."""
     import os
     return os.path.dirname(os.path.abspath(path)) if os.path.isfile(path) else path
+
+
+def _plugin_option(p) -> None:
+    p.add_argument("--plugin", action="append", default=[], metavar="MODULE",
+                   help="import MODULE first (a module of yours that registers an architecture or parts); may be given "
+                        "several times; the environment variable LLAMA_CU_AMD_PLUGINS names modules too")
 
 
 def _engine(args):
@@ -176,6 +183,9 @@ def main(argv: Optional[List[str]] = None) -> int:
     r.add_argument("--seed", type=int, default=0)
     r.add_argument("--dtype", choices=["bfloat16", "float32"], default="bfloat16", help="type of the stored matrices")
     r.add_argument("--std", type=float, default=0.02, help="standard deviation of the matrices' entries")
+    _plugin_option(r)
     r.set_defaults(func=random_model)
     args = ap.parse_args(argv)
+    from .config import load_plugins
+    load_plugins(args.plugin)
     return args.func(args)

@@ -7,8 +7,10 @@ switch is a table that anyone may add to.
 """
 from __future__ import annotations
 
+import importlib
+import os
 from dataclasses import dataclass
-from typing import Any, Callable, Dict, List
+from typing import Any, Callable, Dict, Iterable, List
 
 from .base import ConfigError, read_config_json
 
@@ -40,8 +42,37 @@ def architecture_of(data: Dict[str, Any], where: str = "config.json") -> Archite
     arch = _REGISTRY.get(names[0])
     if arch is None:
         raise ConfigError(f"{where}: architecture {names[0]!r} is not registered; "
-                          f"registered: {registered_architectures()}")
+                          f"registered: {registered_architectures()} (a module that registers another one is "
+                          f"named with --plugin or in {PLUGINS_ENV})")
     return arch
+
+
+PLUGINS_ENV = "LLAMA_CU_AMD_PLUGINS"
+_loaded_plugins: List[str] = []
+
+
+def load_plugins(names: Iterable[str]) -> List[str]:
+    """Import the modules ``names`` (found as any module is, on ``sys.path``): modules of the user's that call
+    ``register_architecture`` and ``register_part`` when they are imported, so that the command line, the replay
+    program and the Python entry point know an architecture or a part that is no file of this package.  A module
+    is imported once; one that cannot be imported raises a ConfigError that names it."""
+    done = []
+    for name in names:
+        name = name.strip()
+        if not name or name in _loaded_plugins:
+            continue
+        try:
+            importlib.import_module(name)
+        except Exception as e:
+            raise ConfigError(f"plugin module {name!r} could not be imported: {type(e).__name__}: {e}") from e
+        _loaded_plugins.append(name)
+        done.append(name)
+    return done
+
+
+def load_plugins_from_env() -> List[str]:
+    """The modules named in the environment variable LLAMA_CU_AMD_PLUGINS (separated by commas)."""
+    return load_plugins(os.environ.get(PLUGINS_ENV, "").split(","))
 
 
 def load_config(folder: str):

@@ -8,7 +8,7 @@ import random
 import subprocess
 import sys
 import tempfile
-from typing import Dict, List, Optional, Sequence
+from typing import Dict, List, Optional, Sequence, Tuple
 
 import numpy as np
 import torch
@@ -196,12 +196,14 @@ def run_trace_inprocess(folder: str, dtype: str, steps, max_tokens: int, stats: 
     return outputs
 
 
-def run_trace_program(folder: str, dtype: str, steps, max_tokens: int, vocab: int, extra: Sequence[str] = ()) -> Dict[int, np.ndarray]:
+def run_trace_program(folder: str, dtype: str, steps, max_tokens: int, vocab: int, extra: Sequence[str] = (),
+                      env: Optional[dict] = None) -> Dict[int, np.ndarray]:
     """Through ``bin/trace_run`` as a user runs it."""
     out_dir = tempfile.mkdtemp(prefix="lcu_trace_")
     text = "".join(json.dumps(s) + "\n" for s in steps)
     proc = subprocess.run([os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", dtype, "--out", out_dir,
-                           "--max-tokens", str(max_tokens)] + list(extra), input=text, capture_output=True, text=True, timeout=600)
+                           "--max-tokens", str(max_tokens)] + list(extra), input=text, capture_output=True, text=True, timeout=600,
+                          env=env)
     assert proc.returncode == 0, proc.stderr[-2000:]
     done = [l for l in proc.stdout.splitlines() if l.startswith("done ")]
     assert done == [f"done {s['step']}" for s in steps]
@@ -235,3 +237,86 @@ def assert_matches_plain(got: Dict[str, Dict[int, np.ndarray]], want: Dict[str, 
             err = float(np.abs(got[name][pos].astype(np.float64) - ref[pos]).max())
             assert np.isfinite(err) and err <= rel * scale, \
                 f"{what}: request {name}, first wrong position {pos} of {ref.shape[0]}: error {err:.3e} > {rel * scale:.3e}"
+
+
+# ----------------------------------------------------------------------------- a plugin
+# A module of a user's, as a file outside the package: an architecture of its own (the Llama layout, but the layer
+# that config.json's "mean_layer" names mixes with a running mean of its inputs, whose state of fixed size lives in
+# the engine's state slots) with a part of its own.  Named with --plugin or in LLAMA_CU_AMD_PLUGINS.
+TOY_PLUGIN = '''
+import dataclasses
+
+import torch
+
+from llama_cu_amd import register_architecture, register_part
+from llama_cu_amd.config import LlamaConfig
+from llama_cu_amd.models.llama import llama_spec
+from llama_cu_amd.parts import Part, PartSpec, SlotState, TensorSpec
+
+
+class RunningMean(Part):
+    def __init__(self, hidden_size):
+        self.d = hidden_size
+
+    def tensors(self):
+        return {"mix.weight": TensorSpec((self.d, self.d))}
+
+    def cache_need(self):
+        return SlotState((self.d,), torch.float32)
+
+    def load(self, tensors, build):
+        self.w = tensors["mix.weight"].float()
+
+    def forward(self, h, step, cache):
+        out = torch.empty_like(h)
+        start = 0
+        for r, n in enumerate(step.q_lens):
+            slot = step.state_slots[r]
+            first = step.ctx_lens[r] - n
+            if first == 0:
+                cache.state[slot].zero_()
+            sums = cache.state[slot] + torch.cumsum(h[start:start + n].float(), 0)
+            counts = torch.arange(first + 1, first + n + 1, device=h.device, dtype=torch.float32)[:, None]
+            out[start:start + n] = ((sums / counts) @ self.w.T).to(h.dtype)
+            cache.state[slot] = sums[-1]
+            start += n
+        return out
+
+
+@dataclasses.dataclass(frozen=True)
+class ToyMeanConfig:
+    base: LlamaConfig
+    mean_layer: int
+
+    @staticmethod
+    def from_dict(d):
+        d = dict(d)
+        mean_layer = int(d.pop("mean_layer"))
+        d["architectures"] = ["LlamaForCausalLM"]
+        base = LlamaConfig.from_dict(d)
+        if not 0 <= mean_layer < base.num_hidden_layers:
+            raise ValueError("mean_layer names no layer")
+        return ToyMeanConfig(base, mean_layer)
+
+    def to_dict(self):
+        return dict(self.base.to_dict(), architectures=["ToyMeanForCausalLM"], mean_layer=self.mean_layer)
+
+
+def toy_mean_spec(cfg):
+    spec = llama_spec(cfg.base)
+    spec.layers[cfg.mean_layer].params["mixer"] = PartSpec("running_mean", {"hidden_size": cfg.base.hidden_size}, "toy")
+    return spec
+
+
+register_part("mixer", "running_mean", RunningMean, replace=True)
+register_architecture("ToyMeanForCausalLM", ToyMeanConfig.from_dict, toy_mean_spec, replace=True)
+'''
+
+
+def write_toy_plugin(folder: str, name: str = "lcu_toy_plugin") -> Tuple[str, dict]:
+    """Writes the module into ``folder``; returns its name and an environment in which a child process finds it."""
+    with open(os.path.join(folder, name + ".py"), "w") as f:
+        f.write(TOY_PLUGIN)
+    env = dict(os.environ)
+    env["PYTHONPATH"] = folder + os.pathsep + env.get("PYTHONPATH", "")
+    return name, env

@@ -1,6 +1,7 @@
 """Configuration and registry: every size and constant comes from config.json's keys,
 errors name the key, and the architecture's name picks the model."""
 import json
+import os
 
 import pytest
 
@@ -140,3 +141,37 @@ def test_decode_attention_split_rule():
         assert decode_splits(b, 32, 8, 2100) == 1            # up to 4k keys: one part
     assert decode_splits(20, 32, 8, 8192) == 3 and decode_splits(48, 32, 8, 8192) == 1 and decode_splits(64, 32, 8, 8192) == 1
     assert decode_splits(20, 32, 8, 4097) == 3 and decode_splits(20, 32, 8, 4096) == 1
+
+
+def test_a_module_of_the_user_s_registers_an_architecture_for_the_command_line(tmp_path):
+    """--plugin MODULE (and LLAMA_CU_AMD_PLUGINS) import a module that is no file of the package before a model is
+    looked up: an architecture and a part that only that module knows are then found by the registry, here by
+    ``random-model``, which writes the folder of such a model."""
+    import json
+    import subprocess
+    import sys
+    from llama_cu_amd.config import ConfigError, load_plugins
+    from llama_cu_amd.weights.safetensors_io import open_safetensors
+    name, env = common.write_toy_plugin(str(tmp_path))
+    cfg = dict(common.TINY_A, architectures=["ToyMeanForCausalLM"], mean_layer=1)
+    (tmp_path / "config.json").write_text(json.dumps(cfg))
+    tool = os.path.join(common.ROOT, "bin", "llama.cu_amd")
+    # without the module: one line that says what is registered and how to name a module
+    bare = subprocess.run([tool, "random-model", str(tmp_path / "config.json"), str(tmp_path / "m0")], capture_output=True, text=True, env=env)
+    assert bare.returncode != 0 and "ToyMeanForCausalLM" in bare.stderr and "--plugin" in bare.stderr
+    ok = subprocess.run([tool, "random-model", str(tmp_path / "config.json"), str(tmp_path / "m1"), "--plugin", name, "--dtype", "float32"],
+                        capture_output=True, text=True, env=env)
+    assert ok.returncode == 0, ok.stderr[-2000:]
+    names = [n for f in open_safetensors(str(tmp_path / "m1")) for n in f.names()]
+    assert "model.layers.1.toy.mix.weight" in names and "model.layers.1.self_attn.q_proj.weight" not in names
+    assert "model.layers.0.self_attn.q_proj.weight" in names
+    assert json.loads((tmp_path / "m1" / "config.json").read_text())["mean_layer"] == 1
+    # the environment variable does the same for every entry point
+    env2 = dict(env, LLAMA_CU_AMD_PLUGINS=name)
+    via_env = subprocess.run([sys.executable, "-c", "import sys; sys.path.insert(0, %r); import llama_cu_amd; "
+                              "from llama_cu_amd.config import registered_architectures; print(registered_architectures())" % common.ROOT],
+                             capture_output=True, text=True, env=env2)
+    assert via_env.returncode == 0 and "ToyMeanForCausalLM" in via_env.stdout, via_env.stderr[-2000:]
+    # a module that cannot be imported is named
+    with pytest.raises(ConfigError, match="no_such_module_anywhere"):
+        load_plugins(["no_such_module_anywhere"])

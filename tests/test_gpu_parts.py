@@ -3,6 +3,7 @@ composition: a run order that names a layer twice and lets a layer read another'
 a window with pages of its own, and a toy mixer with per-request state that is defined
 here, registered, built and stepped without a change to the framework."""
 import copy
+import os
 
 import pytest
 import torch
@@ -274,6 +275,23 @@ def test_a_layer_with_pages_of_its_own_size(dtype):
 
 
 # ----------------------------------------------------------------------------- a toy mixer with state of its own
+def toy_mean_direct(cfg_d, w, toks):
+    """The logits of the toy model whose layer 1 mixes with a running mean (layer 0 is a Llama layer), computed
+    directly from the plain implementation's functions."""
+    pcfg = plain.PlainConfig.from_dict(cfg_d)
+    sin, cos = plain.rope_tables(len(toks), 16, pcfg.rope_theta)
+    x = plain.embedding(w["model.embed_tokens.weight"], toks)
+    p = "model.layers.0."
+    x = x + plain.attention_block(pcfg, w, p, plain.rms_norm(x, w[p + "input_layernorm.weight"], 1e-5), list(range(len(toks))), sin, cos)
+    x = x + plain.feed_forward(w, p, plain.rms_norm(x, w[p + "post_attention_layernorm.weight"], 1e-5))
+    p = "model.layers.1."
+    h = plain.rms_norm(x, w[p + "input_layernorm.weight"], 1e-5)
+    mean = torch.cumsum(h, 0) / torch.arange(1, len(toks) + 1, dtype=torch.float64)[:, None]
+    x = x + mean @ w[p + "toy.mix.weight"].double().T
+    x = x + plain.feed_forward(w, p, plain.rms_norm(x, w[p + "post_attention_layernorm.weight"], 1e-5))
+    return plain.linear(plain.rms_norm(x, w["model.norm.weight"], 1e-5), w["lm_head.weight"])
+
+
 def test_a_toy_mixer_with_state_is_registered_built_and_stepped():
     """The mixer ``running_mean`` is defined here: its output at a token is a matrix times
     the mean of its inputs up to that token.  Its state per request (the running sum, of
@@ -325,18 +343,7 @@ def test_a_toy_mixer_with_state_is_registered_built_and_stepped():
     assert not runner.use_graphs                # the toy reads lengths on the host: its steps are not captured
 
     def direct(toks):
-        pcfg = plain.PlainConfig.from_dict(cfg_d)
-        sin, cos = plain.rope_tables(len(toks), 16, pcfg.rope_theta)
-        x = plain.embedding(w["model.embed_tokens.weight"], toks)
-        p = "model.layers.0."
-        x = x + plain.attention_block(pcfg, w, p, plain.rms_norm(x, w[p + "input_layernorm.weight"], 1e-5), list(range(len(toks))), sin, cos)
-        x = x + plain.feed_forward(w, p, plain.rms_norm(x, w[p + "post_attention_layernorm.weight"], 1e-5))
-        p = "model.layers.1."
-        h = plain.rms_norm(x, w[p + "input_layernorm.weight"], 1e-5)
-        mean = torch.cumsum(h, 0) / torch.arange(1, len(toks) + 1, dtype=torch.float64)[:, None]
-        x = x + mean @ w[p + "toy.mix.weight"].double().T
-        x = x + plain.feed_forward(w, p, plain.rms_norm(x, w[p + "post_attention_layernorm.weight"], 1e-5))
-        return plain.linear(plain.rms_norm(x, w["model.norm.weight"], 1e-5), w["lm_head.weight"])
+        return toy_mean_direct(cfg_d, w, toks)
 
     reqs = common.random_requests(256, [40, 9, 77, 30, 5], 12)
     want = {k: direct(v) for k, v in reqs.items()}
@@ -653,3 +660,29 @@ def test_an_end_learned_late_with_a_cache_that_cannot_be_cut_back(kind):
         whole = fresh.generate([prompt + probe[:at + 1] + more], max_steps=len(want[1][0]), ignore_eos=True)[0]
         stop = want[1][0].index(eos) + 1 if eos in want[1][0] else len(want[1][0])
         assert want[1][0][:stop] == whole[:stop]
+
+
+def test_an_architecture_of_a_module_outside_the_package_through_the_programs(tmp_path):
+    """A whole architecture with a part of its own, defined in a module that is no file of the package and named
+    with --plugin: ``random-model`` writes its folder, ``bin/trace_run`` replays a mixed trace on it (config.json's
+    architecture picks the model, as everywhere) and agrees with a direct computation, ``generate`` generates."""
+    import json
+    import subprocess
+    from llama_cu_amd.weights.safetensors_io import open_safetensors
+    name, env = common.write_toy_plugin(str(tmp_path))
+    cfg_d = dict(common.TINY_A)
+    (tmp_path / "config.json").write_text(json.dumps(dict(cfg_d, architectures=["ToyMeanForCausalLM"], mean_layer=1)))
+    tool = os.path.join(common.ROOT, "bin", "llama.cu_amd")
+    folder = str(tmp_path / "model")
+    made = subprocess.run([tool, "random-model", str(tmp_path / "config.json"), folder, "--plugin", name, "--dtype", "float32", "--std", "0.15",
+                           "--seed", "4"], capture_output=True, text=True, env=env, timeout=300)
+    assert made.returncode == 0, made.stderr[-2000:]
+    w = {n: f.tensor(n).double() for f in open_safetensors(folder) for n in f.names()}
+    reqs = common.random_requests(256, [40, 9, 77, 30], 21)
+    want = {k: toy_mean_direct(cfg_d, w, v) for k, v in reqs.items()}
+    steps, _ = common.trace_mixed(reqs, max_live=3)
+    outputs = common.run_trace_program(folder, "float32", steps, 256, 256, extra=["--plugin", name, "--max-live", "3"], env=env)
+    common.assert_matches_plain(common.collect(steps, outputs, 256), want, "float32", "architecture of a plugin")
+    gen = subprocess.run([tool, "generate", folder, "--plugin", name, "--dtype", "float32", "--max-steps", "6", "-p", "ab"],
+                         capture_output=True, text=True, env=env, timeout=300)
+    assert gen.returncode == 0 and "n toks = " in gen.stderr + gen.stdout, (gen.stdout + gen.stderr)[-2000:]
