@@ -107,7 +107,7 @@ def library_friendly_rows(di: int, d: int, device) -> int:
     """The number of rows to which each half of a bfloat16 gate/up matrix ``[2 * di, d]`` is filled up
     with rows of zeros for the library's product of many rows.  The library's choice of kernel
     depends on the number of output features in ways that no rule predicts: with 2,048 rows and
-    K = 4096 it takes 420 us for 22,016 features (the Llama-2-7B shape) and 278 us for 24,576.
+    K = 4096 it takes 417 us for 22,016 features (the Llama-2-7B shape) and 320 us for 24,576.
     So a large matrix is timed once, at 2,048 rows, as it is and with each half filled up to the
     next multiples of 1024, 2048 and 4096; rows are added only if that is at least 15 % faster.
     The rows of zeros give zeros (silu(0) * 0), which whoever multiplies next leaves out."""
@@ -121,7 +121,11 @@ def library_friendly_rows(di: int, d: int, device) -> int:
         x = torch.randn(2048, d, device=device, dtype=torch.bfloat16)
         times = {}
         for rows in sorted({di} | {-(-di // m) * m for m in (1024, 2048, 4096)}):
+            # numbers as a model's, zeros only where the rows of zeros would be: with a matrix of zeros the card's clock is
+            # higher (its power limit is further away) and the comparison another
             w = torch.zeros(2 * rows, d, device=device, dtype=torch.bfloat16)
+            for half in (0, 1):
+                w[half * rows:half * rows + di].normal_(0.0, 0.02)
             for _ in range(2):
                 torch.matmul(x, w.t())
             start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
