@@ -51,6 +51,9 @@ class StepContext:
     # to be taken from row feed_src[i] of that step's sampled ids, on the device
     feed_src: Optional[torch.Tensor] = None
     feed_dst: Optional[torch.Tensor] = None
+    # the requests' indices, the one that holds most tokens first: the order in which the decode attention starts its
+    # workgroups (those that walk the most keys must not start last)
+    decode_order: Optional[torch.Tensor] = None
 
     def block_table(self, group: int) -> torch.Tensor:
         return self.block_tables[group]
@@ -84,7 +87,7 @@ class BatchBuilder:
         self.device = device
         n, r = self.max_tokens, self.max_reqs
         sizes = [("tokens", n), ("positions", n), ("req_of_token", n), ("logit_rows", n),
-                 ("q_start", r + 1), ("ctx_len", r), ("state_slot", r), ("feed_src", r), ("feed_dst", r)]
+                 ("q_start", r + 1), ("ctx_len", r), ("state_slot", r), ("feed_src", r), ("feed_dst", r), ("decode_order", r)]
         for g, mp in enumerate(self.max_pages):
             sizes += [(f"slots{g}", n), (f"block_table{g}", r * mp)]
         self.offsets = {}
@@ -149,11 +152,12 @@ class BatchBuilder:
         self.cache.fill_batch(req_ids, n_new, ptr("positions"), ptr("req_of_token"), ptr("q_start"), ptr("ctx_len"),
                               ptr("state_slot"), [ptr(f"block_table{g}") for g in range(len(self.max_pages))],
                               self.max_pages, [ptr(f"slots{g}") for g in range(len(self.max_pages))])
+        ctx_lens = self._h("ctx_len")[:n_req].tolist()
+        self._h("decode_order")[:n_req] = torch.tensor(sorted(range(n_req), key=lambda i: -ctx_lens[i]), dtype=torch.int32)
         self.dev.copy_(self.host, non_blocking=True)
         if self.device.type == "cuda":
             self._copied = torch.cuda.Event()
             self._copied.record()
-        ctx_lens = self._h("ctx_len")[:n_req].tolist()
         return StepContext(
             n=n, n_req=n_req, tokens=self._d("tokens", n), positions=self._d("positions", n),
             req_of_token=self._d("req_of_token", n), q_start=self._d("q_start", n_req + 1),
@@ -164,4 +168,5 @@ class BatchBuilder:
             q_lens=n_new, ctx_lens=ctx_lens, req_ids=list(req_ids),
             state_slots=self._h("state_slot")[:n_req].tolist(),
             feed_src=self._d("feed_src", len(feed)) if feed else None,
-            feed_dst=self._d("feed_dst", len(feed)) if feed else None)
+            feed_dst=self._d("feed_dst", len(feed)) if feed else None,
+            decode_order=self._d("decode_order", n_req))

@@ -440,15 +440,17 @@ def paged_attention(q: torch.Tensor, out: torch.Tensor, cache: torch.Tensor, ste
                         page_size)
     if step.decode_only:
         splits = step.attn_splits or decode_splits(step.n_req, n_heads, n_kv_heads, step.max_ctx_len)
+        # the workgroups start in the order of the requests' list: the requests with the most keys first, where the
+        # batch says which they are (64 requests of 150 to 2,200 keys: the step 11.2 -> 11.0 ms)
         return attention_decode(q, out, cache, bt, step.q_start, step.ctx_len, step.n_req, n_heads, n_kv_heads, head_dim,
-                                page_size, scale, window, splits)
+                                page_size, scale, window, splits, req_list=step.decode_order)
     # a mixed batch: the requests that decode one token go to the decode kernel, the portions
     # to the prefill kernel (each would be slow at the other's work)
     lib = build.load("attention_mfma")
     tpt = lib.lcu_attention_prefill_tokens_per_task(n_heads, n_kv_heads)
     key = ("attention_tasks", tpt)
     if key not in step.scratch:
-        singles = [r for r, n in enumerate(step.q_lens) if n == 1]
+        singles = sorted((r for r, n in enumerate(step.q_lens) if n == 1), key=lambda r: -step.ctx_lens[r])    # most keys first
         use_decode = len(singles) >= 1
         tasks = prefill_tasks(step.q_lens, step.ctx_lens, tpt, q.device, skip_single=use_decode)
         req_list = to_device(singles, torch.int32, q.device) if use_decode else None

@@ -360,6 +360,11 @@ def test_attention_decode_kernel(nh, nkv, dh, page, window, splits):
     out = torch.empty(q.shape[0], nh * dh, dtype=torch.bfloat16, device="cuda")
     ops.paged_attention(q.cuda(), out, cache.cuda(), step, 0, nh, nkv, dh, page, dh ** -0.5, window)
     close(out, want, "bfloat16")
+    # the order in which the workgroups take the requests (the batch builder names the longest first) changes no bit
+    step.decode_order = torch.tensor([5, 4, 3, 2, 1, 0], dtype=torch.int32, device="cuda")
+    ordered = torch.full_like(out, float("nan"))
+    ops.paged_attention(q.cuda(), ordered, cache.cuda(), step, 0, nh, nkv, dh, page, dh ** -0.5, window)
+    assert torch.equal(ordered, out)
 
 
 @pytest.mark.parametrize("nh,nkv,dh,page", [(8, 2, 128, 16), (4, 1, 64, 32)])
