@@ -158,6 +158,7 @@ class ModelRunner:
         self.use_graphs = bool(use_graphs) and self.model.graph_safe
         self._graphs: Dict[tuple, Any] = {}        # (batch size, key parts) -> (graph, its logits)
         self._seen: Dict[tuple, int] = {}
+        self.graph_replays: Dict[tuple, int] = {}  # how often each was replayed
 
     # ------------------------------------------------------------ construction helpers
     @classmethod
@@ -278,6 +279,7 @@ class ModelRunner:
             entry = self._graphs[key] = (graph, logits)
         graph, logits = entry
         graph.replay()
+        self.graph_replays[key] = self.graph_replays.get(key, 0) + 1
         return logits
 
     def _decode_splits(self, batch: int, max_ctx_len: int) -> int:

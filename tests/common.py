@@ -63,8 +63,10 @@ def plain_logits(folder: str, reqs: Dict[str, List[int]]) -> Dict[str, torch.Ten
 
 
 # ----------------------------------------------------------------------------- traces
-def ceil64(n: int) -> int:
-    return (n + 63) // 64 * 64
+def ceil64(n: int, page: int = 16) -> int:
+    """What a request of ``n`` tokens counts for in ``--max-tokens``: ``n`` rounded up to a multiple of 64, or to
+    whole pages where that is more (pages that do not divide 64)."""
+    return max((n + 63) // 64 * 64, (n + page - 1) // page * page)
 
 
 def _want(name, first, n, keep):
@@ -73,16 +75,16 @@ def _want(name, first, n, keep):
     return [k for k in range(n) if keep is None or keep(name, first + k)]
 
 
-def trace_whole(reqs, keep=None):
+def trace_whole(reqs, keep=None, page=16):
     """Each request alone and whole: one step with all its tokens, all logits wanted."""
     steps = []
     for name, toks in reqs.items():
         steps.append({"step": len(steps), "entries": [{"id": name, "tokens": toks, "want": _want(name, 0, len(toks), keep)}],
                       "end": [name]})
-    return steps, max(ceil64(len(t)) for t in reqs.values())
+    return steps, max(ceil64(len(t), page) for t in reqs.values())
 
 
-def trace_tail_decode(reqs, tail=32, keep=None):
+def trace_tail_decode(reqs, tail=32, keep=None, page=16):
     """Most of a request in one step, its last ``tail`` tokens one by one."""
     steps = []
     for name, toks in reqs.items():
@@ -93,10 +95,10 @@ def trace_tail_decode(reqs, tail=32, keep=None):
         for i in range(head, len(toks)):
             steps.append({"step": len(steps), "entries": [{"id": name, "tokens": [toks[i]], "want": _want(name, i, 1, keep)}],
                           "end": [name] if i == len(toks) - 1 else []})
-    return steps, max(ceil64(len(t)) for t in reqs.values())
+    return steps, max(ceil64(len(t), page) for t in reqs.values())
 
 
-def trace_portions(reqs, sizes=(7, 2, 16, 3, 48, 2, 1, 33, 5, 2), keep=None):
+def trace_portions(reqs, sizes=(7, 2, 16, 3, 48, 2, 1, 33, 5, 2), keep=None, page=16):
     """Portions of changing size, down to two tokens (and one), across page edges."""
     steps = []
     k = 0
@@ -108,12 +110,13 @@ def trace_portions(reqs, sizes=(7, 2, 16, 3, 48, 2, 1, 33, 5, 2), keep=None):
             steps.append({"step": len(steps), "entries": [{"id": name, "tokens": toks[fed:fed + n], "want": _want(name, fed, n, keep)}],
                           "end": [name] if fed + n == len(toks) else []})
             fed += n
-    return steps, max(ceil64(len(t)) for t in reqs.values())
+    return steps, max(ceil64(len(t), page) for t in reqs.values())
 
 
-def trace_mixed(reqs, seed=0, max_live=4, tail=12, sizes=(2, 2, 3, 5, 7, 16, 17, 31, 48), keep=None, preempt=0.0):
+def trace_mixed(reqs, seed=0, max_live=4, tail=12, sizes=(2, 2, 3, 5, 7, 16, 17, 31, 48), keep=None, preempt=0.0, page=16):
     """Up to ``max_live`` requests at a time: portions of some beside single tokens of
-    others; requests sit steps out; finished requests' pages go to the next ones.  ``preempt``:
+    others; requests sit steps out; finished requests' pages go to the next ones.  ``page``: the
+    tokens of a page of the engine that will replay it (for the count of tokens only).  ``preempt``:
     the chance per step that one live request loses its pages (it is computed again when it next
     appears).  Returns the steps and the smallest ``--max-tokens`` that holds them."""
     rng = random.Random(seed)
@@ -143,7 +146,7 @@ def trace_mixed(reqs, seed=0, max_live=4, tail=12, sizes=(2, 2, 3, 5, 7, 16, 17,
             toks, fed = reqs[name], live[name]
             entries.append({"id": name, "tokens": toks[fed:fed + 1], "want": _want(name, fed, 1, keep)})
             live[name] = fed + 1
-        need = max(need, sum(ceil64(v) for v in live.values()))
+        need = max(need, sum(ceil64(v, page) for v in live.values()))
         for name in list(live):
             if live[name] == len(reqs[name]):
                 end.append(name)
@@ -320,3 +323,27 @@ def write_toy_plugin(folder: str, name: str = "lcu_toy_plugin") -> Tuple[str, di
     env = dict(os.environ)
     env["PYTHONPATH"] = folder + os.pathsep + env.get("PYTHONPATH", "")
     return name, env
+
+
+# ----------------------------------------------------------------------------- a sweep of configurations
+def sweep_configuration(seed: int):
+    """A configuration, a page size and request lengths drawn from ``seed``: the generator of a search for wrong
+    logits over some 1,700 seeds.  Among them are the widest and deepest models that tests replay (width up to
+    512, three layers), where bfloat16 rounding adds up to the most."""
+    rng = random.Random(seed * 7919)
+    mfma = rng.random() < 0.6
+    nkv = rng.choice([1, 2, 3, 4, 8])
+    g = rng.choice([1, 2, 4, 8, 16]) if mfma else rng.choice([1, 2, 3, 5, 7])
+    dh = rng.choice([32, 64, 96, 128]) if mfma else rng.choice([16, 48, 80, 112, 144, 256])
+    cfg = dict(architectures=["LlamaForCausalLM"], num_hidden_layers=rng.choice([1, 2, 3]),
+               hidden_size=rng.choice([64, 72, 128, 136, 192, 256, 320, 384, 512, 8 * rng.randrange(5, 40)]),
+               num_attention_heads=nkv * g, num_key_value_heads=nkv, head_dim=dh,
+               intermediate_size=rng.choice([56, 128, 172, 352, 2 * rng.randrange(4, 300), 16 * rng.randrange(1, 40),
+                                             8 * rng.randrange(1, 80)]),
+               vocab_size=rng.choice([257, 384, 1000, 16 * rng.randrange(4, 80), rng.randrange(50, 1500)]),
+               max_position_embeddings=512, rope_theta=rng.choice([1e4, 5e5]),
+               rms_norm_eps=rng.choice([1e-5, 1e-6]), tie_word_embeddings=rng.random() < 0.5,
+               rope_interleaved=rng.random() < 0.2)
+    page = rng.choice([16, 32, 48, 64, 128])
+    lens = [rng.randrange(1, 140) for _ in range(rng.choice([2, 3, 4]))]
+    return cfg, page, lens

@@ -21,6 +21,16 @@ import torch
 F64 = torch.float64
 
 
+def rounded(x: torch.Tensor, rounding: Optional[str]) -> torch.Tensor:
+    """``x`` as a tensor of the type ``rounding`` holds it (None: as it is; "bfloat16": rounded to 32-bit, as
+    a kernel's accumulator holds it, and then to bfloat16, as the kernel stores it)."""
+    if rounding is None:
+        return x
+    if rounding != "bfloat16":
+        raise ValueError(f"rounding {rounding!r}: None or 'bfloat16'")
+    return x.to(torch.float32).to(torch.bfloat16).to(F64)
+
+
 # --------------------------------------------------------------------------- parts
 
 
@@ -102,7 +112,7 @@ def rope(x: torch.Tensor, pos: Sequence[int], sin: torch.Tensor, cos: torch.Tens
 
 
 def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float,
-              first_pos: int = 0, window: Optional[int] = None) -> torch.Tensor:
+              first_pos: int = 0, window: Optional[int] = None, rounding: Optional[str] = None) -> torch.Tensor:
     """Causal attention of the queries ``q [nq, nh, dh]`` over the keys ``k, v [nk, nkvh, dh]``.
 
     The call contract is llama.cu/src/exec/step.rs:162-178: causal mask with the
@@ -111,7 +121,9 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float,
     operator itself lies outside the reference's tree; taken as usual: head ``h`` reads
     the key/value head ``h // (nh/nkvh)``, scores are scaled by ``scale``
     (``dh**-0.5`` for Llama), softmax over the visible keys.  ``window`` (not used by
-    Llama) limits a query to the last ``window`` keys, itself included.
+    Llama) limits a query to the last ``window`` keys, itself included.  ``rounding``: the
+    weights ``exp(s - max)`` are rounded to that type before they multiply the values, and the
+    sum that divides them is that of the unrounded weights.
     """
     q, k, v = q.to(F64), k.to(F64), v.to(F64)
     nq, nh, dh = q.shape
@@ -126,8 +138,11 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float,
             s = (k[lo:p + 1, kv, :] @ q[t, h, :]) * scale
             s = s - s.max()
             e = torch.exp(s)
-            a = e / e.sum()
-            out[t, h, :] = a @ v[lo:p + 1, kv, :]
+            if rounding is None:
+                a = e / e.sum()
+                out[t, h, :] = a @ v[lo:p + 1, kv, :]
+            else:
+                out[t, h, :] = (rounded(e, rounding) @ v[lo:p + 1, kv, :]) / e.sum()
     return out
 
 
@@ -178,7 +193,8 @@ class PlainConfig:
 
 
 def attention_block(cfg: PlainConfig, w: Dict[str, torch.Tensor], prefix: str, x1: torch.Tensor,
-                    pos: Sequence[int], sin, cos, shared_kv=None, keep_kv: Optional[list] = None) -> torch.Tensor:
+                    pos: Sequence[int], sin, cos, shared_kv=None, keep_kv: Optional[list] = None,
+                    rounding: Optional[str] = None) -> torch.Tensor:
     """q, k, v projections, rotation of q and k, causal attention, output projection,
 for one whole sequence: ``pos`` (the positions the rotation uses) may start anywhere,
 the mask only counts places in the sequence.
@@ -189,30 +205,33 @@ the mask only counts places in the sequence.
     """
     n = x1.shape[0]
     nh, nkvh, dh = cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim
-    q = linear(x1, w[prefix + "self_attn.q_proj.weight"]).view(n, nh, dh)
-    q = rope(q, pos, sin, cos, cfg.rope_pairing)
+    R = lambda t: rounded(t, rounding)
+    q = R(linear(x1, w[prefix + "self_attn.q_proj.weight"])).view(n, nh, dh)
+    q = R(rope(q, pos, sin, cos, cfg.rope_pairing))
     if shared_kv is not None:          # not Llama's: a layer that reads the keys and values another one made
         k, v = shared_kv
     else:
-        k = linear(x1, w[prefix + "self_attn.k_proj.weight"]).view(n, nkvh, dh)
-        v = linear(x1, w[prefix + "self_attn.v_proj.weight"]).view(n, nkvh, dh)
-        k = rope(k, pos, sin, cos, cfg.rope_pairing)
+        k = R(linear(x1, w[prefix + "self_attn.k_proj.weight"])).view(n, nkvh, dh)
+        v = R(linear(x1, w[prefix + "self_attn.v_proj.weight"])).view(n, nkvh, dh)
+        k = R(rope(k, pos, sin, cos, cfg.rope_pairing))
     if keep_kv is not None:
         keep_kv.append((k, v))
-    o = attention(q, k, v, dh ** -0.5, first_pos=0, window=cfg.window)
-    return linear(o.reshape(n, nh * dh), w[prefix + "self_attn.o_proj.weight"])
+    o = R(attention(q, k, v, dh ** -0.5, first_pos=0, window=cfg.window, rounding=rounding))
+    return R(linear(o.reshape(n, nh * dh), w[prefix + "self_attn.o_proj.weight"]))
 
 
-def feed_forward(w: Dict[str, torch.Tensor], prefix: str, x2: torch.Tensor) -> torch.Tensor:
+def feed_forward(w: Dict[str, torch.Tensor], prefix: str, x2: torch.Tensor, rounding: Optional[str] = None) -> torch.Tensor:
     """``down(swiglu(gate(x), up(x)))``: llama.cu/src/model/mod.rs:140-154 (gate rows
     first, then up, in the reference's one matrix; here two)."""
-    gate = linear(x2, w[prefix + "mlp.gate_proj.weight"])
-    up = linear(x2, w[prefix + "mlp.up_proj.weight"])
-    return linear(swiglu(gate, up), w[prefix + "mlp.down_proj.weight"])
+    R = lambda t: rounded(t, rounding)
+    gate = R(linear(x2, w[prefix + "mlp.gate_proj.weight"]))
+    up = R(linear(x2, w[prefix + "mlp.up_proj.weight"]))
+    return R(linear(R(swiglu(gate, up)), w[prefix + "mlp.down_proj.weight"]))
 
 
 def forward(cfg: PlainConfig, w: Dict[str, torch.Tensor], tokens: Sequence[int],
-            logits_at: Optional[Sequence[int]] = None) -> torch.Tensor:
+            logits_at: Optional[Sequence[int]] = None, rounding: Optional[str] = None,
+            states: Optional[list] = None) -> torch.Tensor:
     """Logits ``[n, vocab]`` at every position of one whole sequence that starts at 0
     (``logits_at``: at these positions only, ``[len(logits_at), vocab]``: the output selects
     its rows before the final norm, llama.cu/src/exec/output_head.rs:74-78).
@@ -222,6 +241,13 @@ def forward(cfg: PlainConfig, w: Dict[str, torch.Tensor], tokens: Sequence[int],
     the residual is added in the output and down projections: llama.cu/src/op/linear.rs:35-62).
     Output: final norm, then the output matrix, which is the embedding table when the
     file holds none (llama.cu/src/model/mod.rs:83-88,158-168; llama.cu/src/exec/output_head.rs:80-100).
+
+    ``rounding="bfloat16"``: the model of an engine that keeps its activations in bfloat16, as the reference keeps
+    them in float16 (llama.cu/src/model/mod.rs:78: the activations' type is the matrices'): what a norm, a
+    projection, the rotation, the attention and the activation function give is rounded to that type where it is
+    stored, the softmax's weights before they multiply the values; sums inside a product, the residual stream
+    and the logits are not.  ``states``: a list that takes the residual stream ``[n, d]`` before every entry of
+    the run order and after the last.
     """
     n = len(tokens)
     pos = list(range(n))
@@ -234,16 +260,20 @@ def forward(cfg: PlainConfig, w: Dict[str, torch.Tensor], tokens: Sequence[int],
     for entry in order:
         layer, cache_of = entry if isinstance(entry, tuple) else (entry, None)
         p = f"model.layers.{layer}."
-        x1 = rms_norm(x, w[p + "input_layernorm.weight"], cfg.rms_norm_eps)
+        if states is not None:
+            states.append(x.clone())
+        x1 = rounded(rms_norm(x, w[p + "input_layernorm.weight"], cfg.rms_norm_eps), rounding)
         made = []
         x = x + attention_block(cfg, w, p, x1, pos, sin, cos,
-                                shared_kv=kept[cache_of] if cache_of is not None else None, keep_kv=made)
+                                shared_kv=kept[cache_of] if cache_of is not None else None, keep_kv=made, rounding=rounding)
         kept.append(made[0] if cache_of is None else None)
-        x2 = rms_norm(x, w[p + "post_attention_layernorm.weight"], cfg.rms_norm_eps)
-        x = x + feed_forward(w, p, x2)
+        x2 = rounded(rms_norm(x, w[p + "post_attention_layernorm.weight"], cfg.rms_norm_eps), rounding)
+        x = x + feed_forward(w, p, x2, rounding=rounding)
+    if states is not None:
+        states.append(x.clone())
     if logits_at is not None:
         x = x[list(logits_at)]
-    y = rms_norm(x, w["model.norm.weight"], cfg.rms_norm_eps)
+    y = rounded(rms_norm(x, w["model.norm.weight"], cfg.rms_norm_eps), rounding)
     head = w["model.embed_tokens.weight"] if (cfg.tie_word_embeddings or "lm_head.weight" not in w) \
         else w["lm_head.weight"]
     return linear(y, head)

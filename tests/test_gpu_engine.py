@@ -46,7 +46,7 @@ def test_seeded_temperature_sampling_with_portions(folder_b):
     reqs = list(common.random_requests(384, [1, 40, 97, 130], seed=2).values())
     params = SamplingParams(temperature=0.8, seed=1234)
     engine = Engine.from_folder(folder_b, dtype="float32", max_tokens=1024, max_seqs=4, max_batch_tokens=64,
-                                prefill_chunk=48)
+                                prefill_chunk=48, page_size=32)
     got = engine.generate(reqs, params, max_steps=24, ignore_eos=True)
     cfg, w = plain.load_folder(folder_b)
     for rid, (prompt, out) in enumerate(zip(reqs, got)):
@@ -63,7 +63,7 @@ def test_seeded_temperature_sampling_with_portions(folder_b):
                 assert tok in (lo, hi), (rid, len(toks), tok, want)
             toks.append(tok)          # follow the engine's choice
     # the same seed gives the same tokens when the requests run alone (another batch)
-    engine2 = Engine.from_folder(folder_b, dtype="float32", max_tokens=512, max_seqs=1)
+    engine2 = Engine.from_folder(folder_b, dtype="float32", max_tokens=512, max_seqs=1, page_size=16)
     for rid, prompt in enumerate(reqs):
         rid2 = engine2.add_request(prompt, params, 24, req_id=rid, ignore_eos=True)
         out = []
@@ -110,8 +110,8 @@ def test_greedy_generation_in_bfloat16_through_scheduler_and_sampler(name, run_a
     cfg_d = common.TINY[name]
     folder = common.make_folder(cfg_d, seed=31, dtype=torch.bfloat16, std=0.1)
     prompts = list(common.random_requests(cfg_d["vocab_size"], [3, 40, 77, 21, 60], seed=5).values())
-    engine = Engine.from_folder(folder, dtype="bfloat16", max_tokens=224, max_seqs=4, max_batch_tokens=48, prefill_chunk=32,
-                                run_ahead=run_ahead)
+    engine = Engine.from_folder(folder, dtype="bfloat16", max_tokens=256, max_seqs=4, max_batch_tokens=48, prefill_chunk=32,
+                                run_ahead=run_ahead, page_size={"B": 32, "D": 64}[name])
     steps = 40
     got = engine.generate(prompts, max_steps=steps, ignore_eos=True)
     assert engine.sched.preemptions > 0                                # the pool was too small for all of them

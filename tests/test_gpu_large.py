@@ -188,6 +188,60 @@ def test_steps_of_33_to_64_rows_at_full_layer_sizes(big, dtype, monkeypatch):
     common.assert_matches_plain(got, want, dtype, f"8B-sized layers, 33 to 64 rows/{dtype}")
 
 
+_plain_rows = {}
+
+
+def plain_rows_after(prompt, generated):
+    """The plain model's logits at the places where the tokens of ``generated`` were chosen, given the prompt and
+    the tokens chosen before (computed once per sequence: the engines under test mostly agree)."""
+    key = (tuple(prompt), tuple(generated[:-1]))
+    if key not in _plain_rows:
+        pcfg = plain.PlainConfig.from_dict(SHAPE)
+        at = list(range(len(prompt) - 1, len(prompt) - 1 + len(generated)))
+        print(f"plain: {len(prompt) + len(generated) - 1} tokens, logits at {len(at)} positions", flush=True)
+        _plain_rows[key] = plain.forward(pcfg, host_weights(), list(prompt) + list(generated[:-1]), logits_at=at)
+    return _plain_rows[key]
+
+
+@pytest.mark.parametrize("run_ahead", [False, True])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_engine_generates_the_plain_models_tokens_at_full_layer_sizes(dtype, run_ahead):
+    """The whole engine (scheduler, portions of prompts under a token budget, decoding with captured steps whose
+    keys are cut into parts, the arg-max kernel, running ahead with the ids fed on the device, a pool so small that
+    a request loses its pages and is computed again) at the layer sizes of the Llama-3-8B shape: prompts of 30,
+    1,000 and 1,100 tokens, 48 greedy tokens each, so that two contexts pass 1,024 keys while decoding.  Every
+    token is the plain implementation's arg-max given the same tokens before it, or one whose plain logit lies
+    within the type's tolerance of the best."""
+    from llama_cu_amd.engine.engine import Engine
+    rng = np.random.default_rng(12)
+    prompts = [[int(t) for t in rng.integers(SHAPE["vocab_size"], size=n)] for n in (30, 1000, 1100)]
+    steps = 48
+    # at the end the three requests hold 80 + 1,056 + 1,152 tokens' worth of pages: the pool is a little less
+    engine = Engine.from_config(config(), SEED, dtype=dtype, stored="bfloat16", page_size=16, max_tokens=2256, max_seqs=4,
+                                max_batch_tokens=512, prefill_chunk=384, run_ahead=run_ahead)
+    got = engine.generate(prompts, max_steps=steps, ignore_eos=True)
+    assert engine.sched.preemptions >= 1, "the pool was meant to be too small"
+    engine.runner.cache.check()
+    assert engine.runner.cache.free_pages(0) == engine.runner.num_pages
+    replayed = {key: n for key, n in engine.runner.graph_replays.items() if n > 0}
+    print(f"{dtype}, run_ahead={run_ahead}: {engine.steps} steps, {engine.sched.preemptions} preemptions, replays {replayed}", flush=True)
+    if dtype == "bfloat16":
+        assert any(key[1] > 1 for key in replayed), replayed           # decode steps with the keys cut into parts, from a graph
+    exact = total = 0
+    for prompt, out in zip(prompts, got):
+        assert len(out) == steps
+        logits = plain_rows_after(prompt, out)
+        tol = common.REL_TOL[dtype] * float(logits.abs().max())
+        for i, tok in enumerate(out):
+            best = float(logits[i].max())
+            assert float(logits[i][tok]) >= best - tol, \
+                f"token {i} after a prompt of {len(prompt)}: logit {float(logits[i][tok])} against the best {best} (tolerance {tol})"
+            exact += int(tok == int(torch.argmax(logits[i])))
+            total += 1
+    print(f"{dtype}, run_ahead={run_ahead}: {exact} of {total} tokens are the plain arg-max", flush=True)
+    assert exact >= (0.97 if dtype == "float32" else 0.85) * total, (exact, total)
+
+
 def test_captured_steps_of_36_requests_equal_eager_ones(big):
     """36 requests decode together: the steps replayed from a captured graph (the kernel for 33 to
     64 rows and its planes of partial sums inside it) give the bits of eager steps on every replay,

@@ -11,6 +11,8 @@ pytestmark = pytest.mark.gpu
 
 LENGTHS = {"A": [5, 17, 33, 70, 128, 40], "B": [1, 40, 97, 130, 256, 66], "C": [2, 65, 150, 31, 200],
            "D": [40, 100, 128, 70, 33]}
+# tokens per page of the cache: each configuration has its own (A and B the ones their workloads name)
+PAGE = {"A": 16, "B": 32, "C": 48, "D": 64}
 
 
 @pytest.fixture(scope="module")
@@ -34,16 +36,16 @@ TRACES = {"whole": common.trace_whole, "tail": common.trace_tail_decode, "portio
 @pytest.mark.parametrize("mode", ["whole", "tail", "portions", "mixed"])
 def test_replay_matches_plain(models, name, dtype, mode, monkeypatch):
     folder, reqs, want = models[(name, dtype)]
-    steps, max_tokens = TRACES[mode](reqs)
+    steps, max_tokens = TRACES[mode](reqs, page=PAGE[name])
     vocab = common.TINY[name]["vocab_size"]
-    print(f"replay {name} {dtype} {mode}: {len(steps)} steps, max-tokens {max_tokens}", flush=True)
+    print(f"replay {name} {dtype} {mode}: {len(steps)} steps, max-tokens {max_tokens}, pages of {PAGE[name]}", flush=True)
     calls = []
     if name == "D" and dtype == "bfloat16":
         from llama_cu_amd.kernels import ops
         real = ops.gemm_mid
         monkeypatch.setattr(ops, "gemm_mid", lambda *a, **kw: (calls.append(a[0].shape[0]), real(*a, **kw))[1])
     stats = {}
-    outputs = common.run_trace_inprocess(folder, dtype, steps, max_tokens, stats=stats)
+    outputs = common.run_trace_inprocess(folder, dtype, steps, max_tokens, stats=stats, page_size=PAGE[name])
     got = common.collect(steps, outputs, vocab)
     common.assert_matches_plain(got, want, dtype, f"{name}/{dtype}/{mode}")
     if mode == "mixed":
@@ -69,10 +71,10 @@ def test_replay_with_requests_that_lose_their_pages_and_are_computed_again(model
     names it computes all its earlier tokens again beside its new ones, in one batch with the
     other requests.  The logits are those of the plain implementation all the same."""
     folder, reqs, want = models[("B", dtype)]
-    steps, max_tokens = common.trace_mixed(reqs, seed=7, preempt=0.2)
+    steps, max_tokens = common.trace_mixed(reqs, seed=7, preempt=0.2, page=PAGE["B"])
     assert sum(len(s.get("preempt", [])) for s in steps) >= 3
     stats = {}
-    outputs = common.run_trace_inprocess(folder, dtype, steps, max_tokens, stats=stats)
+    outputs = common.run_trace_inprocess(folder, dtype, steps, max_tokens, stats=stats, page_size=PAGE["B"])
     got = common.collect(steps, outputs, common.TINY_B["vocab_size"])
     common.assert_matches_plain(got, want, dtype, f"preempted/{dtype}")
     assert stats["pages_used_again"] > 0
@@ -112,9 +114,9 @@ def test_float32_does_not_depend_on_cutting(models):
     folder, reqs, _ = models[("B", "float32")]
     vocab = common.TINY_B["vocab_size"]
     results = []
-    for mode in ("whole", "tail", "portions", "mixed"):
-        steps, max_tokens = TRACES[mode](reqs)
-        results.append(common.collect(steps, common.run_trace_inprocess(folder, "float32", steps, max_tokens), vocab))
+    for mode, page in (("whole", 32), ("tail", 16), ("portions", 64), ("mixed", 32)):     # nor on the pages' size
+        steps, max_tokens = TRACES[mode](reqs, page=page)
+        results.append(common.collect(steps, common.run_trace_inprocess(folder, "float32", steps, max_tokens, page_size=page), vocab))
     for other in results[1:]:
         for name in reqs:
             for pos in results[0][name]:
@@ -141,12 +143,13 @@ def test_random_configurations_match_plain(seed):
                rms_norm_eps=rng.choice([1e-5, 1e-6, 1e-3]), tie_word_embeddings=rng.random() < 0.5,
                rope_interleaved=rng.random() < 0.3)
     lens = [rng.randrange(1, 150) for _ in range(4)]
+    page = rng.choice([16, 32, 48, 64, 128])
     for dtype, tdt, std in (("float32", torch.float32, 0.15), ("bfloat16", torch.bfloat16, common.BF16_STD)):
         folder = common.make_folder(cfg, seed=seed, dtype=tdt, std=std)
         reqs = common.random_requests(cfg["vocab_size"], lens, seed=seed)
         want = common.plain_logits(folder, reqs)
         for mode in ("whole", "tail", "portions", "mixed"):
-            steps, max_tokens = TRACES[mode](reqs)
-            outputs = common.run_trace_inprocess(folder, dtype, steps, max_tokens)
+            steps, max_tokens = TRACES[mode](reqs, page=page)
+            outputs = common.run_trace_inprocess(folder, dtype, steps, max_tokens, page_size=page)
             got = common.collect(steps, outputs, cfg["vocab_size"])
-            common.assert_matches_plain(got, want, dtype, f"{cfg}/{dtype}/{mode}")
+            common.assert_matches_plain(got, want, dtype, f"{cfg}/pages of {page}/{dtype}/{mode}")

@@ -250,3 +250,32 @@ def test_sampling_frequencies_follow_softmax():
         cnt[plain.sample(l, T, 1.0, 2, float(u))] += 1
     q = p.copy(); q[[1, 2]] = 0; q /= q.sum()
     assert np.abs(cnt / n - q).max() < 0.015
+
+
+def test_rounding_model_rounds_what_is_stored_and_nothing_else():
+    """``forward(..., rounding="bfloat16")``: with weights and activations that bfloat16 holds exactly all the way (a
+    model of zeros and ones: the embedding rows are unit vectors scaled by powers of two, the projections pick
+    coordinates) the rounding changes nothing; with ordinary weights it moves the logits by about 2^-8 of their
+    size, not by 2^-16 (nothing rounded) and not by 2^-4 (something rounded that must not be: the sums of a
+    product, the residual stream)."""
+    cfg = plain.PlainConfig(num_hidden_layers=2, hidden_size=32, num_attention_heads=2, num_key_value_heads=1, head_dim=16,
+                            intermediate_size=48, vocab_size=64, max_position_embeddings=64)
+    w = plain.random_weights(cfg, 3, std=0.2)
+    w = {k: v.to(torch.bfloat16).float() for k, v in w.items()}
+    toks = [3, 9, 27, 1, 60, 33, 7]
+    a = plain.forward(cfg, w, toks)
+    b = plain.forward(cfg, w, toks, rounding="bfloat16")
+    rel = float((a - b).abs().max() / a.abs().max())
+    assert 2.0 ** -12 < rel < 2.0 ** -5, rel
+    # the residual stream is not rounded: a stream that bfloat16 cannot hold (1 + 2^-12) survives a layer whose
+    # branches give zero
+    for k in w:
+        if "o_proj" in k or "down_proj" in k:
+            w[k] = torch.zeros_like(w[k])
+    w["model.embed_tokens.weight"] = torch.full_like(w["model.embed_tokens.weight"], 1.0 + 2.0 ** -12)
+    w["model.embed_tokens.weight"][:, 0] = 3.0
+    st = []
+    plain.forward(cfg, w, toks, rounding="bfloat16", states=st)
+    assert len(st) == cfg.num_hidden_layers + 1
+    assert all(torch.equal(s, st[0]) for s in st) and float(st[-1][0, 1]) == 1.0 + 2.0 ** -12
+    assert float(plain.rounded(st[-1], "bfloat16")[0, 1]) == 1.0
