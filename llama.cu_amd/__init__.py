@@ -15,6 +15,20 @@ import os
 _engines: dict = {}
 
 
+def _folder_stamp(folder: str):
+    """Sizes and modification times of the folder's configuration and weight files: a folder that was written
+    again is another model."""
+    stamp = []
+    try:
+        for name in sorted(os.listdir(folder)):
+            if name == "config.json" or name.endswith(".safetensors") or name.endswith(".safetensors.index.json"):
+                st = os.stat(os.path.join(folder, name))
+                stamp.append((name, st.st_size, st.st_mtime_ns))
+    except OSError:
+        pass
+    return tuple(stamp)
+
+
 def Engine(model: str, dtype: str = "bfloat16", device: str = "cuda:0", **kw):
     """The engine for the model folder ``model`` (see engine.engine.Engine)."""
     from .engine.engine import Engine as _Engine
@@ -27,9 +41,11 @@ def generate(model: str, prompts, sampling: SamplingParams = SamplingParams(), m
     encodes) with the model of the folder ``model``; returns token ids, or strings for
     string prompts."""
     from . import text
-    key = (os.path.abspath(model), dtype, str(device), tuple(sorted(kw.items())))
+    # a model is loaded once per process, folder as it is on the disk (its files' sizes and times) and set of
+    # options; the engine is idle between calls, and a call's draws do not depend on the calls before it
+    key = (os.path.abspath(model), _folder_stamp(model), dtype, str(device), repr(sorted(kw.items())))
     engine = _engines.get(key)
-    if engine is None:                       # a model is loaded once per process and set of options
+    if engine is None:
         _engines.clear()
         engine = _engines[key] = Engine(model, dtype=dtype, device=device, **kw)
     as_text = len(prompts) > 0 and isinstance(prompts[0], str)

@@ -28,6 +28,8 @@ class CacheGroup:
     num_pages: int
     page_size: int
     window: int = 0      # 0: all tokens are kept
+    slack: int = 0       # a window gives a page back only when a request cut back by up to this many tokens would not
+                         # see it either (1 for an engine that runs one round ahead of its sampler's results)
 
 
 _STATUS = {1: "not enough free pages", 2: "no free state slot", -1: "unknown request", -2: "request exists already",
@@ -55,16 +57,17 @@ def _ints(values: Sequence[int]):
 
 class CacheManager:
     def __init__(self, groups: Sequence[CacheGroup], n_slots: int, can_truncate: bool = True):
-        """``can_truncate``: whether all that the model keeps for a request can be cut back to a
-        shorter length (pages can, a state of fixed size cannot); if not, ``truncate`` to less than
-        a request holds raises."""
+        """``can_truncate``: whether the state of fixed size that the model keeps for a request (if any) can be
+        cut back to a shorter length; if not, ``truncate`` to less than a request holds raises, and
+        ``truncate_or_reset`` sets the request to length 0 with its pages kept."""
         self.groups = list(groups)
         self.can_truncate = bool(can_truncate)
         self.n_slots = int(n_slots)
         self._lib = _lib()
         self._h = ctypes.c_void_p(self._lib.lcu_cache_create(
             len(self.groups), _ints([g.num_pages for g in self.groups]), _ints([g.page_size for g in self.groups]),
-            _ints([g.window for g in self.groups]), self.n_slots, int(self.can_truncate)))
+            _ints([g.window for g in self.groups]), _ints([g.slack for g in self.groups]), self.n_slots,
+            int(self.can_truncate)))
         if not self._h:
             raise CacheError("cache manager: bad group description")
 
@@ -106,6 +109,16 @@ class CacheManager:
         st = self._lib.lcu_cache_truncate(self._h, ctypes.c_longlong(req), int(new_len))
         if st:
             self._raise(st, f"truncate request {req} to {new_len}")
+
+    def truncate_or_reset(self, req: int, new_len: int) -> bool:
+        """``truncate`` where everything the request holds can be cut back (True).  Where something cannot (a state
+        of fixed size, a window that has given back a page the shorter request would see), only that is given up:
+        the request's length becomes 0, groups without a window keep their pages up to ``new_len``, and the request
+        is to be computed again from its first token (False)."""
+        st = self._lib.lcu_cache_truncate_or_reset(self._h, ctypes.c_longlong(req), int(new_len))
+        if st not in (0, 3):
+            self._raise(st, f"cut request {req} back to {new_len}")
+        return st == 0
 
     def release(self, req: int) -> None:
         st = self._lib.lcu_cache_release(self._h, ctypes.c_longlong(req))

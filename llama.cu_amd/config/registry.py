@@ -10,7 +10,7 @@ from __future__ import annotations
 import importlib
 import os
 from dataclasses import dataclass
-from typing import Any, Callable, Dict, Iterable, List
+from typing import Any, Callable, Dict, Iterable, List, Tuple
 
 from .base import ConfigError, read_config_json
 
@@ -20,15 +20,20 @@ class Architecture:
     name: str
     config_from_dict: Callable[[Dict[str, Any]], Any]   # dict of config.json -> typed configuration
     build_spec: Callable[[Any], Any]                    # typed configuration -> parts.ModelSpec
+    ignored_tensors: Tuple[str, ...] = ()               # regular expressions: tensors that this architecture's files may
+                                                        # carry beside the weights, which the loader passes over
 
 
 _REGISTRY: Dict[str, Architecture] = {}
 
 
-def register_architecture(name: str, config_from_dict, build_spec, replace: bool = False) -> None:
+def register_architecture(name: str, config_from_dict, build_spec, replace: bool = False,
+                          ignored_tensors: Iterable[str] = ()) -> None:
+    """``ignored_tensors``: regular expressions (matched from a tensor name's start) for tensors that files of this
+    architecture may hold and that are no weights; every other tensor that the model does not expect is an error."""
     if name in _REGISTRY and not replace:
         raise ValueError(f"architecture {name!r} is already registered")
-    _REGISTRY[name] = Architecture(name, config_from_dict, build_spec)
+    _REGISTRY[name] = Architecture(name, config_from_dict, build_spec, tuple(ignored_tensors))
 
 
 def registered_architectures() -> List[str]:

@@ -11,12 +11,12 @@ using namespace lcu;
 
 #define API extern "C" __attribute__((visibility("default")))
 
-API void *lcu_cache_create(int n_groups, const int *num_pages, const int *page_size, const int *window, int n_slots,
-                           int can_truncate) {
+API void *lcu_cache_create(int n_groups, const int *num_pages, const int *page_size, const int *window, const int *slack,
+                           int n_slots, int can_truncate) {
     std::vector<GroupDesc> g;
     for (int i = 0; i < n_groups; ++i) {
-        if (num_pages[i] < 0 || page_size[i] <= 0 || window[i] < 0) return nullptr;
-        g.push_back({num_pages[i], page_size[i], window[i]});
+        if (num_pages[i] < 0 || page_size[i] <= 0 || window[i] < 0 || slack[i] < 0) return nullptr;
+        g.push_back({num_pages[i], page_size[i], window[i], slack[i]});
     }
     if (n_slots < 0) return nullptr;
     return new CacheManager(g, n_slots, can_truncate != 0);
@@ -26,6 +26,7 @@ API int lcu_cache_add(void *h, long long id) { return ((CacheManager *)h)->add(i
 API int lcu_cache_reserve(void *h, long long id, int new_len) { return ((CacheManager *)h)->reserve(id, new_len); }
 API int lcu_cache_commit(void *h, long long id) { return ((CacheManager *)h)->commit(id); }
 API int lcu_cache_truncate(void *h, long long id, int new_len) { return ((CacheManager *)h)->truncate(id, new_len); }
+API int lcu_cache_truncate_or_reset(void *h, long long id, int new_len) { return ((CacheManager *)h)->truncate_or_reset(id, new_len); }
 API int lcu_cache_release(void *h, long long id) { return ((CacheManager *)h)->release(id); }
 API int lcu_cache_has(void *h, long long id) { return ((CacheManager *)h)->has(id) ? 1 : 0; }
 API int lcu_cache_len(void *h, long long id) {

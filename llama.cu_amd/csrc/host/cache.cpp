@@ -87,11 +87,11 @@ int CacheManager::commit(int64_t id) {
     RequestCache &rc = it->second;
     rc.len = rc.reserved;
     // A window has passed a page when the next query (at position len) cannot see any of its
-    // tokens: the first key it sees is len - window + 1.
+    // tokens: the first key it sees is len - window + 1 (with slack: the query at len - slack).
     for (size_t g = 0; g < groups_.size(); ++g) {
         const int w = groups_[g].window;
         if (w <= 0) continue;
-        const int first_key = rc.len - w + 1;
+        const int first_key = rc.len - groups_[g].slack - w + 1;
         if (first_key <= 0) continue;
         const int first_page = first_key / groups_[g].page_size;
         auto &tab = rc.tables[g];
@@ -130,6 +130,25 @@ int CacheManager::truncate(int64_t id, int new_len) {
     }
     rc.len = rc.reserved = new_len;
     return CACHE_OK;
+}
+
+int CacheManager::truncate_or_reset(int64_t id, int new_len) {
+    const int st = truncate(id, new_len);
+    if (st != CACHE_CANNOT_TRUNCATE && st != CACHE_WINDOW_PASSED) return st;
+    RequestCache &rc = reqs_.at(id);
+    int reserved = new_len;
+    for (size_t g = 0; g < groups_.size(); ++g) {
+        auto &tab = rc.tables[g];
+        const int keep = groups_[g].window > 0 ? 0 : pages_for(new_len, groups_[g].page_size);
+        while ((int)tab.size() > keep) {
+            if (tab.back() >= 0 && !pools_[g].give(tab.back())) return CACHE_CORRUPT;
+            tab.pop_back();
+        }
+        reserved = std::min(reserved, (int)tab.size() * groups_[g].page_size);
+    }
+    rc.len = 0;
+    rc.reserved = reserved;
+    return CACHE_RESET;
 }
 
 int CacheManager::release(int64_t id) {

@@ -20,6 +20,9 @@ struct GroupDesc {
     int num_pages;   // pages in this group's pool
     int page_size;   // tokens per page
     int window;      // 0: all tokens are kept; w > 0: a token sees the last w tokens, itself included
+    int slack = 0;   // a window gives a page back only when a request cut back by up to this many tokens
+                     // would not see it either (an engine that runs one round ahead of its sampler's
+                     // results cuts a request back by the one token it computed beyond its end)
 };
 
 class PagePool {
@@ -47,6 +50,7 @@ enum CacheStatus {
     CACHE_OK = 0,
     CACHE_NO_PAGES = 1,       // not enough free pages: nothing was changed
     CACHE_NO_SLOT = 2,        // all state slots are taken
+    CACHE_RESET = 3,          // truncate_or_reset: the request was not cut back but set to length 0
     CACHE_UNKNOWN_REQUEST = -1,
     CACHE_DUPLICATE_REQUEST = -2,
     CACHE_BAD_ARGUMENT = -3,
@@ -66,6 +70,15 @@ class CacheManager {
     int reserve(int64_t id, int new_len);      // pages for tokens [len, new_len) in every group, all or nothing
     int commit(int64_t id);                    // the reserved tokens are written; windows slide
     int truncate(int64_t id, int new_len);     // forget the tokens at and after new_len, give tail pages back
+    // truncate where everything the request holds can be cut back to new_len.  Where something cannot (a
+    // state of fixed size; a window that has given back a page that the shorter request would see), the
+    // request has to be computed again from its first token, and only what cannot be cut is given up:
+    // the request's length becomes 0, every group without a window keeps its pages up to new_len (the
+    // recomputation writes the same keys and values into them and asks the pool for nothing), a group
+    // with a window gives its pages back (their place in the table depends on where the window stood),
+    // the slot stays (its owner starts the state anew at position 0).  CACHE_OK: cut back; CACHE_RESET:
+    // set to 0; anything else: an error, nothing changed.
+    int truncate_or_reset(int64_t id, int new_len);
     int release(int64_t id);                   // give everything back
     bool has(int64_t id) const { return reqs_.count(id) != 0; }
     const RequestCache *get(int64_t id) const;

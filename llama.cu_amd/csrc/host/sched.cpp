@@ -28,7 +28,7 @@ int Scheduler::extend(int64_t id, const int *tokens, int n, int max_new) {
     r.max_new = max_new;
     r.generated = 0;
     r.reason = NOT_FINISHED;
-    if (!cache_->has(id)) r.computed = 0;       // the cache was not kept (or was taken away)
+    if (!cache_->has(id) || cache_->get(id)->len < r.computed) r.computed = 0;       // the cache was not kept (or was taken away)
     waiting_.push_back(id);
     return CACHE_OK;
 }
@@ -223,13 +223,18 @@ int Scheduler::finish_now(int64_t id, int reason, int n_tokens) {
         r.tokens.resize(n_tokens);
         if (r.computed > n_tokens - 1) {
             r.computed = n_tokens - 1;
-            if (cache_->has(id) && cache_->get(id)->len > r.computed && cache_->truncate(id, r.computed) != CACHE_OK) {
-                // What was computed beyond the end cannot be taken back: a window has given back a page
-                // that the shorter request would still see, or the model keeps a state that has folded
-                // the tokens in.  The request loses its cache; if it goes on (a kept request's next
-                // turn), it is computed again from its tokens.
-                cache_->release(id);
-                r.computed = 0;
+            if (cache_->has(id) && cache_->get(id)->len > r.computed) {
+                // What was computed beyond the end may not be there to take back: a window has given back a
+                // page that the shorter request would still see, or the model keeps a state that has folded
+                // the tokens in.  Then the request gives up what cannot be cut (its other pages stay its
+                // own) and, if it goes on (a kept request's next turn), is computed again from its tokens.
+                const int st = cache_->truncate_or_reset(id, r.computed);
+                if (st == CACHE_RESET) {
+                    r.computed = 0;
+                } else if (st != CACHE_OK) {
+                    cache_->release(id);
+                    r.computed = 0;
+                }
             }
         }
     }

@@ -78,7 +78,8 @@ class Scheduler {
     // the request had ended when that token was appended.  A request that ended by count at the
     // same token takes the new reason.  Where the cache cannot be cut back (a window has passed a
     // page that the shorter request would see, or the model keeps a state of fixed size), the
-    // request's cache is given back instead and a later turn computes it again from its tokens.
+    // request gives up what cannot be cut (CacheManager::truncate_or_reset) and a later turn
+    // computes it again from its tokens.
     int finish_now(int64_t id, int reason, int n_tokens);
 
     const SchedRequest *get(int64_t id) const;

@@ -466,15 +466,25 @@ static int launch_decode(const void *q, int q_stride, void *out, int out_stride,
 // if req_list is null) feed exactly one token each.
 // part_o: [n_req * nh * n_splits * dh] floats, part_ml: [n_req * nh * n_splits * 2] (unused
 // when n_splits == 1).  bfloat16 only; head_dim 32, 64, 96 or 128; page_size a multiple of 16.
+// What both decode entry points ask of their sizes (the parts' memory apart): LCU_OK or why not.
+static int decode_arguments(int q_stride, int out_stride, int max_pages, int nh, int nkvh, int dh, int page, int window,
+                            int n_splits) {
+    if (nh <= 0 || nkvh <= 0 || nh % nkvh || dh <= 0 || page <= 0 || page % 16 || max_pages <= 0 || window < 0 || n_splits < 1 ||
+        n_splits > 65535 || q_stride % 8 || out_stride % 4)
+        return LCU_BAD_ARGUMENT;
+    if (dh != 32 && dh != 64 && dh != 96 && dh != 128) return LCU_UNSUPPORTED;
+    if ((unsigned long long)kv_page_elems(nkvh, dh, page) * 2ull >= (1ull << 31)) return LCU_UNSUPPORTED;
+    return LCU_OK;
+}
+
 LCU_API int lcu_attention_decode_bf16(const void *q, int q_stride, void *out, int out_stride, const void *cache,
                                       const int *block_table, int max_pages, const int *q_start, const int *ctx_len,
                                       const int *req_list, int n_req, int nh, int nkvh, int dh, int page, float scale,
                                       int window, int n_splits, float *part_o, float *part_ml, hipStream_t stream) {
     if (n_req <= 0) return LCU_OK;
-    if (nh > 0 && nkvh > 0 && page > 0 && (unsigned long long)kv_page_elems(nkvh, dh, page) * 2ull >= (1ull << 31)) return LCU_UNSUPPORTED;
-    if (nh <= 0 || nkvh <= 0 || nh % nkvh || page <= 0 || page % 16 || max_pages <= 0 || window < 0 || n_splits < 1 ||
-        n_splits > 65535 || (n_splits > 1 && (!part_o || !part_ml)) || q_stride % 8 || out_stride % 4)
-        return LCU_BAD_ARGUMENT;
+    const int args = decode_arguments(q_stride, out_stride, max_pages, nh, nkvh, dh, page, window, n_splits);
+    if (args != LCU_OK) return args;
+    if (n_splits > 1 && (!part_o || !part_ml)) return LCU_BAD_ARGUMENT;
 #define GO(D) return launch_decode<D>(q, q_stride, out, out_stride, cache, block_table, max_pages, q_start, ctx_len, req_list, n_req, nh, nkvh, page, scale, window, n_splits, part_o, part_ml, stream)
     if (dh == 128) GO(128);
     if (dh == 64) GO(64);
@@ -494,18 +504,16 @@ constexpr int STATIC_MAX_DEVICES = 64;
 static void *scratch_on_device[STATIC_MAX_DEVICES];     // per device: each holds its own copy at its own address
 static std::mutex scratch_lock;
 
-// The buffer's address on the current device, looked up at the first call there.
+// The buffer's address on the current device, looked up at the first call there.  LCU_OK, LCU_UNSUPPORTED
+// (a device number beyond the table) or LCU_RUNTIME_ERROR (the runtime refused the look-up).
 static int static_scratch(void **ptr) {
     int dev = -1;
-    hipError_t e = hipGetDevice(&dev);
-    if (e != hipSuccess) return (int)e;
+    if (hipGetDevice(&dev) != hipSuccess) return LCU_RUNTIME_ERROR;
     if (dev < 0 || dev >= STATIC_MAX_DEVICES) return LCU_UNSUPPORTED;
     std::lock_guard<std::mutex> guard(scratch_lock);
     if (!scratch_on_device[dev]) {
         void *p = nullptr;
-        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
-        if (e != hipSuccess) return (int)e;
-        if (!p) return LCU_UNSUPPORTED;
+        if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) return LCU_RUNTIME_ERROR;
         scratch_on_device[dev] = p;
     }
     *ptr = scratch_on_device[dev];
@@ -521,7 +529,9 @@ LCU_API long long lcu_attention_static_scratch_bytes(void) { return (long long)L
 
 LCU_API long long lcu_attention_static_scratch_needed(int n_req, int nh, int dh, int n_splits) {
     if (n_req <= 0 || nh <= 0 || dh <= 0 || n_splits <= 1) return 0;
-    return (long long)n_req * nh * n_splits * (dh + 2) * (long long)sizeof(float);
+    // sizes so large that the product leaves 63 bits need more than any buffer: the largest number says so
+    const unsigned __int128 bytes = (unsigned __int128)n_req * (unsigned)nh * (unsigned)n_splits * (unsigned)(dh + 2) * sizeof(float);
+    return bytes > (unsigned __int128)0x7fffffffffffffffll ? 0x7fffffffffffffffll : (long long)bytes;
 }
 
 LCU_API int lcu_attention_decode_bf16_static(const void *q, int q_stride, void *out, int out_stride, const void *cache,
@@ -529,9 +539,12 @@ LCU_API int lcu_attention_decode_bf16_static(const void *q, int q_stride, void *
                                              const int *req_list, int n_req, int nh, int nkvh, int dh, int page, float scale,
                                              int window, int n_splits, hipStream_t stream) {
     if (n_req <= 0) return LCU_OK;
+    // the arguments first, as the other entry point checks them: a call with bad sizes is told so, whatever
+    // buffer it would need
+    const int args = decode_arguments(q_stride, out_stride, max_pages, nh, nkvh, dh, page, window, n_splits);
+    if (args != LCU_OK) return args;
     float *part_o = nullptr, *part_ml = nullptr;
     if (n_splits > 1) {
-        if (nh <= 0 || dh <= 0 || dh % 4) return LCU_BAD_ARGUMENT;
         if (lcu_attention_static_scratch_needed(n_req, nh, dh, n_splits) > (long long)LCU_ATTENTION_STATIC_SCRATCH_BYTES)
             return LCU_SCRATCH_EXCEEDED;
         void *base = nullptr;
@@ -1033,12 +1046,19 @@ static int launch_prefill_as(const void *q, int q_stride, void *out, int out_str
     if (n_wg > 0x7fffffffll) return LCU_BAD_ARGUMENT;
     dim3 grid((unsigned)n_wg), block(PRE_THREADS);
     constexpr size_t lds_bytes = (size_t)PRE_RING * 8 * DH * sizeof(u32x4);
-    static bool allowed = false;                   // more than 64 KB of LDS must be asked for once
-    if (!allowed) {
-        const hipError_t e = hipFuncSetAttribute((const void *)attention_prefill_kernel<DH, PAGE16, FLAT>,
-                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
-        if (e != hipSuccess) return (int)e;
-        allowed = true;
+    // more than 64 KB of LDS must be asked for once, on every device that runs the kernel
+    static std::mutex lock;
+    static bool allowed[STATIC_MAX_DEVICES] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= STATIC_MAX_DEVICES) return LCU_RUNTIME_ERROR;
+    {
+        std::lock_guard<std::mutex> guard(lock);
+        if (!allowed[dev]) {
+            const hipError_t e = hipFuncSetAttribute((const void *)attention_prefill_kernel<DH, PAGE16, FLAT>,
+                                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+            if (e != hipSuccess) return (int)e;
+            allowed[dev] = true;
+        }
     }
     attention_prefill_kernel<DH, PAGE16, FLAT><<<grid, block, lds_bytes, stream>>>(
         (const bf16_t *)q, q_stride, (bf16_t *)out, out_stride, (const bf16_t *)cache, cache_bytes, block_table, max_pages, q_start,

@@ -21,15 +21,18 @@
 //     current) by lcu_attention_static_init or by the entry point's first call on the device; call
 //     lcu_attention_static_init beforehand where even that look-up is unwelcome (before a capture).
 //
-// All other arguments are those of lcu_attention_decode_bf16.
+// All other arguments are those of lcu_attention_decode_bf16, and they are checked as there (and first: a call
+// with sizes that no kernel takes gets LCU_BAD_ARGUMENT or LCU_UNSUPPORTED, not LCU_SCRATCH_EXCEEDED).
 #pragma once
 #include <hip/hip_runtime.h>
 
 #define LCU_ATTENTION_STATIC_SCRATCH_BYTES (16u << 20)
 #define LCU_SCRATCH_EXCEEDED (-3)
+#define LCU_RUNTIME_ERROR (-4)      // the HIP runtime refused a call that is no launch (the buffer's address, the device)
 
 extern "C" {
-// Looks the buffer's address up for the current device; 0, or a HIP error code.
+// Looks the buffer's address up for the current device; 0, LCU_UNSUPPORTED (-2: a device number of 64 or more)
+// or LCU_RUNTIME_ERROR.
 int lcu_attention_static_init(void);
 // The size of the buffer in bytes.
 long long lcu_attention_static_scratch_bytes(void);

@@ -37,6 +37,7 @@ class _Request:
     params: SamplingParams
     prompt_len: int
     ignore_eos: bool = False
+    draw_id: int = 0                  # what its random draws are keyed by beside the seed (default: its id)
     unknown: Optional[int] = None     # index of a token that is sampled but not read yet
     done: bool = False                # its end has been reported (or it was aborted)
     turn: int = 0                     # counts continuations: a row of an earlier turn is stale
@@ -84,9 +85,12 @@ class Engine:
 
     # ---------------------------------------------------------------- requests
     def add_request(self, tokens: Sequence[int], params: SamplingParams = GREEDY, max_steps: int = 1000,
-                    req_id: Optional[int] = None, keep: bool = False, ignore_eos: bool = False) -> int:
+                    req_id: Optional[int] = None, keep: bool = False, ignore_eos: bool = False,
+                    draw_id: Optional[int] = None) -> int:
         """A new request; ``max_steps`` is the number of tokens to generate, the first
-        included (llama.cu/src/exec/engine_manager.rs:118-122)."""
+        included (llama.cu/src/exec/engine_manager.rs:118-122).  A random draw is a function of
+        (the parameters' seed, ``draw_id``, the index of the drawn token); ``draw_id`` is the
+        request's id unless given."""
         tokens = [int(t) for t in tokens]
         if not tokens:
             raise ValueError("a request needs at least one prompt token")
@@ -97,7 +101,7 @@ class Engine:
         rid = self._next_id if req_id is None else int(req_id)
         self._next_id = max(self._next_id, rid + 1)
         self.sched.add(rid, tokens, max_steps, keep)
-        self.requests[rid] = _Request(tokens, params, len(tokens), ignore_eos)
+        self.requests[rid] = _Request(tokens, params, len(tokens), ignore_eos, draw_id=rid if draw_id is None else int(draw_id))
         return rid
 
     def continue_request(self, rid: int, tokens: Sequence[int], max_steps: int = 1000) -> None:
@@ -175,7 +179,7 @@ class Engine:
         if not rows:
             return None
         params = [self.requests[e.req].params for e in rows]
-        keys = [(e.req, len(self.requests[e.req].tokens)) for e in rows]
+        keys = [(self.requests[e.req].draw_id, len(self.requests[e.req].tokens)) for e in rows]
         sampled = self.sampler.sample_device(logits, params, keys)
         host = torch.empty(len(rows), dtype=torch.int32, pin_memory=True)
         host.copy_(sampled, non_blocking=True)
@@ -236,7 +240,7 @@ class Engine:
             rows = [e for e in plan if e.want_logits]
             if rows:
                 params = [self.requests[e.req].params for e in rows]
-                keys = [(e.req, len(self.requests[e.req].tokens)) for e in rows]
+                keys = [(self.requests[e.req].draw_id, len(self.requests[e.req].tokens)) for e in rows]
                 sampled = self.sampler.sample(logits, params, keys)
                 for e, tok in zip(rows, sampled):
                     r = self.requests[e.req]
@@ -254,24 +258,40 @@ class Engine:
                  max_steps: int = 1000, ignore_eos: bool = False,
                  on_token: Optional[Callable[[int, int], None]] = None) -> List[List[int]]:
         """Generate for every prompt (lists of token ids); returns the generated tokens of
-        each, an end-of-sequence token included if one ended it."""
+        each, an end-of-sequence token included if one ended it.  The random draws of prompt ``i``
+        are keyed by ``i``: the same call gives the same tokens however many requests the engine
+        has served before.  If it raises, its requests are taken out of the engine again."""
         plist = [params] * len(prompts) if isinstance(params, SamplingParams) else list(params)
-        ids = [self.add_request(p, sp, max_steps, ignore_eos=ignore_eos) for p, sp in zip(prompts, plist)]
-        out: Dict[int, List[int]] = {i: [] for i in ids}
-        live = set(ids)
-        while live:
-            results = self.step()
-            if not results and self.idle:
-                break
-            for o in results:
-                if o.req not in out:
-                    continue
-                if o.token is not None:
-                    out[o.req].append(o.token)
-                    if on_token:
-                        on_token(ids.index(o.req), o.token)
-                if o.finished:
-                    live.discard(o.req)
+        if len(plist) != len(prompts):
+            raise ValueError(f"{len(prompts)} prompts but {len(plist)} sets of sampling parameters")
+        ids: List[int] = []
+        try:
+            for i, (p, sp) in enumerate(zip(prompts, plist)):
+                ids.append(self.add_request(p, sp, max_steps, ignore_eos=ignore_eos, draw_id=i))
+            out: Dict[int, List[int]] = {i: [] for i in ids}
+            live = set(ids)
+            while live:
+                results = self.step()
+                if not results and self.idle:
+                    break
+                for o in results:
+                    if o.req not in out:
+                        continue
+                    if o.token is not None:
+                        out[o.req].append(o.token)
+                        if on_token:
+                            on_token(ids.index(o.req), o.token)
+                    if o.finished:
+                        live.discard(o.req)
+        except BaseException:
+            # what this call put into the engine goes out again: the engine may serve other calls
+            for i in ids:
+                try:
+                    self.abort(i)
+                    self.drop(i)
+                except Exception:
+                    pass
+            raise
         for i in ids:
             self.drop(i)
         return [out[i] for i in ids]

@@ -17,6 +17,7 @@ import torch
 
 from ..cache import CacheGroup, CacheManager, OutOfPages
 from ..config import load_config
+from ..kernels import ops
 from ..parts import BuildContext, CacheNeed, DecoderModel, LayerCache, ModelSpec
 from ..weights import load_weights, open_safetensors, random_tensors
 from ..weights.loader import convert
@@ -99,6 +100,7 @@ class ModelRunner:
         self.max_model_len = min(int(max_model_len or spec.max_positions), spec.max_positions)
         self.max_seqs, self.max_batch_tokens = int(max_seqs), int(max_batch_tokens)
         torch.cuda.set_device(self.device)
+        ops.tune_for(self.device)
         self.model = DecoderModel(spec)
         if pack_weights is None:
             # the second, packed copy of the matrices is worth its memory only while most of the
@@ -133,8 +135,11 @@ class ModelRunner:
             tokens = max(self.page_size, min(by_memory, by_need))
         # every pool holds the same number of tokens, in pages of its own size
         self.num_pages = (tokens + self.page_size - 1) // self.page_size
-        self.groups = [CacheGroup((tokens + ps - 1) // ps, ps, p[0]) for p, ps in zip(pools, page_of)]
-        # a request's cache can be cut back to a shorter length only if every need's can
+        # a window keeps its pages one token longer than the next query needs: the engine runs one round ahead of
+        # its sampler's results and cuts a request back by the token it computed beyond an end of sequence
+        self.groups = [CacheGroup((tokens + ps - 1) // ps, ps, p[0], slack=1 if p[0] else 0) for p, ps in zip(pools, page_of)]
+        # whether every need's state of fixed size can be cut back to a shorter length (the manager knows what its
+        # pages and windows can); a request that cannot be cut back gives up what cannot and is computed again
         self.can_truncate = all(n.can_truncate for n in needs if n is not None)
         self.cache = CacheManager(self.groups, self.max_seqs, can_truncate=self.can_truncate)
         self.caches: List[LayerCache] = []
@@ -176,7 +181,8 @@ class ModelRunner:
                                                       kw.get("max_tokens"), kw.get("num_pages"), int(kw.get("max_seqs", 8)),
                                                       int(kw.get("max_batch_tokens", 2048)), float(kw.get("kv_fraction", 0.85))))
         tensors = load_weights(files, model.tensors(), DTYPES[dtype], device, groups=model.fused_groups(DTYPES[dtype], device),
-                               log=lambda line: print(f"[llama.cu_amd] {line}", file=sys.stderr, flush=True))
+                               log=lambda line: print(f"[llama.cu_amd] {line}", file=sys.stderr, flush=True),
+                               ignored=arch.ignored_tensors)
         runner = cls(spec, tensors, dtype, device, **kw)
         runner.config = cfg
         return runner

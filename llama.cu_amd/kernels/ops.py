@@ -13,7 +13,7 @@ from typing import Optional
 import torch
 
 from . import build
-from .tuning import TUNING, Tuning  # noqa: F401  (ops.TUNING may be replaced to try other numbers)
+from .tuning import TUNING, Tuning, for_device  # noqa: F401  (ops.TUNING may be replaced to try other numbers)
 
 F32, BF16 = 0, 1
 _TYPE = {torch.float32: F32, torch.bfloat16: BF16}
@@ -21,6 +21,23 @@ _TYPE = {torch.float32: F32, torch.bfloat16: BF16}
 
 class KernelError(RuntimeError):
     pass
+
+
+def tune_for(device) -> None:
+    """Put the facts of the card at ``device`` (its number of compute units) into ``TUNING``."""
+    global TUNING
+    TUNING = for_device(TUNING, device)
+
+
+_said: set = set()
+
+
+def say_once(line: str) -> None:
+    """A line for the log (standard error), once per process however often the same thing happens."""
+    if line not in _said:
+        _said.add(line)
+        import sys
+        print(f"[llama.cu_amd] {line}", file=sys.stderr, flush=True)
 
 
 def _type(t: torch.Tensor, what: str) -> int:
@@ -105,6 +122,10 @@ def _check(rc: int, name: str) -> None:
         raise KernelError(f"{name}: the kernel refused its arguments (unsupported size or shape)")
     if rc == -2:
         raise KernelError(f"{name}: unsupported configuration")
+    if rc == -3:
+        raise KernelError(f"{name}: the call needs more scratch memory than the library's fixed buffer holds")
+    if rc == -4:
+        raise KernelError(f"{name}: the HIP runtime refused a call that is no launch (device or symbol look-up)")
     raise KernelError(f"{name}: launch failed with HIP error {rc}")
 
 
@@ -336,13 +357,25 @@ def gemm_nt(a: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = None
     return out
 
 
-def mfma_attention_supported(q: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: int, page_size: int) -> bool:
-    """Whether the matrix-core attention kernels take this shape (the generic kernel takes
-    the rest): bfloat16, head_dim 32, 64, 96 or 128, pages of a multiple of 16 tokens, groups of
-    at most 16 heads or of a multiple of 16."""
+def mfma_attention_refusal(dtype: torch.dtype, n_heads: int, n_kv_heads: int, head_dim: int, page_size: int) -> Optional[str]:
+    """None if the matrix-core attention kernels take this shape, else why not (the generic kernel, one wave per
+    token and head with plain multiply-adds, takes the rest): bfloat16, head_dim 32, 64, 96 or 128, pages of a
+    multiple of 16 tokens, groups of at most 16 heads or of a multiple of 16."""
     g = n_heads // n_kv_heads
-    return (q.dtype == torch.bfloat16 and head_dim in (32, 64, 96, 128) and page_size % 16 == 0 and (g <= 16 or g % 16 == 0)
-            and q.stride(0) % 8 == 0)
+    if dtype != torch.bfloat16:
+        return f"the type is {dtype}, not bfloat16"
+    if head_dim not in (32, 64, 96, 128):
+        return f"the head size is {head_dim}, not 32, 64, 96 or 128"
+    if page_size % 16:
+        return f"a page holds {page_size} tokens, no multiple of 16"
+    if not (g <= 16 or g % 16 == 0):
+        return f"{g} heads share a key/value head: more than 16 and no multiple of 16"
+    return None
+
+
+def mfma_attention_supported(q: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: int, page_size: int) -> bool:
+    """Whether the matrix-core attention kernels take these queries (``mfma_attention_refusal`` says why not)."""
+    return mfma_attention_refusal(q.dtype, n_heads, n_kv_heads, head_dim, page_size) is None and q.stride(0) % 8 == 0
 
 
 def attention_decode(q, out, cache, block_table, q_start, ctx_len, n_req, n_heads, n_kv_heads, head_dim, page_size,
@@ -364,19 +397,23 @@ def attention_decode(q, out, cache, block_table, q_start, ctx_len, n_req, n_head
     return out
 
 
-def prefill_tasks(q_lens, ctx_lens, tokens_per_task: int, device, skip_single: bool = False, per_wg: int = 1):
+def prefill_tasks(q_lens, ctx_lens, tokens_per_task: int, device, skip_single: bool = False, per_wg: int = 1,
+                  window: int = 0):
     """Cut the batch into the prefill kernel's tasks: (request index, first token) pairs.  Workgroups start in the
     order of the list, two to a compute unit, and the card fills the compute units' first places in turn before their
     second ones: so the longer half of the tasks (those that walk the most keys) comes first, longest first, and the
     shorter half follows shortest first; a compute unit then holds a long task beside a short one, and the long ones
     do not start last and leave the other compute units waiting for them.  (Against all tasks longest first: 60.4 ->
     57.8 us for 2,048 tokens over 2k keys, 251.6 -> 242.7 us over 8k; a long and a short one in turns, or as one
-    workgroup's two tasks, was slower.)  ``per_wg`` tasks go to one workgroup, one after the other."""
+    workgroup's two tasks, was slower.)  ``per_wg`` tasks go to one workgroup, one after the other.  ``window``: a
+    task of a layer with a window walks no more keys than its tokens and the window."""
     tasks = []
     start = 0
     for r, n in enumerate(q_lens):
         for t in range(0, n if not (skip_single and n == 1) else 0, tokens_per_task):
             keys = ctx_lens[r] - n + min(t + tokens_per_task, n)        # keys the task's last token sees
+            if window > 0:
+                keys = min(keys, window + tokens_per_task)
             tasks.append((-keys, r, start + t))
         start += n
     tasks.sort()
@@ -448,11 +485,11 @@ def paged_attention(q: torch.Tensor, out: torch.Tensor, cache: torch.Tensor, ste
     # to the prefill kernel (each would be slow at the other's work)
     lib = build.load("attention_mfma")
     tpt = lib.lcu_attention_prefill_tokens_per_task(n_heads, n_kv_heads)
-    key = ("attention_tasks", tpt)
+    key = ("attention_tasks", tpt, int(window))
     if key not in step.scratch:
         singles = sorted((r for r, n in enumerate(step.q_lens) if n == 1), key=lambda r: -step.ctx_lens[r])    # most keys first
         use_decode = len(singles) >= 1
-        tasks = prefill_tasks(step.q_lens, step.ctx_lens, tpt, q.device, skip_single=use_decode)
+        tasks = prefill_tasks(step.q_lens, step.ctx_lens, tpt, q.device, skip_single=use_decode, window=window)
         req_list = to_device(singles, torch.int32, q.device) if use_decode else None
         max_ctx = max([step.ctx_lens[r] for r in singles], default=0)
         step.scratch[key] = (tasks, req_list, len(singles) if use_decode else 0, max_ctx)

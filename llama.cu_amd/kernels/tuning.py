@@ -27,7 +27,7 @@ class Tuning:
     skinny_four_tiles_from: int = 65536  # ... four for the widest, with more than 8 rows
     skinny_workgroups_per_cu: int = 4   # plain: as many tiles as still leave this many workgroups for each compute unit
     skinny_eight_waves_to: int = 8192   # eight waves share a workgroup's K up to this many output features, four beyond
-    compute_units: int = 256
+    compute_units: int = 256            # of the card the numbers were measured on; ``for_device`` puts in the card's own
     # ---- the product that shares the rows through LDS (gemm_mid.hip, up to 128 rows)
     mid_long_k: int = 8192              # with a plain (not packed) weight only weights with a longer K than this (the down
                                         # projection) go to it at all; a packed weight with a longer K goes to it
@@ -48,3 +48,13 @@ class Tuning:
 
 
 TUNING = Tuning()
+
+
+def for_device(tuning: Tuning, device) -> Tuning:
+    """``tuning`` with the facts of the card at ``device`` in the fields that are the card's (the number of compute
+    units), not choices."""
+    import dataclasses
+
+    import torch
+    units = int(torch.cuda.get_device_properties(device).multi_processor_count)
+    return tuning if units == tuning.compute_units or units <= 0 else dataclasses.replace(tuning, compute_units=units)

@@ -41,4 +41,7 @@ def llama_spec(cfg: LlamaConfig) -> ModelSpec:
         eos_token_ids=cfg.eos_token_ids)
 
 
-register_architecture("LlamaForCausalLM", LlamaConfig.from_dict, llama_spec)
+# files of this architecture may carry each layer's rotation frequencies, which are no weights (the tables are made
+# from rope_theta)
+register_architecture("LlamaForCausalLM", LlamaConfig.from_dict, llama_spec,
+                      ignored_tensors=[r".*\.rotary_emb\.inv_freq$"])

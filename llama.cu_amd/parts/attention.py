@@ -70,6 +70,15 @@ class Attention(Part):
         self._rotation_only = type(self.position).apply is Part.apply
         self.page_size = build.page_size
         self.dtype = build.dtype
+        if self.dtype == torch.bfloat16:
+            # a bfloat16 model whose attention the matrix-core kernels do not take still runs, on the generic
+            # kernel: correct, and several times slower over long contexts, so the log says so and why
+            why = ops.mfma_attention_refusal(self.dtype, self.heads, self.kv_heads, self.head_dim, self.own_page_size or self.page_size)
+            if why is None and self.position.score_slopes() is not None:
+                why = "the position encoding is a bias inside the scores, which the matrix-core kernels do not take"
+            if why is not None:
+                ops.say_once(f"attention with {self.heads} heads of {self.head_dim} in {self.kv_heads} groups runs on the generic "
+                             f"kernel, not on the matrix cores: {why}")
 
     # forward(..., into=(residual, norm)) may end with the residual sum and that norm's weight
     # in the output projection and return ScaledRows instead of the branch's output

@@ -29,8 +29,9 @@ import torch
 
 @dataclass(frozen=True)
 class TensorSpec:
-    """One tensor a part binds: its shape, and how a random model fills it
-    (``normal``: N(0, std); ``one_plus_normal``: 1 + N(0, std), for norm weights).
+    """One tensor a part binds: its shape, and how a random model fills it: the name of an
+    initialiser (``normal``: N(0, std); ``one_plus_normal``: 1 + N(0, std), for norm weights;
+    ``zeros``; ``ones``; or one that ``weights.register_initialiser`` has made known).
     ``integer`` tensors are kept as int32, all others follow the weight policy."""
     shape: Tuple[int, ...]
     init: str = "normal"

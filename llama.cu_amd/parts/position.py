@@ -16,6 +16,8 @@ token's place.  The interface:
 """
 from __future__ import annotations
 
+import weakref
+
 import numpy as np
 import torch
 
@@ -35,6 +37,19 @@ class NoPosition(Part):
         ``slope[h] * (key position - query position)`` added to the scaled score.  The mixer hands it to
         the attention kernel (the generic one: the matrix-core kernels take no bias)."""
         return None
+
+
+class _Tables:
+    """The cosine and sine tables of one (theta, rotated dims, positions) on one device."""
+
+    def __init__(self, cos: torch.Tensor, sin: torch.Tensor):
+        self.cos, self.sin = cos, sin
+
+
+# The tables depend on (theta, rotated dims, positions, device) alone, so the layers of a model that agree in
+# these share one pair: 32 layers at 131,072 positions would else build and hold 32 x 67 MB.  The table lives as
+# long as a part holds it.
+_tables: "weakref.WeakValueDictionary" = weakref.WeakValueDictionary()
 
 
 class Rotary(NoPosition):
@@ -69,9 +84,14 @@ class Rotary(NoPosition):
         return np.cos(ang).astype(np.float32), np.sin(ang).astype(np.float32)
 
     def load(self, tensors, build: BuildContext) -> None:
-        cos, sin = self.host_tables()
-        self.cos = torch.from_numpy(cos).to(build.device).contiguous()
-        self.sin = torch.from_numpy(sin).to(build.device).contiguous()
+        key = (self.theta, self.rot_dim, self.max_positions, str(torch.device(build.device)))
+        tables = _tables.get(key)
+        if tables is None:
+            cos, sin = self.host_tables()
+            tables = _tables[key] = _Tables(torch.from_numpy(cos).to(build.device).contiguous(),
+                                            torch.from_numpy(sin).to(build.device).contiguous())
+        self._tables = tables                  # keeps the shared pair alive
+        self.cos, self.sin = tables.cos, tables.sin
 
     def rotary_tables(self):
         return self.cos, self.sin, self.rot_dim, 1 if self.interleaved else 0

@@ -23,18 +23,18 @@ import torch
 from ..parts.base import TensorSpec
 from .safetensors_io import SafetensorsFile
 
-# tensors that files of this ecosystem may carry and that hold no weights
-IGNORED = [re.compile(r".*\.rotary_emb\.inv_freq$")]
-
 
 class WeightError(ValueError):
     """The weight files do not fit the model; the message lists every problem."""
 
 
-def check_tensors(expected: Dict[str, TensorSpec], found: Dict[str, Tuple[int, ...]]) -> None:
-    """Raise one WeightError that lists missing and unexpected tensors and wrong shapes."""
+def check_tensors(expected: Dict[str, TensorSpec], found: Dict[str, Tuple[int, ...]], ignored: Sequence[str] = ()) -> None:
+    """Raise one WeightError that lists missing and unexpected tensors and wrong shapes.  ``ignored``: regular
+    expressions for tensors that the files may hold beside the weights (the architecture's registry entry names
+    them); they are passed over."""
+    patterns = [re.compile(p) for p in ignored]
     missing = sorted(n for n, s in expected.items() if n not in found and not s.optional)
-    unexpected = sorted(n for n in found if n not in expected and not any(p.match(n) for p in IGNORED))
+    unexpected = sorted(n for n in found if n not in expected and not any(p.match(n) for p in patterns))
     wrong = sorted((n, tuple(found[n]), tuple(s.shape)) for n, s in expected.items()
                    if n in found and tuple(found[n]) != tuple(s.shape))
     if not (missing or unexpected or wrong):
@@ -160,14 +160,15 @@ class _Stager:
 
 
 def load_weights(files: List[SafetensorsFile], expected: Dict[str, TensorSpec], compute: torch.dtype,
-                 device: torch.device, groups: Sequence[FusedGroup] = (), log=None) -> Dict[str, torch.Tensor]:
+                 device: torch.device, groups: Sequence[FusedGroup] = (), log=None,
+                 ignored: Sequence[str] = ()) -> Dict[str, torch.Tensor]:
     """All expected tensors, checked, converted and on ``device``, as views of one allocation
     (the reference lays all weights out in one region too, llama.cu/src/load/mod.rs:28-44).  The
     members of a fused group stand one after the other in it.  The bytes go through pinned host
     buffers, two in turn; a tensor whose file stores another type than the engine keeps is staged
     on the device and converted there, so the most that is ever allocated beside the weights
     themselves is one tensor.  ``log``: a function that takes the line with the size and the rate
-    (llama.cu/src/load/mod.rs:110-117 logs the same)."""
+    (llama.cu/src/load/mod.rs:110-117 logs the same).  ``ignored``: as in ``check_tensors``."""
     import time
     device = torch.device(device)
     where: Dict[str, SafetensorsFile] = {}
@@ -179,7 +180,7 @@ def load_weights(files: List[SafetensorsFile], expected: Dict[str, TensorSpec], 
             where[n] = f
     if dup:
         raise WeightError("tensors that more than one file holds: " + ", ".join(sorted(dup)))
-    check_tensors(expected, {n: f.shape(n) for n, f in where.items()})
+    check_tensors(expected, {n: f.shape(n) for n, f in where.items()}, ignored)
     stored = {n: where[n].dtype(n) for n in expected if n in where}
     for n, dt in stored.items():
         try:

@@ -14,7 +14,7 @@ from __future__ import annotations
 import ctypes
 import json
 import os
-from typing import Dict
+from typing import Callable, Dict, List
 
 import torch
 
@@ -65,6 +65,30 @@ def fill_normal(out: torch.Tensor, key: int, std: float, shift: float = 0.0) -> 
     return out
 
 
+# How the random mode fills a tensor, by the name that ``TensorSpec.init`` holds: ``fill(out, key, std)`` fills the
+# contiguous float32 or bfloat16 tensor ``out`` (on the host or on the GPU) in place; ``key`` is the tensor's stream
+# (``fill_normal(out, key, ...)`` gives the same bits on both sides), ``std`` the scale that the caller asked for.
+_INITIALISERS: Dict[str, Callable[[torch.Tensor, int, float], None]] = {}
+
+
+def register_initialiser(name: str, fill: Callable[[torch.Tensor, int, float], None], replace: bool = False) -> None:
+    """Make ``name`` known as a value of ``TensorSpec.init``: a part whose tensors need another start than a
+    normal distribution (zeros, a decay in some range, a bias) registers its own and names it in ``tensors()``."""
+    if name in _INITIALISERS and not replace:
+        raise ValueError(f"initialiser {name!r} is already registered")
+    _INITIALISERS[name] = fill
+
+
+def registered_initialisers() -> List[str]:
+    return sorted(_INITIALISERS)
+
+
+register_initialiser("normal", lambda out, key, std: fill_normal(out, key, std))                   # N(0, std): matrices
+register_initialiser("one_plus_normal", lambda out, key, std: fill_normal(out, key, std, 1.0))    # 1 + N(0, std): norm weights
+register_initialiser("zeros", lambda out, key, std: out.zero_())
+register_initialiser("ones", lambda out, key, std: out.fill_(1.0))
+
+
 def random_tensors(expected: Dict[str, TensorSpec], seed: int, dtype: torch.dtype = torch.bfloat16,
                    std: float = 0.02, device="cpu", vector_dtype=None) -> Dict[str, torch.Tensor]:
     """A tensor for every expected name that the random mode makes (a tied model gets no
@@ -80,8 +104,11 @@ def random_tensors(expected: Dict[str, TensorSpec], seed: int, dtype: torch.dtyp
             continue
         dt = (vector_dtype or dtype) if len(spec.shape) == 1 else dtype
         made = dt if dt in (torch.float32, torch.bfloat16) else torch.float32
+        fill = _INITIALISERS.get(spec.init)
+        if fill is None:
+            raise ValueError(f"tensor {name!r}: no initialiser {spec.init!r}; registered: {registered_initialisers()}")
         t = torch.empty(spec.shape, dtype=made, device=dev)
-        fill_normal(t, stream_key(seed, name), std, 1.0 if spec.init == "one_plus_normal" else 0.0)
+        fill(t, stream_key(seed, name), std)
         out[name] = t if made == dt else t.to(dt)
     return out
 

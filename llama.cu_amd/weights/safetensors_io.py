@@ -38,15 +38,24 @@ def read_safetensors_header(path: str) -> Tuple[Dict[str, dict], int]:
             header = json.loads(f.read(hlen))
         except (json.JSONDecodeError, UnicodeDecodeError) as e:
             raise SafetensorsError(f"{path}: header is not valid JSON: {e}") from None
+    if not isinstance(header, dict):
+        raise SafetensorsError(f"{path}: the header is no JSON object")
     header.pop("__metadata__", None)
     base = 8 + hlen
     for name, info in header.items():
+        if not isinstance(info, dict):
+            raise SafetensorsError(f"{path}: the header's entry for tensor {name!r} is no object")
         dt = DTYPES.get(info.get("dtype"))
         if dt is None:
             raise SafetensorsError(f"{path}: tensor {name!r} has unsupported dtype {info.get('dtype')!r}")
-        a, b = info["data_offsets"]
+        shape, offsets = info.get("shape"), info.get("data_offsets")
+        if not isinstance(shape, list) or not all(isinstance(x, int) and x >= 0 for x in shape):
+            raise SafetensorsError(f"{path}: tensor {name!r}: 'shape' is missing or no list of sizes")
+        if not isinstance(offsets, list) or len(offsets) != 2 or not all(isinstance(x, int) for x in offsets):
+            raise SafetensorsError(f"{path}: tensor {name!r}: 'data_offsets' is missing or no pair of offsets")
+        a, b = offsets
         n = 1
-        for s in info["shape"]:
+        for s in shape:
             n *= s
         if b - a != n * torch.empty(0, dtype=dt).element_size():
             raise SafetensorsError(f"{path}: tensor {name!r}: {b - a} bytes do not hold shape {info['shape']} of {info['dtype']}")
@@ -99,8 +108,15 @@ def open_safetensors(folder: str) -> List[SafetensorsFile]:
     if os.path.isfile(single):
         return [SafetensorsFile(single)]
     if os.path.isfile(index):
-        with open(index) as f:
-            shards = sorted(set(json.load(f)["weight_map"].values()))
+        try:
+            with open(index) as f:
+                weight_map = json.load(f)["weight_map"]
+            shards = sorted(set(weight_map.values()))
+        except (json.JSONDecodeError, UnicodeDecodeError, KeyError, TypeError, AttributeError) as e:
+            raise SafetensorsError(f"{index}: no JSON object with a 'weight_map' from tensor names to files ({type(e).__name__}: {e})") from None
+        absent = [s for s in shards if not os.path.isfile(os.path.join(folder, str(s)))]
+        if absent:
+            raise SafetensorsError(f"{index} names files that are not in {folder!r}: {', '.join(map(str, absent))}")
         return [SafetensorsFile(os.path.join(folder, s)) for s in shards]
     raise SafetensorsError(f"no model.safetensors (or model.safetensors.index.json) in {folder!r}")
 

@@ -187,3 +187,54 @@ def test_a_cache_with_state_that_cannot_be_cut_back_refuses_to_truncate():
         m.truncate(1, 39)
     assert m.length(1) == 40
     m.check()
+
+
+def test_a_request_that_cannot_be_cut_back_gives_up_only_what_cannot_be_cut():
+    """``truncate_or_reset``: where a plain ``truncate`` works it is one; where the state of fixed size cannot be
+    cut back the request's length becomes 0 with its pages kept; where a window has given back a page that the
+    shorter request would see, that group's pages go back to the pool and the other group's stay."""
+    m = CacheManager([CacheGroup(8, 16)], 2, can_truncate=True)
+    m.add(1); m.reserve(1, 40); m.commit(1)
+    assert m.truncate_or_reset(1, 30) and m.length(1) == 30 and len(m.table(1)) == 2
+    m = CacheManager([CacheGroup(8, 16)], 2, can_truncate=False)
+    m.add(1); m.reserve(1, 40); m.commit(1)
+    assert not m.truncate_or_reset(1, 30)
+    assert m.length(1) == 0 and m.reserved(1) == 30 and len(m.table(1)) == 2 and m.free_pages() == 6
+    assert m.reserve(1, 30) and m.free_pages() == 6        # computing it again asks the pool for nothing
+    m.commit(1)
+    assert m.length(1) == 30
+    m.check()
+    m = CacheManager([CacheGroup(8, 16), CacheGroup(8, 16, window=20)], 2)
+    m.add(1); m.reserve(1, 70); m.commit(1)
+    assert m.table(1, 1)[:3] == [-1, -1, -1]
+    assert not m.truncate_or_reset(1, 60)                  # the query at 60 would see keys from 41: page 2 is gone
+    assert m.length(1) == 0 and m.reserved(1) == 0
+    assert len(m.table(1, 0)) == 4 and m.table(1, 1) == [] and m.free_pages(1) == 8 and m.free_pages(0) == 4
+    assert m.reserve(1, 60) and m.free_pages(0) == 4 and m.free_pages(1) == 4
+    m.commit(1)
+    m.check()
+    m.release(1)
+    assert m.free_pages(0) == 8 and m.free_pages(1) == 8 and m.free_slots() == 2
+
+
+def test_a_windows_slack_keeps_what_a_request_cut_back_by_that_much_would_see():
+    for slack in (0, 1, 5):
+        m = CacheManager([CacheGroup(8, 4, window=6, slack=slack)], 2)
+        m.add(1)
+        for n in range(1, 60):
+            assert m.reserve(1, n)
+            m.commit(1)
+            t = m.table(1)
+            first_key = max(n - slack - 5, 0)              # what the query at n - slack sees first
+            for p, page in enumerate(t):
+                assert (page == -1) == (p < first_key // 4), (slack, n, t)
+            # cutting back by up to the slack works at every length; by more, not at every length
+            for cut in range(0, slack + 1):
+                if n - cut >= 0:
+                    probe = CacheManager([CacheGroup(8, 4, window=6, slack=slack)], 2)
+                    probe.add(1)
+                    for k in range(1, n + 1):
+                        probe.reserve(1, k); probe.commit(1)
+                    probe.truncate(1, n - cut)
+                    probe.check()
+        m.check()

@@ -73,6 +73,34 @@ def test_seeded_temperature_sampling_with_portions(folder_b):
         assert out == got[rid]
 
 
+def test_the_entry_point_gives_the_same_draws_on_every_call_and_is_clean_after_an_error(folder_b):
+    """``llama_cu_amd.generate`` keeps the engine of a folder between calls.  A call's random draws are keyed by the
+    prompt's place in the call, so the same call gives the same tokens the second time; a call that fails half
+    way (a token outside the vocabulary in its second prompt) leaves nothing of itself in the engine; a folder
+    that is written again is loaded again."""
+    import llama_cu_amd
+    from llama_cu_amd.sampling import SamplingParams
+    prompts = list(common.random_requests(384, [7, 30, 12], seed=4).values())
+    params = SamplingParams(temperature=0.9, top_p=0.95, seed=99)
+    kw = dict(max_steps=12, dtype="float32", max_tokens=512, max_seqs=4)
+    first = llama_cu_amd.generate(folder_b, prompts, params, **kw)
+    engine = next(iter(llama_cu_amd._engines.values()))
+    with pytest.raises(ValueError, match="outside the vocabulary"):
+        llama_cu_amd.generate(folder_b, [prompts[0], [1, 2, 9999]], params, **kw)
+    assert engine.idle and not engine.requests and engine.runner.cache.live_requests() == 0
+    second = llama_cu_amd.generate(folder_b, prompts, params, **kw)
+    assert next(iter(llama_cu_amd._engines.values())) is engine            # the same engine served all three calls
+    assert second == first and len(set(map(tuple, first))) == 3
+    # another order of the prompts is another set of draws for each (the key is the place in the call)
+    assert llama_cu_amd.generate(folder_b, prompts[::-1], params, **kw)[::-1] != first
+    # the folder written again (other weights): not the engine of before
+    common.make_folder(common.TINY_B, seed=77, dtype=torch.float32, folder=folder_b)
+    other = llama_cu_amd.generate(folder_b, prompts, params, **kw)
+    assert next(iter(llama_cu_amd._engines.values())) is not engine and other != first
+    common.make_folder(common.TINY_B, seed=22, dtype=torch.float32, folder=folder_b)      # as the fixture made it
+    assert llama_cu_amd.generate(folder_b, prompts, params, **kw) == first
+
+
 def test_few_pages_preemption_changes_no_token(folder_a):
     """A pool too small for all requests at once: the scheduler preempts and recomputes;
     the generated tokens are those of an ample pool."""

@@ -561,8 +561,9 @@ def test_a_toy_position_encoding_that_is_a_bias_inside_the_scores():
     runner.cache.check()
 
 
-def _engine_turns(engine, prompt, eos, more, steps):
-    """A kept request: one turn until the end-of-sequence token, then a turn with ``more``."""
+def _engine_turns(engine, prompt, eos, more, steps, seen=None):
+    """A kept request: one turn until the end-of-sequence token, then a turn with ``more``.  ``seen``: takes what
+    the request has computed and which pages it holds between the turns."""
     from llama_cu_amd.sampling import GREEDY
     engine.eos = {eos} if eos is not None else set()
     rid = engine.add_request(prompt, GREEDY, steps, keep=True, ignore_eos=eos is None)
@@ -576,6 +577,9 @@ def _engine_turns(engine, prompt, eos, more, steps):
                 why = o.finished or why
         turns.append((toks, why))
         if turn == 0:
+            if seen is not None:
+                seen["computed"] = engine.sched.info(rid).computed
+                seen["pages"] = [len(engine.runner.cache.table(rid, g)) for g in range(len(engine.runner.groups))]
             engine.continue_request(rid, more, steps)
     engine.drop(rid)
     engine.runner.cache.check()
@@ -653,8 +657,18 @@ def test_an_end_learned_late_with_a_cache_that_cannot_be_cut_back(kind):
         want = _engine_turns(engine(False), prompt, eos, more, 10)
         assert want[0] == (probe[:at + 1], "eos")
         e = engine(True)
-        got = _engine_turns(e, prompt, eos, more, 10)
+        seen = {}
+        got = _engine_turns(e, prompt, eos, more, 10, seen)
         assert got == want, f"end-of-sequence token at {at}"
+        held = len(prompt) + at                  # tokens before the end-of-sequence token
+        if kind == "window":
+            # the window keeps its pages a token longer than the next query needs, so the one token computed
+            # beyond the end is cut away and nothing is computed again
+            assert seen["computed"] == held, seen
+        else:
+            # the state cannot be cut back: the request starts again at its first token, but the pages of the
+            # layer that has pages stayed its own
+            assert seen["computed"] == 0 and seen["pages"] == [(held + 7) // 8], seen
         # the second turn is what a fresh request with the whole context generates
         fresh = engine(False)
         whole = fresh.generate([prompt + probe[:at + 1] + more], max_steps=len(want[1][0]), ignore_eos=True)[0]

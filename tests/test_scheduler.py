@@ -262,12 +262,13 @@ def test_an_end_by_count_at_the_same_token_takes_the_late_reason():
     assert cache.free_pages(0) == 64
 
 
-def test_an_end_learned_late_at_a_windows_edge_gives_the_cache_back_and_the_next_turn_recomputes():
+def test_an_end_learned_late_at_a_windows_edge_gives_the_windows_pages_back_and_the_next_turn_recomputes():
     """Window 4, pages of 4: once token 7 is in the cache, page 0 is given back (the next query, at
     8, sees keys 5..8).  If the request is then cut back to 6 tokens, the next query, at 6, would
-    see keys 3..6, and key 3 lay in page 0, which is gone.  The scheduler then gives the whole
-    cache back and a later turn starts at token 0."""
-    cache = CacheManager([CacheGroup(16, 4, window=4)], 4)
+    see keys 3..6, and key 3 lay in page 0, which is gone.  The request then gives up the pages of
+    the group with the window, keeps those of the group without one, and a later turn starts at
+    token 0 without asking that group's pool for anything."""
+    cache = CacheManager([CacheGroup(16, 4, window=4), CacheGroup(16, 4)], 4)
     s = Scheduler(cache, 4, 64, 32, 512)
     s.add(0, list(range(6)), 10, keep=True)
     run_round(s, next_token=lambda req, n: 0)            # tokens 0..5 computed, placeholder 6
@@ -276,15 +277,42 @@ def test_an_end_learned_late_at_a_windows_edge_gives_the_cache_back_and_the_next
     assert cache.length(0) == 8 and cache.table(0)[0] == -1
     # the token at index 6 was the end of the sequence: 7 tokens remain, 6 of them in the cache
     assert s.finish(0, "eos", 7) == "eos"
-    assert not cache.has(0) and s.info(0).computed == 0
-    assert cache.free_pages(0) == 16
+    assert cache.has(0) and cache.length(0) == 0 and s.info(0).computed == 0
+    assert cache.free_pages(0) == 16                       # the window's pages are back in the pool
+    assert cache.table(0, 1) and cache.free_pages(1) == 14 and len(cache.table(0, 1)) == 2     # pages for 6 tokens stay
     cache.check()
     s.extend(0, [5, 6], 3)
     plan = s.plan()
     assert [(e.req, e.start, e.count) for e in plan] == [(0, 0, 9)]
+    assert cache.free_pages(1) == 13                       # one more page for tokens 8: the first two were its own already
     s.commit()
     s.abort(0); s.drop(0)
     cache.check()
+    assert cache.free_pages(0) == 16 and cache.free_pages(1) == 16
+
+
+def test_a_window_with_a_token_of_slack_can_be_cut_back_by_the_token_computed_beyond_the_end():
+    """An engine that runs one round ahead computes one token beyond an end of sequence: here token 6, the end,
+    is in the cache (7 tokens) when the end is learned, and the request is to be cut back to 6.  The query at 7
+    sees keys 4..7, so without slack page 0 went when token 6 came, and the query at 6 (keys 3..6) has lost key 3.
+    With ``slack=1`` (what the engine asks for) page 0 is still there, the request is cut back, and nothing is
+    computed again."""
+    for slack in (0, 1):
+        cache = CacheManager([CacheGroup(16, 4, window=4, slack=slack)], 4)
+        s = Scheduler(cache, 4, 64, 32, 512)
+        s.add(0, list(range(6)), 10, keep=True)
+        for _ in range(2):
+            run_round(s, next_token=lambda req, n: 0)
+        assert cache.length(0) == 7 and (cache.table(0)[0] >= 0) == (slack == 1)
+        assert s.finish(0, "eos", 7) == "eos"
+        assert cache.has(0) and cache.length(0) == (6 if slack else 0) and s.info(0).computed == (6 if slack else 0)
+    s.extend(0, [5, 6], 3)
+    assert [(e.req, e.start, e.count) for e in s.plan()] == [(0, 6, 3)]
+    s.commit()
+    assert cache.table(0)[0] == -1                         # with 9 tokens in, the query at 8 sees keys 5..8: page 0 goes
+    s.abort(0); s.drop(0)
+    cache.check()
+    assert cache.free_pages(0) == 16
 
 
 def test_an_end_learned_late_with_state_that_cannot_be_cut_back_recomputes_the_next_turn():
@@ -296,8 +324,11 @@ def test_an_end_learned_late_with_state_that_cannot_be_cut_back_recomputes_the_n
     run_round(s, next_token=lambda req, n: 0)
     run_round(s, next_token=lambda req, n: 0)
     assert cache.length(0) == 9
+    free = cache.free_pages(0)
     assert s.finish(0, "eos", 8) == "eos"                 # one token computed beyond the end
-    assert not cache.has(0) and s.info(0).computed == 0
+    # the state cannot be cut back: the request starts again at 0, but its pages (for 7 tokens) stay its own
+    assert cache.has(0) and cache.length(0) == 0 and s.info(0).computed == 0
+    assert len(cache.table(0)) == 2 and cache.free_pages(0) == free + 1
     # request 1 ended by count with nothing computed beyond its end: its cache stays
     assert s.info(1).reason == "max_steps" and cache.has(1) and cache.length(1) == 4
     s.extend(0, [5], 2)

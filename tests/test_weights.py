@@ -70,8 +70,24 @@ def test_broken_files_are_refused(tmp_path):
     open(path, "wb").write(struct.pack("<Q", 5) + b"{oops")
     with pytest.raises(SafetensorsError, match="JSON"):
         open_safetensors(str(tmp_path))
+    # header entries without their keys
+    for entry, what in (({"dtype": "F32", "data_offsets": [0, 4]}, "shape"), ({"dtype": "F32", "shape": [1]}, "data_offsets"),
+                        ({"dtype": "F32", "shape": [1], "data_offsets": [0]}, "data_offsets"), ("F32", "no object")):
+        blob = json.dumps({"a": entry}).encode()
+        open(path, "wb").write(struct.pack("<Q", len(blob)) + blob + b"\0" * 4)
+        with pytest.raises(SafetensorsError, match=what):
+            open_safetensors(str(tmp_path))
     os.remove(path)
     with pytest.raises(SafetensorsError, match="no model.safetensors"):
+        open_safetensors(str(tmp_path))
+    # an index that names a file that is not there, and one that is no index
+    index = os.path.join(str(tmp_path), "model.safetensors.index.json")
+    json.dump({"weight_map": {"a": "model-00001-of-00002.safetensors", "b": "model-00002-of-00002.safetensors"}}, open(index, "w"))
+    write_safetensors(os.path.join(str(tmp_path), "model-00001-of-00002.safetensors"), {"a": torch.zeros(2)})
+    with pytest.raises(SafetensorsError, match="model-00002-of-00002.safetensors"):
+        open_safetensors(str(tmp_path))
+    json.dump({"weights": {}}, open(index, "w"))
+    with pytest.raises(SafetensorsError, match="weight_map"):
         open_safetensors(str(tmp_path))
 
 
@@ -86,12 +102,19 @@ def test_one_error_lists_missing_unexpected_and_wrong_shapes(tmp_path):
     w["model.layers.7.extra.weight"] = torch.zeros(2)
     w["model.layers.0.self_attn.rotary_emb.inv_freq"] = torch.zeros(8)      # carried by some files, holds no weight
     write_safetensors(os.path.join(folder, "model.safetensors"), w)
+    # which tensors a file may hold beside the weights is the architecture's business: its registry entry names them
+    from llama_cu_amd.config import architecture_of
+    ignored = architecture_of(common.TINY_A).ignored_tensors
+    assert ignored
     with pytest.raises(WeightError) as err:
-        load_weights(open_safetensors(folder), expected(common.TINY_A), torch.float32, torch.device("cpu"))
+        load_weights(open_safetensors(folder), expected(common.TINY_A), torch.float32, torch.device("cpu"), ignored=ignored)
     msg = str(err.value)
     assert "missing tensors (2)" in msg and "model.layers.1.mlp.up_proj.weight" in msg and "model.norm.weight" in msg
     assert "unexpected tensors (1)" in msg and "model.layers.7.extra.weight" in msg and "inv_freq" not in msg
     assert "wrong shapes (1)" in msg and "found [64, 63], expected [64, 64]" in msg
+    # the loader itself knows no such tensor
+    with pytest.raises(WeightError, match=r"unexpected tensors \(2\)"):
+        load_weights(open_safetensors(folder), expected(common.TINY_A), torch.float32, torch.device("cpu"))
 
 
 def test_tied_and_untied_output_matrix(tmp_path):
@@ -251,3 +274,29 @@ def test_weights_lie_in_one_allocation_and_fused_tensors_stand_in_place(tmp_path
     expected = {"g": TensorSpec((5, 8)), "u": TensorSpec((5, 8)), "x": TensorSpec((3,))}
     place, total = plan_arena(expected, {n: torch.bfloat16 for n in expected}, torch.bfloat16, [FusedGroup(("g", "u"), 8)])
     assert place["u"][0] - place["g"][0] == 8 * 8 * 2 and place["x"][0] >= place["u"][0] + 8 * 8 * 2 and total % 256 == 0
+
+
+def test_a_part_names_how_its_tensors_start_and_may_bring_its_own_way():
+    """``TensorSpec.init`` names an initialiser of a registry: zeros and ones are there beside the two normal ones, a
+    part from outside registers its own (here a decay spread evenly over a range, made from the tensor's own stream),
+    and a name that nothing registers is an error that lists the registered ones."""
+    from llama_cu_amd.weights import fill_normal, random_tensors, register_initialiser, registered_initialisers
+
+    def decay(out, key, std):
+        fill_normal(out, key, 1.0)                              # the tensor's stream: the same bits on host and GPU
+        out.copy_(torch.sigmoid(out.float()) * 0.5 + 0.4)       # into (0.4, 0.9)
+
+    register_initialiser("toy_decay", decay, replace=True)
+    assert {"normal", "one_plus_normal", "zeros", "ones", "toy_decay"} <= set(registered_initialisers())
+    want = {"a.weight": TensorSpec((8, 16)), "a.bias": TensorSpec((8,), init="zeros"), "a.gain": TensorSpec((8,), init="ones"),
+            "a.decay": TensorSpec((64,), init="toy_decay")}
+    t = random_tensors(want, 5, dtype=torch.float32, std=0.02)
+    assert float(t["a.bias"].abs().max()) == 0.0 and bool((t["a.gain"] == 1.0).all())
+    assert 0.4 < float(t["a.decay"].min()) and float(t["a.decay"].max()) < 0.9 and float(t["a.decay"].std()) > 0.05
+    assert 0.01 < float(t["a.weight"].std()) < 0.03
+    again = random_tensors(want, 5, dtype=torch.float32, std=0.02)
+    assert all(torch.equal(t[k], again[k]) for k in t)
+    with pytest.raises(ValueError, match="registered"):
+        random_tensors({"b.weight": TensorSpec((2, 2), init="no_such_start")}, 1)
+    with pytest.raises(ValueError, match="already registered"):
+        register_initialiser("zeros", decay)

@@ -49,8 +49,12 @@ def test_decode_attention_that_allocates_nothing_equals_the_one_that_is_given_it
                  torch.empty(n * nh * splits * 2, dtype=torch.float32, device="cuda"))
         assert _decode(lib, "lcu_attention_decode_bf16", q, want, cache, step, nh, nkv, dh, page, splits, parts) == 0
         got = torch.full_like(want, float("nan"))
+        torch.cuda.synchronize()
+        free_before = torch.cuda.mem_get_info()[0]
         assert _decode(lib, "lcu_attention_decode_bf16_static", q, got, cache, step, nh, nkv, dh, page, splits) == 0
         torch.cuda.synchronize()
+        # the call took no memory from the driver (the kernels are loaded: the other entry point has just run them)
+        assert torch.cuda.mem_get_info()[0] == free_before, (free_before, torch.cuda.mem_get_info()[0])
         assert torch.isfinite(want.float()).all()
         assert torch.equal(got, want), f"{n} requests in {splits} parts"
     # more than the buffer holds: refused, nothing launched, the output untouched
@@ -67,3 +71,14 @@ def test_decode_attention_that_allocates_nothing_equals_the_one_that_is_given_it
                                               ctypes.c_float(1.0), 0, splits, stream)
     torch.cuda.synchronize()
     assert rc == -3 and bool((out == 3.0).all())
+    # sizes that no kernel takes are told so, also where the parts would not fit the buffer: the arguments are
+    # checked first, as the other entry point checks them
+    for bad in (dict(nkv=3), dict(page=24), dict(dh=40)):
+        a = {"nkv": nkv, "page": page, "dh": dh, **bad}
+        rc = lib.lcu_attention_decode_bf16_static(_ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(cache), _ptr(bt), 4,
+                                                  _ptr(ones), _ptr(ones), _ptr(None), n, nh, a["nkv"], a["dh"], a["page"],
+                                                  ctypes.c_float(1.0), 0, splits, stream)
+        assert rc in (-1, -2), (bad, rc)
+    assert lib.lcu_attention_static_scratch_needed(2 ** 31 - 1, 2 ** 31 - 1, 2 ** 31 - 3, 2 ** 31 - 1) == 2 ** 63 - 1
+    torch.cuda.synchronize()
+    assert bool((out == 3.0).all())
