@@ -131,7 +131,7 @@ def run_prefill(engine, cfg, rng, sync, repeats=3, history=0):
 
 
 def run_mixed(engine, cfg, n_requests, rng, sync, new_tokens=128, lo=16, hi=2048):
-    """The mixed batch of BASELINE's Llama-2-7B workload: ``n_requests`` requests at once, prompt
+    """A mixed batch (the workload that goes with the Llama-2-7B shape): ``n_requests`` requests at once, prompt
     lengths uniform in [lo, hi], ``new_tokens`` greedy tokens each, through the scheduler under its
     token budget (prompt portions beside decoding requests).  Returns a dict of what was measured:
     the reference's bench prints the same (llama.cu/xtask/src/bench.rs:63-80: time to the first
@@ -166,6 +166,55 @@ def run_mixed(engine, cfg, n_requests, rng, sync, new_tokens=128, lo=16, hi=2048
     return {"requests": n_requests, "prompt_tokens": sum(lens), "new_tokens": produced, "seconds": dt,
             "all_prompts_in_ms": first_all * 1e3, "prefill_steps": first_steps, "steps": steps,
             "decode_step_median_ms": decode_steps[len(decode_steps) // 2], "preemptions": engine.sched.preemptions}
+
+
+def run_arrivals(engine, cfg, batch, steps, rng, sync, every=2, arrival_len=16, arrival_tokens=2):
+    """``batch`` requests decode (after prompts of PROMPT_LEN tokens) while a new request with a prompt of
+    ``arrival_len`` tokens arrives every ``every`` steps, generates ``arrival_tokens`` tokens and leaves: steps in
+    which a prompt portion stands beside the decoding requests alternate with steps that only decode.  Returns what
+    the engine's timeline says of the timed steps: wall time per step, the host's time per step from the plan to
+    the last launch, and the fraction of the time in which the GPU had a step's work (events around each step)."""
+    from llama_cu_amd.sampling import GREEDY
+    total = steps + 64
+    ids = [engine.add_request([rng.randrange(cfg.vocab_size) for _ in range(PROMPT_LEN)], GREEDY, max_steps=total + 8 * batch,
+                              ignore_eos=True) for _ in range(batch)]
+    while any(engine.sched.info(i).generated == 0 for i in ids):
+        engine.step()
+    arrivals = []
+
+    def rounds(n, timed):
+        for k in range(n):
+            if k % every == 0:
+                arrivals.append(engine.add_request([rng.randrange(cfg.vocab_size) for _ in range(arrival_len)], GREEDY,
+                                                   max_steps=arrival_tokens, ignore_eos=True))
+            engine.step()
+    rounds(32, False)                                # every kind of step has come often enough to be captured, if it can be
+    sync()
+    engine.timeline = []
+    t0 = time.perf_counter()
+    rounds(steps, True)
+    sync()
+    dt = time.perf_counter() - t0
+    line, engine.timeline = engine.timeline, None
+    for i in ids:
+        engine.abort(i)
+        engine.drop(i)
+    while not engine.idle:
+        engine.step()
+    for i in arrivals:
+        engine.drop(i)
+    busy = sum(e["first"].elapsed_time(e["last"]) for e in line)
+    span = line[0]["first"].elapsed_time(line[-1]["last"])
+    kinds = {}
+    for e in line:
+        k = kinds.setdefault((e["tokens"], e["requests"], e["graph"]), [0, 0.0, 0.0])
+        k[0] += 1
+        k[1] += e["host_ms"]
+        k[2] += e["first"].elapsed_time(e["last"])
+    return {"steps": len(line), "ms_per_step": dt / steps * 1e3, "host_ms_per_step": sum(e["host_ms"] for e in line) / len(line),
+            "gpu_busy_frac": busy / span,
+            "kinds": [{"tokens": t, "requests": r, "from_graph": g, "steps": n, "host_ms": h / n, "gpu_ms": u / n}
+                      for (t, r, g), (n, h, u) in sorted(kinds.items())]}
 
 
 def library_product(cfg, sync, calls=400):
@@ -239,10 +288,12 @@ def main() -> int:
                          "limit grows with it)")
     ap.add_argument("--dtype", choices=["bfloat16", "float32"], default="bfloat16")
     ap.add_argument("--page-size", type=int, default=16, help="tokens in a page of the cache (a multiple of 16)")
-    ap.add_argument("--workload", choices=["decode", "mixed"], default="decode",
+    ap.add_argument("--workload", choices=["decode", "mixed", "arrivals"], default="decode",
                     help="decode: --batch requests decode together after prompts of --prompt-len (the default); mixed: "
                          "--batch requests at once with prompt lengths uniform in [16, 2048], 128 tokens each, through the "
-                         "scheduler (BASELINE's Llama-2-7B workload: --shape llama2-7b --batch 64)")
+                         "scheduler (the workload that goes with --shape llama2-7b --batch 64); arrivals: --batch requests "
+                         "decode while a prompt of 16 tokens arrives every second step (host time and the GPU's busy "
+                         "fraction per kind of step)")
     ap.add_argument("--no-points", action="store_true", help="skip decoding at batch 1 and 64 and the prefill")
     ap.add_argument("--only-prefill", action="store_true", help="time the 2048-token prefill alone (for profiles)")
     ap.add_argument("--prefill-history", type=int, default=0,
@@ -282,13 +333,22 @@ def main() -> int:
         print(json.dumps({"library_product": library_product(cfg, sync), "rows": PREFILL_TOKENS,
                           "in": cfg.hidden_size, "out": 2 * cfg.intermediate_size, "dtype": "bf16"}))
         return 0
-    biggest = max(args.batch, 1 if (args.no_points or args.only_prefill or args.workload == "mixed") else 64)
+    biggest = max(args.batch, 1 if (args.no_points or args.only_prefill or args.workload != "decode") else 64)
     # a request decodes while later ones still prefill: room for that too
     per_req = max(args.prompt_len, PROMPT_LEN) + grow
     engine = Engine.from_config(cfg, seed=0, dtype=args.dtype, page_size=page,
                                 max_tokens=biggest * ((per_req + page - 1) // page * page) + args.prefill_history + PREFILL_TOKENS + page,
                                 max_seqs=biggest + 2, max_batch_tokens=max(PREFILL_TOKENS, biggest), prefill_chunk=PREFILL_TOKENS)
 
+    if args.workload == "arrivals":
+        a = run_arrivals(engine, cfg, args.batch, args.steps, rng, sync)
+        print(json.dumps({"metric": f"ms a step ({shape_name} shape, {args.batch} requests decode, a prompt of 16 tokens arrives "
+                                    f"every second step)", "value": round(a["ms_per_step"], 4), "unit": "ms", "n_gpus": 1,
+                          "steps": a["steps"], "higher_is_better": False, "dtype": dt_name, "data": "synthetic",
+                          "host_ms_per_step": round(a["host_ms_per_step"], 3), "gpu_busy_frac": round(a["gpu_busy_frac"], 4),
+                          "kinds": [{k: (round(v, 3) if isinstance(v, float) else v) for k, v in kind.items()} for kind in a["kinds"]]}),
+              flush=True)
+        return 0
     if args.workload == "mixed":
         run_mixed(engine, cfg, min(args.batch, 8), rng, sync, new_tokens=8)          # builds, loads and captures
         m = run_mixed(engine, cfg, args.batch, rng, sync)

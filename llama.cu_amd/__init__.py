@@ -9,6 +9,7 @@ from .config import LlamaConfig, register_architecture
 from .parts import register_part
 
 from .sampling import SamplingParams
+from .engine.config import EngineConfig
 
 import os
 
@@ -29,10 +30,11 @@ def _folder_stamp(folder: str):
     return tuple(stamp)
 
 
-def Engine(model: str, dtype: str = "bfloat16", device: str = "cuda:0", **kw):
-    """The engine for the model folder ``model`` (see engine.engine.Engine)."""
+def Engine(model: str, config: EngineConfig = None, **fields):
+    """The engine for the model folder ``model`` (see engine.engine.Engine); ``config`` holds the engine's
+    constants, ``fields`` replace single ones (``dtype="float32", max_seqs=4, ...``)."""
     from .engine.engine import Engine as _Engine
-    return _Engine.from_folder(model, dtype=dtype, device=device, **kw)
+    return _Engine.from_folder(model, config, **fields)
 
 
 def generate(model: str, prompts, sampling: SamplingParams = SamplingParams(), max_steps: int = 1000,
@@ -56,7 +58,7 @@ def generate(model: str, prompts, sampling: SamplingParams = SamplingParams(), m
 
 
 __all__ = ["config", "parts", "models", "weights", "LlamaConfig", "register_architecture", "register_part",
-           "SamplingParams", "Engine", "generate"]
+           "SamplingParams", "EngineConfig", "Engine", "generate"]
 
 # modules of the user's that register further architectures or parts (LLAMA_CU_AMD_PLUGINS=module[,module]): imported
 # last, when everything they may import from here is there

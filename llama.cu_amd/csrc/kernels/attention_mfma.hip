@@ -896,7 +896,8 @@ __global__ void __launch_bounds__(PRE_THREADS, LCU_PRE_MIN_WAVES)
 attention_prefill_kernel(const bf16_t *__restrict__ q, int q_stride, bf16_t *__restrict__ out, int out_stride,
                            const bf16_t *__restrict__ cache, uint32_t cache_bytes, const int *__restrict__ block_table, int max_pages,
                            const int *__restrict__ q_start, const int *__restrict__ ctx_len,
-                           const int *__restrict__ task_req, const int *__restrict__ task_tok0, int n_tasks,
+                           const int *__restrict__ task_req, const int *__restrict__ task_tok0, int max_tasks,
+                           const int *__restrict__ n_tasks_dev,
                            int tasks_per_wg, int nh, int nkvh, int page, uint32_t tile_magic, float scale_log2, int window) {
     extern __shared__ u32x4 lds_ring[];            // [PRE_RING][8 * DH]
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
@@ -908,6 +909,9 @@ attention_prefill_kernel(const bf16_t *__restrict__ q, int q_stride, bf16_t *__r
     const int g = nh / nkvh;
     const int chunks = (g + 15) / 16;
     const int head_chunk = blockIdx.x % (nkvh * chunks), wg = blockIdx.x / (nkvh * chunks);
+    // the grid is made for max_tasks; how many of them the list holds may stand in memory (so that a launch recorded
+    // into a graph serves steps with other lists): workgroups beyond the list's end have nothing to do
+    const int n_tasks = n_tasks_dev ? min(*n_tasks_dev, max_tasks) : max_tasks;
     for (int task = wg * tasks_per_wg; task < (wg + 1) * tasks_per_wg && task < n_tasks; ++task) {
     __syncthreads();                               // the last task's use of LDS is over (it waited for its copies)
     const int n = lane & 31, hi = lane >> 5;
@@ -1039,8 +1043,8 @@ attention_prefill_kernel(const bf16_t *__restrict__ q, int q_stride, bf16_t *__r
 template <int DH, bool PAGE16, bool FLAT>
 static int launch_prefill_as(const void *q, int q_stride, void *out, int out_stride, const void *cache, uint32_t cache_bytes,
                              const int *block_table, int max_pages, const int *q_start, const int *ctx_len,
-                             const int *task_req, const int *task_tok0, int n_tasks, int tasks_per_wg, int nh, int nkvh,
-                             int page, float scale, int window, hipStream_t stream) {
+                             const int *task_req, const int *task_tok0, int n_tasks, const int *n_tasks_dev, int tasks_per_wg,
+                             int nh, int nkvh, int page, float scale, int window, hipStream_t stream) {
     const int g = nh / nkvh, chunks = (g + 15) / 16;
     const long long n_wg = (long long)((n_tasks + tasks_per_wg - 1) / tasks_per_wg) * nkvh * chunks;
     if (n_wg > 0x7fffffffll) return LCU_BAD_ARGUMENT;
@@ -1062,7 +1066,7 @@ static int launch_prefill_as(const void *q, int q_stride, void *out, int out_str
     }
     attention_prefill_kernel<DH, PAGE16, FLAT><<<grid, block, lds_bytes, stream>>>(
         (const bf16_t *)q, q_stride, (bf16_t *)out, out_stride, (const bf16_t *)cache, cache_bytes, block_table, max_pages, q_start,
-        ctx_len, task_req, task_tok0, n_tasks, tasks_per_wg, nh, nkvh, page,
+        ctx_len, task_req, task_tok0, n_tasks, n_tasks_dev, tasks_per_wg, nh, nkvh, page,
         page == 16 ? 0u : (uint32_t)(0x100000000ull / (unsigned)(page / 16)) + 1u, scale * 1.4426950408889634f, window);
     LCU_LAUNCH_CHECK();
     return LCU_OK;
@@ -1072,11 +1076,11 @@ static int launch_prefill_as(const void *q, int q_stride, void *out, int out_str
 template <int DH>
 static int launch_prefill(const void *q, int q_stride, void *out, int out_stride, const void *cache, long long cache_pages,
                           const int *block_table, int max_pages, const int *q_start, const int *ctx_len,
-                          const int *task_req, const int *task_tok0, int n_tasks, int tasks_per_wg, int nh, int nkvh,
-                          int page, float scale, int window, hipStream_t stream) {
+                          const int *task_req, const int *task_tok0, int n_tasks, const int *n_tasks_dev, int tasks_per_wg,
+                          int nh, int nkvh, int page, float scale, int window, hipStream_t stream) {
     const unsigned long long bytes = (unsigned long long)cache_pages * kv_page_elems(nkvh, DH, page) * sizeof(bf16_t);
     const bool flat = bytes < (1ull << 32);
-#define AS(P, F) return launch_prefill_as<DH, P, F>(q, q_stride, out, out_stride, cache, (uint32_t)(F ? bytes : 0), block_table, max_pages, q_start, ctx_len, task_req, task_tok0, n_tasks, tasks_per_wg, nh, nkvh, page, scale, window, stream)
+#define AS(P, F) return launch_prefill_as<DH, P, F>(q, q_stride, out, out_stride, cache, (uint32_t)(F ? bytes : 0), block_table, max_pages, q_start, ctx_len, task_req, task_tok0, n_tasks, n_tasks_dev, tasks_per_wg, nh, nkvh, page, scale, window, stream)
     if (page == 16) {
         if (flat) AS(true, true);
         AS(true, false);
@@ -1098,18 +1102,20 @@ LCU_API int lcu_attention_prefill_tokens_per_task(int nh, int nkvh) {
 
 // task_req / task_tok0: [n_tasks], tasks cut from the batch with the size above; a
 // request's last task may be shorter.  Workgroup i takes tasks i*tasks_per_wg .. + tasks_per_wg-1.
+// n_tasks_dev (may be null): a number on the device, read when the kernel runs: the lists hold that many tasks
+// (at most n_tasks, for which the grid is made), so that one recorded launch serves lists of other lengths.
 // bfloat16 only; head_dim 32, 64, 96 or 128; page_size a multiple of 16.
 LCU_API int lcu_attention_prefill_bf16(const void *q, int q_stride, void *out, int out_stride, const void *cache,
                                        long long cache_pages, const int *block_table, int max_pages, const int *q_start, const int *ctx_len,
-                                       const int *task_req, const int *task_tok0, int n_tasks, int tasks_per_wg,
-                                       int nh, int nkvh, int dh, int page, float scale, int window,
+                                       const int *task_req, const int *task_tok0, int n_tasks, const int *n_tasks_dev,
+                                       int tasks_per_wg, int nh, int nkvh, int dh, int page, float scale, int window,
                                        hipStream_t stream) {
     if (n_tasks <= 0) return LCU_OK;
     if ((unsigned long long)kv_page_elems(nkvh, dh, page) * 2ull >= (1ull << 31)) return LCU_UNSUPPORTED;
     if (cache_pages <= 0 || tasks_per_wg < 1 || lcu_attention_prefill_tokens_per_task(nh, nkvh) == 0 || page <= 0 || page % 16 || max_pages <= 0 ||
         window < 0 || q_stride % 8 || out_stride % 4 || nkvh * ((nh / nkvh + 15) / 16) > 65535)
         return LCU_BAD_ARGUMENT;
-#define GO(D) return launch_prefill<D>(q, q_stride, out, out_stride, cache, cache_pages, block_table, max_pages, q_start, ctx_len, task_req, task_tok0, n_tasks, tasks_per_wg, nh, nkvh, page, scale, window, stream)
+#define GO(D) return launch_prefill<D>(q, q_stride, out, out_stride, cache, cache_pages, block_table, max_pages, q_start, ctx_len, task_req, task_tok0, n_tasks, n_tasks_dev, tasks_per_wg, nh, nkvh, page, scale, window, stream)
     if (dh == 128) GO(128);
     if (dh == 64) GO(64);
     if (dh == 96) GO(96);

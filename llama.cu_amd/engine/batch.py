@@ -54,6 +54,15 @@ class StepContext:
     # the requests' indices, the one that holds most tokens first: the order in which the decode attention starts its
     # workgroups (those that walk the most keys must not start last)
     decode_order: Optional[torch.Tensor] = None
+    # who built the step, if its memory can take more arrays (``extra``)
+    builder: Optional["BatchBuilder"] = None
+
+    def extra(self, name: str, size: int):
+        """``(host, device)``: two int32 arrays of ``size`` entries under ``name`` in the step's own memory, for what
+        a part derives from the batch on the host before the step runs (``Part.prepare``): the host array goes to
+        the device with the batch's one copy, and the device array's address is the same in every step, so a
+        captured graph reads the new step's values.  None if the step was not made by a builder."""
+        return self.builder.extra(name, size) if self.builder is not None else None
 
     def block_table(self, group: int) -> torch.Tensor:
         return self.block_tables[group]
@@ -80,7 +89,9 @@ class BatchBuilder:
     never change (a captured graph can read them)."""
 
     def __init__(self, cache: CacheManager, max_tokens: int, max_reqs: int, max_pages: Sequence[int],
-                 device: torch.device):
+                 device: torch.device, extra_ints: Optional[int] = None):
+        """``extra_ints``: room for the arrays that parts add to a step (``StepContext.extra``); by default two
+        entries per token and eight per request."""
         self.cache = cache
         self.max_tokens, self.max_reqs = int(max_tokens), int(max_reqs)
         self.max_pages = [int(m) for m in max_pages]
@@ -90,6 +101,10 @@ class BatchBuilder:
                  ("q_start", r + 1), ("ctx_len", r), ("state_slot", r), ("feed_src", r), ("feed_dst", r), ("decode_order", r)]
         for g, mp in enumerate(self.max_pages):
             sizes += [(f"slots{g}", n), (f"block_table{g}", r * mp)]
+        self.extra_ints = int(extra_ints) if extra_ints is not None else 2 * n + 8 * r + 256
+        sizes.append(("extra", self.extra_ints))
+        self._extra_used = 0
+        self._extras = {}                       # name -> (offset in the extra area, size): the same in every step
         self.offsets = {}
         total = 0
         for name, size in sizes:
@@ -108,12 +123,35 @@ class BatchBuilder:
         o, s = self.offsets[name]
         return self.dev[o:o + count]
 
+    def extra(self, name: str, size: int):
+        """``(host, device)`` views of ``size`` entries that ``name`` owns from its first call on (the same
+        addresses in every step)."""
+        at = self._extras.get(name)
+        if at is None:
+            if self._extra_used + size > self.extra_ints:
+                raise ValueError(f"the step's memory has no room for {size} more entries under {name!r} "
+                                 f"({self._extra_used} of {self.extra_ints} are taken): build with a larger extra_ints")
+            at = self._extras[name] = (self._extra_used, int(size))
+            self._extra_used += (int(size) + 3) // 4 * 4
+        if at[1] < size:
+            raise ValueError(f"{name!r} holds {at[1]} entries, {size} were asked for")
+        o = self.offsets["extra"][0] + at[0]
+        return self.host[o:o + size], self.dev[o:o + size]
+
+    def upload(self) -> None:
+        """The step's arrays go to the device (one copy on the current stream)."""
+        self.dev.copy_(self.host, non_blocking=True)
+        if self.device.type == "cuda":
+            self._copied = torch.cuda.Event()
+            self._copied.record()
+
     def build(self, req_ids: Sequence[int], tokens: Sequence[Sequence[int]], want: Sequence[Sequence[int]],
-              vocab_size: int, feed: Sequence[tuple] = ()) -> StepContext:
+              vocab_size: int, feed: Sequence[tuple] = (), upload: bool = True) -> StepContext:
         """The batch in which request ``req_ids[i]`` feeds ``tokens[i]`` and wants the logits
         at the places ``want[i]`` among them.  The requests' pages must be reserved.
         ``feed``: pairs (row of the last step's sampled ids, request index here) for requests
-        whose last token here is a placeholder that the device fills in."""
+        whose last token here is a placeholder that the device fills in.  ``upload=False``: the
+        caller lets parts add their arrays (``StepContext.extra``) and calls ``upload`` then."""
         n_req = len(req_ids)
         n_new = [len(t) for t in tokens]
         n = sum(n_new)
@@ -154,10 +192,8 @@ class BatchBuilder:
                               self.max_pages, [ptr(f"slots{g}") for g in range(len(self.max_pages))])
         ctx_lens = self._h("ctx_len")[:n_req].tolist()
         self._h("decode_order")[:n_req] = torch.tensor(sorted(range(n_req), key=lambda i: -ctx_lens[i]), dtype=torch.int32)
-        self.dev.copy_(self.host, non_blocking=True)
-        if self.device.type == "cuda":
-            self._copied = torch.cuda.Event()
-            self._copied.record()
+        if upload:
+            self.upload()
         return StepContext(
             n=n, n_req=n_req, tokens=self._d("tokens", n), positions=self._d("positions", n),
             req_of_token=self._d("req_of_token", n), q_start=self._d("q_start", n_req + 1),
@@ -169,4 +205,4 @@ class BatchBuilder:
             state_slots=self._h("state_slot")[:n_req].tolist(),
             feed_src=self._d("feed_src", len(feed)) if feed else None,
             feed_dst=self._d("feed_dst", len(feed)) if feed else None,
-            decode_order=self._d("decode_order", n_req))
+            decode_order=self._d("decode_order", n_req), builder=self)

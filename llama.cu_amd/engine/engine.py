@@ -13,6 +13,7 @@ beyond an end-of-sequence token that was learned late is cut away again.  With
 """
 from __future__ import annotations
 
+import time
 from dataclasses import dataclass
 from typing import Callable, Dict, List, Optional, Sequence, Union
 
@@ -20,6 +21,7 @@ import torch
 
 from ..kernels import ops
 from ..sampling import GREEDY, Sampler, SamplingParams
+from .config import EngineConfig
 from .runner import ModelRunner
 from .scheduler import Scheduler
 
@@ -70,18 +72,34 @@ class Engine:
         self.requests: Dict[int, _Request] = {}
         self._next_id = 0
         self.steps = 0
+        # measurement (``timeline = []`` switches it on): per launched round the host's time from the plan to the
+        # last launch, the round's tokens and requests, whether it was replayed from a graph, and two events on
+        # the stream around its work (the gap between one round's last and the next one's first is a GPU that waits)
+        self.timeline: Optional[List[dict]] = None
 
     @classmethod
-    def from_folder(cls, folder: str, dtype: str = "bfloat16", device: str = "cuda:0",
-                    prefill_chunk: Optional[int] = None, run_ahead: bool = True, **runner_kw) -> "Engine":
-        return cls(ModelRunner.from_folder(folder, dtype=dtype, device=device, **runner_kw), prefill_chunk,
-                   run_ahead=run_ahead)
+    def from_folder(cls, folder: str, config: Optional[EngineConfig] = None, **fields) -> "Engine":
+        """The engine for a model folder.  ``config``: the engine's constants (``EngineConfig``); ``fields``
+        replace single ones (``dtype="float32", max_seqs=4, ...``)."""
+        ec = EngineConfig.of(config, **fields)
+        engine = cls(ModelRunner.from_folder(folder, **ec.runner_kwargs()), ec.prefill_chunk, run_ahead=ec.run_ahead)
+        engine.config = ec
+        return engine
 
     @classmethod
-    def from_config(cls, cfg, seed: int, dtype: str = "bfloat16", device: str = "cuda:0",
-                    prefill_chunk: Optional[int] = None, run_ahead: bool = True, **runner_kw) -> "Engine":
-        return cls(ModelRunner.from_config(cfg, seed, dtype=dtype, device=device, **runner_kw), prefill_chunk,
-                   run_ahead=run_ahead)
+    def from_config(cls, cfg, seed: int, config: Optional[EngineConfig] = None, std: float = 0.02, stored=None,
+                    **fields) -> "Engine":
+        """The engine for a model configuration with random weights made on the device from ``seed`` (``std``,
+        ``stored``: as in ``ModelRunner.from_config``)."""
+        ec = EngineConfig.of(config, **fields)
+        engine = cls(ModelRunner.from_config(cfg, seed, std=std, stored=stored, **ec.runner_kwargs()), ec.prefill_chunk,
+                     run_ahead=ec.run_ahead)
+        engine.config = ec
+        return engine
+
+    def export_weights(self):
+        """The model's weights by the names that files use, on the host (``ModelRunner.export_weights``)."""
+        return self.runner.export_weights()
 
     # ---------------------------------------------------------------- requests
     def add_request(self, tokens: Sequence[int], params: SamplingParams = GREEDY, max_steps: int = 1000,
@@ -150,9 +168,14 @@ class Engine:
     def _launch(self) -> Optional[_Flight]:
         """Plan and launch a round; the ids it samples stay on the device, and the requests
         get placeholders for them."""
+        t_plan = time.perf_counter()
         plan = self.sched.plan()
         if not plan:
             return None
+        first = None
+        if self.timeline is not None:
+            first = torch.cuda.Event(enable_timing=True)
+            first.record()
         before = self._flight
         row_of = {rid: i for i, rid in enumerate(before.rows)} if before is not None else {}
         ids, toks, want, feed = [], [], [], []
@@ -185,6 +208,11 @@ class Engine:
         host.copy_(sampled, non_blocking=True)
         copied = torch.cuda.Event()
         copied.record()
+        if first is not None:
+            last = torch.cuda.Event(enable_timing=True)
+            last.record()
+            self.timeline.append({"host_ms": (time.perf_counter() - t_plan) * 1e3, "tokens": step.n, "requests": step.n_req,
+                                  "graph": self.runner.last_run_was_replay, "first": first, "last": last})
         flight = _Flight([e.req for e in rows], [], [], [], [], sampled, host, copied)
         for e in rows:
             r = self.requests[e.req]

@@ -74,7 +74,7 @@ def engine_bytes(spec: ModelSpec, expected, dtype: torch.dtype, device, page_siz
     total += max(tokens, 0) * token_bytes
     widest = max([max(t.shape) for t in expected.values() if len(t.shape) == 2] + [1])
     total += 16 * int(max_batch_tokens) * widest * 4 + (256 << 20)        # a step's buffers and the library's workspace
-    return total
+    return total + total // 32                                             # and what the allocator's rounding adds
 
 
 def require_gpu(device) -> torch.device:
@@ -152,18 +152,31 @@ class ModelRunner:
             else:
                 group = pools.index(need.pool()) if need.pool() is not None else -1
                 pages, ps = (self.groups[group].num_pages, page_of[group]) if group >= 0 else (self.num_pages, self.page_size)
-                self.caches.append(need.allocate(group, pages, ps, self.max_seqs, self.dtype, self.device))
+                try:
+                    made = need.allocate(group, pages, ps, self.max_seqs, self.dtype, self.device)
+                except torch.cuda.OutOfMemoryError:
+                    # what torch's allocator holds without a tensor in it (the rest of a piece reserved for another
+                    # engine, say) goes back to the driver, and the allocation is tried once more
+                    torch.cuda.empty_cache()
+                    made = need.allocate(group, pages, ps, self.max_seqs, self.dtype, self.device)
+                self.caches.append(made)
         max_pages = [(self.max_model_len + g.page_size - 1) // g.page_size for g in self.groups]
         self.builder = BatchBuilder(self.cache, self.max_batch_tokens, self.max_seqs, max_pages, self.device)
         # a debugging aid: pages that were given back, or went to another request, since the last step are
         # filled with NaN before the step runs, so that a read of memory that its request does not own shows
         self.poison_freed = bool(poison_freed)
         self._owners: Optional[List[List[int]]] = None
-        # captured decode steps, by batch size: (graph, its logits tensor)
+        # captured steps: for steps of single tokens by batch size and key parts: (graph, its logits tensor)
         self.use_graphs = bool(use_graphs) and self.model.graph_safe
+        self.tensors: Dict[str, torch.Tensor] = tensors      # by the names that files use (views of the load's one allocation)
         self._graphs: Dict[tuple, Any] = {}        # (batch size, key parts) -> (graph, its logits)
         self._seen: Dict[tuple, int] = {}
         self.graph_replays: Dict[tuple, int] = {}  # how often each was replayed
+        self._step_graphs: Dict[tuple, Any] = {}   # the same for steps that are not all single tokens, by their sizes
+        self.step_graph_replays: Dict[tuple, int] = {}
+        self._last_use: Dict[tuple, int] = {}
+        self._clock = 0
+        self.last_run_was_replay = False
 
     # ------------------------------------------------------------ construction helpers
     @classmethod
@@ -185,6 +198,7 @@ class ModelRunner:
                                ignored=arch.ignored_tensors)
         runner = cls(spec, tensors, dtype, device, **kw)
         runner.config = cfg
+        runner.tensors = tensors
         return runner
 
     @classmethod
@@ -207,7 +221,13 @@ class ModelRunner:
         tensors = {n: convert(t, expected[n], DTYPES[dtype]) for n, t in tensors.items()}
         runner = cls(spec, tensors, dtype, device, **kw)
         runner.config = cfg
+        runner.tensors = tensors
         return runner
+
+    def export_weights(self) -> Dict[str, torch.Tensor]:
+        """The weights as the engine holds them, under the names that files use, copied to the host (for a
+        plain model in a test, or to write a folder with ``weights.write_safetensors``)."""
+        return {name: t.detach().to("cpu") for name, t in self.tensors.items()}
 
     # ------------------------------------------------------------ the step function
     def prepare(self, req_ids: Sequence[int], tokens: Sequence[Sequence[int]], want: Sequence[Sequence[int]],
@@ -236,7 +256,10 @@ class ModelRunner:
             raise
         if self.poison_freed:
             self._poison_pages_that_changed_hands()
-        return self.builder.build(req_ids, tokens, want, self.spec.vocab_size, feed)
+        step = self.builder.build(req_ids, tokens, want, self.spec.vocab_size, feed, upload=False)
+        self.model.prepare(step)                   # what the parts derive from the batch on the host joins the step's arrays
+        self.builder.upload()
+        return step
 
     def _poison_pages_that_changed_hands(self) -> None:
         """Called when a step's pages are reserved and nothing of it has run: every page that a request
@@ -255,25 +278,49 @@ class ModelRunner:
                 if c.group == g and c.writes and c.pages is not None:
                     c.pages.index_fill_(0, index, float("nan"))
 
-    GRAPH_AFTER = 2          # a batch size is captured when it comes for the third time
+    GRAPH_AFTER = 2          # a kind of step is captured when it comes for the third time
     GRAPH_MAX_BATCH = 256
+    GRAPH_MAX_TOKENS = 256   # steps that are not all single tokens are captured up to this many tokens (beyond, the
+                             # GPU's step takes far longer than the host's launches, and a graph would hold much memory)
+    GRAPH_MAX_KINDS = 64     # so many kinds of such steps are kept; the one replayed longest ago goes first
 
     def run(self, step: StepContext) -> torch.Tensor:
-        """The model on the batch.  A step in which every request decodes one token and
-        wants its logits is launch-bound, so such steps are captured per batch size into a
-        HIP graph and replayed: the batch arrays live at fixed device addresses (the
-        builder's buffer), so a replay reads the new step's tokens, positions and block
-        tables.  (The reference captures everything between two attentions per token-count
-        bucket, llama.cu/src/exec/step.rs:82-96; here the whole step is one graph.)"""
+        """The model on the batch.  Small steps are launch-bound (a step of the model is some two hundred to
+        four hundred launches), so they are captured into HIP graphs and replayed: the batch arrays, and what
+        the parts derive from them on the host (``Part.prepare``), live at fixed device addresses, so a replay
+        reads the new step's tokens, positions, block tables and task lists.  A graph fits every step with the same
+        sizes: for steps in which every request decodes one token the number of requests and the number of parts
+        into which the decode attention cuts the keys; for any other step (a prompt portion beside decoding
+        requests, say) the numbers of tokens, requests, single tokens and wanted rows, and what the parts' plans
+        say fixes their launches (``signature``).  (The reference captures everything between two attentions per
+        token-count bucket, llama.cu/src/exec/step.rs:82-96; here the whole step is one graph.)"""
         b = step.n_req
-        if not (self.use_graphs and step.decode_only and step.n_logits == b and b <= self.GRAPH_MAX_BATCH):
+        self.last_run_was_replay = False
+        if not self.use_graphs:
             return self.model.forward(step, self.caches)
-        # the number of key parts of the decode attention must not change between replays: a
-        # graph is made for a batch size and a number of parts (which follows the longest
-        # context rounded up to a power of two, so it changes rarely)
-        step.attn_splits = self._decode_splits(b, step.max_ctx_len)
-        key = (b, step.attn_splits)
-        entry = self._graphs.get(key)
+        if step.decode_only:
+            if not (step.n_logits == b and b <= self.GRAPH_MAX_BATCH):
+                return self.model.forward(step, self.caches)
+            # the number of key parts of the decode attention must not change between replays: a
+            # graph is made for a batch size and a number of parts (which follows the longest
+            # context rounded up to a power of two, so it changes rarely)
+            step.attn_splits = self._decode_splits(b, step.max_ctx_len)
+            return self._run_captured(self._graphs, (b, step.attn_splits), step, self.graph_replays)
+        if step.n > self.GRAPH_MAX_TOKENS:
+            return self.model.forward(step, self.caches)
+        plans = tuple(sorted((k, v.signature) for k, v in step.scratch.items() if hasattr(v, "signature")))
+        key = (step.n, b, step.n_logits, step.logits_all, plans)
+        logits = self._run_captured(self._step_graphs, key, step, self.step_graph_replays)
+        if len(self._step_graphs) > self.GRAPH_MAX_KINDS:
+            oldest = min((k for k in self._step_graphs if k != key), key=lambda k: self._last_use.get(k, 0))
+            del self._step_graphs[oldest]
+        return logits
+
+    def _run_captured(self, graphs: Dict[tuple, Any], key: tuple, step: StepContext, replays: Dict[tuple, int]) -> torch.Tensor:
+        """Replay the graph of ``key`` (capture it first if the key has come often enough; before that, run eagerly)."""
+        self._clock += 1
+        self._last_use[key] = self._clock
+        entry = graphs.get(key)
         if entry is None:
             self._seen[key] = self._seen.get(key, 0) + 1
             if self._seen[key] <= self.GRAPH_AFTER:
@@ -282,10 +329,11 @@ class ModelRunner:
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph):
                 logits = self.model.forward(step, self.caches)
-            entry = self._graphs[key] = (graph, logits)
+            entry = graphs[key] = (graph, logits)
         graph, logits = entry
         graph.replay()
-        self.graph_replays[key] = self.graph_replays.get(key, 0) + 1
+        self.last_run_was_replay = True
+        replays[key] = replays.get(key, 0) + 1
         return logits
 
     def _decode_splits(self, batch: int, max_ctx_len: int) -> int:

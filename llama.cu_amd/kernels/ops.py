@@ -397,16 +397,16 @@ def attention_decode(q, out, cache, block_table, q_start, ctx_len, n_req, n_head
     return out
 
 
-def prefill_tasks(q_lens, ctx_lens, tokens_per_task: int, device, skip_single: bool = False, per_wg: int = 1,
-                  window: int = 0):
-    """Cut the batch into the prefill kernel's tasks: (request index, first token) pairs.  Workgroups start in the
-    order of the list, two to a compute unit, and the card fills the compute units' first places in turn before their
-    second ones: so the longer half of the tasks (those that walk the most keys) comes first, longest first, and the
-    shorter half follows shortest first; a compute unit then holds a long task beside a short one, and the long ones
-    do not start last and leave the other compute units waiting for them.  (Against all tasks longest first: 60.4 ->
-    57.8 us for 2,048 tokens over 2k keys, 251.6 -> 242.7 us over 8k; a long and a short one in turns, or as one
-    workgroup's two tasks, was slower.)  ``per_wg`` tasks go to one workgroup, one after the other.  ``window``: a
-    task of a layer with a window walks no more keys than its tokens and the window."""
+def cut_into_tasks(q_lens, ctx_lens, tokens_per_task: int, skip_single: bool = False, window: int = 0):
+    """Cut the batch into the prefill kernel's tasks: (request index, first token) pairs, in the order in which the
+    workgroups should start.  Workgroups start in the order of the list, two to a compute unit, and the card fills
+    the compute units' first places in turn before their second ones: so the longer half of the tasks (those that
+    walk the most keys) comes first, longest first, and the shorter half follows shortest first; a compute unit then
+    holds a long task beside a short one, and the long ones do not start last and leave the other compute units
+    waiting for them.  (Against all tasks longest first: 60.4 -> 57.8 us for 2,048 tokens over 2k keys, 251.6 ->
+    242.7 us over 8k; a long and a short one in turns, or as one workgroup's two tasks, was slower.)  ``skip_single``:
+    requests that feed one token get no task (they go to the decode kernel).  ``window``: a task of a layer with a
+    window walks no more keys than its tokens and the window."""
     tasks = []
     start = 0
     for r, n in enumerate(q_lens):
@@ -417,25 +417,104 @@ def prefill_tasks(q_lens, ctx_lens, tokens_per_task: int, device, skip_single: b
             tasks.append((-keys, r, start + t))
         start += n
     tasks.sort()
-    if not tasks:
-        return None, None, 0, 1
     half = len(tasks) // 2
     tasks = tasks[:half] + tasks[half:][::-1]
-    both = to_device([[t[1] for t in tasks], [t[2] for t in tasks]], torch.int32, device)
+    return [(t[1], t[2]) for t in tasks]
+
+
+def prefill_tasks(q_lens, ctx_lens, tokens_per_task: int, device, skip_single: bool = False, per_wg: int = 1,
+                  window: int = 0):
+    """``cut_into_tasks`` as two arrays on the device, with their length; ``per_wg`` tasks go to one workgroup, one
+    after the other."""
+    tasks = cut_into_tasks(q_lens, ctx_lens, tokens_per_task, skip_single, window)
+    if not tasks:
+        return None, None, 0, 1
+    both = to_device([[t[0] for t in tasks], [t[1] for t in tasks]], torch.int32, device)
     return both[0], both[1], len(tasks), per_wg
 
 
 def attention_prefill(q, out, cache, block_table, q_start, ctx_len, task_req, task_tok0, n_tasks, tasks_per_wg, n_heads,
-                      n_kv_heads, head_dim, page_size, scale, window) -> torch.Tensor:
-    """Matrix-core attention for any mix of portions and single tokens."""
-    _i32(task_req, "task_req", n_tasks); _i32(task_tok0, "task_tok0", n_tasks)
+                      n_kv_heads, head_dim, page_size, scale, window, n_tasks_dev: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Matrix-core attention for any mix of portions and single tokens.  ``n_tasks_dev`` (int32 on the device, one
+    entry): the lists hold that many tasks, at most ``n_tasks``, for which the grid is made."""
+    if task_req.numel() < n_tasks or task_tok0.numel() < n_tasks:
+        raise KernelError(f"attention_prefill: the task lists hold fewer than {n_tasks} entries")
+    _i32(task_req, "task_req"); _i32(task_tok0, "task_tok0")
+    if n_tasks_dev is not None:
+        _gpu(n_tasks_dev)
+        _i32(n_tasks_dev, "n_tasks_dev")
     lib = build.load("attention_mfma")
     _check(lib.lcu_attention_prefill_bf16(_ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(cache),
                                           ctypes.c_longlong(cache.shape[0]), _ptr(block_table),
                                           block_table.shape[1], _ptr(q_start), _ptr(ctx_len), _ptr(task_req),
-                                          _ptr(task_tok0), n_tasks, tasks_per_wg, n_heads, n_kv_heads, head_dim, page_size,
-                                          ctypes.c_float(scale), int(window), _stream()), "attention_prefill")
+                                          _ptr(task_tok0), n_tasks, _ptr(n_tasks_dev), tasks_per_wg, n_heads, n_kv_heads, head_dim,
+                                          page_size, ctypes.c_float(scale), int(window), _stream()), "attention_prefill")
     return out
+
+
+class AttentionPlan:
+    """How the matrix-core kernels share out a step that is not all single tokens: the requests that feed one token go
+    to the decode kernel (``singles``: their indices, most keys first), every other request's tokens are cut into the
+    prefill kernel's tasks (``task_req``, ``task_tok0``; ``n_tasks`` on the device says how many).  The launches' sizes
+    (``max_tasks``, ``n_single``, ``single_splits``) follow from the step's sizes and the longest context rounded up to
+    a power of two; what the lists hold is data."""
+    __slots__ = ("task_req", "task_tok0", "n_tasks_dev", "max_tasks", "per_wg", "singles", "n_single", "single_splits")
+
+    @property
+    def signature(self):
+        """What fixes the launches that ``paged_attention`` makes with this plan: two steps with equal signatures are
+        served by the same recorded launches."""
+        return (self.max_tasks, self.per_wg, self.n_single, self.single_splits)
+
+
+def plan_attention(step, n_heads: int, n_kv_heads: int, window: int = 0) -> Optional[AttentionPlan]:
+    """The AttentionPlan of ``step`` for layers with these heads and this window (one per step and kind of layer,
+    kept in ``step.scratch``); None for a step of single tokens only, which needs none.  Called before the step's
+    arrays go to the device (``Part.prepare``) it lays its lists into the step's own memory (``step.extra``): their
+    addresses are then the same in every step, and launches recorded into a graph read the new step's lists.
+    Called later (a step made by hand) it brings its lists to the device itself."""
+    if step.decode_only:
+        return None
+    lib = build.load("attention_mfma")
+    tpt = lib.lcu_attention_prefill_tokens_per_task(n_heads, n_kv_heads)
+    if tpt <= 0:
+        return None
+    key = ("attention_plan", tpt, int(window))
+    plan = step.scratch.get(key)
+    if plan is not None:
+        return plan
+    singles = sorted((r for r, n in enumerate(step.q_lens) if n == 1), key=lambda r: -step.ctx_lens[r])    # most keys first
+    tasks = cut_into_tasks(step.q_lens, step.ctx_lens, tpt, skip_single=bool(singles), window=window)
+    plan = AttentionPlan()
+    plan.per_wg = 1
+    plan.n_single = len(singles)
+    # the most tasks that a step of these sizes can have: a request of q tokens has at most q / tpt + 1
+    plan.max_tasks = (step.n - len(singles)) // tpt + (step.n_req - len(singles))
+    plan.single_splits = decode_splits(len(singles), n_heads, n_kv_heads, max([step.ctx_lens[r] for r in singles], default=0)) if singles else 1
+    builder = getattr(step, "builder", None)
+    if builder is not None:
+        cap_tasks = builder.max_tokens // tpt + builder.max_reqs
+        host, dev = step.extra(f"attention/{tpt}/{int(window)}", 4 + 2 * cap_tasks + builder.max_reqs)
+        host[0] = len(tasks)
+        if tasks:
+            host[4:4 + len(tasks)] = torch.tensor([t[0] for t in tasks], dtype=torch.int32)
+            host[4 + cap_tasks:4 + cap_tasks + len(tasks)] = torch.tensor([t[1] for t in tasks], dtype=torch.int32)
+        if singles:
+            host[4 + 2 * cap_tasks:4 + 2 * cap_tasks + len(singles)] = torch.tensor(singles, dtype=torch.int32)
+        plan.n_tasks_dev = dev[0:1]
+        plan.task_req = dev[4:4 + cap_tasks]
+        plan.task_tok0 = dev[4 + cap_tasks:4 + 2 * cap_tasks]
+        plan.singles = dev[4 + 2 * cap_tasks:4 + 2 * cap_tasks + len(singles)] if singles else None
+    else:
+        room = max(plan.max_tasks, 1)
+        flat = to_device([len(tasks)] + [t[0] for t in tasks] + [0] * (room - len(tasks)) + [t[1] for t in tasks]
+                         + [0] * (room - len(tasks)) + singles, torch.int32, step.tokens.device)
+        plan.n_tasks_dev = flat[0:1]
+        plan.task_req = flat[1:1 + room]
+        plan.task_tok0 = flat[1 + room:1 + 2 * room]
+        plan.singles = flat[1 + 2 * room:] if singles else None
+    step.scratch[key] = plan
+    return plan
 
 
 def decode_splits(n_req: int, n_heads: int, n_kv_heads: int, max_ctx_len: int) -> int:
@@ -483,23 +562,13 @@ def paged_attention(q: torch.Tensor, out: torch.Tensor, cache: torch.Tensor, ste
                                 page_size, scale, window, splits, req_list=step.decode_order)
     # a mixed batch: the requests that decode one token go to the decode kernel, the portions
     # to the prefill kernel (each would be slow at the other's work)
-    lib = build.load("attention_mfma")
-    tpt = lib.lcu_attention_prefill_tokens_per_task(n_heads, n_kv_heads)
-    key = ("attention_tasks", tpt, int(window))
-    if key not in step.scratch:
-        singles = sorted((r for r, n in enumerate(step.q_lens) if n == 1), key=lambda r: -step.ctx_lens[r])    # most keys first
-        use_decode = len(singles) >= 1
-        tasks = prefill_tasks(step.q_lens, step.ctx_lens, tpt, q.device, skip_single=use_decode, window=window)
-        req_list = to_device(singles, torch.int32, q.device) if use_decode else None
-        max_ctx = max([step.ctx_lens[r] for r in singles], default=0)
-        step.scratch[key] = (tasks, req_list, len(singles) if use_decode else 0, max_ctx)
-    (task_req, task_tok0, n_tasks, per_wg), req_list, n_single, max_ctx = step.scratch[key]
-    if n_single:
-        attention_decode(q, out, cache, bt, step.q_start, step.ctx_len, n_single, n_heads, n_kv_heads, head_dim, page_size,
-                         scale, window, decode_splits(n_single, n_heads, n_kv_heads, max_ctx), req_list=req_list)
-    if n_tasks:
-        attention_prefill(q, out, cache, bt, step.q_start, step.ctx_len, task_req, task_tok0, n_tasks, per_wg, n_heads,
-                          n_kv_heads, head_dim, page_size, scale, window)
+    plan = plan_attention(step, n_heads, n_kv_heads, window)
+    if plan.n_single:
+        attention_decode(q, out, cache, bt, step.q_start, step.ctx_len, plan.n_single, n_heads, n_kv_heads, head_dim, page_size,
+                         scale, window, plan.single_splits, req_list=plan.singles)
+    if plan.max_tasks:
+        attention_prefill(q, out, cache, bt, step.q_start, step.ctx_len, plan.task_req, plan.task_tok0, plan.max_tasks,
+                          plan.per_wg, n_heads, n_kv_heads, head_dim, page_size, scale, window, n_tasks_dev=plan.n_tasks_dev)
     return out
 
 

@@ -80,6 +80,15 @@ class Attention(Part):
                 ops.say_once(f"attention with {self.heads} heads of {self.head_dim} in {self.kv_heads} groups runs on the generic "
                              f"kernel, not on the matrix cores: {why}")
 
+    def prepare(self, step) -> None:
+        """The lists by which the matrix-core kernels share out a step that is not all single tokens are made here, on
+        the host, and go to the device with the step's arrays; ``forward`` then launches work whose sizes follow from
+        the step's sizes alone."""
+        page_size = self.own_page_size or self.page_size
+        if self.dtype == torch.bfloat16 and self.position.score_slopes() is None \
+                and ops.mfma_attention_refusal(self.dtype, self.heads, self.kv_heads, self.head_dim, page_size) is None:
+            ops.plan_attention(step, self.heads, self.kv_heads, self.window)
+
     # forward(..., into=(residual, norm)) may end with the residual sum and that norm's weight
     # in the output projection and return ScaledRows instead of the branch's output
     ends_in_norm = True

@@ -228,6 +228,13 @@ class Part:
     def load(self, tensors: Dict[str, torch.Tensor], build: BuildContext) -> None:
         pass
 
+    def prepare(self, step) -> None:
+        """Called once per step for every layer, on the host, before the step's arrays go to the device and
+        before anything of the step runs or is replayed from a graph: a part that derives arrays from the batch
+        (lists of tasks, orders) writes them into ``step.extra(name, size)`` here, so that its ``forward`` launches
+        work whose shape depends on the step's sizes alone and a graph-safe part stays one."""
+        pass
+
     def fused_groups(self, dtype: torch.dtype, device: torch.device) -> List[Tuple[Tuple[str, ...], int]]:
         """Tensors that this part multiplies as one matrix: ``[(names in row order, rows to which each
         is filled up with zeros, or 0)]``.  The weight loader lays such tensors out one after the other,

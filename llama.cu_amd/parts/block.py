@@ -51,6 +51,10 @@ class PreNormBlock(Part):
     def cache_need(self):
         return self.mixer.cache_need()
 
+    def prepare(self, step) -> None:
+        for _, part in self._children():
+            part.prepare(step)
+
     def decode_splits(self, batch: int, max_ctx_len: int) -> int:
         return int(self.mixer.decode_splits(batch, max_ctx_len))
 

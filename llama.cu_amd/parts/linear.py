@@ -117,7 +117,8 @@ def library_friendly_rows(di: int, d: int, device) -> int:
     if key not in _friendly_rows:
         free, _ = torch.cuda.mem_get_info(device)
         if free < 4 * (2 * (di + 4096) * d * 2):
-            return di                               # no room to try (and none to spare for rows of zeros)
+            _friendly_rows[key] = di                # no room to try (and none to spare for rows of zeros): decided once, so
+            return di                               # that the loader's layout and the part's agree
         x = torch.randn(2048, d, device=device, dtype=torch.bfloat16)
         times = {}
         for rows in sorted({di} | {-(-di // m) * m for m in (1024, 2048, 4096)}):

@@ -132,6 +132,11 @@ class DecoderModel:
         return needs
 
     # ---- one step
+    def prepare(self, step) -> None:
+        """What the parts derive from the batch on the host (``Part.prepare``), before the step runs."""
+        for layer in self.layers:
+            layer.prepare(step)
+
     def forward(self, step, caches) -> torch.Tensor:
         """Logits ``[len(step.logit_rows), vocab]`` (float32) for the batch ``step``;
         ``caches[i]`` is the cache of run-order entry ``i``."""

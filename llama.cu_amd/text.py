@@ -50,19 +50,26 @@ class StreamDecoder:
     """Turns tokens into text piece by piece; bytes of a character that is not yet whole
     are held back (the reference's ``TextBuf``, llama.cu/xtask/src/generate.rs:44,56)."""
 
+    # how many tokens before the pending ones are decoded along with them: a tokenizer may render a token
+    # differently after another (a leading space), so a piece is what a short context adds to its rendering
+    CONTEXT = 8
+
     def __init__(self, tokenizer):
         self.tokenizer = tokenizer
         self.ids: List[int] = []
-        self.shown = ""
+        self.done = 0                  # tokens whose text has been handed out
 
     def push(self, token: int) -> str:
+        """The text that ``token`` completes ("" while a character's bytes are not all there).  Only the last few
+        tokens are decoded, not the whole sequence so far."""
         self.ids.append(token)
-        text = self.tokenizer.decode(self.ids)
-        if text.endswith("�"):
+        start = max(self.done - self.CONTEXT, 0)
+        before = self.tokenizer.decode(self.ids[start:self.done])
+        text = self.tokenizer.decode(self.ids[start:])
+        if text.endswith("�") and len(self.ids) - self.done < 8:
             return ""
-        piece = text[len(self.shown):]
-        self.shown = text
-        return piece
+        self.done = len(self.ids)
+        return text[len(before):] if text.startswith(before) else text
 
 
 DEFAULT_TEMPLATE = ("{% for message in messages %}{{ message['role'] + ': ' + message['content'].strip() + '\\n' }}"

@@ -175,3 +175,20 @@ def test_a_module_of_the_user_s_registers_an_architecture_for_the_command_line(t
     # a module that cannot be imported is named
     with pytest.raises(ConfigError, match="no_such_module_anywhere"):
         load_plugins(["no_such_module_anywhere"])
+
+
+def test_the_engines_constants_are_one_typed_record():
+    """``EngineConfig``: defaults, replacement of single fields, and errors that name the field."""
+    from llama_cu_amd import EngineConfig
+    base = EngineConfig()
+    assert (base.dtype, base.page_size, base.max_batch_tokens, base.run_ahead) == ("bfloat16", 16, 2048, True)
+    ec = EngineConfig.of(base, dtype="float32", page_size=32, max_tokens=4096, prefill_chunk=48)
+    assert ec.page_size == 32 and ec.runner_kwargs()["max_tokens"] == 4096 and "num_pages" not in ec.runner_kwargs()
+    assert "prefill_chunk" not in ec.runner_kwargs() and "run_ahead" not in ec.runner_kwargs()
+    for bad, word in ((dict(page_size=12), "page_size"), (dict(dtype="float16"), "dtype"), (dict(max_seqs=0), "max_seqs"),
+                      (dict(num_pages=4, max_tokens=64), "num_pages"), (dict(kv_fraction=1.5), "kv_fraction"),
+                      (dict(prefill_chunk=-1), "prefill_chunk")):
+        with pytest.raises(ValueError, match=word):
+            EngineConfig.of(**bad)
+    with pytest.raises(TypeError, match="page_sise"):
+        EngineConfig.of(page_sise=16)

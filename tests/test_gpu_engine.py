@@ -315,6 +315,52 @@ def test_captured_decode_steps_equal_eager_ones():
         assert torch.equal(a, b), f"decode step {i} differs between eager and captured"
 
 
+@pytest.mark.parametrize("name", ["B", "D"])
+def test_captured_steps_with_a_prompt_portion_beside_decoding_requests_equal_eager_ones(name):
+    """Steps that are not all single tokens are captured too, by their sizes: three requests decode while a fourth
+    feeds five tokens of its prompt (a new request in some steps, the next portion of a long one in others, so the
+    lists of the attention kernels' tasks, the contexts and the pages differ from replay to replay while the sizes
+    stay).  Every replay gives the bits of the eager step, with eager work and synchronisations in between."""
+    from llama_cu_amd.engine.runner import ModelRunner
+    cfg = common.TINY[name]
+    vocab = cfg["vocab_size"]
+    folder = common.make_folder(cfg, seed=35, dtype=torch.bfloat16, std=common.BF16_STD)
+    reqs = list(common.random_requests(vocab, [9, 40, 33], seed=8).values())
+    rng = np.random.default_rng(1)
+    plan = []
+    for i in range(14):
+        singles = [[int(rng.integers(vocab))] for _ in range(3)]
+        portion = [int(t) for t in rng.integers(vocab, size=5)]
+        plan.append((singles, portion, i % 3 == 2))               # every third step: a new request's first tokens
+
+    def run(use_graphs):
+        runner = ModelRunner.from_folder(folder, dtype="bfloat16", max_tokens=1024, max_seqs=6, use_graphs=use_graphs,
+                                         page_size={"B": 32, "D": 16}[name])
+        runner.step([0, 1, 2], reqs)
+        outs, fresh = [], 100
+        for i, (singles, portion, new) in enumerate(plan):
+            if new:
+                rid, fresh = fresh, fresh + 1
+            else:
+                rid = 3                                           # the long request goes on: its history grows by five a step
+            ids, toks = [0, 1, rid, 2], [singles[0], singles[1], portion, singles[2]]
+            outs.append(runner.step(ids, toks, [[0], [0], [1, 4], [0]]).float().cpu())
+            if new:
+                runner.end(rid)
+            if i == 7:                                            # eager work between replays: another kind of step
+                runner.step([50], [[1, 2, 3]])
+                runner.end(50)
+            torch.cuda.synchronize()
+        return outs, runner
+
+    eager, _ = run(False)
+    graphed, runner = run(True)
+    assert len(runner._step_graphs) == 1 and sum(runner.step_graph_replays.values()) == len(plan) - 2, runner.step_graph_replays
+    for i, (a, b) in enumerate(zip(eager, graphed)):
+        assert torch.isfinite(a).all() and a.shape == (5, vocab)
+        assert torch.equal(a, b), f"step {i} differs between eager and captured"
+
+
 def test_the_packed_copy_of_the_weights_changes_no_logit():
     """With and without the second copy of the matrices in the decode kernels' order the
     model gives the same bits, prompt and decoding; the copy is made by default where the
