@@ -713,37 +713,27 @@ __device__ __forceinline__ const u32x4 *lane_values(const u32x4 *buf, int n, int
 template <int DH>
 __device__ __forceinline__ const u32x4 *lane_keys(const u32x4 *buf, int n, int hi) { return buf + (n >> 4) * 2 * DH + hi * 16 + (n & 15); }
 
-__device__ __forceinline__ uint32_t lds_address(const void *p) {
-    return (uint32_t)(__SIZE_TYPE__)(__attribute__((address_space(3))) const void *)p;
-}
-
 // f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>): a loop whose index is a constant in its body.
 template <int... I, class F>
 __device__ __forceinline__ void static_for_impl(std::integer_sequence<int, I...>, F &&f) { (f(std::integral_constant<int, I>{}), ...); }
 template <int N, class F>
 __device__ __forceinline__ void static_for(F &&f) { static_for_impl(std::make_integer_sequence<int, N>{}, f); }
 
-// The 16 bytes at LDS address `addr` + OFF into the registers of `r`, as an instruction of its own: `r` is
-// read and written ("+v"), so the read stands behind every instruction that uses the old contents and takes
-// no registers of its own (as a plain load the compiler read into new registers, all at once and early, and
-// copied them over at the end of every turn).  The compiler does not know that the data is still on its way:
-// NOTHING may touch `r` before operands_arrived().
-template <int OFF>
-__device__ __forceinline__ void lds_read_in_place(u32x4 &r, uint32_t addr) {
-    static_assert(OFF >= 0 && OFF < 65536 && OFF % 16 == 0, "the instruction's offset has 16 bits");
-    asm volatile("ds_read_b128 %0, %1 offset:%2" : "+v"(r) : "v"(addr), "n"(OFF));
+// Chunk CHUNK behind `from` in LDS into the registers of `r`: an ordinary load, which the compiler waits for where the
+// register is used, by its own count.  The fence keeps the load where it stands, behind the instruction that used the
+// register's old contents: the old and the new value then never live at once, and the register allocator gives both
+// the same register (without the fence the scheduler read all keys early into new registers and copied them over at
+// the end of every turn, 24 copies a turn).  `from` is derived from a __restrict__ parameter of the function that also
+// issues the copies into LDS, so the read does not wait for them (through an integer address the compiler put a wait
+// for every copy in flight before the reads).
+template <int CHUNK>
+__device__ __forceinline__ void lds_read_plain(u32x4 &r, const u32x4 *from) {
+    r = from[CHUNK];
+    __builtin_amdgcn_sched_barrier(0);
 }
 
-// Waits until at most LEFT of the wave's reads from LDS are on their way (they arrive in the order in which
-// they were issued; scalar loads in flight count with them, which makes the wait longer, never shorter),
-// and says that the operands are defined here: nothing that uses them moves above.
-template <int LEFT, int N>
-__device__ __forceinline__ void operands_arrived(u32x4 (&r)[N]) {
-    static_assert(LEFT >= 0 && LEFT < 16, "lgkmcnt has four bits");
-    __builtin_amdgcn_s_waitcnt(0xc07f | (LEFT << 8));          // vmcnt and expcnt: no wait
-#pragma unroll
-    for (int i = 0; i < N; ++i) asm volatile("" : "+v"(r[i]));
-}
+// Nothing that uses the operands read so far moves above this point, and nothing that stands above moves below.
+__device__ __forceinline__ void operands_fence() { __builtin_amdgcn_sched_barrier(0); }
 
 // One turn of a wave: the output of step e - 1 and the scores and the softmax of step e, 32 keys each, for
 // the wave's 32 rows.
@@ -784,10 +774,10 @@ __device__ __forceinline__ void attn_turn(const u32x4 *__restrict__ next, u32x4 
     // the values of step e - 1: on their way during the scores' matrix instructions (they stand before the
     // branch below, in a block of their own: in one block with the matrix instructions the compiler's
     // scheduler put them behind most of those, and the wait for them was 5 % of the kernel's time)
-    const uint32_t ka = lds_address(lane_keys<DH>(next, n, hi)), va = lds_address(lane_values<DH>(next, n, hi));
+    const u32x4 *ka = lane_keys<DH>(next, n, hi), *va = lane_values<DH>(next, n, hi);
     static_for<2 * (DH / 32)>([&](auto i) {
         constexpr int kk = decltype(i)::value / (DH / 32), t = decltype(i)::value % (DH / 32);
-        lds_read_in_place<(kk * 2 * DH + 32 * t) * 16>(v[decltype(i)::value], va);
+        lds_read_plain<kk * 2 * DH + 32 * t>(v[decltype(i)::value], va);
     });
     // the output so far goes over to the reference point that the turn before has chosen (here, and not where
     // that turn made the factor: a branch behind the softmax would cut it off the block of the matrix
@@ -804,10 +794,10 @@ __device__ __forceinline__ void attn_turn(const u32x4 *__restrict__ next, u32x4 
     static_for<DH / 16>([&](auto i) {
         constexpr int sidx = decltype(i)::value;
         s = mfma32(k[sidx], q[sidx], s);
-        lds_read_in_place<32 * 16 * sidx>(k[sidx], ka);            // the keys of step e + 1
+        lds_read_plain<32 * sidx>(k[sidx], ka);                    // the keys of step e + 1
     });
-    operands_arrived<DH / 16>(v);                  // all but the reads of the keys, which came later
-    ask_pages();                                   // (scalar loads: behind the wait, which they would make longer)
+    operands_fence();
+    ask_pages();                                   // (scalar loads: behind the matrix instructions and the reads from LDS)
     if (maskv) {
 #pragma unroll
         for (int kk = 0; kk < 2; ++kk) {
@@ -841,7 +831,7 @@ __device__ __forceinline__ void attn_turn(const u32x4 *__restrict__ next, u32x4 
     // the keys of the next turn: here rather than at the turn's end (it costs nothing: the other workgroup's
     // waves have work), so that the long block below, where registers are scarce, is outside the stretch
     // in which the keys' registers may not be touched
-    operands_arrived<0>(k);
+    operands_fence();
     // the output's matrix instructions stand here, beside the softmax that does not need them: the
     // compiler's scheduler puts vector instructions between them (its own mix was the fastest: with ten
     // vector instructions forced behind each matrix instruction the kernel was 11 % slower, with all the

@@ -129,31 +129,6 @@ def _compiler(name: str) -> str:
     return hipcc
 
 
-# Kernels that read into registers with instructions of their own, which the compiler does not know to be
-# on their way: a register that the compiler saved to memory in between would be saved with its old
-# contents.  Such a kernel must be compiled without any spill (its resource report says so), or the build fails.
-NO_SPILL_KERNELS = {"attention_mfma": ("attention_prefill_kernel",)}
-
-
-def _check_no_spill(name: str, log: str) -> None:
-    """Reads the compiler's resource report (-Rpass-analysis=kernel-resource-usage) in ``log``."""
-    import re
-    current, seen = None, 0
-    for line in log.splitlines():
-        m = re.search(r"Function Name: (\S+)", line)
-        if m:
-            current = m.group(1)
-            continue
-        m = re.search(r"ScratchSize \[bytes/lane\]: (\d+)", line)
-        if m and current and any(k in current for k in NO_SPILL_KERNELS[name]):
-            seen += 1
-            if int(m.group(1)) != 0:
-                raise BuildError(f"{name}: the kernel {current} was compiled with {m.group(1)} bytes of spilled registers per "
-                                 "lane; it reads into registers behind the compiler's back and must not spill")
-    if seen == 0:
-        raise BuildError(f"{name}: the compiler's resource report names none of {NO_SPILL_KERNELS[name]}")
-
-
 def build(name: str, force: bool = False) -> str:
     """Compile one library if it is missing (or always with ``force``); returns its path."""
     out = library_path(name)
@@ -162,7 +137,7 @@ def build(name: str, force: bool = False) -> str:
     cc = _compiler(name)
     flags = HOST_FLAGS if name == HOST_LIBRARY else HIP_FLAGS
     tmp = f"{out}.tmp{os.getpid()}"
-    cmd = [cc] + flags + (["-Rpass-analysis=kernel-resource-usage"] if name in NO_SPILL_KERNELS else []) + ["-o", tmp] + _sources(name)
+    cmd = [cc] + flags + ["-o", tmp] + _sources(name)
     env = dict(os.environ)
     env.setdefault("HOME", tempfile.gettempdir())      # hipcc wants a home for its caches
     t0 = time.time()
@@ -183,12 +158,6 @@ def build(name: str, force: bool = False) -> str:
         if os.path.exists(tmp):
             os.remove(tmp)
         raise BuildError(f"building {name} failed ({' '.join(cmd)}):\n{log}")
-    if name in NO_SPILL_KERNELS:
-        try:
-            _check_no_spill(name, log)
-        except BuildError:
-            os.remove(tmp)
-            raise
     os.replace(tmp, out)
     # older builds of the same library are of no use any more
     for f in os.listdir(os.path.dirname(out)):
