@@ -130,6 +130,49 @@ def run_prefill(engine, cfg, rng, sync, repeats=3, history=0):
     return best
 
 
+def run_first_token(engine, cfg, n_requests, prompt_len, rng, sync, repeats=4):
+    """Time to the first token: ``n_requests`` requests with prompts of ``prompt_len`` tokens arrive together at an
+    idle engine; the time until every one of them has its first token on the host (the reference's own headline,
+    llama.cu/xtask/src/generate.rs:41-52: its "prefill" is the time until the first token was received).  The best
+    of ``repeats`` (the first ones build, load and capture)."""
+    from llama_cu_amd.sampling import GREEDY
+    best = None
+    for _ in range(repeats):
+        prompts = [[rng.randrange(cfg.vocab_size) for _ in range(prompt_len)] for _ in range(n_requests)]
+        sync()
+        t0 = time.perf_counter()
+        ids = [engine.add_request(p, GREEDY, max_steps=1, ignore_eos=True) for p in prompts]
+        got = 0
+        while got < n_requests:
+            got += sum(1 for o in engine.step() if o.token is not None)
+        dt = time.perf_counter() - t0
+        while not engine.idle:
+            engine.step()
+        for i in ids:
+            engine.drop(i)
+        best = dt if best is None else min(best, dt)
+    return best
+
+
+def run_prefill_step(engine, cfg, n_requests, prompt_len, rng, sync, repeats=4):
+    """Best time of ONE step that holds the whole prompts of ``n_requests`` requests, ``prompt_len`` tokens each
+    (many short tasks for the prefill attention)."""
+    best = None
+    for k in range(repeats):
+        ids = [20_000 + k * n_requests + i for i in range(n_requests)]
+        toks = [[rng.randrange(cfg.vocab_size) for _ in range(prompt_len)] for _ in ids]
+        sync()
+        t0 = time.perf_counter()
+        engine.runner.step(ids, toks)
+        sync()
+        dt = time.perf_counter() - t0
+        for i in ids:
+            engine.runner.end(i)
+        if k > 0:
+            best = dt if best is None else min(best, dt)
+    return best
+
+
 def run_mixed(engine, cfg, n_requests, rng, sync, new_tokens=128, lo=16, hi=2048):
     """A mixed batch (the workload that goes with the Llama-2-7B shape): ``n_requests`` requests at once, prompt
     lengths uniform in [lo, hi], ``new_tokens`` greedy tokens each, through the scheduler under its
@@ -244,28 +287,31 @@ def library_product(cfg, sync, calls=400):
     return out
 
 
-def kernel_summary(db: str, steps: int) -> int:
+def kernel_summary(db: str, steps: int, launches: int = 0) -> int:
     """Per-step table of kernels from the database that ``rocprofv3 --kernel-trace`` wrote for a
     run of this program: the kernels between two embedding gathers are one step of the model;
-    the last ``steps`` steps are averaged."""
+    the last ``steps`` steps are averaged (with ``launches``: the last ``steps`` steps of exactly that
+    many kernel launches, to tell the kinds of steps of a mixed workload apart)."""
     import re
     import sqlite3
     con = sqlite3.connect(db)
     rows = con.execute("select name, start, end from kernels order by start").fetchall()
     marks = [i for i, r in enumerate(rows) if "embedding_gather" in r[0]]
-    if len(marks) < steps + 1:
-        print(f"bench.py: {db} holds {len(marks)} steps, fewer than the {steps + 1} needed")
+    spans = [(a, b) for a, b in zip(marks[:-1], marks[1:]) if not launches or b - a == launches]
+    if len(spans) < steps:
+        kinds = sorted({b - a for a, b in zip(marks[:-1], marks[1:])})
+        print(f"bench.py: {db} holds {len(spans)} such steps, fewer than the {steps} needed (launches a step: {kinds})")
         return 1
-    sel = marks[-(steps + 1):]
+    spans = spans[-steps:]
     agg = {}
-    for a, b in zip(sel[:-1], sel[1:]):
+    for a, b in spans:
         for name, t0, t1 in rows[a:b]:
             short = re.sub(r"\(.*", "", name).replace("void ", "")
             short = re.sub(r"_SN_LDSB.*", "", short)[:70]
             item = agg.setdefault(short, [0, 0.0])
             item[0] += 1
             item[1] += (t1 - t0) / 1e3
-    wall = (rows[sel[-1]][1] - rows[sel[0]][1]) / 1e3 / steps
+    wall = sum(rows[b][1] - rows[a][1] for a, b in spans) / 1e3 / steps
     busy = sum(v[1] for v in agg.values()) / steps
     print(f"steps averaged: {steps}; wall {wall:.1f} us/step, kernels busy {busy:.1f} us/step\n")
     print("| kernel | launches/step | us/step | avg us | % of busy |")
@@ -295,6 +341,10 @@ def main() -> int:
                          "decode while a prompt of 16 tokens arrives every second step (host time and the GPU's busy "
                          "fraction per kind of step)")
     ap.add_argument("--no-points", action="store_true", help="skip decoding at batch 1 and 64 and the prefill")
+    ap.add_argument("--points", choices=["default", "all"], default="default",
+                    help="all: beside decoding at batch 1 and 64 also the time to the first token at 1 and 8 requests for "
+                         "prompts of 16, 128, 512 and 8192 tokens, one prefill step of 16 prompts of 128 tokens and of 64 of "
+                         "32, and decoding at 256 requests over 512 keys")
     ap.add_argument("--only-prefill", action="store_true", help="time the 2048-token prefill alone (for profiles)")
     ap.add_argument("--prefill-history", type=int, default=0,
                     help="with --only-prefill: time the 2048 tokens that follow this many tokens of the same prompt")
@@ -302,9 +352,11 @@ def main() -> int:
                     help="time the library's gate/up product of 2048 rows with random rows and with rows of zeros, and exit")
     ap.add_argument("--kernel-summary", metavar="DB", help="print the per-step kernel table of a rocprofv3 database and exit")
     ap.add_argument("--summary-steps", type=int, default=8)
+    ap.add_argument("--summary-launches", type=int, default=0,
+                    help="with --kernel-summary: only steps of exactly this many kernel launches (0: all)")
     args = ap.parse_args()
     if args.kernel_summary:
-        return kernel_summary(args.kernel_summary, args.summary_steps)
+        return kernel_summary(args.kernel_summary, args.summary_steps, args.summary_launches)
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported (no multi-GPU path)")
         return 2
@@ -320,7 +372,7 @@ def main() -> int:
     if args.layers:
         shape["num_hidden_layers"] = args.layers
     grow = args.steps + args.warmup + 2 * max(args.batch, 64) * rounds_of(args.prompt_len) + 64
-    need_ctx = max(args.prompt_len + grow + 64, args.prefill_history + PREFILL_TOKENS)
+    need_ctx = max(args.prompt_len + grow + 64, args.prefill_history + PREFILL_TOKENS, 8192 + 64 if args.points == "all" else 0)
     while shape["max_position_embeddings"] < need_ctx:
         shape["max_position_embeddings"] *= 2
     cfg = LlamaConfig.from_dict(shape)
@@ -333,7 +385,8 @@ def main() -> int:
         print(json.dumps({"library_product": library_product(cfg, sync), "rows": PREFILL_TOKENS,
                           "in": cfg.hidden_size, "out": 2 * cfg.intermediate_size, "dtype": "bf16"}))
         return 0
-    biggest = max(args.batch, 1 if (args.no_points or args.only_prefill or args.workload != "decode") else 64)
+    all_points = args.points == "all" and not args.no_points
+    biggest = max(args.batch, 1 if (args.no_points or args.only_prefill or args.workload != "decode") else (256 if all_points else 64))
     # a request decodes while later ones still prefill: room for that too
     per_req = max(args.prompt_len, PROMPT_LEN) + grow
     engine = Engine.from_config(cfg, seed=0, dtype=args.dtype, page_size=page,
@@ -402,6 +455,15 @@ def main() -> int:
         for b in (1, 64):
             s, p, _ = run_decode(engine, cfg, b, max(16, args.steps // 4), 4, rng, sync)
             points[f"decode_b{b}"] = round(p / s, 2)
+        if all_points:
+            s, p, _ = run_decode(engine, cfg, 256, max(16, args.steps // 4), 4, rng, sync, prompt_len=512)
+            points["decode_b256_ctx512"] = round(p / s, 2)
+            for b in (1, 8):
+                for n in (16, 128, 512, 8192):
+                    points[f"first_token_ms_b{b}_prompt{n}"] = round(run_first_token(engine, cfg, b, n, rng, sync) * 1e3, 3)
+            for b, n in ((16, 128), (64, 32)):
+                t = run_prefill_step(engine, cfg, b, n, rng, sync)
+                points[f"prefill_step_ms_{b}x{n}"] = round(t * 1e3, 3)
         line["points"] = points
     print(json.dumps(line), flush=True)
     return 0
