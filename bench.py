@@ -260,6 +260,41 @@ def run_arrivals(engine, cfg, batch, steps, rng, sync, every=2, arrival_len=16, 
                       for (t, r, g), (n, h, u) in sorted(kinds.items())]}
 
 
+def check_against_float32(engine, cfg, rng, sync, prompt_len=48, decode_steps=6):
+    """The benchmarked bfloat16 model against the true 32-bit path with the same weights, at the benchmark's full depth:
+    a prompt in one step (logits at every position) and some single-token steps after it, through both runners.  The
+    32-bit path is the one that the tests hold against the plain implementation; here it says whether the bfloat16
+    kernels that were just timed still compute the model.  Returns the largest difference of a logit as a fraction of
+    the largest logit, the root mean square difference as a fraction of the logits' root mean square, and how many of
+    the positions agree on the arg-max."""
+    import torch
+    from llama_cu_amd.engine.runner import ModelRunner
+    ref = ModelRunner.from_config(cfg, seed=0, dtype="float32", stored="bfloat16", page_size=16, max_tokens=256, max_seqs=2,
+                                  max_batch_tokens=256, one_piece=False)
+    toks = [rng.randrange(cfg.vocab_size) for _ in range(prompt_len)]
+    rid = 30_000
+    want = list(range(prompt_len))
+    a = engine.runner.step([rid], [toks], [want])
+    b = ref.step([rid], [toks], [want])
+    worst, scale, same, total, err2, ref2, count = 0.0, 0.0, 0, 0, 0.0, 0.0, 0
+    for _ in range(decode_steps + 1):
+        worst = max(worst, float((a - b).abs().max()))
+        scale = max(scale, float(b.abs().max()))
+        err2 += float(((a - b).double() ** 2).sum())
+        ref2 += float((b.double() ** 2).sum())
+        count += a.numel()
+        same += int((a.argmax(-1) == b.argmax(-1)).sum())
+        total += a.shape[0]
+        nxt = int(b[-1].argmax())
+        a = engine.runner.step([rid], [[nxt]])
+        b = ref.step([rid], [[nxt]])
+    sync()
+    engine.runner.end(rid)
+    del ref
+    torch.cuda.empty_cache()
+    return worst / scale, (err2 / ref2) ** 0.5, same, total
+
+
 def library_product(cfg, sync, calls=400):
     """Time of the library's gate/up product of a 2,048-token prefill (the largest of a layer's four), once with
     random rows and once with rows of zeros: the same instructions on the same addresses, but zeros switch far fewer
@@ -340,7 +375,9 @@ def main() -> int:
                          "scheduler (the workload that goes with --shape llama2-7b --batch 64); arrivals: --batch requests "
                          "decode while a prompt of 16 tokens arrives every second step (host time and the GPU's busy "
                          "fraction per kind of step)")
-    ap.add_argument("--no-points", action="store_true", help="skip decoding at batch 1 and 64 and the prefill")
+    ap.add_argument("--no-points", action="store_true", help="skip decoding at batch 1 and 64, the prefill and the check")
+    ap.add_argument("--no-check", action="store_true",
+                    help="skip the comparison of the benchmarked model's logits with the 32-bit path's (same weights, all layers)")
     ap.add_argument("--points", choices=["default", "all"], default="default",
                     help="all: beside decoding at batch 1 and 64 also the time to the first token at 1 and 8 requests for "
                          "prompts of 16, 128, 512 and 8192 tokens, one prefill step of 16 prompts of 128 tokens and of 64 of "
@@ -465,7 +502,18 @@ def main() -> int:
                 t = run_prefill_step(engine, cfg, b, n, rng, sync)
                 points[f"prefill_step_ms_{b}x{n}"] = round(t * 1e3, 3)
         line["points"] = points
+        if not args.no_check and args.dtype == "bfloat16":
+            rel, rms, same, total = check_against_float32(engine, cfg, rng, sync)
+            # bfloat16 rounding through all layers moves the logits by a few hundredths of their size (measured:
+            # root mean square 0.04 of the logits' own, largest 0.05 of the largest); a kernel that computes
+            # something else moves them by their size
+            line["check"] = {"against": "float32 path, same weights, all layers", "positions": total,
+                             "rms_error_of_rms_logit": round(rms, 5), "max_error_of_largest_logit": round(rel, 5),
+                             "same_argmax": same, "ok": bool(rms < 0.1 and rel < 0.2)}
     print(json.dumps(line), flush=True)
+    if "check" in line and not line["check"]["ok"]:
+        print("bench.py: the benchmarked model's logits differ from the 32-bit path's", file=sys.stderr)
+        return 1
     return 0
 
 

@@ -468,3 +468,38 @@ LCU_API int lcu_sample(const float *logits, int ld, int rows, int vocab, const f
     LCU_LAUNCH_CHECK();
     return LCU_OK;
 }
+
+// ---------------------------------------------------------------- the chosen token's log-probability
+// out[r] = logits[r][tokens[r]] - log(sum_j exp(logits[r][j])), the natural logarithm of the token's probability under
+// the softmax of the row at temperature 1 (what the model itself gives the token, whatever the draw's temperature and
+// cuts were).  One workgroup a row; the maximum first, then the sum of exp(l - max) in a fixed order.  A token outside
+// the row gives NaN.
+__global__ void __launch_bounds__(SAMPLE_THREADS)
+token_logprob_kernel(const float *__restrict__ logits, int ld, int vocab, const int *__restrict__ tokens, float *__restrict__ out) {
+    __shared__ float scratch[16];
+    const float *row = logits + (size_t)blockIdx.x * ld;
+    float mx = -INFINITY;
+    scan_part(row, 0, vocab, [&](int, float v) { mx = fmaxf(mx, v); });
+    mx = wave_max(mx);
+    const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
+    if (lane == 0) scratch[wave] = mx;
+    __syncthreads();
+    mx = scratch[0];
+    for (int i = 1; i < SAMPLE_THREADS / WAVE; ++i) mx = fmaxf(mx, scratch[i]);
+    float sum = 0.f;
+    scan_part(row, 0, vocab, [&](int, float v) { sum += expf(v - mx); });
+    sum = block_sum(sum, scratch);
+    if (threadIdx.x == 0) {
+        const int t = tokens[blockIdx.x];
+        out[blockIdx.x] = (t >= 0 && t < vocab) ? row[t] - mx - logf(sum) : NAN;
+    }
+}
+
+// logits: [rows, ld] float32 with vocab <= ld; tokens: [rows] int32; out: [rows] float32.
+LCU_API int lcu_token_logprob(const float *logits, int ld, int rows, int vocab, const int *tokens, float *out, hipStream_t stream) {
+    if (rows <= 0) return LCU_OK;
+    if (vocab <= 0 || ld < vocab || !logits || !tokens || !out) return LCU_BAD_ARGUMENT;
+    token_logprob_kernel<<<dim3(rows), dim3(SAMPLE_THREADS), 0, stream>>>(logits, ld, vocab, tokens, out);
+    LCU_LAUNCH_CHECK();
+    return LCU_OK;
+}

@@ -25,6 +25,7 @@ class EngineConfig:
     use_graphs: bool = True                 # replay decode steps from captured graphs
     pack_weights: Optional[bool] = None     # a second copy of the matrices in the decode kernels' order (default: if memory allows)
     run_ahead: bool = True                  # launch a round before the round before has been read
+    logprobs: bool = False                  # every sampled token comes with the log of the probability the model gave it
     poison_freed: bool = False              # debugging: fill pages that change hands with NaN
 
     def __post_init__(self):

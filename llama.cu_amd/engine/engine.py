@@ -20,7 +20,7 @@ from typing import Callable, Dict, List, Optional, Sequence, Union
 import torch
 
 from ..kernels import ops
-from ..sampling import GREEDY, Sampler, SamplingParams
+from ..sampling import GREEDY, Sampler, SamplingParams, token_logprobs
 from .config import EngineConfig
 from .runner import ModelRunner
 from .scheduler import Scheduler
@@ -31,6 +31,7 @@ class StepOutput:
     req: int
     token: Optional[int]          # the sampled token (None if the request ended without one)
     finished: Optional[str]       # None, "eos", "max_steps", "length", "aborted"
+    logprob: Optional[float] = None   # log of the probability the model gave the token (an engine made with ``logprobs``)
 
 
 @dataclass
@@ -56,13 +57,17 @@ class _Flight:
     sampled: torch.Tensor             # the ids on the device
     host: torch.Tensor                # and where the copy to the host lands
     copied: torch.cuda.Event
+    host_logprobs: Optional[torch.Tensor] = None
 
 
 class Engine:
     def __init__(self, runner: ModelRunner, prefill_chunk: Optional[int] = None, eos_token_ids: Sequence[int] = (),
-                 run_ahead: bool = True):
+                 run_ahead: bool = True, logprobs: bool = False):
+        """``logprobs``: every sampled token comes with the logarithm of the probability that the model gave it
+        (``StepOutput.logprob``; one more small kernel and copy a round)."""
         self.runner = runner
         self.run_ahead = bool(run_ahead)
+        self.logprobs = bool(logprobs)
         self._flight: Optional[_Flight] = None
         self._awaiting: set = set()    # ended by count at launch, token not read yet
         self.sched = Scheduler(runner.cache, runner.max_seqs, runner.max_batch_tokens,
@@ -82,7 +87,8 @@ class Engine:
         """The engine for a model folder.  ``config``: the engine's constants (``EngineConfig``); ``fields``
         replace single ones (``dtype="float32", max_seqs=4, ...``)."""
         ec = EngineConfig.of(config, **fields)
-        engine = cls(ModelRunner.from_folder(folder, **ec.runner_kwargs()), ec.prefill_chunk, run_ahead=ec.run_ahead)
+        engine = cls(ModelRunner.from_folder(folder, **ec.runner_kwargs()), ec.prefill_chunk, run_ahead=ec.run_ahead,
+                     logprobs=ec.logprobs)
         engine.config = ec
         return engine
 
@@ -93,7 +99,7 @@ class Engine:
         ``stored``: as in ``ModelRunner.from_config``)."""
         ec = EngineConfig.of(config, **fields)
         engine = cls(ModelRunner.from_config(cfg, seed, std=std, stored=stored, **ec.runner_kwargs()), ec.prefill_chunk,
-                     run_ahead=ec.run_ahead)
+                     run_ahead=ec.run_ahead, logprobs=ec.logprobs)
         engine.config = ec
         return engine
 
@@ -206,6 +212,10 @@ class Engine:
         sampled = self.sampler.sample_device(logits, params, keys)
         host = torch.empty(len(rows), dtype=torch.int32, pin_memory=True)
         host.copy_(sampled, non_blocking=True)
+        host_lp = None
+        if self.logprobs:
+            host_lp = torch.empty(len(rows), dtype=torch.float32, pin_memory=True)
+            host_lp.copy_(token_logprobs(logits, sampled), non_blocking=True)
         copied = torch.cuda.Event()
         copied.record()
         if first is not None:
@@ -213,7 +223,7 @@ class Engine:
             last.record()
             self.timeline.append({"host_ms": (time.perf_counter() - t_plan) * 1e3, "tokens": step.n, "requests": step.n_req,
                                   "graph": self.runner.last_run_was_replay, "first": first, "last": last})
-        flight = _Flight([e.req for e in rows], [], [], [], [], sampled, host, copied)
+        flight = _Flight([e.req for e in rows], [], [], [], [], sampled, host, copied, host_lp)
         for e in rows:
             r = self.requests[e.req]
             r.unknown = len(r.tokens)
@@ -232,8 +242,9 @@ class Engine:
         an end-of-sequence token ends."""
         flight.copied.synchronize()
         outputs: List[StepOutput] = []
-        for rid, index, reason, turn, owner, tok in zip(flight.rows, flight.index, flight.reasons, flight.turns,
-                                                        flight.owners, flight.host.tolist()):
+        lps = flight.host_logprobs.tolist() if flight.host_logprobs is not None else [None] * len(flight.rows)
+        for rid, index, reason, turn, owner, tok, lp in zip(flight.rows, flight.index, flight.reasons, flight.turns,
+                                                            flight.owners, flight.host.tolist(), lps):
             r = self.requests.get(rid)
             if r is not owner or r.done or r.turn != turn:
                 continue                                    # ended earlier; this row ran for nothing
@@ -248,7 +259,7 @@ class Engine:
             if reason:
                 r.done = True
                 self._awaiting.discard(rid)
-            outputs.append(StepOutput(rid, tok, reason))
+            outputs.append(StepOutput(rid, tok, reason, lp))
         return outputs
 
     def _step_in_turn(self) -> List[StepOutput]:
@@ -270,11 +281,14 @@ class Engine:
                 params = [self.requests[e.req].params for e in rows]
                 keys = [(self.requests[e.req].draw_id, len(self.requests[e.req].tokens)) for e in rows]
                 sampled = self.sampler.sample(logits, params, keys)
-                for e, tok in zip(rows, sampled):
+                lps = [None] * len(sampled)
+                if self.logprobs:
+                    lps = token_logprobs(logits, ops.to_device(sampled, torch.int32, logits.device)).tolist()
+                for e, tok, lp in zip(rows, sampled, lps):
                     r = self.requests[e.req]
                     r.tokens.append(tok)
                     reason = self.sched.append(e.req, tok, (tok in self.eos) and not r.ignore_eos)
-                    outputs.append(StepOutput(e.req, tok, reason))
+                    outputs.append(StepOutput(e.req, tok, reason, lp))
         reported = {o.req for o in outputs if o.finished}
         for rid in self.sched.take_finished():
             if rid not in reported:

@@ -77,6 +77,22 @@ def sample_rows(logits: torch.Tensor, temperature: Sequence[float], top_p: Seque
     return out
 
 
+def token_logprobs(logits: torch.Tensor, tokens: torch.Tensor) -> torch.Tensor:
+    """``log softmax(logits[r])[tokens[r]]`` for every row: the natural logarithm of the probability that the model
+    gives each row's token (float32, on the device).  The reference hands back the chosen token's value beside its
+    index (``KVPair``, llama.cu/src/op/random_sample/mod.rs:29-36); this is that value made comparable across rows."""
+    _gpu(logits, tokens)
+    if logits.dim() != 2 or logits.dtype != torch.float32 or logits.stride(1) != 1:
+        raise KernelError("token_logprobs: logits must be float32 [rows, vocab] with contiguous rows")
+    rows, vocab = logits.shape
+    if tokens.dtype != torch.int32 or tokens.numel() != rows or not tokens.is_contiguous():
+        raise KernelError(f"token_logprobs: tokens must be a contiguous int32 tensor of {rows} entries")
+    out = torch.empty(rows, dtype=torch.float32, device=logits.device)
+    lib = build.load("sampling")
+    _check(lib.lcu_token_logprob(_ptr(logits), logits.stride(0), rows, vocab, _ptr(tokens), _ptr(out), _stream()), "token_logprobs")
+    return out
+
+
 class Sampler:
     def sample_device(self, logits: torch.Tensor, params: Sequence[SamplingParams],
                       keys: Sequence[Tuple[int, int]]) -> torch.Tensor:

@@ -135,3 +135,49 @@ def test_per_row_parameters_and_sampler_mix():
         p = params[r]
         want = plain.sample(l[r], p.temperature, p.top_p, min(p.top_k, 10 ** 9), uniform(p.seed, *keys[r]))
         assert got[r] == want
+
+
+def test_the_chosen_tokens_log_probability():
+    """``token_logprobs`` against ``torch.log_softmax`` in 64-bit, on rows of a vocabulary that is no power of two with a
+    stride of its own, one row sharp (a logit far above the rest) and one flat; and through the engine: the tokens of an
+    engine made with ``logprobs`` come with the plain model's log-probabilities."""
+    from llama_cu_amd.sampling import token_logprobs
+    g = torch.Generator().manual_seed(3)
+    rows, vocab = 7, 128256 + 3
+    buf = torch.randn(rows, vocab + 5, generator=g) * 3.0
+    buf[2, 777] = 60.0
+    buf[4, :] = 0.25
+    logits = buf.cuda()[:, :vocab]
+    tokens = torch.tensor([0, vocab - 1, 777, 5, 9, 100000, 31], dtype=torch.int32)
+    got = token_logprobs(logits, tokens.cuda()).cpu().double()
+    want = torch.log_softmax(buf[:, :vocab].double(), dim=-1)[torch.arange(rows), tokens.long()]
+    assert float((got - want).abs().max()) < 1e-4, (got, want)
+    assert abs(float(got[2])) < 1e-6 and abs(float(got[4]) + float(torch.log(torch.tensor(float(vocab))))) < 1e-4
+    assert torch.isnan(token_logprobs(logits[:1], torch.tensor([vocab], dtype=torch.int32).cuda())).all()
+
+
+@pytest.mark.parametrize("run_ahead", [False, True])
+def test_an_engine_made_with_logprobs_hands_them_out_with_its_tokens(run_ahead):
+    import common
+    import plain
+    from llama_cu_amd.engine.engine import Engine
+    from llama_cu_amd.sampling import SamplingParams
+    folder = common.make_folder(common.TINY_A, seed=5, dtype=torch.float32)
+    engine = Engine.from_folder(folder, dtype="float32", max_tokens=512, max_seqs=4, run_ahead=run_ahead, logprobs=True)
+    prompts = list(common.random_requests(256, [9, 30], seed=2).values())
+    params = [SamplingParams(), SamplingParams(temperature=0.9, seed=4)]
+    ids = [engine.add_request(p, sp, 6, ignore_eos=True) for p, sp in zip(prompts, params)]
+    got = {i: [] for i in ids}
+    while not engine.idle:
+        for o in engine.step():
+            if o.token is not None:
+                assert o.logprob is not None
+                got[o.req].append((o.token, o.logprob))
+    cfg, w = plain.load_folder(folder)
+    for rid, prompt in zip(ids, prompts):
+        toks = list(prompt)
+        assert len(got[rid]) == 6
+        for tok, lp in got[rid]:
+            want = torch.log_softmax(plain.forward(cfg, w, toks)[-1], dim=-1)[tok]
+            assert abs(lp - float(want)) < 1e-3, (rid, len(toks), lp, float(want))
+            toks.append(tok)
