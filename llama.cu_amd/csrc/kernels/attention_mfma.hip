@@ -72,6 +72,10 @@ struct KVFrag {
     u32x2 v[DH / 16][2];    // dim 16*dt + lane%16, keys 16*t + 4*grp .. + 3
 };
 
+// The decode kernel reads a request's keys and values once a step: its loads are non-temporal (see gemm_skinny.hip's
+// stream_load), so that they do not displace the weights' neighbours and the rows in the caches.
+constexpr int DEC_STREAM = 2;
+
 // The numbers of the two pages that hold the keys k0 .. k0+15 and k0+16 .. k0+31 (k0 the same in
 // all lanes: the table is read through the scalar unit).
 __device__ __forceinline__ void kv_pages(int (&pid)[2], const int *__restrict__ bt, int max_pages, int page, int k0) {
@@ -106,10 +110,10 @@ __device__ __forceinline__ void load_kv(KVFrag<DH> &f, const bf16_t *__restrict_
         const uint32_t k_off = k_lane + tok0 * 8 * E, v_off = v_lane + tok0 * E;
 #pragma unroll
         for (int kb = 0; kb < DH / 32; ++kb)
-            f.k[t][kb] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(pg, k_off, k_head + (uint32_t)(4 * kb) * page * 8 * E, 0));
+            f.k[t][kb] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(pg, k_off, k_head + (uint32_t)(4 * kb) * page * 8 * E, DEC_STREAM));
 #pragma unroll
         for (int dt = 0; dt < DH / 16; ++dt)
-            f.v[dt][t] = __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(pg, v_off, v_head + (uint32_t)(16 * dt) * page * E, 0));
+            f.v[dt][t] = __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(pg, v_off, v_head + (uint32_t)(16 * dt) * page * E, DEC_STREAM));
     }
 }
 
@@ -128,10 +132,10 @@ __device__ __forceinline__ void load_kv_flat(KVFrag<DH> &f, const bf16_t *__rest
         const int tok0 = j % page;
         const bf16_t *kp = pg + ((size_t)kvh * (DH / 8) * page + tok0 + l16) * 8;
 #pragma unroll
-        for (int kb = 0; kb < DH / 32; ++kb) f.k[t][kb] = *(const u32x4 *)(kp + (size_t)(4 * kb + grp) * page * 8);
+        for (int kb = 0; kb < DH / 32; ++kb) f.k[t][kb] = __builtin_nontemporal_load((const u32x4 *)(kp + (size_t)(4 * kb + grp) * page * 8));
         const bf16_t *vp = pg + v_off + tok0;
 #pragma unroll
-        for (int dt = 0; dt < DH / 16; ++dt) f.v[dt][t] = *(const u32x2 *)(vp + (size_t)(16 * dt + l16) * page);
+        for (int dt = 0; dt < DH / 16; ++dt) f.v[dt][t] = __builtin_nontemporal_load((const u32x2 *)(vp + (size_t)(16 * dt + l16) * page));
     }
 }
 

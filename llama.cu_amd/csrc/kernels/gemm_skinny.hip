@@ -78,6 +78,11 @@ struct Frag {
     u32x4 x[MT][4];
 };
 
+// A weight is read once per product and never again before the caches have turned over: its loads are marked
+// non-temporal, so that they do not displace what is used again (the rows, the next kernel's operands).  A kernel
+// that only reads memory moves 6.2 to 6.4 TB/s of a 235 MB stretch with such loads and 5.7 with ordinary ones.
+__device__ __forceinline__ u32x4 stream_load(const u32x4 *p) { return __builtin_nontemporal_load(p); }
+
 // The lane's loads of macro-step s: k = 128 s + 32 grp + 8 j .. + 7 for j = 0..3.
 template <int NT, int MT>
 __device__ __forceinline__ void load_frag(Frag<NT, MT> &f, const bf16_t *const (&wrow)[NT], const bf16_t *const (&xrow)[MT],
@@ -91,7 +96,7 @@ __device__ __forceinline__ void load_frag(Frag<NT, MT> &f, const bf16_t *const (
 #pragma unroll
         for (int t = 0; t < NT; ++t)
 #pragma unroll
-            for (int j = 0; j < 4; ++j) f.w[t][j] = *(const u32x4 *)(wrow[t] + w0 + wj * j);
+            for (int j = 0; j < 4; ++j) f.w[t][j] = stream_load((const u32x4 *)(wrow[t] + w0 + wj * j));
 #pragma unroll
         for (int m = 0; m < MT; ++m)
 #pragma unroll
@@ -100,7 +105,7 @@ __device__ __forceinline__ void load_frag(Frag<NT, MT> &f, const bf16_t *const (
 #pragma unroll
         for (int t = 0; t < NT; ++t)
 #pragma unroll
-            for (int j = 0; j < 4; ++j) f.w[t][j] = (kb + 8 * j + 8 <= K) ? *(const u32x4 *)(wrow[t] + kb + 8 * j) : zero;
+            for (int j = 0; j < 4; ++j) f.w[t][j] = (kb + 8 * j + 8 <= K) ? stream_load((const u32x4 *)(wrow[t] + kb + 8 * j)) : zero;
 #pragma unroll
         for (int m = 0; m < MT; ++m)
 #pragma unroll
