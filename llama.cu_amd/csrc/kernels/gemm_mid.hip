@@ -44,7 +44,7 @@ constexpr int MID_STAGE_TILES = LCU_MID_STAGES;    // tiles of W in flight per w
 #define LCU_MID_CONSUMERS 4
 #endif
 constexpr int MID_CONSUMERS = LCU_MID_CONSUMERS;
-constexpr int MID_STREAM = 2;                 // the loads of W are non-temporal (read once; see gemm_skinny.hip's stream_load)
+constexpr int MID_STREAM = 2;                 // the loads of a packed W are non-temporal (read once; see gemm_skinny.hip's stream_load)
 constexpr int MID_XROW = 272;                 // bytes between the rows of X in LDS (256 + 16)
 constexpr int MID_XBUFS = 3;
 
@@ -186,7 +186,7 @@ gemm_mid_kernel(const bf16_t *__restrict__ X, int ldx, const bf16_t *__restrict_
     u32x4 w[MID_STAGES][NT][4];
 #define MID_LOAD_W(i, step)                                                                                     \
     _Pragma("unroll") for (int t = 0; t < NT; ++t) _Pragma("unroll") for (int j = 0; j < 4; ++j) w[i][t][j] =  \
-        __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(wb[t], w_lane + (uint32_t)(step) * w_step + w_j * j, 0, MID_STREAM))
+        __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(wb[t], w_lane + (uint32_t)(step) * w_step + w_j * j, 0, PACKED ? MID_STREAM : 0))
 #pragma unroll
     for (int i = 0; i < MID_STAGES; ++i) MID_LOAD_W(i, i);
     if (scales) {

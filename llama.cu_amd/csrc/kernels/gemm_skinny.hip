@@ -78,25 +78,29 @@ struct Frag {
     u32x4 x[MT][4];
 };
 
-// A weight is read once per product and never again before the caches have turned over: its loads are marked
-// non-temporal, so that they do not displace what is used again (the rows, the next kernel's operands).  A kernel
-// that only reads memory moves 6.2 to 6.4 TB/s of a 235 MB stretch with such loads and 5.7 with ordinary ones.
+// A weight is read once per product and never again before the caches have turned over: the loads of a packed
+// weight are marked non-temporal, so that they do not displace what is used again (the rows, the next kernel's
+// operands).  A kernel that only reads memory moves 6.2 to 6.4 TB/s of a 235 MB stretch with such loads and 5.7
+// with ordinary ones.  Only where a load instruction of a wave takes whole 128-byte lines, as it does from a packed
+// weight: from plain rows, where eight instructions share a line, such loads fetch the line again and again (the
+// decode step of 8 requests took 5.5 ms with them and plain rows).
 __device__ __forceinline__ u32x4 stream_load(const u32x4 *p) { return __builtin_nontemporal_load(p); }
 
 // The lane's loads of macro-step s: k = 128 s + 32 grp + 8 j .. + 7 for j = 0..3.
-template <int NT, int MT>
+template <int NT, int MT, bool PACKED>
 __device__ __forceinline__ void load_frag(Frag<NT, MT> &f, const bf16_t *const (&wrow)[NT], const bf16_t *const (&xrow)[MT],
-                                          const bool (&xvalid)[MT], int s, int grp, int K, int packed) {
+                                          const bool (&xvalid)[MT], int s, int grp, int K) {
     const int kb = 128 * s + 32 * grp;
     const u32x4 zero = u32x4{0u, 0u, 0u, 0u};
     if (128 * (s + 1) <= K) {
         // packed: wrow is the lane's place in the tile's first block; blocks are 2048 elements,
         // the four loads of a block 512 apart
-        const int w0 = packed ? 2048 * s : kb, wj = packed ? 512 : 8;
+        const int w0 = PACKED ? 2048 * s : kb, wj = PACKED ? 512 : 8;
 #pragma unroll
         for (int t = 0; t < NT; ++t)
 #pragma unroll
-            for (int j = 0; j < 4; ++j) f.w[t][j] = stream_load((const u32x4 *)(wrow[t] + w0 + wj * j));
+            for (int j = 0; j < 4; ++j)
+                f.w[t][j] = PACKED ? stream_load((const u32x4 *)(wrow[t] + w0 + wj * j)) : *(const u32x4 *)(wrow[t] + w0 + wj * j);
 #pragma unroll
         for (int m = 0; m < MT; ++m)
 #pragma unroll
@@ -105,7 +109,7 @@ __device__ __forceinline__ void load_frag(Frag<NT, MT> &f, const bf16_t *const (
 #pragma unroll
         for (int t = 0; t < NT; ++t)
 #pragma unroll
-            for (int j = 0; j < 4; ++j) f.w[t][j] = (kb + 8 * j + 8 <= K) ? stream_load((const u32x4 *)(wrow[t] + kb + 8 * j)) : zero;
+            for (int j = 0; j < 4; ++j) f.w[t][j] = (kb + 8 * j + 8 <= K) ? *(const u32x4 *)(wrow[t] + kb + 8 * j) : zero;
 #pragma unroll
         for (int m = 0; m < MT; ++m)
 #pragma unroll
@@ -124,10 +128,10 @@ __device__ __forceinline__ void mul_frag(const Frag<NT, MT> &f, f32x4 (&acc)[NT]
             for (int m = 0; m < MT; ++m) acc[t][m] = mfma16(f.w[t][j], f.x[m][j], acc[t][m]);
 }
 
-template <int NT, int MT, int EPI, int SK_WAVES>
+template <int NT, int MT, int EPI, int SK_WAVES, bool PACKED>
 __global__ void __launch_bounds__(SK_WAVES *WAVE)
 gemm_skinny_kernel(const bf16_t *__restrict__ X, int ldx, const bf16_t *__restrict__ W, int ldw, void *__restrict__ Y,
-                   int ldy, int M, int N, int K, int w_packed, SkinnyExtra ex) {
+                   int ldy, int M, int N, int K, SkinnyExtra ex) {
     __shared__ float red[SK_WAVES][NT * MT * 4][WAVE];
     __shared__ float row_scale[16 * MT];
     const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
@@ -147,7 +151,7 @@ gemm_skinny_kernel(const bf16_t *__restrict__ X, int ldx, const bf16_t *__restri
         if (EPI == EPI_QKV_ROPE) row = rope_head * ex.head_dim + t * (ex.head_dim / 2) + 16 * rope_c + l16;
         const int limit = EPI == EPI_SWIGLU ? (half + 1) * n_out : N;
         row = row < limit ? row : limit - 1;                          // a row beyond the end is read, not stored
-        wrow[t] = w_packed ? W + ((size_t)(row / 16) * (K / 128)) * 2048 + (size_t)lane * 8   // (the tile of the row)
+        wrow[t] = PACKED ? W + ((size_t)(row / 16) * (K / 128)) * 2048 + (size_t)lane * 8   // (the tile of the row)
                            : W + (size_t)row * ldw;
     }
     const bf16_t *xrow[MT];
@@ -201,7 +205,7 @@ gemm_skinny_kernel(const bf16_t *__restrict__ X, int ldx, const bf16_t *__restri
     int s = wave;
 #pragma unroll
     for (int i = 0; i < STAGES; ++i)
-        if (s + i * SK_WAVES < nsteps) load_frag<NT, MT>(f[i], wrow, xrow, xvalid, s + i * SK_WAVES, grp, K, w_packed);
+        if (s + i * SK_WAVES < nsteps) load_frag<NT, MT, PACKED>(f[i], wrow, xrow, xvalid, s + i * SK_WAVES, grp, K);
     for (; s < nsteps; s += STAGES * SK_WAVES) {
 #pragma unroll
         for (int i = 0; i < STAGES; ++i) {
@@ -209,7 +213,7 @@ gemm_skinny_kernel(const bf16_t *__restrict__ X, int ldx, const bf16_t *__restri
             if (cur < nsteps) {
                 mul_frag<NT, MT>(f[i], acc);
                 if (cur + STAGES * SK_WAVES < nsteps)
-                    load_frag<NT, MT>(f[i], wrow, xrow, xvalid, cur + STAGES * SK_WAVES, grp, K, w_packed);
+                    load_frag<NT, MT, PACKED>(f[i], wrow, xrow, xvalid, cur + STAGES * SK_WAVES, grp, K);
             }
         }
     }
@@ -355,7 +359,11 @@ static int launch_epi(const void *X, int ldx, const void *W, int ldw, void *Y, i
                       int packed, const SkinnyExtra &ex, hipStream_t stream) {
     dim3 block(WAVES * WAVE);
     const dim3 grid((N + 16 * NT - 1) / (16 * NT));
-#define GO(E) gemm_skinny_kernel<NT, MT, E, WAVES><<<grid, block, 0, stream>>>((const bf16_t *)X, ldx, (const bf16_t *)W, ldw, Y, ldy, M, N, K, packed, ex)
+#define GO(E)                                                                                                                      \
+    do {                                                                                                                           \
+        if (packed) gemm_skinny_kernel<NT, MT, E, WAVES, true><<<grid, block, 0, stream>>>((const bf16_t *)X, ldx, (const bf16_t *)W, ldw, Y, ldy, M, N, K, ex); \
+        else gemm_skinny_kernel<NT, MT, E, WAVES, false><<<grid, block, 0, stream>>>((const bf16_t *)X, ldx, (const bf16_t *)W, ldw, Y, ldy, M, N, K, ex);       \
+    } while (0)
     switch (epi) {
     case EPI_BF16: GO(EPI_BF16); break;
     case EPI_F32: GO(EPI_F32); break;
@@ -366,8 +374,10 @@ static int launch_epi(const void *X, int ldx, const void *W, int ldw, void *Y, i
     case EPI_QKV_ROPE:
         if constexpr (MT <= 2 && NT == 2) {
             const dim3 rgrid((ex.heads + 2 * ex.kv_heads) * (ex.head_dim / 32));
-            gemm_skinny_kernel<NT, MT, EPI_QKV_ROPE, WAVES><<<rgrid, block, 0, stream>>>(
-                (const bf16_t *)X, ldx, (const bf16_t *)W, ldw, Y, ldy, M, N, K, packed, ex);
+            if (packed) gemm_skinny_kernel<NT, MT, EPI_QKV_ROPE, WAVES, true><<<rgrid, block, 0, stream>>>(
+                (const bf16_t *)X, ldx, (const bf16_t *)W, ldw, Y, ldy, M, N, K, ex);
+            else gemm_skinny_kernel<NT, MT, EPI_QKV_ROPE, WAVES, false><<<rgrid, block, 0, stream>>>(
+                (const bf16_t *)X, ldx, (const bf16_t *)W, ldw, Y, ldy, M, N, K, ex);
             break;
         }
         return LCU_UNSUPPORTED;
@@ -382,8 +392,10 @@ template <int NT, int MT, int WAVES>
 static int launch_swiglu(const void *X, int ldx, const void *W, int ldw, void *Y, int ldy, int M, int N, int K,
                          int packed, const SkinnyExtra &ex, hipStream_t stream) {
     const int groups = (N / 2 + 8 * NT - 1) / (8 * NT);
-    gemm_skinny_kernel<NT, MT, EPI_SWIGLU, WAVES><<<dim3(groups), dim3(WAVES * WAVE), 0, stream>>>(
-        (const bf16_t *)X, ldx, (const bf16_t *)W, ldw, Y, ldy, M, N, K, packed, ex);
+    if (packed) gemm_skinny_kernel<NT, MT, EPI_SWIGLU, WAVES, true><<<dim3(groups), dim3(WAVES * WAVE), 0, stream>>>(
+        (const bf16_t *)X, ldx, (const bf16_t *)W, ldw, Y, ldy, M, N, K, ex);
+    else gemm_skinny_kernel<NT, MT, EPI_SWIGLU, WAVES, false><<<dim3(groups), dim3(WAVES * WAVE), 0, stream>>>(
+        (const bf16_t *)X, ldx, (const bf16_t *)W, ldw, Y, ldy, M, N, K, ex);
     LCU_LAUNCH_CHECK();
     return LCU_OK;
 }
