@@ -1,15 +1,16 @@
-// Y[M, N] = X[M, K] * W[N, K]^T for 17 to 128 rows (decoding many requests), bfloat16 operands,
+// Y[M, N] = X[M, K] * W[N, K]^T for 17 to 256 rows (decoding many requests), bfloat16 operands,
 // 32-bit accumulation on the matrix cores.  W is streamed once from HBM; what sets this kernel
 // apart from the one for few rows is where X comes from.  With 64 rows a wave that loads its own
 // piece of X moves twice as many bytes of X as of W and has no registers left to keep loads of W
 // in flight.  Here
 //
-//   * a workgroup is four consumer waves and one producer wave (two from 65 rows on, 64 rows
-//     each).  The four consumers work on the
+//   * a workgroup is four consumer waves and one producer wave for every 64 rows.  The four
+//     consumers work on the
 //     same k at the same time, each on its own tile of 16 output features (for SwiGLU a gate
 //     tile and the up tile that belongs to it), so one piece of X serves all of them;
 //   * the producer wave does nothing but copy X, macro-step (128 k) by macro-step, from memory
-//     (it comes from the L2 cache) into a ring of three buffers in LDS, two macro-steps ahead.
+//     (it comes from the L2 cache) into a ring of three buffers in LDS, two macro-steps ahead
+//     (beyond 128 rows three buffers do not fit: two buffers, one macro-step ahead).
 //     Its waits for its loads do not touch the consumers' loads: a wave's loads come back in
 //     order, so a consumer that waited for X would wait for every load of W issued before it;
 //   * a consumer keeps the loads of W of several macro-steps in flight (16 registers a tile and step),
@@ -46,14 +47,14 @@ constexpr int MID_STAGE_TILES = LCU_MID_STAGES;    // tiles of W in flight per w
 constexpr int MID_CONSUMERS = LCU_MID_CONSUMERS;
 constexpr int MID_STREAM = 2;                 // the loads of a packed W are non-temporal (read once; see gemm_skinny.hip's stream_load)
 constexpr int MID_XROW = 272;                 // bytes between the rows of X in LDS (256 + 16)
-constexpr int MID_XBUFS = 3;
+constexpr int mid_xbufs(int MT) { return MT > 8 ? 2 : 3; }      // buffers of the ring of X (160 KB of LDS: 256 rows fit twice)
 
 __device__ __forceinline__ f32x4 mid_mfma(u32x4 a, u32x4 b, f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
 }
 
-constexpr int mid_producers(int MT) { return MT > 4 ? 2 : 1; }
-constexpr int mid_lds_bytes(int MT) { return MID_XBUFS * 16 * MT * MID_XROW + 16 * MT * (int)sizeof(float); }
+constexpr int mid_producers(int MT) { return (MT + 3) / 4; }
+constexpr int mid_lds_bytes(int MT) { return mid_xbufs(MT) * 16 * MT * MID_XROW + 16 * MT * (int)sizeof(float); }
 
 // Producer wave P copies the rows 64 P .. of X, macro-step by macro-step, into the ring in LDS.
 // chunk c = 64 i + lane of a macro-step: row 64 P + c / 16, 16 bytes at k = 8 (c % 16).  The loads
@@ -64,8 +65,10 @@ constexpr int mid_lds_bytes(int MT) { return MID_XBUFS * 16 * MT * MID_XROW + 16
 // lane's offset against the end, not the scalar one).
 template <int MT, int P>
 __device__ __forceinline__ void mid_produce(char *xs, const bf16_t *__restrict__ X, int ldx, int M, int s_begin, int nst, int lane) {
-    constexpr int LOADS = (P == 0 ? (MT < 4 ? MT : 4) : MT - 4) * 4;      // four rows a load
+    constexpr int ROWS16 = MT - 4 * P < 4 ? MT - 4 * P : 4;              // tiles of 16 rows that this producer copies
+    constexpr int LOADS = ROWS16 * 4;                                     // four rows a load
     constexpr int BUF = 16 * MT * MID_XROW;
+    constexpr int XB = mid_xbufs(MT), AHEAD = XB - 1;                     // the copy runs this many macro-steps ahead
     const __amdgpu_buffer_rsrc_t xb = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<bf16_t *>(X + (size_t)128 * s_begin), 0, (uint32_t)(((size_t)(M - 1) * ldx + 128 * nst) * 2), 0x00020000);
     uint32_t src[LOADS];
@@ -80,18 +83,18 @@ __device__ __forceinline__ void mid_produce(char *xs, const bf16_t *__restrict__
 #define MID_LOAD_X(b, step)                                                                                         \
     _Pragma("unroll") for (int i = 0; i < LOADS; ++i) xr[b][i] =                                                   \
         __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(xb, src[i] + (uint32_t)(step) * 256u, 0, 0))
-    // macro-steps 0 and 1 go straight into their buffers
+    // the first AHEAD macro-steps go straight into their buffers
     MID_LOAD_X(0, 0);
-    MID_LOAD_X(1, 1);
+    if (AHEAD > 1) MID_LOAD_X(1, 1);
 #pragma unroll
-    for (int b = 0; b < 2; ++b)
+    for (int b = 0; b < AHEAD; ++b)
 #pragma unroll
         for (int i = 0; i < LOADS; ++i) *(u32x4 *)(xs + b * BUF + dst[i]) = xr[b][i];
-    MID_LOAD_X(0, 2);
-    MID_LOAD_X(1, 3);
+    MID_LOAD_X(0, AHEAD);
+    MID_LOAD_X(1, AHEAD + 1);
     lds_barrier();
-    // in iteration s: macro-step s + 2 goes into buffer (s + 2) % 3, the loads of s + 4 start
-    int buf = 2;
+    // in iteration s: macro-step s + AHEAD goes into buffer (s + AHEAD) % XB, the loads of s + AHEAD + 2 start
+    int buf = AHEAD;
     for (int s = 0; s < nst; s += 2) {
 #pragma unroll
         for (int b = 0; b < 2; ++b) {
@@ -99,8 +102,8 @@ __device__ __forceinline__ void mid_produce(char *xs, const bf16_t *__restrict__
             if (cur < nst) {
 #pragma unroll
                 for (int i = 0; i < LOADS; ++i) *(u32x4 *)(xs + buf * BUF + dst[i]) = xr[b][i];
-                MID_LOAD_X(b, cur + 4);
-                buf = buf == MID_XBUFS - 1 ? 0 : buf + 1;
+                MID_LOAD_X(b, cur + AHEAD + 2);
+                buf = buf == XB - 1 ? 0 : buf + 1;
                 lds_barrier();
             }
         }
@@ -115,7 +118,8 @@ gemm_mid_kernel(const bf16_t *__restrict__ X, int ldx, const bf16_t *__restrict_
                 float eps) {
     extern __shared__ __attribute__((aligned(16))) char xs[];      // the ring of X, then the rows' factors
     constexpr int BUF = 16 * MT * MID_XROW;
-    float *row_scale = (float *)(xs + MID_XBUFS * BUF);
+    constexpr int XB = mid_xbufs(MT);
+    float *row_scale = (float *)(xs + XB * BUF);
     const int lane = threadIdx.x & (WAVE - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
     const int l16 = lane & 15, grp = lane >> 4;
@@ -131,6 +135,18 @@ gemm_mid_kernel(const bf16_t *__restrict__ X, int ldx, const bf16_t *__restrict_
     if constexpr (MT > 4) {
         if (wave == MID_CONSUMERS + 1) {
             mid_produce<MT, 1>(xs, X, ldx, M, s_begin, nst, lane);
+            return;
+        }
+    }
+    if constexpr (MT > 8) {
+        if (wave == MID_CONSUMERS + 2) {
+            mid_produce<MT, 2>(xs, X, ldx, M, s_begin, nst, lane);
+            return;
+        }
+    }
+    if constexpr (MT > 12) {
+        if (wave == MID_CONSUMERS + 3) {
+            mid_produce<MT, 3>(xs, X, ldx, M, s_begin, nst, lane);
             return;
         }
     }
@@ -182,7 +198,9 @@ gemm_mid_kernel(const bf16_t *__restrict__ X, int ldx, const bf16_t *__restrict_
             for (int i = grp; i < n_in; i += 4) scale_ss += p[i];
         }
     }
-    constexpr int MID_STAGES = (MT > 4 && NT > 1 ? MID_STAGE_TILES * 3 / 4 : MID_STAGE_TILES) / NT;
+    // loads of W in flight: fewer where the sums take more registers (beyond 128 rows half as many)
+    constexpr int MID_STAGES = (MT > 8 ? MID_STAGE_TILES / 2 : MT > 4 && NT > 1 ? MID_STAGE_TILES * 3 / 4 : MID_STAGE_TILES) / NT;
+    constexpr int MCHUNK = MT > 8 ? MT / 2 : MT;          // row tiles whose operands are read from LDS at a time
     u32x4 w[MID_STAGES][NT][4];
 #define MID_LOAD_W(i, step)                                                                                     \
     _Pragma("unroll") for (int t = 0; t < NT; ++t) _Pragma("unroll") for (int j = 0; j < 4; ++j) w[i][t][j] =  \
@@ -204,16 +222,20 @@ gemm_mid_kernel(const bf16_t *__restrict__ X, int ldx, const bf16_t *__restrict_
             if (cur < nst) {
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    u32x4 xf[MT];
 #pragma unroll
-                    for (int m = 0; m < MT; ++m) xf[m] = *(const u32x4 *)(xs + buf * BUF + x_off + 16 * m * MID_XROW + 16 * j);
+                    for (int m0 = 0; m0 < MT; m0 += MCHUNK) {
+                        u32x4 xf[MCHUNK];
 #pragma unroll
-                    for (int t = 0; t < NT; ++t)
+                        for (int m = 0; m < MCHUNK; ++m)
+                            xf[m] = *(const u32x4 *)(xs + buf * BUF + x_off + 16 * (m0 + m) * MID_XROW + 16 * j);
 #pragma unroll
-                        for (int m = 0; m < MT; ++m) acc[t][m] = mid_mfma(w[i][t][j], xf[m], acc[t][m]);
+                        for (int t = 0; t < NT; ++t)
+#pragma unroll
+                            for (int m = 0; m < MCHUNK; ++m) acc[t][m0 + m] = mid_mfma(w[i][t][j], xf[m], acc[t][m0 + m]);
+                    }
                 }
                 MID_LOAD_W(i, cur + MID_STAGES);
-                buf = buf == MID_XBUFS - 1 ? 0 : buf + 1;
+                buf = buf == XB - 1 ? 0 : buf + 1;
                 lds_barrier();
             }
         }
@@ -292,14 +314,16 @@ static int mid_launch(const void *X, int ldx, const void *W, int ldw, void *Y, i
     else if (M <= 48) GO_MT(3);
     else if (M <= 64) GO_MT(4);
     else if (M <= 96) GO_MT(6);
-    else GO_MT(8);
+    else if (M <= 128) GO_MT(8);
+    else if (M <= 192) GO_MT(12);
+    else GO_MT(16);
 #undef GO_MT
 #undef GO
     LCU_LAUNCH_CHECK();
     return LCU_OK;
 }
 
-// X: [M, K] bfloat16 rows ldx apart, M <= 128 (rows that wait for their normalisation: M <= 64); W: [N, K] bfloat16, rows ldw apart or packed; K a
+// X: [M, K] bfloat16 rows ldx apart, M <= 256 (rows that wait for their normalisation: M <= 64); W: [N, K] bfloat16, rows ldw apart or packed; K a
 // multiple of 128, N of 16 (SwiGLU: of 32; W holds N/2 gate rows, then N/2 up rows).
 // epilogue MID_EPI_BF16: Y [M, N] bfloat16 rows ldy apart (slices must be 1);
 //          MID_EPI_SWIGLU: Y [M, N/2] bfloat16 = silu(gate) * up (slices must be 1);
@@ -315,7 +339,7 @@ LCU_API int lcu_gemm_mid_planes(int K, int slices) {
 static int mid_bf16(const void *X, int ldx, const void *W, int ldw, void *Y, int ldy, int M, int N, int K, int epilogue,
                     int slices, int w_packed, const MidScale &sc, hipStream_t stream) {
     if (M <= 0 || N <= 0) return LCU_OK;
-    if (M > 128 || (sc.sumsq_in && M > 64) || K <= 0 || K % 128 || N % 16 || ldx % 8 || ldx < K || slices <= 0 || slices > 64) return LCU_BAD_ARGUMENT;
+    if (M > 256 || (sc.sumsq_in && M > 64) || K <= 0 || K % 128 || N % 16 || ldx % 8 || ldx < K || slices <= 0 || slices > 64) return LCU_BAD_ARGUMENT;
     if (!w_packed && (ldw % 8 || ldw < K)) return LCU_BAD_ARGUMENT;
     if ((uintptr_t)X % 16 || (uintptr_t)W % 16 || (uintptr_t)Y % 16 || (uintptr_t)sc.sumsq_in % 16) return LCU_BAD_ARGUMENT;
     switch (epilogue) {

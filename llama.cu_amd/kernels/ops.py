@@ -698,12 +698,12 @@ def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = 
     return out
 
 
-MID_MAX_ROWS = 128
+MID_MAX_ROWS = 256
 MID_MAX_SCALED_ROWS = 64
 
 
 def mid_supported(x: torch.Tensor, w: torch.Tensor) -> bool:
-    """Whether ``gemm_mid`` takes these operands: up to 128 bfloat16 rows with K a multiple of 128
+    """Whether ``gemm_mid`` takes these operands: up to 256 bfloat16 rows with K a multiple of 128
     and a bfloat16 weight of a multiple of 16 rows."""
     return (x.is_cuda and w.is_cuda and x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and x.dim() == 2
             and w.dim() == 2 and 0 < x.shape[0] <= MID_MAX_ROWS and x.shape[1] == w.shape[1] and w.shape[1] % 128 == 0
@@ -721,7 +721,7 @@ def mid_planes(k: int, slices: int) -> int:
 def gemm_mid(x: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = None, swiglu: bool = False,
              slices: Optional[int] = None, packed: bool = False, row_sumsq: Optional[torch.Tensor] = None,
              norm_width: int = 0, eps: float = 0.0) -> torch.Tensor:
-    """``x @ w.T`` for up to 128 rows of bfloat16 ``x`` (chosen from 12 to 33 rows on, by the product), streaming ``w`` once while
+    """``x @ w.T`` for up to 256 rows of bfloat16 ``x`` (chosen from 12 to 33 rows on, by the product), streaming ``w`` once while
     the waves of a workgroup share ``x`` through LDS.  ``slices=None``: ``out [m, n]`` bfloat16
     (``swiglu``: ``w`` holds gate rows, then up rows, ``out [m, n/2] = silu(gate) * up``).
     ``slices=s``: K is cut into (at most) ``s`` slices and ``out [planes, m, n]`` float32 holds

@@ -28,13 +28,19 @@ class Tuning:
     skinny_workgroups_per_cu: int = 4   # plain: as many tiles as still leave this many workgroups for each compute unit
     skinny_eight_waves_to: int = 8192   # eight waves share a workgroup's K up to this many output features, four beyond
     compute_units: int = 256            # of the card the numbers were measured on; ``for_device`` puts in the card's own
-    # ---- the product that shares the rows through LDS (gemm_mid.hip, up to 128 rows)
+    # ---- the product that shares the rows through LDS (gemm_mid.hip, up to 256 rows)
     mid_long_k: int = 8192              # with a plain (not packed) weight only weights with a longer K than this (the down
                                         # projection) go to it at all; a packed weight with a longer K goes to it
     mid_long_k_rows: int = 11           # ... above this many rows (whole decode steps: 0.9 % faster at 12 rows, 3 % at 16;
                                         # 0.3 % slower at 11: below, the weight-streaming kernel with the norm in its epilogue)
     mid_swiglu_features: int = 8192     # gate/up with SwiGLU goes to it from this many rows of the weight on,
     mid_swiglu_rows: int = 14           # above this many rows of the batch (0.4 % at 16 rows, nothing below 15)
+    mid_swiglu_max_rows: int = 128      # ... up to this many (at 128 rows 61 us against the library's 59 with the activation
+                                        # kernel, beyond that the library is ahead: 69 against 63 at 160 rows, 80 against 72 at 256)
+    mid_long_k_max_rows: int = 256      # the products cut over K go to it up to this many rows with a long K (the down
+                                        # projection: 42 us against the library's 85 at 160 rows, 55 against 65 at 256)
+    mid_short_k_max_rows: int = 192     # ... and up to this many with a shorter one (the output projection: 19 us against 25 to
+                                        # 28 at 160 to 192 rows, no gain beyond)
     mid_min_slice_steps: int = 4        # a slice of K keeps at least this many macro-steps of 128
     mid_max_slices: int = 8
     # ---- the decode attention's cut of a request's keys into parts (attention_mfma.hip)

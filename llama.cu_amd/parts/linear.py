@@ -148,7 +148,7 @@ def library_friendly_rows(di: int, d: int, device) -> int:
 
 
 def _mid_slices(n_features: int, k: int) -> int:
-    """Into how many slices of K the kernel that shares the rows through LDS (up to 128 rows) cuts a product, so that about one
+    """Into how many slices of K the kernel that shares the rows through LDS (up to 256 rows) cuts a product, so that about one
     workgroup (64 features and a slice) stands on each compute unit; a slice keeps at least four
     macro-steps of 128."""
     t = ops.TUNING
@@ -157,7 +157,7 @@ def _mid_slices(n_features: int, k: int) -> int:
 
 
 def mid_takes(n_rows: int, weight: Union[torch.Tensor, Weight]) -> bool:
-    """Whether the kernel that shares the rows through LDS (up to 128 rows) is the faster choice for this many bfloat16 rows and
+    """Whether the kernel that shares the rows through LDS (up to 256 rows) is the faster choice for this many bfloat16 rows and
     this weight (measured against the library on the Llama-3-8B shapes: the products with few
     output features, which are cut over K, 10 to 30 % faster with a packed weight at 64 rows and
     more beyond, the down projection with a plain one too).  A packed weight with a long K (the
@@ -168,7 +168,8 @@ def mid_takes(n_rows: int, weight: Union[torch.Tensor, Weight]) -> bool:
     w, packed = _split(weight)
     long_k = w.dim() == 2 and w.shape[1] > t.mid_long_k
     fewest = t.mid_long_k_rows if (packed is not None and long_k) else t.skinny_rows_short_k
-    if not (fewest < n_rows <= ops.MID_MAX_ROWS and w.dtype == torch.bfloat16 and w.is_cuda and w.dim() == 2
+    most = min(ops.MID_MAX_ROWS, t.mid_long_k_max_rows if long_k else t.mid_short_k_max_rows)
+    if not (fewest < n_rows <= most and w.dtype == torch.bfloat16 and w.is_cuda and w.dim() == 2
             and w.shape[1] % 128 == 0 and w.shape[0] % 16 == 0):
         return False
     # products that are not cut over K stay with the library; a plain weight only with a long K (measured: the
@@ -192,7 +193,7 @@ def mid_swiglu_takes(n_rows: int, weight: Union[torch.Tensor, Weight]) -> bool:
     activation kernel after it, and from 15 rows on than the weight-streaming kernel: 46 against
     48 us at 16 rows, 52 to 55 from 17 on, on the Llama-3-8B shape)."""
     w, packed = _split(weight)
-    return (ops.TUNING.mid_swiglu_rows < n_rows <= ops.MID_MAX_ROWS and packed is not None and w.shape[0] % 32 == 0
+    return (ops.TUNING.mid_swiglu_rows < n_rows <= min(ops.MID_MAX_ROWS, ops.TUNING.mid_swiglu_max_rows) and packed is not None and w.shape[0] % 32 == 0
             and w.shape[1] % 128 == 0 and w.shape[0] >= ops.TUNING.mid_swiglu_features)
 
 

@@ -587,8 +587,8 @@ def test_gemm_skinny_refuses_what_it_cannot_take():
     assert not ops.skinny_supported(rnd(33, 64).to(torch.bfloat16).cuda(), rnd(16, 64).to(torch.bfloat16).cuda(), torch.bfloat16)
 
 
-# ------------------------------------------------------------------ product for 33 to 64 rows
-@pytest.mark.parametrize("m", [5, 33, 47, 48, 64, 65, 96, 97, 128])
+# ------------------------------------------------------------------ product that shares the rows through LDS (to 256 rows)
+@pytest.mark.parametrize("m", [5, 33, 47, 48, 64, 65, 96, 97, 128, 129, 177, 192, 193, 256])
 @pytest.mark.parametrize("n,k", [(16, 128), (208, 384), (1008, 1024), (64, 2176)])
 @pytest.mark.parametrize("packed", [False, True])
 def test_gemm_mid(m, n, k, packed):
@@ -614,7 +614,8 @@ def test_gemm_mid(m, n, k, packed):
         close(planes[0], plain.linear(x[:, :half], w[:, :half]), "float32", "first slice")
 
 
-@pytest.mark.parametrize("m,di,k", [(33, 16, 128), (40, 176, 256), (64, 1008, 640), (90, 176, 384), (128, 1008, 256)])
+@pytest.mark.parametrize("m,di,k", [(33, 16, 128), (40, 176, 256), (64, 1008, 640), (90, 176, 384), (128, 1008, 256),
+                                    (130, 176, 640), (192, 1008, 384), (255, 48, 1152), (256, 176, 128)])
 @pytest.mark.parametrize("packed", [False, True])
 def test_gemm_mid_swiglu(m, di, k, packed):
     from llama_cu_amd.kernels import ops
@@ -649,25 +650,26 @@ def test_gemm_mid_rows_that_wait_for_their_normalisation(m, di, k, parts):
 
 def test_gemm_mid_result_does_not_depend_on_the_batch_and_equals_the_sum_of_the_products():
     from llama_cu_amd.kernels import ops
-    x = rnd(110, 512, seed=1).to(torch.bfloat16).cuda()
+    x = rnd(250, 512, seed=1).to(torch.bfloat16).cuda()
     w = rnd(304, 512, seed=2).to(torch.bfloat16).cuda()
-    whole = ops.gemm_mid(x, w, slices=2)
-    one = ops.gemm_mid(x[23:24], w, slices=2)
-    assert torch.equal(whole[:, 23:24], one)
-    assert torch.equal(whole[:, 70:110], ops.gemm_mid(x[70:110], w, slices=2))
-    again = ops.gemm_mid(x, w, slices=2)
-    assert torch.equal(whole, again)
+    for rows in (110, 250):
+        whole = ops.gemm_mid(x[:rows], w, slices=2)
+        one = ops.gemm_mid(x[23:24], w, slices=2)
+        assert torch.equal(whole[:, 23:24], one)
+        assert torch.equal(whole[:, 70:110], ops.gemm_mid(x[70:110], w, slices=2))
+        again = ops.gemm_mid(x[:rows], w, slices=2)
+        assert torch.equal(whole, again)
 
 
 def test_gemm_mid_refuses_what_it_cannot_take():
     from llama_cu_amd.kernels import ops
     w = rnd(16, 128).to(torch.bfloat16).cuda()
-    assert not ops.mid_supported(rnd(129, 128).to(torch.bfloat16).cuda(), w)                # too many rows
+    assert not ops.mid_supported(rnd(257, 128).to(torch.bfloat16).cuda(), w)                # too many rows
     assert not ops.mid_supported(rnd(40, 136).to(torch.bfloat16).cuda(), rnd(16, 136).to(torch.bfloat16).cuda())   # K no multiple of 128
     assert not ops.mid_supported(rnd(40, 128).to(torch.bfloat16).cuda(), rnd(24, 128).to(torch.bfloat16).cuda())   # features no multiple of 16
     assert not ops.mid_supported(rnd(40, 128).cuda(), w)                                      # float32 rows
     with pytest.raises(ops.KernelError):
-        ops.gemm_mid(rnd(129, 128).to(torch.bfloat16).cuda(), w)
+        ops.gemm_mid(rnd(257, 128).to(torch.bfloat16).cuda(), w)
     with pytest.raises(ops.KernelError):                                                      # rows that wait for their factor: at most 64
         ops.gemm_mid(rnd(65, 128).to(torch.bfloat16).cuda(), w, row_sumsq=torch.ones(65, 4, device="cuda"), norm_width=128, eps=1e-5)
     with pytest.raises(ops.KernelError):

@@ -83,7 +83,7 @@ def test_long_requests_at_full_layer_sizes_through_the_four_traces(long_requests
     """Two layers of the Llama-3-8B shape with random weights from a seed, requests of 100, 1,300,
     2,500 and 600 tokens: whole; with the last 32 tokens decoded one by one (the decode kernel cuts
     2,500 keys into parts, and its steps are replayed from a captured graph); in portions of 1 to
-    700 tokens (prefill over a history of up to 2,000 keys); and mixed, four live requests with a
+    700 tokens (150 and 200 among them: the widest steps of the kernel that shares the rows through LDS) (prefill over a history of up to 2,000 keys); and mixed, four live requests with a
     pool so small that pages are used again, one of them losing its pages on the way and computed
     again.  Logits at the kept positions against the plain implementation."""
     from llama_cu_amd.engine.trace import TraceReplayer
@@ -93,7 +93,7 @@ def test_long_requests_at_full_layer_sizes_through_the_four_traces(long_requests
     elif mode == "tail":
         steps, max_tokens = common.trace_tail_decode(reqs, keep=keep)
     elif mode == "portions":
-        steps, max_tokens = common.trace_portions(reqs, sizes=(300, 2, 700, 17, 1, 512, 64, 5), keep=keep)
+        steps, max_tokens = common.trace_portions(reqs, sizes=(300, 2, 200, 700, 17, 1, 150, 512, 64, 5), keep=keep)
     else:
         steps, max_tokens = common.trace_mixed(reqs, seed=2, tail=20, sizes=(2, 3, 17, 48, 130, 300, 640), keep=keep,
                                                preempt=0.04)
@@ -186,6 +186,51 @@ def test_steps_of_33_to_64_rows_at_full_layer_sizes(big, dtype, monkeypatch):
     else:
         assert calls == {"planes": 0, "swiglu": 0}
     common.assert_matches_plain(got, want, dtype, f"8B-sized layers, 33 to 64 rows/{dtype}")
+
+
+def test_steps_of_129_to_256_rows_at_full_layer_sizes(long_requests, monkeypatch):
+    """Steps of 250, 192 (two requests) and 129 rows in bfloat16: the down projection of each, and the output
+    projection up to 192 rows, leave planes of partial sums from the kernel that shares the rows through LDS (its
+    ring of two buffers and three or four producer waves); gate/up stays with the library there."""
+    from llama_cu_amd.kernels import ops
+    calls = {"planes": 0, "swiglu": 0}
+    real = ops.gemm_mid
+
+    def counted(*a, **kw):
+        calls["swiglu" if kw.get("swiglu") else "planes"] += 1
+        return real(*a, **kw)
+    monkeypatch.setattr(ops, "gemm_mid", counted)
+    reqs, keep, want = long_requests
+    names = list(reqs)
+    a, b = names[1], names[3]                       # 1,300 and 600 tokens
+    runner = runner_for("bfloat16", max_tokens=1024, max_seqs=4)
+    got = {a: {}, b: {}}
+
+    def run(ids, parts, at0):
+        wanted = [[k for k in range(len(p)) if keep(n, o + k)] for n, p, o in zip(ids, parts, at0)]
+        logits = runner.step([names.index(n) for n in ids], parts, wanted).cpu().numpy()
+        row = 0
+        for n, o, w in zip(ids, at0, wanted):
+            for k in w:
+                got[n][o + k] = logits[row]; row += 1
+    run([a], [reqs[a][:250]], [0])
+    run([a, b], [reqs[a][250:400], reqs[b][:42]], [250, 0])
+    run([a], [reqs[a][400:529]], [400])
+    # of the two layers the last one's down projection ends in ordinary rows (the wanted rows are gathered before the
+    # final norm): 1 + 0 products in the step of 250 rows, 2 + 1 in each of the others
+    assert calls == {"planes": 7, "swiglu": 0}, calls
+    rel = common.REL_TOL["bfloat16"]
+    for n in (a, b):
+        at, ref = want[n]
+        ref = ref.numpy()
+        scale = float(np.abs(ref).max())
+        seen = 0
+        for row, pos in enumerate(at):
+            if pos in got[n]:
+                err = float(np.abs(got[n][pos].astype(np.float64) - ref[row]).max())
+                assert np.isfinite(err) and err <= rel * scale, f"request {n}, position {pos}: error {err:.3e} > {rel * scale:.3e}"
+                seen += 1
+        assert seen >= 3
 
 
 _plain_rows = {}
