@@ -30,6 +30,7 @@
 // wave w loads the shares of rows 16 w .. 16 w + 15 before its first loads of W, so they are back
 // first, adds them in a fixed order and leaves the factors in LDS for the epilogue.
 #include "common.h"
+#include "kv_layout.h"
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
@@ -371,3 +372,231 @@ LCU_API int lcu_gemm_mid_bf16_scaled(const void *X, int ldx, const void *W, int 
     const MidScale sc = {sumsq_in, n_in, norm_width, eps};
     return mid_bf16(X, ldx, W, ldw, Y, ldy, M, N, K, epilogue, slices, w_packed, sc, stream);
 }
+
+// ------------------------------------------------------------------------------------------------
+// The q, k, v product of an attention layer with the rotation and the cache write in its epilogue,
+// for more rows than gemm_skinny.hip's takes.  W holds the rows of the q heads, the k heads and the v
+// heads, head_dim each.  A rotation pairs dim i of a head with dim i + head_dim/2, so a workgroup takes
+// two tiles of one head, dims 16 c .. and head_dim/2 + 16 c .., over all of K; with so few features a
+// workgroup there are workgroups enough (192 for 48 heads of 128) without cutting K over workgroups,
+// which a rotation in the epilogue could not have.  Instead the four consumer waves share each
+// macro-step of 128 k: wave w multiplies the k that the w-th matrix instruction of a macro-step takes
+// (in the packed layout the w-th KB of a tile's 4 KB block), all four read the same rows of X from the
+// ring, and at the end they add their sums through LDS in the order of the waves.  Wave w then holds
+// the row tiles w, w + 4, .. of both tiles: it rounds q and k to bfloat16 (as the plain product
+// stores them for the rotation kernel), rotates them by the token's position, writes q to q_out and
+// k and v into the token's place in its page.
+template <int MT, bool PACKED>
+__global__ void __launch_bounds__((MID_CONSUMERS + mid_producers(MT)) * WAVE)
+gemm_mid_qkv_kernel(const bf16_t *__restrict__ X, int ldx, const bf16_t *__restrict__ W, int ldw, int M, int K,
+                    bf16_t *__restrict__ q_out, int ldq, const int *__restrict__ positions, const int *__restrict__ slots,
+                    const float *__restrict__ cos_t, const float *__restrict__ sin_t, int max_pos, bf16_t *__restrict__ cache,
+                    int heads, int kv_heads, int head_dim, int page) {
+    static_assert(MID_CONSUMERS == 4, "the four matrix instructions of a macro-step go to four waves");
+    extern __shared__ __attribute__((aligned(16))) char xs[];      // the ring of X; at the end the waves' sums
+    constexpr int BUF = 16 * MT * MID_XROW;
+    constexpr int XB = mid_xbufs(MT);
+    const int lane = threadIdx.x & (WAVE - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
+    const int l16 = lane & 15, grp = lane >> 4;
+    const int nst = K / 128;
+    if (wave == MID_CONSUMERS) {
+        mid_produce<MT, 0>(xs, X, ldx, M, 0, nst, lane);
+        return;
+    }
+    if constexpr (MT > 4) {
+        if (wave == MID_CONSUMERS + 1) {
+            mid_produce<MT, 1>(xs, X, ldx, M, 0, nst, lane);
+            return;
+        }
+    }
+    if constexpr (MT > 8) {
+        if (wave == MID_CONSUMERS + 2) {
+            mid_produce<MT, 2>(xs, X, ldx, M, 0, nst, lane);
+            return;
+        }
+    }
+    if constexpr (MT > 12) {
+        if (wave == MID_CONSUMERS + 3) {
+            mid_produce<MT, 3>(xs, X, ldx, M, 0, nst, lane);
+            return;
+        }
+    }
+    const int per_head = head_dim / 32;
+    const int head = blockIdx.x / per_head, c = blockIdx.x % per_head;
+    __amdgpu_buffer_rsrc_t wb[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+        const int tile = head * (head_dim / 16) + c + t * per_head;
+        wb[t] = PACKED ? __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t *>(W + (size_t)tile * nst * 2048), 0, (uint32_t)nst * 4096u, 0x00020000)
+                       : __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t *>(W + (size_t)16 * tile * ldw), 0,
+                                                           (uint32_t)(((size_t)15 * ldw + 128 * nst) * 2), 0x00020000);
+    }
+    const uint32_t w_lane = PACKED ? (uint32_t)lane * 16u + 1024u * wave : (uint32_t)(l16 * ldw + 32 * grp) * 2u + 16u * wave;
+    constexpr uint32_t w_step = PACKED ? 4096u : 256u;
+    f32x4 acc[2][MT];
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int m = 0; m < MT; ++m) acc[t][m] = f32x4{0.f, 0.f, 0.f, 0.f};
+    constexpr int STAGES = MT > 8 ? 8 : 16;            // macro-steps whose loads of W (1 KB a tile) are in flight
+    constexpr int MCHUNK = MT > 8 ? MT / 2 : MT;       // row tiles whose operands are read from LDS at a time
+    u32x4 w[STAGES][2];
+#define QKV_LOAD_W(i, step)                                                                             \
+    _Pragma("unroll") for (int t = 0; t < 2; ++t) w[i][t] = __builtin_bit_cast(                        \
+        u32x4, __builtin_amdgcn_raw_buffer_load_b128(wb[t], w_lane + (uint32_t)(step) * w_step, 0, PACKED ? MID_STREAM : 0))
+#pragma unroll
+    for (int i = 0; i < STAGES; ++i) QKV_LOAD_W(i, i);
+    const int x_off = l16 * MID_XROW + 64 * grp + 16 * wave;
+    lds_barrier();
+    int buf = 0;
+    for (int s = 0; s < nst; s += STAGES) {
+#pragma unroll
+        for (int i = 0; i < STAGES; ++i) {
+            const int cur = s + i;
+            if (cur < nst) {
+#pragma unroll
+                for (int m0 = 0; m0 < MT; m0 += MCHUNK) {
+                    u32x4 xf[MCHUNK];
+#pragma unroll
+                    for (int m = 0; m < MCHUNK; ++m) xf[m] = *(const u32x4 *)(xs + buf * BUF + x_off + 16 * (m0 + m) * MID_XROW);
+#pragma unroll
+                    for (int t = 0; t < 2; ++t)
+#pragma unroll
+                        for (int m = 0; m < MCHUNK; ++m) acc[t][m0 + m] = mid_mfma(w[i][t], xf[m], acc[t][m0 + m]);
+                }
+                QKV_LOAD_W(i, cur + STAGES);
+                buf = buf == XB - 1 ? 0 : buf + 1;
+                lds_barrier();
+            }
+        }
+    }
+#undef QKV_LOAD_W
+    // every wave has passed the last barrier: nobody reads the ring any more, the producers have ended.
+    // The waves' sums: [wave][tile][row tile][lane], 16 bytes each
+    f32x4 *sums = (f32x4 *)xs;
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int m = 0; m < MT; ++m) sums[((wave * 2 + t) * MT + m) * WAVE + lane] = acc[t][m];
+    lds_barrier();
+    const int half_dim = head_dim / 2;
+    const bool is_q = head < heads, is_k = !is_q && head < heads + kv_heads;
+#pragma unroll
+    for (int mi = 0; mi < (MT + MID_CONSUMERS - 1) / MID_CONSUMERS; ++mi) {
+        const int m = wave + MID_CONSUMERS * mi;
+        if (m >= MT) break;
+        f32x4 sum[2];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            sum[t] = sums[((0 * 2 + t) * MT + m) * WAVE + lane];
+#pragma unroll
+            for (int v = 1; v < MID_CONSUMERS; ++v) {
+                const f32x4 o = sums[((v * 2 + t) * MT + m) * WAVE + lane];
+                sum[t][0] += o[0]; sum[t][1] += o[1]; sum[t][2] += o[2]; sum[t][3] += o[3];
+            }
+        }
+        // the lane holds dims i0 .. i0 + 3 (tile 0) and head_dim/2 + i0 .. (tile 1) of token 16 m + l16
+        const int tok = 16 * m + l16;
+        if (tok >= M) continue;
+        const int i0 = 16 * c + 4 * grp;
+        const int pos = positions[tok];
+        const bool in_table = pos >= 0 && pos < max_pos;
+        const int slot = slots ? slots[tok] : -1;
+        bf16_t *pg = nullptr;
+        int place = 0;
+        if (!is_q && slot >= 0) {
+            pg = cache + (size_t)(slot / page) * kv_page_elems(kv_heads, head_dim, page);
+            place = slot % page;
+        }
+        bf16_t va[4], vb[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            // rounded to bfloat16 before the rotation, as the plain product stores them for the rotation
+            // kernel: a token's query and key are made the same way whichever kernel makes them
+            float a = to_f32(from_f32<bf16_t>(sum[0][r])), b = to_f32(from_f32<bf16_t>(sum[1][r]));
+            if (is_q || is_k) {
+                float cs = __uint_as_float(0x7fc00000u), sn = cs;         // a position outside the table gives NaN
+                if (in_table) { cs = cos_t[(size_t)pos * half_dim + i0 + r]; sn = sin_t[(size_t)pos * half_dim + i0 + r]; }
+                float ra, rb;
+                rotate_pair(a, b, cs, sn, ra, rb);
+                a = ra; b = rb;
+            }
+            va[r] = from_f32<bf16_t>(a);
+            vb[r] = from_f32<bf16_t>(b);
+        }
+        if (is_q) {
+            bf16_t *qo = q_out + (size_t)tok * ldq + (size_t)head * head_dim;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) { qo[i0 + r] = va[r]; qo[i0 + half_dim + r] = vb[r]; }
+        } else if (pg) {
+            if (is_k) {
+                const int kvh = head - heads;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    pg[kv_key_offset(kvh, place, i0 + r, head_dim, page)] = va[r];
+                    pg[kv_key_offset(kvh, place, i0 + half_dim + r, head_dim, page)] = vb[r];
+                }
+            } else {
+                const int kvh = head - heads - kv_heads;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    pg[kv_value_offset(kv_heads, kvh, place, i0 + r, head_dim, page)] = va[r];
+                    pg[kv_value_offset(kv_heads, kvh, place, i0 + half_dim + r, head_dim, page)] = vb[r];
+                }
+            }
+        }
+    }
+}
+
+// X: [M, K] bfloat16 rows ldx apart, M <= 256, K a multiple of 128; W: [(heads + 2 kv_heads) * head_dim, K] bfloat16 (q heads,
+// then k heads, then v heads), rows ldw apart or packed; head_dim a multiple of 32.  q_out: [M, heads * head_dim] rows
+// ldq apart takes the rotated queries; the rotated keys and the values go to cache (this layer's pages, laid out as
+// kv_layout.h says) at slots[m] (page * page_size + place; negative or slots null: nothing is stored).  cos_t, sin_t:
+// [max_pos, head_dim / 2] float32; pairs are (i, i + head_dim / 2).
+LCU_API int lcu_gemm_mid_bf16_qkv_rope(const void *X, int ldx, const void *W, int ldw, int M, int K, void *q_out, int ldq,
+                                       const int *positions, const int *slots, const float *cos_t, const float *sin_t,
+                                       int max_pos, void *cache, int heads, int kv_heads, int head_dim, int page,
+                                       int w_packed, hipStream_t stream) {
+    if (M <= 0) return LCU_OK;
+    if (M > 256 || K <= 0 || K % 128 || heads <= 0 || kv_heads <= 0 || head_dim <= 0 || head_dim % 32 || page <= 0 || page % 8 ||
+        !q_out || !positions || !cos_t || !sin_t || max_pos <= 0 || !cache || ldq < heads * head_dim || ldx % 8 || ldx < K)
+        return LCU_BAD_ARGUMENT;
+    if (!w_packed && (ldw % 8 || ldw < K)) return LCU_BAD_ARGUMENT;
+    if ((uintptr_t)X % 16 || (uintptr_t)W % 16) return LCU_BAD_ARGUMENT;
+    const dim3 grid((heads + 2 * kv_heads) * (head_dim / 32));
+#define GO(MT_, P_)                                                                                                         \
+    do {                                                                                                                    \
+        auto kernel = gemm_mid_qkv_kernel<MT_, P_>;                                                                         \
+        constexpr int lds = mid_xbufs(MT_) * 16 * MT_ * MID_XROW;                                                           \
+        static_assert(lds >= MID_CONSUMERS * 2 * MT_ * WAVE * 16, "the waves' sums lie over the ring");                     \
+        if (lds > 64 * 1024) {                                                                                              \
+            static bool asked = false;                                                                                      \
+            if (!asked) {                                                                                                   \
+                hipError_t e = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds); \
+                if (e != hipSuccess) return (int)e;                                                                         \
+                asked = true;                                                                                               \
+            }                                                                                                               \
+        }                                                                                                                   \
+        kernel<<<grid, dim3((MID_CONSUMERS + mid_producers(MT_)) * WAVE), lds, stream>>>(                                   \
+            (const bf16_t *)X, ldx, (const bf16_t *)W, ldw, M, K, (bf16_t *)q_out, ldq, positions, slots, cos_t, sin_t,    \
+            max_pos, (bf16_t *)cache, heads, kv_heads, head_dim, page);                                                     \
+    } while (0)
+#define GO_MT(MT_)                   \
+    do {                             \
+        if (w_packed) GO(MT_, true); \
+        else GO(MT_, false);         \
+    } while (0)
+    if (M <= 32) GO_MT(2);
+    else if (M <= 48) GO_MT(3);
+    else if (M <= 64) GO_MT(4);
+    else if (M <= 96) GO_MT(6);
+    else if (M <= 128) GO_MT(8);
+    else if (M <= 192) GO_MT(12);
+    else GO_MT(16);
+#undef GO_MT
+#undef GO
+    LCU_LAUNCH_CHECK();
+    return LCU_OK;
+}
+

@@ -853,6 +853,42 @@ def gemm_skinny_qkv_rope(x: torch.Tensor, w: torch.Tensor, positions: torch.Tens
     return q
 
 
+def mid_qkv_rope_supported(x: torch.Tensor, w: torch.Tensor, heads: int, kv_heads: int, head_dim: int) -> bool:
+    """Whether ``gemm_mid_qkv_rope`` takes these operands: what ``gemm_mid`` takes, and whole heads whose halves
+    are multiples of 16."""
+    return (head_dim % 32 == 0 and w.dim() == 2 and w.shape[0] == (heads + 2 * kv_heads) * head_dim and mid_supported(x, w))
+
+
+def gemm_mid_qkv_rope(x: torch.Tensor, w: torch.Tensor, positions: torch.Tensor, slots: torch.Tensor,
+                      cos: torch.Tensor, sin: torch.Tensor, cache: torch.Tensor, heads: int, kv_heads: int,
+                      head_dim: int, page_size: int, packed: bool = False) -> torch.Tensor:
+    """``gemm_skinny_qkv_rope`` for 17 to 256 rows: the q, k, v product with the rotation and the cache write in its
+    epilogue, by the kernel that shares the rows through LDS (its four consumer waves share each 128 k and add
+    their sums at the end; nothing is cut over workgroups).  Returns the rotated queries ``[rows, heads * head_dim]``."""
+    _gpu(x, w, positions, slots, cos, sin, cache)
+    if packed and not (packable(w) and w.is_contiguous()):
+        raise KernelError("gemm_mid_qkv_rope: a packed weight is a contiguous result of pack_weight")
+    _rows(x, "mid x"); _rows(w, "mid w")
+    m, k = x.shape
+    if w.shape[1] != k or not mid_qkv_rope_supported(x, w, heads, kv_heads, head_dim):
+        raise KernelError(f"gemm_mid_qkv_rope: x {tuple(x.shape)} {x.dtype} with w {tuple(w.shape)} {w.dtype}, {heads} + 2 * "
+                          f"{kv_heads} heads of {head_dim} is not supported")
+    _i32(positions, "positions", m); _i32(slots, "cache slots", m)
+    if cos.shape != sin.shape or cos.dtype != torch.float32 or sin.dtype != torch.float32 or cos.dim() != 2 \
+            or cos.shape[1] * 2 != head_dim or not cos.is_contiguous() or not sin.is_contiguous():
+        raise KernelError("rotation tables must be two contiguous float32 tensors [max_pos, head_dim/2]")
+    _contig(cache, "cache")
+    if cache.dtype != torch.bfloat16 or cache.dim() != 3 or cache.shape[1] != 2 \
+            or cache.shape[2] != kv_heads * head_dim * page_size or page_size % 8:
+        raise KernelError(f"cache: {cache.dtype} {tuple(cache.shape)}, expected bfloat16 [pages, 2, {kv_heads * head_dim * page_size}]")
+    q = torch.empty((m, heads * head_dim), dtype=torch.bfloat16, device=x.device)
+    lib = build.load("gemm_mid")
+    _check(lib.lcu_gemm_mid_bf16_qkv_rope(_ptr(x), x.stride(0), _ptr(w), w.stride(0), m, k, _ptr(q), q.stride(0),
+                                          _ptr(positions), _ptr(slots), _ptr(cos), _ptr(sin), cos.shape[0], _ptr(cache),
+                                          heads, kv_heads, head_dim, page_size, int(packed), _stream()), "gemm_mid_qkv_rope")
+    return q
+
+
 def skinny_f32_supported(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype) -> bool:
     """Whether the float32 weight-streaming kernel takes this product: all float32, K a
     multiple of 4 (16-byte loads)."""

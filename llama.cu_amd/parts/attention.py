@@ -15,7 +15,7 @@ import torch
 
 from ..kernels import ops
 from .base import BuildContext, PagedKV, Part, PartSpec, ScaledRows, TensorSpec, make_part, register_part
-from .linear import (Weight, linear, linear_into_norm, linear_planes, linear_qkv_rope, linear_scaled, mid_takes,
+from .linear import (Weight, linear, linear_into_norm, linear_planes, linear_qkv_rope, linear_scaled, mid_qkv_takes, mid_takes,
                      skinny_takes)
 from ..weights.loader import fused_rows
 
@@ -113,8 +113,9 @@ class Attention(Part):
         n_rows = (h.rows if isinstance(h, ScaledRows) else h).shape[0]
         qkv = None
         if store and self._rotation_only and rot is not None and pairing == 0 and rot_dim == dh \
-                and self.dtype == torch.bfloat16 and skinny_takes(n_rows, self.w_qkv, preferred=True):
-            # few rows: the product rotates q and k and writes k and v into the pages itself
+                and self.dtype == torch.bfloat16 and (skinny_takes(n_rows, self.w_qkv, preferred=True)
+                                                      or (not isinstance(h, ScaledRows) and mid_qkv_takes(n_rows, self.w_qkv))):
+            # up to 256 rows: the product rotates q and k and writes k and v into the pages itself
             qkv = linear_qkv_rope(h, self.w_qkv, step.positions, step.slots(cache.group), cos, sin, cache.pages,
                                   nh, nkv, dh, page_size)
         if qkv is None:

@@ -109,10 +109,14 @@ def library_friendly_rows(di: int, d: int, device) -> int:
     depends on the number of output features in ways that no rule predicts: with 2,048 rows and
     K = 4096 it takes 417 us for 22,016 features (the Llama-2-7B shape) and 320 us for 24,576.
     So a large matrix is timed once, at 2,048 rows, as it is and with each half filled up to the
-    next multiples of 1024, 2048 and 4096; rows are added only if that is at least 15 % faster.
+    next multiples of 1024, 2048 and 4096; rows are added only if that is at least 15 % faster
+    (``TUNING.library_rows`` fixes the answer instead, for runs that must not depend on a timing).
     The rows of zeros give zeros (silu(0) * 0), which whoever multiplies next leaves out."""
     if 2 * di * d < (1 << 25):
         return di                                   # small matrices: nothing to gain, and timings of a few us say nothing
+    fixed = ops.TUNING.library_rows                 # a run that must not depend on a timing says so there
+    if fixed >= 0:
+        return di if fixed == 0 else -(-di // fixed) * fixed
     key = (di, d, str(device))
     if key not in _friendly_rows:
         free, _ = torch.cuda.mem_get_info(device)
@@ -232,15 +236,31 @@ def linear_into_norm(a: torch.Tensor, weight: Union[torch.Tensor, Weight], resid
     return ops.gemm_skinny_add_norm(a, weight, residual, norm_weight)
 
 
+def mid_qkv_takes(n_rows: int, weight: Union[torch.Tensor, Weight]) -> bool:
+    """Whether the q, k, v product of this many rows goes to the kernel that shares the rows through LDS, with the
+    rotation and the cache write in its epilogue (with a packed weight, beyond the rows of the weight-streaming
+    kernel: it replaces the library's product and the rotation kernel after it)."""
+    w, packed = _split(weight)
+    t = ops.TUNING
+    return (packed is not None and t.mid_qkv_rows < n_rows <= min(ops.MID_MAX_ROWS, t.mid_qkv_max_rows)
+            and w.dim() == 2 and w.shape[1] % 128 == 0)
+
+
 def linear_qkv_rope(h, weight: Union[torch.Tensor, Weight], positions, slots, cos, sin, cache_pages, heads: int,
                     kv_heads: int, head_dim: int, page_size: int):
     """The q, k, v product with the rotation of q and k and the write of k and v into the cache in
-    its epilogue (``h``: bfloat16 rows or ScaledRows): returns the rotated queries, or None if the
-    kernel for it does not take these operands (then nothing has been done)."""
+    its epilogue (``h``: bfloat16 rows or ScaledRows): returns the rotated queries, or None if no
+    kernel for it takes these operands (then nothing has been done)."""
+    whole = weight
     weight, packed = _split(weight)
     rows = h.rows if isinstance(h, ScaledRows) else h
-    if not (rows.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and cache_pages.dtype == torch.bfloat16
-            and ops.qkv_rope_supported(rows, weight, heads, kv_heads, head_dim)):
+    if not (rows.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and cache_pages.dtype == torch.bfloat16):
+        return None
+    if not isinstance(h, ScaledRows) and mid_qkv_takes(rows.shape[0], whole) \
+            and ops.mid_qkv_rope_supported(rows, weight, heads, kv_heads, head_dim):
+        return ops.gemm_mid_qkv_rope(rows, packed, positions, slots, cos, sin, cache_pages, heads, kv_heads, head_dim,
+                                     page_size, packed=True)
+    if not ops.qkv_rope_supported(rows, weight, heads, kv_heads, head_dim):
         return None
     kw = dict(row_sumsq=h.sumsq, norm_width=h.width, eps=h.eps) if isinstance(h, ScaledRows) else {}
     if packed is not None:
@@ -248,4 +268,3 @@ def linear_qkv_rope(h, weight: Union[torch.Tensor, Weight], positions, slots, co
                                         page_size, packed=True, **kw)
     return ops.gemm_skinny_qkv_rope(rows, weight, positions, slots, cos, sin, cache_pages, heads, kv_heads, head_dim,
                                     page_size, **kw)
-

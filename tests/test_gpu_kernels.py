@@ -838,6 +838,88 @@ def test_gemm_skinny_q_k_v_with_rotation_and_cache_write(m, k, nh, nkv, dh, page
                                  2, 1, 48, page)
 
 
+@pytest.mark.parametrize("m,k,nh,nkv,dh,page,packed", [(5, 128, 4, 2, 32, 8, False), (33, 256, 6, 2, 64, 16, True),
+                                                       (48, 384, 3, 1, 96, 24, False), (64, 512, 8, 8, 128, 32, True),
+                                                       (65, 128, 5, 5, 160, 16, True), (100, 1152, 4, 2, 64, 16, True),
+                                                       (128, 256, 3, 3, 32, 8, False), (129, 640, 8, 2, 128, 16, True),
+                                                       (192, 128, 2, 1, 64, 48, True), (193, 256, 2, 2, 32, 16, False),
+                                                       (256, 2176, 4, 1, 128, 64, True)])
+def test_gemm_mid_q_k_v_with_rotation_and_cache_write(m, k, nh, nkv, dh, page, packed):
+    """The same for up to 256 rows, by the kernel that shares the rows through LDS (its consumer waves share each
+    128 k and add their sums at the end): against product, rotation and cache layout done one after the other; a
+    token that stores nothing; nothing else in the cache is touched; rows beyond the last are poison."""
+    from llama_cu_amd.kernels import ops
+    from llama_cu_amd.parts.position import Rotary
+    max_pos, theta = 700, 10000.0
+    pages = m // page + 4
+    n = (nh + 2 * nkv) * dh
+    cos, sin = Rotary(dh, theta, max_pos).host_tables()
+    sin_p, cos_p = plain.rope_tables(max_pos, dh, theta)
+    x = rnd(m, k, seed=m + k).to(torch.bfloat16)
+    w = rnd(n, k, seed=n, scale=0.3).to(torch.bfloat16)
+    pos = random.Random(1).sample(range(max_pos), m)
+    slots = random.Random(2).sample(range(pages * page), m)
+    if m > 2:
+        slots[2] = -1
+    cache = torch.full((pages, 2, nkv * dh * page), 7.0, dtype=torch.bfloat16).cuda()
+    buf = torch.full((m + 3, k + 8), float("nan"), dtype=torch.bfloat16, device="cuda")
+    buf[:m, :k] = x.cuda()
+    wg = ops.pack_weight(w.cuda()) if packed else w.cuda()
+    q_got = ops.gemm_mid_qkv_rope(buf[:m, :k], wg, torch.tensor(pos, dtype=torch.int32).cuda(),
+                                  torch.tensor(slots, dtype=torch.int32).cuda(), torch.from_numpy(cos).cuda(),
+                                  torch.from_numpy(sin).cuda(), cache, nh, nkv, dh, page, packed=packed)
+    qkv = plain.linear(x.double(), w)
+    q = qkv[:, :nh * dh].view(m, nh, dh)
+    kk = qkv[:, nh * dh:(nh + nkv) * dh].view(m, nkv, dh)
+    v = qkv[:, (nh + nkv) * dh:].view(m, nkv, dh)
+    close(q_got.reshape(m, nh, dh), plain.rope(q, pos, sin_p, cos_p, "half"), "bfloat16", "q")
+    k_want = plain.rope(kk, pos, sin_p, cos_p, "half")
+    flat = cache.cpu().view(pages, -1)
+    expect = torch.full_like(flat, 7.0).double()
+    written = torch.zeros_like(flat, dtype=torch.bool)
+    dims = torch.arange(dh)
+    for t in range(m):
+        if slots[t] < 0:
+            continue
+        pg, tok = slots[t] // page, slots[t] % page
+        for h in range(nkv):
+            ko = torch.tensor([key_offset(h, tok, int(c), dh, page) for c in dims])
+            vo = torch.tensor([value_offset(nkv, h, tok, int(c), dh, page) for c in dims])
+            expect[pg, ko] = k_want[t, h]
+            expect[pg, vo] = v[t, h]
+            written[pg, ko] = True
+            written[pg, vo] = True
+    close(flat, expect, "bfloat16", "cache")
+    assert bool((flat[~written] == 7.0).all())                              # nothing else was touched
+    # the same bits as the product in bfloat16 followed by the rotation kernel, when the sums agree: the product that
+    # shares the rows adds a row's k in another order than this kernel's four waves, so only nearly
+    cache_b = torch.full_like(cache, 7.0)
+    rows = ops.gemm_mid(buf[:m, :k], wg, packed=packed)
+    ops.rope_kv_store(rows, torch.tensor(pos, dtype=torch.int32).cuda(), nh, nkv, dh, torch.from_numpy(cos).cuda(),
+                      torch.from_numpy(sin).cuda(), dh, 0, cache_b, torch.tensor(slots, dtype=torch.int32).cuda(), page)
+    assert float((q_got.float() - rows[:, :nh * dh].float()).abs().max()) <= 0.02 * float(rows.float().abs().max())
+    assert float((cache.float() - cache_b.float()).abs().max()) <= 0.02 * float(cache_b.float().abs().max())
+
+
+def test_gemm_mid_q_k_v_refuses_what_it_cannot_take():
+    from llama_cu_amd.kernels import ops
+    page, max_pos = 16, 64
+    z = lambda *s: torch.zeros(*s, dtype=torch.int32).cuda()
+    tables = lambda dh: (torch.zeros(max_pos, dh // 2).cuda(), torch.zeros(max_pos, dh // 2).cuda())
+    cache = lambda nkv, dh: torch.zeros(2, 2, nkv * dh * page, dtype=torch.bfloat16).cuda()
+    x = rnd(40, 128).to(torch.bfloat16).cuda()
+    with pytest.raises(ops.KernelError):                                    # halves of a head that are no multiple of 16
+        ops.gemm_mid_qkv_rope(x, rnd(4 * 48, 128).to(torch.bfloat16).cuda(), z(40), z(40), *tables(48), cache(1, 48), 2, 1, 48, page)
+    with pytest.raises(ops.KernelError):                                    # more than 256 rows
+        ops.gemm_mid_qkv_rope(rnd(257, 128).to(torch.bfloat16).cuda(), rnd(4 * 64, 128).to(torch.bfloat16).cuda(), z(257), z(257),
+                              *tables(64), cache(1, 64), 2, 1, 64, page)
+    with pytest.raises(ops.KernelError):                                    # K no multiple of 128
+        ops.gemm_mid_qkv_rope(rnd(40, 136).to(torch.bfloat16).cuda(), rnd(4 * 64, 136).to(torch.bfloat16).cuda(), z(40), z(40),
+                              *tables(64), cache(1, 64), 2, 1, 64, page)
+    with pytest.raises(ops.KernelError):                                    # a weight that is not q, k and v heads
+        ops.gemm_mid_qkv_rope(x, rnd(3 * 64, 128).to(torch.bfloat16).cuda(), z(40), z(40), *tables(64), cache(1, 64), 2, 1, 64, page)
+
+
 @pytest.mark.parametrize("m", [1, 17, 32])
 @pytest.mark.parametrize("packed,scaled", [(False, False), (True, True)])
 def test_q_k_v_epilogue_leaves_the_same_bits_as_product_then_rotation_kernel(m, packed, scaled):

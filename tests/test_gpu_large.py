@@ -188,39 +188,38 @@ def test_steps_of_33_to_64_rows_at_full_layer_sizes(big, dtype, monkeypatch):
     common.assert_matches_plain(got, want, dtype, f"8B-sized layers, 33 to 64 rows/{dtype}")
 
 
-def test_steps_of_129_to_256_rows_at_full_layer_sizes(long_requests, monkeypatch):
-    """Steps of 250, 192 (two requests) and 129 rows in bfloat16: the down projection of each, and the output
-    projection up to 192 rows, leave planes of partial sums from the kernel that shares the rows through LDS (its
-    ring of two buffers and three or four producer waves); gate/up stays with the library there."""
+def _wide_steps(long_requests, monkeypatch, plan):
+    """Runs ``plan`` (a list of steps, each a list of (request index, from, to)) in bfloat16 on the requests of 1,300
+    and 600 tokens, compares the kept positions with the plain model and returns how often each kernel of the
+    row-sharing product was called."""
     from llama_cu_amd.kernels import ops
-    calls = {"planes": 0, "swiglu": 0}
-    real = ops.gemm_mid
+    calls = {"planes": 0, "swiglu": 0, "qkv": 0}
+    real, real_qkv = ops.gemm_mid, ops.gemm_mid_qkv_rope
 
     def counted(*a, **kw):
         calls["swiglu" if kw.get("swiglu") else "planes"] += 1
         return real(*a, **kw)
-    monkeypatch.setattr(ops, "gemm_mid", counted)
-    reqs, keep, want = long_requests
-    names = list(reqs)
-    a, b = names[1], names[3]                       # 1,300 and 600 tokens
-    runner = runner_for("bfloat16", max_tokens=1024, max_seqs=4)
-    got = {a: {}, b: {}}
 
-    def run(ids, parts, at0):
-        wanted = [[k for k in range(len(p)) if keep(n, o + k)] for n, p, o in zip(ids, parts, at0)]
-        logits = runner.step([names.index(n) for n in ids], parts, wanted).cpu().numpy()
+    def counted_qkv(*a, **kw):
+        calls["qkv"] += 1
+        return real_qkv(*a, **kw)
+    monkeypatch.setattr(ops, "gemm_mid", counted)
+    monkeypatch.setattr(ops, "gemm_mid_qkv_rope", counted_qkv)
+    reqs, keep, want = long_requests
+    names = [list(reqs)[1], list(reqs)[3]]          # 1,300 and 600 tokens
+    runner = runner_for("bfloat16", max_tokens=1024, max_seqs=4)
+    got = {n: {} for n in names}
+    for step in plan:
+        ids = [names[i] for i, _, _ in step]
+        parts = [reqs[names[i]][lo:hi] for i, lo, hi in step]
+        wanted = [[k for k in range(hi - lo) if keep(names[i], lo + k)] for i, lo, hi in step]
+        logits = runner.step([i for i, _, _ in step], parts, wanted).cpu().numpy()
         row = 0
-        for n, o, w in zip(ids, at0, wanted):
+        for (i, lo, hi), w in zip(step, wanted):
             for k in w:
-                got[n][o + k] = logits[row]; row += 1
-    run([a], [reqs[a][:250]], [0])
-    run([a, b], [reqs[a][250:400], reqs[b][:42]], [250, 0])
-    run([a], [reqs[a][400:529]], [400])
-    # of the two layers the last one's down projection ends in ordinary rows (the wanted rows are gathered before the
-    # final norm): 1 + 0 products in the step of 250 rows, 2 + 1 in each of the others
-    assert calls == {"planes": 7, "swiglu": 0}, calls
+                got[names[i]][lo + k] = logits[row]; row += 1
     rel = common.REL_TOL["bfloat16"]
-    for n in (a, b):
+    for n in names:
         at, ref = want[n]
         ref = ref.numpy()
         scale = float(np.abs(ref).max())
@@ -231,6 +230,26 @@ def test_steps_of_129_to_256_rows_at_full_layer_sizes(long_requests, monkeypatch
                 assert np.isfinite(err) and err <= rel * scale, f"request {n}, position {pos}: error {err:.3e} > {rel * scale:.3e}"
                 seen += 1
         assert seen >= 3
+    return calls
+
+
+def test_steps_of_129_to_256_rows_at_full_layer_sizes(long_requests, monkeypatch):
+    """Steps of 250, 192 (two requests) and 129 rows in bfloat16: the down projection of each, and the output
+    projection up to 192 rows, leave planes of partial sums from the kernel that shares the rows through LDS (its
+    ring of two buffers and three or four producer waves); gate/up and q/k/v stay with the library there."""
+    calls = _wide_steps(long_requests, monkeypatch, [[(0, 0, 250)], [(0, 250, 400), (1, 0, 42)], [(0, 400, 529)]])
+    # of the two layers the last one's down projection ends in ordinary rows (the wanted rows are gathered before the
+    # final norm): 1 + 0 products in the step of 250 rows, 2 + 1 in each of the others
+    assert calls == {"planes": 7, "swiglu": 0, "qkv": 0}, calls
+
+
+def test_steps_of_65_to_128_rows_at_full_layer_sizes(long_requests, monkeypatch):
+    """Steps of 100, 128 (two requests) and 65 rows in bfloat16: q/k/v with the rotation and the cache write in the
+    epilogue of the kernel that shares the rows through LDS, whose waves share each 128 k (the keys that the later
+    steps read were written by it), beside its planes and its SwiGLU."""
+    calls = _wide_steps(long_requests, monkeypatch, [[(0, 0, 100)], [(0, 100, 190), (1, 0, 38)], [(1, 38, 103)]])
+    layers = SHAPE["num_hidden_layers"]
+    assert calls["qkv"] == 3 * layers and calls["swiglu"] >= 3 * (layers - 1) and calls["planes"] >= 3, calls
 
 
 _plain_rows = {}

@@ -30,3 +30,17 @@ def test_the_layers_of_a_model_share_one_pair_of_rotation_tables():
     del parts, p, other, cos, sin
     gc.collect()
     assert len(position._tables) == 0
+
+
+def test_the_rows_of_zeros_for_the_library_can_be_fixed_instead_of_timed(monkeypatch):
+    """``Tuning.library_rows``: 0 never fills the halves of a gate/up matrix up, n fills them up to a multiple of n;
+    neither times anything (the default, -1, times the library on the GPU once per shape)."""
+    import dataclasses
+    from llama_cu_amd.kernels import ops
+    from llama_cu_amd.parts import linear
+    monkeypatch.setattr(ops, "TUNING", dataclasses.replace(ops.TUNING, library_rows=0))
+    assert linear.library_friendly_rows(11008, 4096, "cpu") == 11008
+    monkeypatch.setattr(ops, "TUNING", dataclasses.replace(ops.TUNING, library_rows=2048))
+    assert linear.library_friendly_rows(11008, 4096, "cpu") == 12288
+    assert linear.library_friendly_rows(14336, 4096, "cpu") == 14336
+    assert linear.library_friendly_rows(176, 64, "cpu") == 176            # small matrices stay as they are

@@ -35,12 +35,14 @@ def test_decode_attention_that_allocates_nothing_equals_the_one_that_is_given_it
     limit = lib.lcu_attention_static_scratch_bytes()
     assert limit == 16 << 20
     assert lib.lcu_attention_static_init() == 0
-    nh, nkv, dh, page = 8, 2, 128, 16
     # the first call is the larger one: five requests in six parts; the second, three requests in four parts, runs
-    # over what the first left in the buffer
-    for ctx_lens, splits in (([700, 33, 2049, 1, 512], 6), ([300, 64, 1500], 4), ([90, 17], 1)):
+    # over what the first left in the buffer; then other head sizes, head counts and page sizes over what those left
+    calls = [((8, 2, 128, 16), [700, 33, 2049, 1, 512], 6), ((8, 2, 128, 16), [300, 64, 1500], 4), ((8, 2, 128, 16), [90, 17], 1),
+             ((6, 3, 64, 32), [400, 77, 1030, 2], 5), ((6, 3, 64, 32), [129, 9], 2), ((4, 4, 96, 48), [1000, 333], 3),
+             ((16, 1, 32, 16), [65], 2)]
+    for (nh, nkv, dh, page), ctx_lens, splits in calls:
         n = len(ctx_lens)
-        q, cache, step, _ = paged_case("bfloat16", nh, nkv, dh, page, [1] * n, ctx_lens, 0, seed=n)
+        q, cache, step, _ = paged_case("bfloat16", nh, nkv, dh, page, [1] * n, ctx_lens, 0, seed=n + dh)
         q, cache = q.cuda(), cache.cuda()
         need = lib.lcu_attention_static_scratch_needed(n, nh, dh, splits)
         assert need == (n * nh * splits * (dh + 2) * 4 if splits > 1 else 0) and need <= limit
@@ -56,7 +58,8 @@ def test_decode_attention_that_allocates_nothing_equals_the_one_that_is_given_it
         # the call took no memory from the driver (the kernels are loaded: the other entry point has just run them)
         assert torch.cuda.mem_get_info()[0] == free_before, (free_before, torch.cuda.mem_get_info()[0])
         assert torch.isfinite(want.float()).all()
-        assert torch.equal(got, want), f"{n} requests in {splits} parts"
+        assert torch.equal(got, want), f"{n} requests in {splits} parts, head size {dh}"
+    nh, nkv, dh, page = 8, 2, 128, 16
     # more than the buffer holds: refused, nothing launched, the output untouched
     n, splits = 64, 512
     assert lib.lcu_attention_static_scratch_needed(n, nh, dh, splits) > limit
