@@ -112,8 +112,8 @@ __device__ __forceinline__ void mid_produce(char *xs, const bf16_t *__restrict__
 #undef MID_LOAD_X
 }
 
-template <int NT, int MT, int EPI, bool PACKED>
-__global__ void __launch_bounds__((MID_CONSUMERS + mid_producers(MT)) * WAVE)
+template <int NT, int MT, int EPI, bool PACKED, int C>
+__global__ void __launch_bounds__((C + mid_producers(MT)) * WAVE)
 gemm_mid_kernel(const bf16_t *__restrict__ X, int ldx, const bf16_t *__restrict__ W, int ldw, void *__restrict__ Y, int ldy,
                 int M, int N, int K, int steps_per_slice, const float *__restrict__ sumsq_in, int n_in, int norm_width,
                 float eps) {
@@ -129,24 +129,24 @@ gemm_mid_kernel(const bf16_t *__restrict__ X, int ldx, const bf16_t *__restrict_
     const int s_end = min(steps_total, s_begin + steps_per_slice);
     const int nst = s_end - s_begin;                 // the same for every wave of the workgroup (at least 1)
 
-    if (wave == MID_CONSUMERS) {
+    if (wave == C) {
         mid_produce<MT, 0>(xs, X, ldx, M, s_begin, nst, lane);
         return;
     }
     if constexpr (MT > 4) {
-        if (wave == MID_CONSUMERS + 1) {
+        if (wave == C + 1) {
             mid_produce<MT, 1>(xs, X, ldx, M, s_begin, nst, lane);
             return;
         }
     }
     if constexpr (MT > 8) {
-        if (wave == MID_CONSUMERS + 2) {
+        if (wave == C + 2) {
             mid_produce<MT, 2>(xs, X, ldx, M, s_begin, nst, lane);
             return;
         }
     }
     if constexpr (MT > 12) {
-        if (wave == MID_CONSUMERS + 3) {
+        if (wave == C + 3) {
             mid_produce<MT, 3>(xs, X, ldx, M, s_begin, nst, lane);
             return;
         }
@@ -154,7 +154,7 @@ gemm_mid_kernel(const bf16_t *__restrict__ X, int ldx, const bf16_t *__restrict_
 
     // -------------------------------------------------------------------- consumers of W
     // tile t of the wave: rows of W.  SwiGLU: tile 0 a gate tile, tile 1 the up tile N/2 further.
-    const int tile0 = blockIdx.x * MID_CONSUMERS + wave;
+    const int tile0 = blockIdx.x * C + wave;
     const int n_tiles = (EPI == MID_EPI_SWIGLU ? N / 2 : N) / 16;
     const bool live = tile0 < n_tiles;               // a wave beyond the last tile reads the last one and stores nothing
     // W comes through buffer resources, one per tile, that end with the slice: the loads of the
@@ -284,16 +284,20 @@ struct MidScale {
     float eps;
 };
 
-template <int NT, int EPI>
-static int mid_launch(const void *X, int ldx, const void *W, int ldw, void *Y, int ldy, int M, int N, int K, int packed,
-                      int slices, const MidScale &sc, hipStream_t stream) {
+// The number of consumer waves: four; two for SwiGLU with up to 32 rows, where a workgroup of four takes 128 rows of
+// W and the 224 workgroups of a 28,672-row gate/up matrix leave an eighth of the compute units idle (448 workgroups of
+// two, two to a compute unit: 39.8 against 44.0 us at 24 rows; from 48 rows on the four are faster, each workgroup
+// reads all rows of X).
+template <int NT, int EPI, int C>
+static int mid_launch_c(const void *X, int ldx, const void *W, int ldw, void *Y, int ldy, int M, int N, int K, int packed,
+                        int slices, const MidScale &sc, hipStream_t stream) {
     const int n_tiles = (EPI == MID_EPI_SWIGLU ? N / 2 : N) / 16;
     const int steps = K / 128, per = (steps + slices - 1) / slices;
-    const dim3 grid((n_tiles + MID_CONSUMERS - 1) / MID_CONSUMERS, (steps + per - 1) / per);
-    // the ring of 65 to 128 rows takes more LDS than a kernel has without asking
+    const dim3 grid((n_tiles + C - 1) / C, (steps + per - 1) / per);
+    // the ring of 65 to 256 rows takes more LDS than a kernel has without asking
 #define GO(MT_, P_)                                                                                                         \
     do {                                                                                                                    \
-        auto kernel = gemm_mid_kernel<NT, MT_, EPI, P_>;                                                                    \
+        auto kernel = gemm_mid_kernel<NT, MT_, EPI, P_, C>;                                                                 \
         if (mid_lds_bytes(MT_) > 64 * 1024) {                                                                               \
             static bool asked = false;                                                                                      \
             if (!asked) {                                                                                                   \
@@ -303,7 +307,7 @@ static int mid_launch(const void *X, int ldx, const void *W, int ldw, void *Y, i
                 asked = true;                                                                                               \
             }                                                                                                               \
         }                                                                                                                   \
-        kernel<<<grid, dim3((MID_CONSUMERS + mid_producers(MT_)) * WAVE), mid_lds_bytes(MT_), stream>>>(                    \
+        kernel<<<grid, dim3((C + mid_producers(MT_)) * WAVE), mid_lds_bytes(MT_), stream>>>(                                \
             (const bf16_t *)X, ldx, (const bf16_t *)W, ldw, Y, ldy, M, N, K, per, sc.sumsq_in, sc.n_in, sc.norm_width, sc.eps); \
     } while (0)
 #define GO_MT(MT_)                 \
@@ -311,17 +315,30 @@ static int mid_launch(const void *X, int ldx, const void *W, int ldw, void *Y, i
         if (packed) GO(MT_, true); \
         else GO(MT_, false);       \
     } while (0)
-    if (M <= 32) GO_MT(2);
-    else if (M <= 48) GO_MT(3);
-    else if (M <= 64) GO_MT(4);
-    else if (M <= 96) GO_MT(6);
-    else if (M <= 128) GO_MT(8);
-    else if (M <= 192) GO_MT(12);
-    else GO_MT(16);
+    if constexpr (C < MID_CONSUMERS) {
+        GO_MT(2);                                   // (chosen for up to 32 rows only)
+    } else {
+        if (M <= 32) GO_MT(2);
+        else if (M <= 48) GO_MT(3);
+        else if (M <= 64) GO_MT(4);
+        else if (M <= 96) GO_MT(6);
+        else if (M <= 128) GO_MT(8);
+        else if (M <= 192) GO_MT(12);
+        else GO_MT(16);
+    }
 #undef GO_MT
 #undef GO
     LCU_LAUNCH_CHECK();
     return LCU_OK;
+}
+
+template <int NT, int EPI>
+static int mid_launch(const void *X, int ldx, const void *W, int ldw, void *Y, int ldy, int M, int N, int K, int packed,
+                      int slices, const MidScale &sc, hipStream_t stream) {
+    if constexpr (EPI == MID_EPI_SWIGLU && MID_CONSUMERS == 4) {
+        if (M <= 32) return mid_launch_c<NT, EPI, 2>(X, ldx, W, ldw, Y, ldy, M, N, K, packed, slices, sc, stream);
+    }
+    return mid_launch_c<NT, EPI, MID_CONSUMERS>(X, ldx, W, ldw, Y, ldy, M, N, K, packed, slices, sc, stream);
 }
 
 // X: [M, K] bfloat16 rows ldx apart, M <= 256 (rows that wait for their normalisation: M <= 64); W: [N, K] bfloat16, rows ldw apart or packed; K a
@@ -373,6 +390,7 @@ LCU_API int lcu_gemm_mid_bf16_scaled(const void *X, int ldx, const void *W, int 
     return mid_bf16(X, ldx, W, ldw, Y, ldy, M, N, K, epilogue, slices, w_packed, sc, stream);
 }
 
+#if LCU_MID_CONSUMERS == 4
 // ------------------------------------------------------------------------------------------------
 // The q, k, v product of an attention layer with the rotation and the cache write in its epilogue,
 // for more rows than gemm_skinny.hip's takes.  W holds the rows of the q heads, the k heads and the v
@@ -549,6 +567,8 @@ gemm_mid_qkv_kernel(const bf16_t *__restrict__ X, int ldx, const bf16_t *__restr
     }
 }
 
+#endif
+
 // X: [M, K] bfloat16 rows ldx apart, M <= 256, K a multiple of 128; W: [(heads + 2 kv_heads) * head_dim, K] bfloat16 (q heads,
 // then k heads, then v heads), rows ldw apart or packed; head_dim a multiple of 32.  q_out: [M, heads * head_dim] rows
 // ldq apart takes the rotated queries; the rotated keys and the values go to cache (this layer's pages, laid out as
@@ -564,6 +584,7 @@ LCU_API int lcu_gemm_mid_bf16_qkv_rope(const void *X, int ldx, const void *W, in
         return LCU_BAD_ARGUMENT;
     if (!w_packed && (ldw % 8 || ldw < K)) return LCU_BAD_ARGUMENT;
     if ((uintptr_t)X % 16 || (uintptr_t)W % 16) return LCU_BAD_ARGUMENT;
+#if LCU_MID_CONSUMERS == 4
     const dim3 grid((heads + 2 * kv_heads) * (head_dim / 32));
 #define GO(MT_, P_)                                                                                                         \
     do {                                                                                                                    \
@@ -598,5 +619,8 @@ LCU_API int lcu_gemm_mid_bf16_qkv_rope(const void *X, int ldx, const void *W, in
 #undef GO
     LCU_LAUNCH_CHECK();
     return LCU_OK;
+#else
+    return LCU_BAD_ARGUMENT;       // an experimental build with another number of consumer waves has no such kernel
+#endif
 }
 

@@ -34,7 +34,7 @@ class Tuning:
     mid_long_k_rows: int = 11           # ... above this many rows (whole decode steps: 0.9 % faster at 12 rows, 3 % at 16;
                                         # 0.3 % slower at 11: below, the weight-streaming kernel with the norm in its epilogue)
     mid_swiglu_features: int = 8192     # gate/up with SwiGLU goes to it from this many rows of the weight on,
-    mid_swiglu_rows: int = 14           # above this many rows of the batch (0.4 % at 16 rows, nothing below 15)
+    mid_swiglu_rows: int = 14           # above this many rows of the batch (whole steps: 2.8 % at 16 rows, nothing at 14, slower below)
     mid_swiglu_max_rows: int = 128      # ... up to this many (at 128 rows 61 us against the library's 59 with the activation
                                         # kernel, beyond that the library is ahead: 69 against 63 at 160 rows, 80 against 72 at 256)
     mid_long_k_max_rows: int = 256      # the products cut over K go to it up to this many rows with a long K (the down

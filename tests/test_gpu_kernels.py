@@ -614,7 +614,7 @@ def test_gemm_mid(m, n, k, packed):
         close(planes[0], plain.linear(x[:, :half], w[:, :half]), "float32", "first slice")
 
 
-@pytest.mark.parametrize("m,di,k", [(33, 16, 128), (40, 176, 256), (64, 1008, 640), (90, 176, 384), (128, 1008, 256),
+@pytest.mark.parametrize("m,di,k", [(15, 48, 128), (17, 176, 256), (32, 1008, 384), (33, 16, 128), (40, 176, 256), (64, 1008, 640), (90, 176, 384), (128, 1008, 256),
                                     (130, 176, 640), (192, 1008, 384), (255, 48, 1152), (256, 176, 128)])
 @pytest.mark.parametrize("packed", [False, True])
 def test_gemm_mid_swiglu(m, di, k, packed):
