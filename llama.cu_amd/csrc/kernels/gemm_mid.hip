@@ -154,9 +154,12 @@ gemm_mid_kernel(const bf16_t *__restrict__ X, int ldx, const bf16_t *__restrict_
 
     // -------------------------------------------------------------------- consumers of W
     // tile t of the wave: rows of W.  SwiGLU: tile 0 a gate tile, tile 1 the up tile N/2 further.
-    const int tile0 = blockIdx.x * C + wave;
+    // the workgroups share the tiles evenly, up to C each: workgroup b takes tiles b n / G .. (b + 1) n / G - 1 of n
     const int n_tiles = (EPI == MID_EPI_SWIGLU ? N / 2 : N) / 16;
-    const bool live = tile0 < n_tiles;               // a wave beyond the last tile reads the last one and stores nothing
+    const int tile_begin = (int)((long long)blockIdx.x * n_tiles / gridDim.x);
+    const int tile_end = (int)((long long)(blockIdx.x + 1) * n_tiles / gridDim.x);
+    const int tile0 = tile_begin + wave;
+    const bool live = tile0 < tile_end;              // a wave without a tile reads nothing (a buffer of no bytes) and stores nothing
     // W comes through buffer resources, one per tile, that end with the slice: the loads of the
     // ring stand under no branch, and a macro-step beyond the slice reads zeros (packed) or
     // what lies further in the rows (plain; past the matrix's last row zeros) and is not used.
@@ -165,9 +168,9 @@ gemm_mid_kernel(const bf16_t *__restrict__ X, int ldx, const bf16_t *__restrict_
     for (int t = 0; t < NT; ++t) {
         const int tile = (live ? tile0 : n_tiles - 1) + t * n_tiles;
         wb[t] = PACKED ? __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t *>(W + ((size_t)tile * steps_total + s_begin) * 2048), 0,
-                                                             (uint32_t)nst * 4096u, 0x00020000)
+                                                             live ? (uint32_t)nst * 4096u : 0u, 0x00020000)
                          : __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t *>(W + (size_t)16 * tile * ldw + (size_t)128 * s_begin), 0,
-                                                             (uint32_t)(((size_t)15 * ldw + 128 * nst) * 2), 0x00020000);
+                                                             live ? (uint32_t)(((size_t)15 * ldw + 128 * nst) * 2) : 0u, 0x00020000);
     }
     // the step and the load within it are constants of the instruction, the lane adds its place once a step
     const uint32_t w_lane = PACKED ? (uint32_t)lane * 16u : (uint32_t)(l16 * ldw + 32 * grp) * 2u;
@@ -278,22 +281,42 @@ gemm_mid_kernel(const bf16_t *__restrict__ X, int ldx, const bf16_t *__restrict_
     }
 }
 
+// The number of compute units of the current device (asked once per device).
+static int mid_compute_units() {
+    static int units[64] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
+    if (units[dev] == 0) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) n = 0;
+        units[dev] = n > 0 ? n : -1;
+    }
+    return units[dev] > 0 ? units[dev] : 0;
+}
+
 struct MidScale {
     const float *sumsq_in;
     int n_in, norm_width;
     float eps;
 };
 
-// The number of consumer waves: four; two for SwiGLU with up to 32 rows, where a workgroup of four takes 128 rows of
-// W and the 224 workgroups of a 28,672-row gate/up matrix leave an eighth of the compute units idle (448 workgroups of
-// two, two to a compute unit: 39.8 against 44.0 us at 24 rows; from 48 rows on the four are faster, each workgroup
-// reads all rows of X).
+// The number of consumer waves: four; two for SwiGLU with up to 32 rows (workgroups of two tiles, two to a compute
+// unit: 39.8 against 44.0 us at 24 rows of a 28,672-row gate/up matrix).
 template <int NT, int EPI, int C>
 static int mid_launch_c(const void *X, int ldx, const void *W, int ldw, void *Y, int ldy, int M, int N, int K, int packed,
                         int slices, const MidScale &sc, hipStream_t stream) {
     const int n_tiles = (EPI == MID_EPI_SWIGLU ? N / 2 : N) / 16;
     const int steps = K / 128, per = (steps + slices - 1) / slices;
-    const dim3 grid((n_tiles + C - 1) / C, (steps + per - 1) / per);
+    // workgroups: as many as take C tiles each; where K is not cut and a workgroup reads few rows (up to 64), the next
+    // multiple of the number of compute units, so that none of them idles (28,672 rows of gate/up are 224 workgroups of
+    // four tiles: as 256 workgroups of three and four tiles 41.8 against 45.2 us at 64 rows; beyond 64 rows more
+    // workgroups cost more in reads of X than they gain)
+    int groups = (n_tiles + C - 1) / C;
+    if (slices == 1 && M <= 64) {
+        const int units = mid_compute_units();
+        if (units > 0) groups = min(n_tiles, (groups + units - 1) / units * units);
+    }
+    const dim3 grid(groups, (steps + per - 1) / per);
     // the ring of 65 to 256 rows takes more LDS than a kernel has without asking
 #define GO(MT_, P_)                                                                                                         \
     do {                                                                                                                    \
