@@ -523,10 +523,11 @@ def decode_splits(n_req: int, n_heads: int, n_kv_heads: int, max_ctx_len: int) -
     32 parts (measured from 2k to 128k keys: more parts cost more in the merge than they gain; a
     single request with 128k keys wants 32).  Between half the chip's worth of workgroups and all of
     it (17 to 31 requests of 8 key/value heads), where one part leaves compute units idle and two
-    parts are a wave and a bit: one part up to 4k keys (whole decode steps with 2k keys gained
-    nothing from more), beyond that up to 4 parts of at least 2048 keys, the fewest with which the
-    workgroups fill whole waves of 256 about as well as any (20 requests are 160 workgroups: over 8k
-    keys 161 us in one part, 118 in three, the whole step 8.7 against 7.9 ms).  From 256 workgroups on
+    parts are a wave and a bit: one part up to 1k keys, beyond that up to 4 parts of at least 1024
+    keys, the fewest with which the workgroups fill whole waves of 256 about as well as any (20
+    requests are 160 workgroups: over 8k keys 161 us in one part, 118 in three, the whole step 8.7
+    against 7.9 ms; over 2k keys the step of 17 requests 4.64 against 4.39 ms, of 20 requests 4.72
+    against 4.55).  From 256 workgroups on
     one part: the chip is full, and more parts gained nothing (48 requests over 8k keys: 13.1 ms a
     step in one part, 13.2 in two).  The length counts rounded up to a power of two, so that a
     growing context changes the choice, and with it the rounding of the result and the captured

@@ -137,10 +137,13 @@ def test_decode_attention_split_rule():
     from llama_cu_amd.kernels.ops import decode_splits
     assert decode_splits(1, 32, 8, 2100) == 8 and decode_splits(8, 32, 8, 2100) == 4 and decode_splits(16, 32, 8, 2100) == 2
     assert decode_splits(1, 32, 8, 100) == 1 and decode_splits(1, 32, 8, 200000) == 32
-    for b in (20, 24, 40, 48, 64, 128):
-        assert decode_splits(b, 32, 8, 2100) == 1            # up to 4k keys: one part
+    for b in (28, 40, 48, 64, 128):
+        assert decode_splits(b, 32, 8, 2100) == 1            # parts would fill the chip no better, or it is full
+    for b in (20, 24, 28, 64):
+        assert decode_splits(b, 32, 8, 1024) == 1            # up to 1k keys: one part
+    assert decode_splits(17, 32, 8, 2100) == 3 and decode_splits(20, 32, 8, 2100) == 3 and decode_splits(24, 32, 8, 2100) == 4
     assert decode_splits(20, 32, 8, 8192) == 3 and decode_splits(48, 32, 8, 8192) == 1 and decode_splits(64, 32, 8, 8192) == 1
-    assert decode_splits(20, 32, 8, 4097) == 3 and decode_splits(20, 32, 8, 4096) == 1
+    assert decode_splits(20, 32, 8, 4097) == 3 and decode_splits(20, 32, 8, 1025) == 1
 
 
 def test_a_module_of_the_user_s_registers_an_architecture_for_the_command_line(tmp_path):
