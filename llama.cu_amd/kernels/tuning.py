@@ -18,8 +18,9 @@ class Tuning:
     skinny_rows: int = 16               # up to here it beats the library's product with a plain weight ...
     skinny_rows_packed: int = 24        # ... up to here with a packed weight, whose epilogues save the kernels around it
                                         # (whole decode steps: +9 % at 17 rows, +4 % at 24)
-    skinny_rows_short_k: int = 32       # ... and up to here for packed weights with K <= skinny_short_k (q/k/v, output,
-                                        # gate/up: +4.5 % at 28 rows, +2 % at 32; with the down projection too, 2 % slower)
+    skinny_rows_short_k: int = 24       # ... and up to here for packed weights with K <= skinny_short_k (q/k/v, output,
+                                        # gate/up; it was 32 before the row-sharing product spread its tiles over all compute
+                                        # units: now whole steps of 28 requests are 1 % faster and of 32 requests 2.7 % with 24)
     skinny_short_k: int = 8192
     skinny_rows_any_weight: int = 4     # so few rows always go to it
     skinny_small_weight: int = 1 << 24  # without a packed copy, beyond 4 rows only weights up to this many elements
