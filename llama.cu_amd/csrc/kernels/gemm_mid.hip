@@ -55,6 +55,10 @@ __device__ __forceinline__ f32x4 mid_mfma(u32x4 a, u32x4 b, f32x4 c) {
 }
 
 constexpr int mid_producers(int MT) { return (MT + 3) / 4; }
+// Whether the loops run whole turns of their rings without a test of the step (below); beyond 192 rows, where the
+// sums leave few registers, the loops with the test in every step are the faster ones (measured: 55 against 67 us
+// for the down projection at 256 rows)
+constexpr bool mid_whole_turns(int MT) { return MT <= 12; }
 constexpr int mid_lds_bytes(int MT) { return mid_xbufs(MT) * 16 * MT * MID_XROW + 16 * MT * (int)sizeof(float); }
 
 // Producer wave P copies the rows 64 P .. of X, macro-step by macro-step, into the ring in LDS.
@@ -70,6 +74,10 @@ __device__ __forceinline__ void mid_produce(char *xs, const bf16_t *__restrict__
     constexpr int LOADS = ROWS16 * 4;                                     // four rows a load
     constexpr int BUF = 16 * MT * MID_XROW;
     constexpr int XB = mid_xbufs(MT), AHEAD = XB - 1;                     // the copy runs this many macro-steps ahead
+#ifndef LCU_MID_XDEPTH
+#define LCU_MID_XDEPTH 2
+#endif
+    constexpr int D = LOADS <= 8 ? 2 * LCU_MID_XDEPTH : LCU_MID_XDEPTH;   // macro-steps whose loads are on their way (in registers)
     const __amdgpu_buffer_rsrc_t xb = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<bf16_t *>(X + (size_t)128 * s_begin), 0, (uint32_t)(((size_t)(M - 1) * ldx + 128 * nst) * 2), 0x00020000);
     uint32_t src[LOADS];
@@ -80,35 +88,44 @@ __device__ __forceinline__ void mid_produce(char *xs, const bf16_t *__restrict__
         src[i] = tok < M ? (uint32_t)(tok * ldx + 8 * kc) * 2 : 0x80000000u;
         dst[i] = tok * MID_XROW + 16 * kc;
     }
-    u32x4 xr[2][LOADS];
+    u32x4 xr[D][LOADS];
 #define MID_LOAD_X(b, step)                                                                                         \
     _Pragma("unroll") for (int i = 0; i < LOADS; ++i) xr[b][i] =                                                   \
         __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(xb, src[i] + (uint32_t)(step) * 256u, 0, 0))
     // the first AHEAD macro-steps go straight into their buffers
-    MID_LOAD_X(0, 0);
-    if (AHEAD > 1) MID_LOAD_X(1, 1);
+#pragma unroll
+    for (int b = 0; b < AHEAD; ++b) MID_LOAD_X(b, b);
 #pragma unroll
     for (int b = 0; b < AHEAD; ++b)
 #pragma unroll
         for (int i = 0; i < LOADS; ++i) *(u32x4 *)(xs + b * BUF + dst[i]) = xr[b][i];
-    MID_LOAD_X(0, AHEAD);
-    MID_LOAD_X(1, AHEAD + 1);
+#pragma unroll
+    for (int b = 0; b < D; ++b) MID_LOAD_X(b, AHEAD + b);
     lds_barrier();
-    // in iteration s: macro-step s + AHEAD goes into buffer (s + AHEAD) % XB, the loads of s + AHEAD + 2 start
+    // in iteration s: macro-step s + AHEAD goes into buffer (s + AHEAD) % XB, the loads of s + AHEAD + D start.
+    // Whole turns of the registers' ring stand under no test of the step (see the consumers' loop)
     int buf = AHEAD;
-    for (int s = 0; s < nst; s += 2) {
+#define MID_COPY_X(b, cur)                                                                                          \
+    do {                                                                                                            \
+        _Pragma("unroll") for (int i = 0; i < LOADS; ++i) *(u32x4 *)(xs + buf * BUF + dst[i]) = xr[b][i];          \
+        MID_LOAD_X(b, (cur) + AHEAD + D);                                                                           \
+        buf = buf == XB - 1 ? 0 : buf + 1;                                                                          \
+        lds_barrier();                                                                                              \
+    } while (0)
+    int s = 0;
+    if constexpr (mid_whole_turns(MT)) {
+        for (; s + D <= nst; s += D) {
 #pragma unroll
-        for (int b = 0; b < 2; ++b) {
-            const int cur = s + b;
-            if (cur < nst) {
-#pragma unroll
-                for (int i = 0; i < LOADS; ++i) *(u32x4 *)(xs + buf * BUF + dst[i]) = xr[b][i];
-                MID_LOAD_X(b, cur + AHEAD + 2);
-                buf = buf == XB - 1 ? 0 : buf + 1;
-                lds_barrier();
-            }
+            for (int b = 0; b < D; ++b) MID_COPY_X(b, s + b);
         }
     }
+    for (; s < nst; s += D) {                      // what is left of the steps (at most one turn after whole ones)
+#pragma unroll
+        for (int b = 0; b < D; ++b) {
+            if (s + b < nst) MID_COPY_X(b, s + b);
+        }
+    }
+#undef MID_COPY_X
 #undef MID_LOAD_X
 }
 
@@ -221,31 +238,39 @@ gemm_mid_kernel(const bf16_t *__restrict__ X, int ldx, const bf16_t *__restrict_
     const int x_off = l16 * MID_XROW + 64 * grp;     // the lane's operand of row tile 0, instruction 0
     lds_barrier();                                   // macro-steps 0 and 1 of X are in LDS
     int buf = 0;
-    for (int s = 0; s < nst; s += MID_STAGES) {
+#define MID_STEP(i, cur)                                                                                            \
+    do {                                                                                                            \
+        _Pragma("unroll") for (int j = 0; j < 4; ++j) {                                                            \
+            _Pragma("unroll") for (int m0 = 0; m0 < MT; m0 += MCHUNK) {                                            \
+                u32x4 xf[MCHUNK];                                                                                   \
+                _Pragma("unroll") for (int m = 0; m < MCHUNK; ++m)                                                 \
+                    xf[m] = *(const u32x4 *)(xs + buf * BUF + x_off + 16 * (m0 + m) * MID_XROW + 16 * j);          \
+                _Pragma("unroll") for (int t = 0; t < NT; ++t)                                                     \
+                    _Pragma("unroll") for (int m = 0; m < MCHUNK; ++m)                                             \
+                        acc[t][m0 + m] = mid_mfma(w[i][t][j], xf[m], acc[t][m0 + m]);                               \
+            }                                                                                                       \
+        }                                                                                                           \
+        MID_LOAD_W(i, (cur) + MID_STAGES);                                                                          \
+        buf = buf == XB - 1 ? 0 : buf + 1;                                                                          \
+        lds_barrier();                                                                                              \
+    } while (0)
+    // Whole turns of the ring stand under no test of the step: the compiler then counts the loads that a turn has
+    // issued when it waits for the oldest one.  With a test around every step it assumed that none of them had been
+    // issued and waited for ever more of the ring, until at a turn's last step nothing was in flight.
+    int s = 0;
+    if constexpr (mid_whole_turns(MT)) {
+        for (; s + MID_STAGES <= nst; s += MID_STAGES) {
 #pragma unroll
-        for (int i = 0; i < MID_STAGES; ++i) {
-            const int cur = s + i;
-            if (cur < nst) {
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-#pragma unroll
-                    for (int m0 = 0; m0 < MT; m0 += MCHUNK) {
-                        u32x4 xf[MCHUNK];
-#pragma unroll
-                        for (int m = 0; m < MCHUNK; ++m)
-                            xf[m] = *(const u32x4 *)(xs + buf * BUF + x_off + 16 * (m0 + m) * MID_XROW + 16 * j);
-#pragma unroll
-                        for (int t = 0; t < NT; ++t)
-#pragma unroll
-                            for (int m = 0; m < MCHUNK; ++m) acc[t][m0 + m] = mid_mfma(w[i][t][j], xf[m], acc[t][m0 + m]);
-                    }
-                }
-                MID_LOAD_W(i, cur + MID_STAGES);
-                buf = buf == XB - 1 ? 0 : buf + 1;
-                lds_barrier();
-            }
+            for (int i = 0; i < MID_STAGES; ++i) MID_STEP(i, s + i);
         }
     }
+    for (; s < nst; s += MID_STAGES) {             // what is left of the steps (at most one turn after whole ones)
+#pragma unroll
+        for (int i = 0; i < MID_STAGES; ++i) {
+            if (s + i < nst) MID_STEP(i, s + i);
+        }
+    }
+#undef MID_STEP
 #undef MID_LOAD_W
     if (!live) return;
     // ---- epilogue: the lane holds, per tile, features 4 grp + r of token 16 m + l16
@@ -493,27 +518,36 @@ gemm_mid_qkv_kernel(const bf16_t *__restrict__ X, int ldx, const bf16_t *__restr
     const int x_off = l16 * MID_XROW + 64 * grp + 16 * wave;
     lds_barrier();
     int buf = 0;
-    for (int s = 0; s < nst; s += STAGES) {
+#define QKV_STEP(i, cur)                                                                                      \
+    do {                                                                                                      \
+        _Pragma("unroll") for (int m0 = 0; m0 < MT; m0 += MCHUNK) {                                          \
+            u32x4 xf[MCHUNK];                                                                                 \
+            _Pragma("unroll") for (int m = 0; m < MCHUNK; ++m)                                               \
+                xf[m] = *(const u32x4 *)(xs + buf * BUF + x_off + 16 * (m0 + m) * MID_XROW);                 \
+            _Pragma("unroll") for (int t = 0; t < 2; ++t)                                                    \
+                _Pragma("unroll") for (int m = 0; m < MCHUNK; ++m) acc[t][m0 + m] = mid_mfma(w[i][t], xf[m], acc[t][m0 + m]); \
+        }                                                                                                     \
+        QKV_LOAD_W(i, (cur) + STAGES);                                                                        \
+        buf = buf == XB - 1 ? 0 : buf + 1;                                                                    \
+        lds_barrier();                                                                                        \
+    } while (0)
+    // whole turns of the ring stand under no branch: the compiler then counts the loads of a turn that are on their
+    // way when it waits for the oldest (with a test of the step around each, it assumed none of them and let the
+    // ring run empty once a turn)
+    int s = 0;
+    if constexpr (mid_whole_turns(MT)) {
+        for (; s + STAGES <= nst; s += STAGES) {
 #pragma unroll
-        for (int i = 0; i < STAGES; ++i) {
-            const int cur = s + i;
-            if (cur < nst) {
-#pragma unroll
-                for (int m0 = 0; m0 < MT; m0 += MCHUNK) {
-                    u32x4 xf[MCHUNK];
-#pragma unroll
-                    for (int m = 0; m < MCHUNK; ++m) xf[m] = *(const u32x4 *)(xs + buf * BUF + x_off + 16 * (m0 + m) * MID_XROW);
-#pragma unroll
-                    for (int t = 0; t < 2; ++t)
-#pragma unroll
-                        for (int m = 0; m < MCHUNK; ++m) acc[t][m0 + m] = mid_mfma(w[i][t], xf[m], acc[t][m0 + m]);
-                }
-                QKV_LOAD_W(i, cur + STAGES);
-                buf = buf == XB - 1 ? 0 : buf + 1;
-                lds_barrier();
-            }
+            for (int i = 0; i < STAGES; ++i) QKV_STEP(i, s + i);
         }
     }
+    for (; s < nst; s += STAGES) {                 // what is left of the steps (at most one turn after whole ones)
+#pragma unroll
+        for (int i = 0; i < STAGES; ++i) {
+            if (s + i < nst) QKV_STEP(i, s + i);
+        }
+    }
+#undef QKV_STEP
 #undef QKV_LOAD_W
     // every wave has passed the last barrier: nobody reads the ring any more, the producers have ended.
     // The waves' sums: [wave][tile][row tile][lane], 16 bytes each

@@ -36,8 +36,8 @@ class Tuning:
                                         # 0.3 % slower at 11: below, the weight-streaming kernel with the norm in its epilogue)
     mid_swiglu_features: int = 8192     # gate/up with SwiGLU goes to it from this many rows of the weight on,
     mid_swiglu_rows: int = 14           # above this many rows of the batch (whole steps: 2.8 % at 16 rows, nothing at 14, slower below)
-    mid_swiglu_max_rows: int = 128      # ... up to this many (at 128 rows 61 us against the library's 59 with the activation
-                                        # kernel, beyond that the library is ahead: 69 against 63 at 160 rows, 80 against 72 at 256)
+    mid_swiglu_max_rows: int = 192      # ... up to this many (at 160 and 192 rows 57 and 61 us against the library's 62 and 66 with
+                                        # the activation kernel: whole steps 4 and 6 % faster; at 256 rows 78 against 73)
     mid_long_k_max_rows: int = 256      # the products cut over K go to it up to this many rows with a long K (the down
                                         # projection: 42 us against the library's 85 at 160 rows, 55 against 65 at 256)
     mid_short_k_max_rows: int = 192     # ... and up to this many with a shorter one (the output projection: 19 us against 25 to

@@ -76,7 +76,7 @@ class SwiGLU(Part):
                 raise ops.KernelError("feed-forward: rows that wait for their normalisation need the kernel for few rows")
             act = linear_swiglu(h.rows, self.w_gate_up, row_sumsq=h.sumsq, norm_width=h.width, eps=h.eps)
         elif self.dtype == torch.bfloat16 and mid_swiglu_takes(h.shape[0], self.w_gate_up) and ops.mid_supported(h, self.w_gate_up.plain):
-            # 15 to 128 rows (mid_swiglu_max_rows): the rows shared through LDS, the activation in the product's epilogue
+            # 15 to 192 rows (mid_swiglu_max_rows): the rows shared through LDS, the activation in the product's epilogue
             act = linear_swiglu_mid(h, self.w_gate_up)
         elif (self.dtype == torch.bfloat16 and h.shape[0] <= skinny_row_limit(self.w_gate_up)
               and ops.skinny_supported(h, self.w_gate_up.plain, self.dtype)):
