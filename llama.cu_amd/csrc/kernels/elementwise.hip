@@ -191,7 +191,7 @@ static int rmsnorm_w(void *x, const void *delta, const void *w, int w_type, void
     dim3 grid(n), block(d >= 2048 ? 512 : 256);
     if (d % 4 == 0 && d <= NORM_VTHREADS * NORM_ITEMS * 4) {
 #define FAST(T_, TW_) rmsnorm_fast_kernel<T_, TX, TD, TW_, TO><<<grid, dim3(T_), 0, stream>>>((TX *)x, (const TD *)delta, (const TW_ *)w, (TO *)out, d, eps, write_back, planes, plane_stride)
-        const bool few = n <= 128;
+        const bool few = n <= 192;        // (measured with four planes: steps of 160 and 192 rows 2 % faster with 1024 threads, of 256 rows 1 % slower)
         if (w_type == LCU_F32) {
             if (few) FAST(1024, float); else FAST(256, float);
         } else if (w_type == LCU_BF16) {
