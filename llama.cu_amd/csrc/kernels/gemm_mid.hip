@@ -4,13 +4,13 @@
 // piece of X moves twice as many bytes of X as of W and has no registers left to keep loads of W
 // in flight.  Here
 //
-//   * a workgroup is four consumer waves and one producer wave for every 64 rows.  The four
-//     consumers work on the
-//     same k at the same time, each on its own tile of 16 output features (for SwiGLU a gate
-//     tile and the up tile that belongs to it), so one piece of X serves all of them;
+//   * a workgroup is four consumer waves (two for SwiGLU with up to 32 rows) and one producer
+//     wave for every 64 rows.  The consumers work on the same k at the same time, each on its
+//     own tile of 16 output features (for SwiGLU a gate tile and the up tile that belongs to
+//     it), so one piece of X serves all of them;
 //   * the producer wave does nothing but copy X, macro-step (128 k) by macro-step, from memory
 //     (it comes from the L2 cache) into a ring of three buffers in LDS, two macro-steps ahead
-//     (beyond 128 rows three buffers do not fit: two buffers, one macro-step ahead).
+//     (beyond 128 rows two buffers, one macro-step ahead: 256 rows fit twice into the 160 KB).
 //     Its waits for its loads do not touch the consumers' loads: a wave's loads come back in
 //     order, so a consumer that waited for X would wait for every load of W issued before it;
 //   * a consumer keeps the loads of W of several macro-steps in flight (16 registers a tile and step),
@@ -20,6 +20,9 @@
 //     chip streams W: each slice writes its partial sums as float32 to its own plane of the
 //     output, [slice][M][N], and the kernel that follows (residual sum and norm) adds the planes
 //     in a fixed order.  Nothing is added atomically: results do not depend on timing.
+//
+// A second kernel (gemm_mid_qkv_kernel, below) is the q, k, v product with the rotation and the cache write
+// in its epilogue: there the consumer waves share each macro-step of K instead of the features.
 //
 // W is plain rows or packed as gemm_skinny.hip describes it (16 x 128 blocks of 4 KB).  (The reference
 // gives every product to its vendor library, llama.cu/src/op/linear.rs:91-118; at these row counts the
@@ -46,6 +49,9 @@ constexpr int MID_STAGE_TILES = LCU_MID_STAGES;    // tiles of W in flight per w
 #define LCU_MID_CONSUMERS 4
 #endif
 constexpr int MID_CONSUMERS = LCU_MID_CONSUMERS;
+#ifndef LCU_MID_XDEPTH
+#define LCU_MID_XDEPTH 2                      // macro-steps of X that a producer has on their way in registers (twice as many for up to 32 rows)
+#endif
 constexpr int MID_STREAM = 2;                 // the loads of a packed W are non-temporal (read once; see gemm_skinny.hip's stream_load)
 constexpr int MID_XROW = 272;                 // bytes between the rows of X in LDS (256 + 16)
 constexpr int mid_xbufs(int MT) { return MT > 8 ? 2 : 3; }      // buffers of the ring of X (160 KB of LDS: 256 rows fit twice)
@@ -74,9 +80,6 @@ __device__ __forceinline__ void mid_produce(char *xs, const bf16_t *__restrict__
     constexpr int LOADS = ROWS16 * 4;                                     // four rows a load
     constexpr int BUF = 16 * MT * MID_XROW;
     constexpr int XB = mid_xbufs(MT), AHEAD = XB - 1;                     // the copy runs this many macro-steps ahead
-#ifndef LCU_MID_XDEPTH
-#define LCU_MID_XDEPTH 2
-#endif
     constexpr int D = LOADS <= 8 ? 2 * LCU_MID_XDEPTH : LCU_MID_XDEPTH;   // macro-steps whose loads are on their way (in registers)
     const __amdgpu_buffer_rsrc_t xb = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<bf16_t *>(X + (size_t)128 * s_begin), 0, (uint32_t)(((size_t)(M - 1) * ldx + 128 * nst) * 2), 0x00020000);
