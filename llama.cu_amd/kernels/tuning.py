@@ -42,10 +42,10 @@ class Tuning:
                                         # projection: 42 us against the library's 85 at 160 rows, 55 against 65 at 256)
     mid_short_k_max_rows: int = 192     # ... and up to this many with a shorter one (the output projection: 19 us against 25 to
                                         # 28 at 160 to 192 rows, no gain beyond)
-    mid_qkv_rows: int = 64              # q/k/v with the rotation and the cache write in its epilogue goes to it above this
+    mid_qkv_rows: int = 16              # q/k/v with the rotation and the cache write in its epilogue goes to it above this
     mid_qkv_max_rows: int = 128         # many rows and up to this many, with a packed weight (whole decode steps over short
-                                        # contexts: 2.5 % faster at 80 rows, 3.5 % at 128; 1.5 % slower at 64, where the library
-                                        # has a faster kernel, 3 to 4 % slower at 160 to 192, where the ring has two buffers)
+                                        # contexts: 1 to 2 % faster from 20 to 64 rows, 2.5 % at 80, 3.5 % at 128; 1 to 2 % slower at
+                                        # 14 and 16 rows, 3 to 4 % slower at 160 to 192, where the ring has two buffers)
     mid_min_slice_steps: int = 4        # a slice of K keeps at least this many macro-steps of 128
     mid_max_slices: int = 8
     # ---- the library's product of many rows (parts/linear.library_friendly_rows)
