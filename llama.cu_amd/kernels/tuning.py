@@ -46,6 +46,9 @@ class Tuning:
     mid_qkv_max_rows: int = 128         # many rows and up to this many, with a packed weight (whole decode steps over short
                                         # contexts: 1 to 2 % faster from 20 to 64 rows, 2.5 % at 80, 3.5 % at 128; 1 to 2 % slower at
                                         # 14 and 16 rows, 3 to 4 % slower at 160 to 192, where the ring has two buffers)
+    mid_f32_rows: int = 32              # a product with 32-bit output (the output matrix, 1.05 GB) goes to it, uncut, above this many
+    mid_f32_max_rows: int = 64          # rows and up to this many (whole steps 1.3 % faster at 40 rows, 1.9 % at 48, 0.7 % at 64;
+                                        # nothing at 25 to 32)
     mid_min_slice_steps: int = 4        # a slice of K keeps at least this many macro-steps of 128
     mid_max_slices: int = 8
     # ---- the library's product of many rows (parts/linear.library_friendly_rows)

@@ -75,6 +75,8 @@ def linear(x: torch.Tensor, weight: Union[torch.Tensor, Weight], out_dtype: Opti
             return torch.matmul(x, weight.t())
         return torch.matmul(x, weight.t(), out=out)
     if all_bf16 and out_dtype == torch.float32 and not accumulate and out is None and x.shape[0] > ops.skinny_max_rows(packed is not None):
+        if packed is not None and ops.TUNING.mid_f32_rows < x.shape[0] <= ops.TUNING.mid_f32_max_rows and ops.mid_supported(x, weight):
+            return ops.gemm_mid(x, packed, slices=1, packed=True)[0]  # one plane of 32-bit sums: K is not cut
         return torch.mm(x, weight.t(), out_dtype=torch.float32)      # 32-bit accumulation, stored unrounded (logits)
     if ops.skinny_f32_supported(x, weight, out_dtype):
         return ops.gemm_skinny_f32(x, weight, out=out, accumulate=accumulate)

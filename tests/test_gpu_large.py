@@ -182,7 +182,8 @@ def test_steps_of_33_to_64_rows_at_full_layer_sizes(big, dtype, monkeypatch):
         got["r0"][58 + p] = logits[12 + p]
     layers = SHAPE["num_hidden_layers"]
     if dtype == "bfloat16":
-        assert calls["planes"] == 5 * layers and calls["swiglu"] == 3 * layers, calls
+        # (and the output matrix of the steps of 40 and 39 rows, as one plane of 32-bit sums)
+        assert calls["planes"] == 5 * layers + 2 and calls["swiglu"] == 3 * layers, calls
     else:
         assert calls == {"planes": 0, "swiglu": 0}
     common.assert_matches_plain(got, want, dtype, f"8B-sized layers, 33 to 64 rows/{dtype}")
