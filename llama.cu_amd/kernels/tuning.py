@@ -46,6 +46,8 @@ class Tuning:
     mid_qkv_max_rows: int = 128         # many rows and up to this many, with a packed weight (whole decode steps over short
                                         # contexts: 1 to 2 % faster from 20 to 64 rows, 2.5 % at 80, 3.5 % at 128; 1 to 2 % slower at
                                         # 14 and 16 rows, 3 to 4 % slower at 160 to 192, where the ring has two buffers)
+    mid_qkv_one_round_rows: int = 32    # ... beyond this many rows only if its workgroups (one for every 32 rows of the weight) are
+                                        # no more than the compute units
     mid_f32_rows: int = 32              # a product with 32-bit output (the output matrix, 1.05 GB) goes to it, uncut, above this many
     mid_f32_max_rows: int = 64          # rows and up to this many (whole steps 1.3 % faster at 40 rows, 1.9 % at 48, 0.7 % at 64;
                                         # nothing at 25 to 32)

@@ -244,8 +244,14 @@ def mid_qkv_takes(n_rows: int, weight: Union[torch.Tensor, Weight]) -> bool:
     kernel: it replaces the library's product and the rotation kernel after it)."""
     w, packed = _split(weight)
     t = ops.TUNING
-    return (packed is not None and t.mid_qkv_rows < n_rows <= min(ops.MID_MAX_ROWS, t.mid_qkv_max_rows)
-            and w.dim() == 2 and w.shape[1] % 128 == 0)
+    if not (packed is not None and t.mid_qkv_rows < n_rows <= min(ops.MID_MAX_ROWS, t.mid_qkv_max_rows)
+            and w.dim() == 2 and w.shape[1] % 128 == 0):
+        return False
+    # a workgroup takes 32 of the weight's rows over all of K and reads every row of the batch: beyond 32 rows of the
+    # batch that pays only while the workgroups run in one round (the Llama-3-8B shape has 192 of them; with the 384 of
+    # the Llama-2-7B shape and the 320 of the 70B shape, whole steps of 64 and 128 requests were 4 to 8 % slower than
+    # with the library's product, those of 24 requests 3 to 4 % faster)
+    return n_rows <= t.mid_qkv_one_round_rows or w.shape[0] // 32 <= t.compute_units
 
 
 def linear_qkv_rope(h, weight: Union[torch.Tensor, Weight], positions, slots, cos, sin, cache_pages, heads: int,
