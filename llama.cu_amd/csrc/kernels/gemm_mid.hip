@@ -686,3 +686,147 @@ LCU_API int lcu_gemm_mid_bf16_qkv_rope(const void *X, int ldx, const void *W, in
 #endif
 }
 
+#if LCU_MID_CONSUMERS == 4
+// ------------------------------------------------------------------------------------------------
+// The product that ends a branch, with the residual sum and the next norm's weight in its epilogue, as
+// gemm_skinny.hip has it for few rows: residual[M, N] += X W^T (32-bit, in place), h = bfloat16(residual * norm_w),
+// not yet normalised, and sumsq[M][N / 16], each workgroup's share of the rows' sums of squares (whoever multiplies h
+// next applies rsqrt(sum of a row's shares / N + eps) in its epilogue).  A sum of squares over a row needs the whole
+// of K under it, so K is not cut over workgroups: a workgroup takes one tile of 16 output features over all of K, and
+// its four consumer waves share each macro-step as in the q, k, v kernel above.  For products with a short K (the
+// output projection): every workgroup reads all rows of X.
+template <int MT, bool PACKED>
+__global__ void __launch_bounds__((MID_CONSUMERS + mid_producers(MT)) * WAVE)
+gemm_mid_add_norm_kernel(const bf16_t *__restrict__ X, int ldx, const bf16_t *__restrict__ W, int ldw, float *__restrict__ residual,
+                         int ldr, int M, int N, int K, const void *__restrict__ norm_w, int norm_w_type, bf16_t *__restrict__ h_out,
+                         int ldh, float *__restrict__ sumsq_out) {
+    extern __shared__ __attribute__((aligned(16))) char xs[];      // the ring of X; at the end the waves' sums
+    constexpr int BUF = 16 * MT * MID_XROW;
+    constexpr int XB = mid_xbufs(MT);
+    const int lane = threadIdx.x & (WAVE - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
+    const int l16 = lane & 15, grp = lane >> 4;
+    const int nst = K / 128;
+    if (wave == MID_CONSUMERS) {
+        mid_produce<MT, 0>(xs, X, ldx, M, 0, nst, lane);
+        return;
+    }
+    const int tile = blockIdx.x;
+    const __amdgpu_buffer_rsrc_t wb =
+        PACKED ? __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t *>(W + (size_t)tile * nst * 2048), 0, (uint32_t)nst * 4096u, 0x00020000)
+               : __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t *>(W + (size_t)16 * tile * ldw), 0,
+                                                   (uint32_t)(((size_t)15 * ldw + 128 * nst) * 2), 0x00020000);
+    const uint32_t w_lane = PACKED ? (uint32_t)lane * 16u + 1024u * wave : (uint32_t)(l16 * ldw + 32 * grp) * 2u + 16u * wave;
+    constexpr uint32_t w_step = PACKED ? 4096u : 256u;
+    f32x4 acc[MT];
+#pragma unroll
+    for (int m = 0; m < MT; ++m) acc[m] = f32x4{0.f, 0.f, 0.f, 0.f};
+    constexpr int STAGES = 16;                         // macro-steps whose loads of W (1 KB) are in flight
+    u32x4 w[STAGES];
+#define AN_LOAD_W(i, step) \
+    w[i] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(wb, w_lane + (uint32_t)(step) * w_step, 0, PACKED ? MID_STREAM : 0))
+#pragma unroll
+    for (int i = 0; i < STAGES; ++i) AN_LOAD_W(i, i);
+    const int x_off = l16 * MID_XROW + 64 * grp + 16 * wave;
+    lds_barrier();
+    int buf = 0;
+#define AN_STEP(i, cur)                                                                                       \
+    do {                                                                                                      \
+        u32x4 xf[MT];                                                                                         \
+        _Pragma("unroll") for (int m = 0; m < MT; ++m) xf[m] = *(const u32x4 *)(xs + buf * BUF + x_off + 16 * m * MID_XROW); \
+        _Pragma("unroll") for (int m = 0; m < MT; ++m) acc[m] = mid_mfma(w[i], xf[m], acc[m]);                \
+        AN_LOAD_W(i, (cur) + STAGES);                                                                         \
+        buf = buf == XB - 1 ? 0 : buf + 1;                                                                    \
+        lds_barrier();                                                                                        \
+    } while (0)
+    int s = 0;
+    for (; s + STAGES <= nst; s += STAGES) {           // whole turns of the ring under no test of the step (see above)
+#pragma unroll
+        for (int i = 0; i < STAGES; ++i) AN_STEP(i, s + i);
+    }
+    for (; s < nst; s += STAGES) {
+#pragma unroll
+        for (int i = 0; i < STAGES; ++i) {
+            if (s + i < nst) AN_STEP(i, s + i);
+        }
+    }
+#undef AN_STEP
+#undef AN_LOAD_W
+    // the waves' sums: [wave][row tile][lane], 16 bytes each; wave w then holds the row tiles w, w + 4, ..
+    f32x4 *sums = (f32x4 *)xs;
+#pragma unroll
+    for (int m = 0; m < MT; ++m) sums[(wave * MT + m) * WAVE + lane] = acc[m];
+    lds_barrier();
+    const int parts = gridDim.x;
+#pragma unroll
+    for (int mi = 0; mi < (MT + MID_CONSUMERS - 1) / MID_CONSUMERS; ++mi) {
+        const int m = wave + MID_CONSUMERS * mi;
+        if (m >= MT) break;
+        f32x4 sum = sums[(0 * MT + m) * WAVE + lane];
+#pragma unroll
+        for (int v = 1; v < MID_CONSUMERS; ++v) {
+            const f32x4 o = sums[(v * MT + m) * WAVE + lane];
+            sum[0] += o[0]; sum[1] += o[1]; sum[2] += o[2]; sum[3] += o[3];
+        }
+        // the lane holds features n0 .. n0 + 3 of token 16 m + l16
+        const int tok = 16 * m + l16, n0 = 16 * tile + 4 * grp;
+        float ss = 0.f;
+        if (tok < M) {
+            f32x4 *res = (f32x4 *)(residual + (size_t)tok * ldr + n0);
+            f32x4 xn = *res;
+            xn[0] += sum[0]; xn[1] += sum[1]; xn[2] += sum[2]; xn[3] += sum[3];
+            *res = xn;
+            float wn[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                ss += xn[r] * xn[r];
+                wn[r] = norm_w_type == LCU_F32 ? ((const float *)norm_w)[n0 + r] : to_f32(((const bf16_t *)norm_w)[n0 + r]);
+            }
+            uint2 pk = {pack2_bf16(xn[0] * wn[0], xn[1] * wn[1]), pack2_bf16(xn[2] * wn[2], xn[3] * wn[3])};
+            *(uint2 *)(h_out + (size_t)tok * ldh + n0) = pk;
+        }
+        ss += __shfl_xor(ss, 16, WAVE);                // every lane takes part: the others bring zero
+        ss += __shfl_xor(ss, 32, WAVE);
+        if (grp == 0 && tok < M) sumsq_out[(size_t)tok * parts + blockIdx.x] = ss;
+    }
+}
+#endif
+
+// X: [M, K] bfloat16 rows ldx apart, M <= 64, K a multiple of 128; W: [N, K] bfloat16, N a multiple of 16, rows ldw apart or
+// packed.  residual: [M, N] float32 rows ldr apart (a multiple of 4), updated in place; norm_w: [N] float32 or bfloat16
+// (norm_w_type LCU_F32 or LCU_BF16); h_out: [M, N] bfloat16 rows ldh apart (a multiple of 4); sumsq_out: [M][N / 16] float32.
+LCU_API int lcu_gemm_mid_bf16_add_norm(const void *X, int ldx, const void *W, int ldw, float *residual, int ldr, int M, int N, int K,
+                                       const void *norm_w, int norm_w_type, void *h_out, int ldh, float *sumsq_out, int w_packed,
+                                       hipStream_t stream) {
+    if (M <= 0 || N <= 0) return LCU_OK;
+    if (M > 64 || K <= 0 || K % 128 || N % 16 || ldx % 8 || ldx < K || ldr < N || ldr % 4 || ldh < N || ldh % 4 || !residual || !norm_w ||
+        !h_out || !sumsq_out || (norm_w_type != LCU_F32 && norm_w_type != LCU_BF16))
+        return LCU_BAD_ARGUMENT;
+    if (!w_packed && (ldw % 8 || ldw < K)) return LCU_BAD_ARGUMENT;
+    if ((uintptr_t)X % 16 || (uintptr_t)W % 16 || (uintptr_t)residual % 16 || (uintptr_t)h_out % 8) return LCU_BAD_ARGUMENT;
+#if LCU_MID_CONSUMERS == 4
+    const dim3 grid(N / 16);
+#define GO(MT_, P_)                                                                                                          \
+    do {                                                                                                                     \
+        constexpr int lds = mid_xbufs(MT_) * 16 * MT_ * MID_XROW;                                                            \
+        static_assert(lds >= MID_CONSUMERS * MT_ * WAVE * 16 && lds <= 64 * 1024, "the waves' sums lie over the ring");      \
+        gemm_mid_add_norm_kernel<MT_, P_><<<grid, dim3((MID_CONSUMERS + mid_producers(MT_)) * WAVE), lds, stream>>>(         \
+            (const bf16_t *)X, ldx, (const bf16_t *)W, ldw, residual, ldr, M, N, K, norm_w, norm_w_type, (bf16_t *)h_out, ldh, sumsq_out); \
+    } while (0)
+#define GO_MT(MT_)                   \
+    do {                             \
+        if (w_packed) GO(MT_, true); \
+        else GO(MT_, false);         \
+    } while (0)
+    if (M <= 16) GO_MT(1);
+    else if (M <= 32) GO_MT(2);
+    else if (M <= 48) GO_MT(3);
+    else GO_MT(4);
+#undef GO_MT
+#undef GO
+    LCU_LAUNCH_CHECK();
+    return LCU_OK;
+#else
+    return LCU_BAD_ARGUMENT;       // an experimental build with another number of consumer waves has no such kernel
+#endif
+}

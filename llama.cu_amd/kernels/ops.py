@@ -803,6 +803,36 @@ def gemm_skinny_add_norm(x: torch.Tensor, w: torch.Tensor, residual: torch.Tenso
     return h, sumsq
 
 
+MID_ADD_NORM_MAX_ROWS = 64
+
+
+def gemm_mid_add_norm(x: torch.Tensor, w: torch.Tensor, residual: torch.Tensor, norm_weight: torch.Tensor, packed: bool = False):
+    """``gemm_skinny_add_norm`` for up to 64 rows, by the kernel that shares the rows through LDS: ``residual += x @ w.T``
+    (float32, in place); returns ``(h, sumsq)`` with ``h = bfloat16(residual * norm_weight)``, not yet normalised, and
+    ``sumsq [rows, out / 16]``, the workgroups' shares of each row's sum of squares.  A workgroup takes 16 output
+    features over all of K and reads every row: for products with a short K (the output projection)."""
+    _gpu(x, w, residual, norm_weight)
+    _rows(x, "mid x"); _rows(w, "mid w"); _rows(residual, "residual")
+    if packed and not (packable(w) and w.is_contiguous()):
+        raise KernelError("gemm_mid_add_norm: a packed weight is a contiguous result of pack_weight")
+    m, k = x.shape
+    n = w.shape[0]
+    if w.shape[1] != k or m > MID_ADD_NORM_MAX_ROWS or not mid_supported(x, w):
+        raise KernelError(f"gemm_mid_add_norm: x {tuple(x.shape)} {x.dtype} with w {tuple(w.shape)} {w.dtype} is not supported "
+                          f"(at most {MID_ADD_NORM_MAX_ROWS} bfloat16 rows, K a multiple of 128, a multiple of 16 features)")
+    if residual.dtype != torch.float32 or residual.shape != (m, n) or residual.stride(0) % 4 or residual.data_ptr() % 16:
+        raise KernelError(f"gemm_mid_add_norm: the residual must be float32 {(m, n)} with rows a multiple of 4 elements apart")
+    if norm_weight.shape != (n,) or not norm_weight.is_contiguous():
+        raise KernelError(f"gemm_mid_add_norm: the norm's weight must be a contiguous [{n}] tensor")
+    h = torch.empty((m, n), dtype=torch.bfloat16, device=x.device)
+    sumsq = torch.empty((m, n // 16), dtype=torch.float32, device=x.device)
+    lib = build.load("gemm_mid")
+    _check(lib.lcu_gemm_mid_bf16_add_norm(_ptr(x), x.stride(0), _ptr(w), w.stride(0), _ptr(residual), residual.stride(0), m, n, k,
+                                          _ptr(norm_weight), _type(norm_weight, "norm weight"), _ptr(h), h.stride(0), _ptr(sumsq),
+                                          int(packed), _stream()), "gemm_mid_add_norm")
+    return h, sumsq
+
+
 QKV_ROPE_MAX_ROWS = 32
 
 

@@ -48,6 +48,12 @@ class Tuning:
                                         # 14 and 16 rows, 3 to 4 % slower at 160 to 192, where the ring has two buffers)
     mid_qkv_one_round_rows: int = 32    # ... beyond this many rows only if its workgroups (one for every 32 rows of the weight) are
                                         # no more than the compute units
+    mid_add_norm_rows: int = 16         # a product with a short K that ends a branch (the output projection) goes to it with the residual
+    mid_add_norm_max_rows: int = 32     # sum and the next norm's weight in its epilogue above this many rows and up to this many, while
+                                        # its workgroups (one for 16 output features) run in one round: 11.9 us at 17 to 32 rows (the
+                                        # weight-streaming kernel 13.1 to 16.9, planes and the norm kernel 14.2); whole steps 0.3 %
+                                        # faster at 20 rows, 1.7 % at 32; 2 % slower at 16 and at 40 to 48, where the first product
+                                        # of the feed-forward pays more for the rows' factors than the norm kernel cost
     mid_f32_rows: int = 32              # a product with 32-bit output (the output matrix, 1.05 GB) goes to it, uncut, above this many
     mid_f32_max_rows: int = 64          # rows and up to this many (whole steps 1.3 % faster at 40 rows, 1.9 % at 48, 0.7 % at 64;
                                         # nothing at 25 to 32)

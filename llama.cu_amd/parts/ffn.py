@@ -59,8 +59,12 @@ class SwiGLU(Part):
     def takes_scaled_rows(self, n_rows: int) -> bool:
         """Whether ``forward`` could be given ScaledRows of ``n_rows`` rows in the place of
         plain rows: the factor then goes into the first product's epilogue."""
-        return (self.dtype == torch.bfloat16 and n_rows <= min(ops.ADD_NORM_MAX_ROWS, skinny_row_limit(self.w_gate_up))
-                and skinny_takes(n_rows, self.w_gate_up))
+        if self.dtype != torch.bfloat16:
+            return False
+        if n_rows <= min(ops.ADD_NORM_MAX_ROWS, skinny_row_limit(self.w_gate_up)) and skinny_takes(n_rows, self.w_gate_up):
+            return True
+        # more rows: the kernel that shares the rows through LDS applies the factor too
+        return n_rows <= ops.MID_MAX_SCALED_ROWS and mid_swiglu_takes(n_rows, self.w_gate_up)
 
     # forward(..., into=(residual, norm)) may end with the residual sum and that norm's weight
     # in the down projection and return ScaledRows instead of the branch's output

@@ -224,14 +224,30 @@ def skinny_takes(n_rows: int, weight: Union[torch.Tensor, Weight], preferred: bo
     return not preferred or ops.skinny_preferred(n_rows, w.shape[0], w.shape[1], torch.bfloat16, packed is not None)
 
 
+def mid_add_norm_takes(n_rows: int, weight: Union[torch.Tensor, Weight]) -> bool:
+    """Whether the product that ends a branch goes, with the residual sum and the next norm's weight in its epilogue, to
+    the kernel that shares the rows through LDS: a packed weight with a short K (the output projection), 17 to 32 rows,
+    and no more workgroups (one for 16 output features, each reads every row) than compute units."""
+    w, packed = _split(weight)
+    t = ops.TUNING
+    return (packed is not None and t.mid_add_norm_rows < n_rows <= min(ops.MID_ADD_NORM_MAX_ROWS, t.mid_add_norm_max_rows)
+            and w.dim() == 2 and w.shape[1] % 128 == 0 and w.shape[1] <= t.mid_long_k and w.shape[0] % 16 == 0
+            and w.shape[0] // 16 <= t.compute_units)
+
+
 def linear_into_norm(a: torch.Tensor, weight: Union[torch.Tensor, Weight], residual: torch.Tensor, norm_weight: torch.Tensor):
     """``residual += a @ weight.T`` and the rows for the product after the next norm, in one
     kernel: returns ``(rows, sumsq)`` for a ``ScaledRows``, or None if the kernel for it does
     not take these operands (then nothing has been done)."""
+    whole = weight
     weight, packed = _split(weight)
-    if not (a.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and a.shape[0] <= ops.ADD_NORM_MAX_ROWS
-            and residual.dtype == torch.float32 and ops.skinny_supported(a, weight, torch.float32)
+    if not (a.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and residual.dtype == torch.float32
             and norm_weight.dtype in (torch.bfloat16, torch.float32)):
+        return None
+    if mid_add_norm_takes(a.shape[0], whole) and ops.mid_supported(a, weight) and residual.stride(0) % 4 == 0 \
+            and residual.data_ptr() % 16 == 0:
+        return ops.gemm_mid_add_norm(a, packed, residual, norm_weight, packed=True)
+    if not (a.shape[0] <= ops.ADD_NORM_MAX_ROWS and ops.skinny_supported(a, weight, torch.float32)):
         return None
     if packed is not None:
         return ops.gemm_skinny_add_norm(a, packed, residual, norm_weight, packed=True)

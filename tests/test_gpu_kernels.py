@@ -748,6 +748,51 @@ def test_gemm_skinny_residual_sum_and_norm_weight_in_the_epilogue(m, n, k, tiles
     assert torch.equal(sumsq, sumsq2) and torch.equal(h, h2) and torch.equal(res_g, res_g2)
 
 
+@pytest.mark.parametrize("m,n,k,packed,wdtype", [(1, 16, 128, False, "bfloat16"), (16, 304, 256, True, "float32"),
+                                                 (17, 4096, 1024, True, "bfloat16"), (33, 96, 384, False, "float32"),
+                                                 (48, 1008, 2176, True, "bfloat16"), (49, 64, 128, True, "float32"),
+                                                 (64, 608, 640, True, "bfloat16")])
+def test_gemm_mid_residual_sum_and_norm_weight_in_the_epilogue(m, n, k, packed, wdtype):
+    """The same for up to 64 rows, by the kernel that shares the rows through LDS (a workgroup takes 16 output features
+    over all of K, its waves share each 128 k): ``residual += x w^T``, the new rows times the norm's weight, the
+    workgroups' shares of the sums of squares; the product that follows applies the factor.  The residual's and h's other
+    rows and the rows of x beyond the last are poison."""
+    from llama_cu_amd.kernels import ops
+    eps = 1e-5
+    x = rnd(m, k, seed=m + k).to(torch.bfloat16)
+    w = rnd(n, k, seed=n, scale=0.3).to(torch.bfloat16)
+    res = rnd(m, n, seed=3) * 3.0
+    nw = (1.0 + 0.2 * rnd(n, seed=4)).to(DT[wdtype])
+    buf = torch.full((m + 3, k + 8), float("nan"), dtype=torch.bfloat16, device="cuda")
+    buf[:m, :k] = x.cuda()
+    res_buf = torch.full((m + 2, n + 4), float("nan"), device="cuda")
+    res_buf[:m, :n] = res.cuda()
+    res_g = res_buf[:m, :n]
+    wg = ops.pack_weight(w.cuda()) if packed else w.cuda()
+    h, sumsq = ops.gemm_mid_add_norm(buf[:m, :k], wg, res_g, nw.cuda(), packed=packed)
+    new = res.double() + plain.linear(x, w)
+    close(res_g, new, "float32", "residual")
+    assert bool(torch.isnan(res_buf[m:]).all()) and bool(torch.isnan(res_buf[:, n:]).all())
+    assert sumsq.shape == (m, n // 16)
+    close(sumsq.sum(dim=1), (new ** 2).sum(dim=1), "float32", "sums of squares")
+    close(h, new * nw.double()[None, :], "bfloat16", "rows with the norm's weight")
+    n2 = 80
+    w2 = rnd(2 * n2, n, seed=5, scale=0.2).to(torch.bfloat16)
+    normed = plain.rms_norm(new, nw, eps)
+    gu = plain.linear(normed, w2)
+    if n % 128 == 0:                                  # the product that follows, in the same kernel family
+        got = ops.gemm_mid(h, w2.cuda(), swiglu=True, row_sumsq=sumsq, norm_width=n, eps=eps)
+        close(got, plain.swiglu(gu[:, :n2], gu[:, n2:]), "bfloat16", "scaled product with SwiGLU")
+    if m <= 32 and n % 8 == 0:
+        close(ops.gemm_skinny(h, w2.cuda(), row_sumsq=sumsq, norm_width=n, eps=eps), gu, "bfloat16", "scaled product")
+    res_buf2 = torch.full((m + 2, n + 4), float("nan"), device="cuda")
+    res_buf2[:m, :n] = res.cuda()
+    h2, sumsq2 = ops.gemm_mid_add_norm(buf[:m, :k], wg, res_buf2[:m, :n], nw.cuda(), packed=packed)
+    assert torch.equal(sumsq, sumsq2) and torch.equal(h, h2) and torch.equal(res_g, res_buf2[:m, :n])   # no atomics
+    with pytest.raises(ops.KernelError):
+        ops.gemm_mid_add_norm(rnd(65, k).to(torch.bfloat16).cuda(), wg, torch.zeros(65, n).cuda(), nw.cuda(), packed=packed)
+
+
 @pytest.mark.parametrize("m,n,k", [(1, 16, 128), (8, 304, 256), (16, 4096, 1024), (13, 96, 384), (30, 608, 256)])
 def test_gemm_skinny_with_a_packed_weight_equals_the_plain_one_bit_for_bit(m, n, k):
     """``pack_weight`` only changes where the kernel finds its operands, not what it adds in

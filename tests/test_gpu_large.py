@@ -151,19 +151,24 @@ def test_whole_portions_and_decoding_at_full_layer_sizes(big, dtype):
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_steps_of_33_to_64_rows_at_full_layer_sizes(big, dtype, monkeypatch):
-    """Steps of 40 and 39 rows: in bfloat16 the output and down projections leave planes of partial
-    sums to the norm that follows, and gate/up ends in SwiGLU, in the kernel that shares the rows
-    through LDS; in the step of 24 rows gate/up (with the norm's factor in its epilogue) and the down
-    projection go there."""
+    """Steps of 40, 39 and 24 rows: in bfloat16 the down projection, and the output projection of the steps of 40
+    and 39 rows, leave planes of partial sums to the norm that follows; the output projection of the step of 24 rows
+    ends in the residual sum and the second norm's weight, and gate/up, which applies that norm's factor there, ends in
+    SwiGLU: all in the kernel that shares the rows through LDS."""
     from llama_cu_amd.engine.runner import ModelRunner
     from llama_cu_amd.kernels import ops
-    calls = {"planes": 0, "swiglu": 0}
-    real = ops.gemm_mid
+    calls = {"planes": 0, "swiglu": 0, "add_norm": 0}
+    real, real_add_norm = ops.gemm_mid, ops.gemm_mid_add_norm
 
     def counted(*a, **kw):
         calls["swiglu" if kw.get("swiglu") else "planes"] += 1
         return real(*a, **kw)
+
+    def counted_add_norm(*a, **kw):
+        calls["add_norm"] += 1
+        return real_add_norm(*a, **kw)
     monkeypatch.setattr(ops, "gemm_mid", counted)
+    monkeypatch.setattr(ops, "gemm_mid_add_norm", counted_add_norm)
     _, reqs, want = big[dtype]
     runner = runner_for(dtype, max_tokens=512, max_seqs=4)
     r0, r1 = reqs["r0"], reqs["r1"]
@@ -182,10 +187,12 @@ def test_steps_of_33_to_64_rows_at_full_layer_sizes(big, dtype, monkeypatch):
         got["r0"][58 + p] = logits[12 + p]
     layers = SHAPE["num_hidden_layers"]
     if dtype == "bfloat16":
-        # (and the output matrix of the steps of 40 and 39 rows, as one plane of 32-bit sums)
-        assert calls["planes"] == 5 * layers + 2 and calls["swiglu"] == 3 * layers, calls
+        # the down projection of every step leaves planes, the output projection of the steps of 40 and 39 rows too (and
+        # the output matrix of those steps is one plane of 32-bit sums); the output projection of the step of 24 rows ends
+        # in the residual sum and the second norm's weight
+        assert calls == {"planes": 5 * layers + 2, "swiglu": 3 * layers, "add_norm": layers}, calls
     else:
-        assert calls == {"planes": 0, "swiglu": 0}
+        assert calls == {"planes": 0, "swiglu": 0, "add_norm": 0}
     common.assert_matches_plain(got, want, dtype, f"8B-sized layers, 33 to 64 rows/{dtype}")
 
 
