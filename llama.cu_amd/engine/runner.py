@@ -283,6 +283,7 @@ class ModelRunner:
     GRAPH_MAX_TOKENS = 256   # steps that are not all single tokens are captured up to this many tokens (beyond, the
                              # GPU's step takes far longer than the host's launches, and a graph would hold much memory)
     GRAPH_MAX_KINDS = 64     # so many kinds of such steps are kept; the one replayed longest ago goes first
+    SEEN_MAX_KINDS = 4096    # so many kinds of steps are counted on their way to a graph
 
     def run(self, step: StepContext) -> torch.Tensor:
         """The model on the batch.  Small steps are launch-bound (a step of the model is some two hundred to
@@ -314,6 +315,8 @@ class ModelRunner:
         if len(self._step_graphs) > self.GRAPH_MAX_KINDS:
             oldest = min((k for k in self._step_graphs if k != key), key=lambda k: self._last_use.get(k, 0))
             del self._step_graphs[oldest]
+            self._last_use.pop(oldest, None)
+            self._seen.pop(oldest, None)                 # (it is counted anew if it comes again)
         return logits
 
     def _run_captured(self, graphs: Dict[tuple, Any], key: tuple, step: StepContext, replays: Dict[tuple, int]) -> torch.Tensor:
@@ -322,6 +325,9 @@ class ModelRunner:
         self._last_use[key] = self._clock
         entry = graphs.get(key)
         if entry is None:
+            if len(self._seen) > self.SEEN_MAX_KINDS:    # a long-lived engine meets ever new kinds of steps: the counts of
+                self._seen.clear()                       # those that never came a third time are not kept for ever
+                self._last_use = {k: v for k, v in self._last_use.items() if k in self._graphs or k in self._step_graphs}
             self._seen[key] = self._seen.get(key, 0) + 1
             if self._seen[key] <= self.GRAPH_AFTER:
                 return self.model.forward(step, self.caches)
