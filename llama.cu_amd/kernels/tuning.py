@@ -43,9 +43,9 @@ class Tuning:
     mid_short_k_max_rows: int = 192     # ... and up to this many with a shorter one (the output projection: 19 us against 25 to
                                         # 28 at 160 to 192 rows, no gain beyond)
     mid_qkv_rows: int = 16              # q/k/v with the rotation and the cache write in its epilogue goes to it above this
-    mid_qkv_max_rows: int = 128         # many rows and up to this many, with a packed weight (whole decode steps over short
-                                        # contexts: 1 to 2 % faster from 20 to 64 rows, 2.5 % at 80, 3.5 % at 128; 1 to 2 % slower at
-                                        # 14 and 16 rows, 3 to 4 % slower at 160 to 192, where the ring has two buffers)
+    mid_qkv_max_rows: int = 192         # many rows and up to this many, with a packed weight (whole decode steps over short
+                                        # contexts: 1 to 2 % faster from 20 to 64 rows, 2.5 % at 80, 3.5 % at 128, 5 % at 144, even at 160
+                                        # to 192; 1 to 2 % slower at 14 and 16 rows)
     mid_qkv_one_round_rows: int = 32    # ... beyond this many rows only if its workgroups (one for every 32 rows of the weight) are
                                         # no more than the compute units
     mid_add_norm_rows: int = 16         # a product with a short K that ends a branch (the output projection) goes to it with the residual

@@ -244,13 +244,14 @@ def _wide_steps(long_requests, monkeypatch, plan):
 def test_steps_of_129_to_256_rows_at_full_layer_sizes(long_requests, monkeypatch):
     """Steps of 250, 192 (two requests) and 129 rows in bfloat16: the down projection of each, and the output
     projection up to 192 rows, leave planes of partial sums from the kernel that shares the rows through LDS (its
-    ring of two buffers and three or four producer waves), gate/up with SwiGLU goes there up to 192 rows; q/k/v stays
-    with the library."""
+    ring of two buffers and three or four producer waves), gate/up with SwiGLU and q/k/v with the rotation go there
+    up to 192 rows."""
     calls = _wide_steps(long_requests, monkeypatch, [[(0, 0, 250)], [(0, 250, 400), (1, 0, 42)], [(0, 400, 529)]])
     # of the two layers the last one's down projection ends in ordinary rows (the wanted rows are gathered before the
     # final norm): 1 + 0 products in the step of 250 rows, 2 + 1 in each of the others
     # (and gate/up of both layers in the steps of 192 and 129 rows)
-    assert calls == {"planes": 7, "swiglu": 4, "qkv": 0}, calls
+    # (and q/k/v of both layers there)
+    assert calls == {"planes": 7, "swiglu": 4, "qkv": 4}, calls
 
 
 def test_steps_of_65_to_128_rows_at_full_layer_sizes(long_requests, monkeypatch):
