@@ -326,7 +326,7 @@ def write_toy_plugin(folder: str, name: str = "lcu_toy_plugin") -> Tuple[str, di
 
 
 # ----------------------------------------------------------------------------- a sweep of configurations
-def sweep_configuration(seed: int):
+def sweep_configuration(seed: int, lens_max: int = 140):
     """A configuration, a page size and request lengths drawn from ``seed``: the generator of a search for wrong
     logits over some 1,700 seeds.  Among them are the widest and deepest models that tests replay (width up to
     512, three layers), where bfloat16 rounding adds up to the most."""
@@ -345,5 +345,5 @@ def sweep_configuration(seed: int):
                rms_norm_eps=rng.choice([1e-5, 1e-6]), tie_word_embeddings=rng.random() < 0.5,
                rope_interleaved=rng.random() < 0.2)
     page = rng.choice([16, 32, 48, 64, 128])
-    lens = [rng.randrange(1, 140) for _ in range(rng.choice([2, 3, 4]))]
+    lens = [rng.randrange(1, lens_max) for _ in range(rng.choice([2, 3, 4]))]
     return cfg, page, lens

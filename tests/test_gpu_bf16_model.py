@@ -27,6 +27,10 @@ pytestmark = pytest.mark.gpu
 # and the search's first seventeen
 SEEDS = [1129, 1346, 1383, 2038, 2072, 2173, 2269, 6054, 6355, 6579, 5198, 5211, 5263] + list(range(1, 18))
 
+# three of a later search with requests of up to 200 tokens (steps of 129 to 199 rows when a request runs whole), whose
+# largest error lay above the fixed bound by 12 to 36 %: the rounding model's own lies there too
+LONG_SEEDS = [7095, 7168, 7221]
+
 RMS_RATIO = 1.05
 MAX_RATIO = 1.5
 
@@ -47,9 +51,9 @@ def distances(got, unrounded, rounding):
     return rms(e), rms(r), float(np.abs(e).max()), float(np.abs(r).max())
 
 
-@pytest.mark.parametrize("seed", SEEDS)
+@pytest.mark.parametrize("seed", SEEDS + LONG_SEEDS)
 def test_bfloat16_engine_errs_no_more_than_a_model_that_rounds_where_it_may(seed):
-    cfg, page, lens = common.sweep_configuration(seed)
+    cfg, page, lens = common.sweep_configuration(seed, lens_max=200 if seed in LONG_SEEDS else 140)
     folder = common.make_folder(cfg, seed=seed, dtype=torch.bfloat16, std=common.BF16_STD)
     reqs = common.random_requests(cfg["vocab_size"], lens, seed=seed)
     pcfg, w = plain.load_folder(folder)
